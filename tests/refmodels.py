@@ -1,0 +1,154 @@
+"""Hand-built models and expected outputs of the reference's own unit tests, as plain data.
+
+Each model dict has the keys of oracle.cbm_reader.read_cbm. Sources:
+  catboost/libs/model/ut/lib/model_test_helpers.cpp:186-224 (SimpleFloatModel), :305-319
+  (SimpleDeepTreeModel), :321-388 (SimpleAsymmetricModel), :458-490 (MultiValueFloatModel);
+  expected values catboost/libs/model/ut/formula_evaluator_ut.cpp:16-25, 76-146, 284-307.
+"""
+import numpy as np
+
+from oracle import model_builder as mb
+
+# formula_evaluator_ut.cpp:16-25
+DATA = np.array([
+    [0, 0, 0], [3, 0, 0], [0, 1, 0], [3, 1, 0],
+    [0, 0, 1], [3, 0, 1], [0, 1, 1], [3, 1, 1]], dtype=np.float32)
+
+
+def _raw(float_features, tree_splits, tree_sizes, leaf_values, dim=1, scale=1.0, bias=None):
+    starts = np.concatenate([[0], np.cumsum(tree_sizes)[:-1]]).astype(np.int32) if len(tree_sizes) else np.zeros(0, np.int32)
+    return {
+        "approx_dimension": dim,
+        "tree_splits": np.asarray(tree_splits, np.int32),
+        "tree_sizes": np.asarray(tree_sizes, np.int32),
+        "tree_start_offsets": starts,
+        "float_features": float_features, "cat_features": [], "one_hot_features": [],
+        "leaf_values": np.asarray(leaf_values, np.float64), "leaf_weights": np.zeros(0),
+        "step_nodes": np.zeros((0, 2), np.uint16), "node_id_to_leaf_id": np.zeros(0, np.uint32),
+        "scale": scale, "bias": np.zeros(dim) if bias is None else np.asarray(bias, np.float64),
+        "info": {}, "model_part_ids": [], "ctr_feature_count": 0, "text_feature_count": 0,
+        "estimated_feature_count": 0, "embedding_feature_count": 0,
+    }
+
+
+def _ff(index, borders):
+    f = mb.float_feature(index)
+    f["borders"] = np.asarray(borders, np.float32)
+    return f
+
+
+def simple_float_model(tree_count=1, scale=1.0, bias=None):
+    """Feature 0 has 301 borders -298..2 (two buckets), features 1 and 2 one border 0.5; every
+    tree splits on bin features {300, 301, 302}; leaf values leaf * 10^tree."""
+    ffs = [_ff(0, [-298.0 + i for i in range(301)]), _ff(1, [0.5]), _ff(2, [0.5])]
+    splits, sizes, leaves = [], [], []
+    ten = 1.0
+    for _ in range(tree_count):
+        splits += [300, 301, 302]
+        sizes.append(3)
+        leaves += [leaf * ten for leaf in range(8)]
+        ten *= 10.0
+    return _raw(ffs, splits, sizes, leaves, scale=scale, bias=bias)
+
+
+def simple_deep_tree_model(depth=9):
+    ffs = [_ff(i, [0.5]) for i in range(depth)]
+    return _raw(ffs, list(range(depth)), [depth], [float(v) for v in range(1 << depth)])
+
+
+def deep_tree_data(depth=9):
+    n = 1 << depth
+    data = np.zeros((n, depth), np.float32)
+    for s in range(n):
+        for f in range(depth):
+            data[s, f] = (s >> f) & 1
+    return data
+
+
+def multi_value_float_model():
+    ffs = [_ff(0, [0.5]), _ff(1, [0.5])]
+    leaves = [0., 10., 20., 1., 11., 21., 2., 12., 22., 3., 13., 23.]
+    return _raw(ffs, [0, 1], [2], leaves, dim=3)
+
+
+def simple_asymmetric_trees():
+    """The three trees of SimpleAsymmetricModel as builder input."""
+    t0 = mb.split_node(("float", 0, 0.5),
+                       mb.split_node(("float", 1, 0.5), mb.leaf_node(1.0), mb.leaf_node(2.0)),
+                       mb.leaf_node(3.0))
+    t1 = mb.split_node(("float", 2, 0.5), mb.leaf_node(0.0), mb.leaf_node(10.0))
+    t2 = mb.split_node(("float", 0, 0.5),
+                       mb.leaf_node(100.0),
+                       mb.split_node(("float", 1, 0.5), mb.leaf_node(200.0), mb.leaf_node(300.0)))
+    return [mb.float_feature(i) for i in range(3)], [t0, t1, t2]
+
+
+def simple_asymmetric_model():
+    ffs, heads = simple_asymmetric_trees()
+    return mb.build_non_symmetric(ffs, [], 1, heads)
+
+
+# formula_evaluator_ut.cpp:286-299
+ASYMMETRIC_PREDICTIONS = np.array([101., 203., 102., 303., 111., 213., 112., 313.])
+ASYMMETRIC_LEAF_INDEXES = np.array([
+    [1, 0, 0], [0, 0, 1], [2, 0, 0], [0, 0, 2],
+    [1, 1, 0], [0, 1, 1], [2, 1, 0], [0, 1, 2]], dtype=np.uint32)
+
+# golden predictions held by the binding tests of the reference
+NUMERIC_ONLY_ROWS = np.array([[0.1, 0.3, 0.2], [0.5, 1.5, -2.5], [0.7, 6.4, 2.4], [-2.0, -1.0, 6.0]], np.float32)
+# CatBoostModelTest.java:290, 344-347
+NUMERIC_ONLY_EXPECTED = np.array([0.029172098906116373, 0.03547209874741901, 0.008157865240661602,
+                                  0.009992472030400074])
+
+# rust-package/src/model.rs:325-350 (exact equality asserted there)
+RUST_FLOATS = np.array([[-10.0, 5.0, 753.0], [30.0, 1.0, 760.0], [40.0, 0.1, 705.0]], np.float32)
+RUST_CATS = [["north"], ["south"], ["south"]]
+RUST_EXPECTED = np.array([0.9980003729960197, 0.00249414628534181, -0.0013677527881450977])
+
+# rust-package/src/model.rs:422-456 (tolerance 1e-6 there), node-package/bindings/tests/model.ts:51-56
+QUERYWISE_ROWS_TEXT = [
+    "0.257727	0.0215909	0.171299	1	1	1	1	1	0	0	0	0	0	0	0.431373	0.935065	0.0208333	0.070824	1	0	0.313726	1	1	0	0.937724	0	1	0	0	0	0	0.0566038	0	0	1	0.73929	1	0.000505391	0.885819	0.000172727	0	0	0	0	0	0	0.153262	0.578118	0.222098	1",
+    "0.424438	0.164384	0.572649	1	1	0	1	0	0	1	0	0	0	0	0.360784	0.512195	0.0447049	0.0717587	1	1	0.321569	1	1	0	0.941214	0	1	0	0	0	0	0.275362	1	0.209302	1	0.391239	1	0.0143194	0.885819	0.00140996	0	0	0	0	0	0	0.357143	0.883721	0.820312	1",
+    "0.345548	0.248034	0.0853067	1	1	0	1	0	0	1	0	0	0	0	0.6	0.5	0.114292	0.071371	1	0	0.396078	1	1	0	0.939218	0	1	0	0	0	0	0.0384615	0	0	1	0	0	0	0.885819	0.00224069	0	0	0	0	0	0	0.588235	0.444444	0.608696	1",
+    "0.946305	0.139752	0.429885	1	1	1	1	1	0	1	0	0	0	0	0.811765	0.75	0.119755	0.071636	0	1	0.541176	1	1	0	0.993828	0	1	0	0	0	0	0.509804	1	0.000398	1	1.5	1	0.417659	0.885819	0.00117792	0	0	0	0	0	0	0.52962	0.958103	0.885843	1",
+]
+QUERYWISE_EXPECTED = np.array([0.08819508860736715, 0.043193651033534904, -0.0019333444540111586,
+                               0.0836685835428004])
+
+
+def querywise_rows():
+    return np.array([[float(x) for x in row.split("\t")] for row in QUERYWISE_ROWS_TEXT], dtype=np.float32)
+
+
+# CatBoostModelTest.java:122-134
+HASH_KNOWN_ANSWERS = {"foo": -553946371, "bar": 50123586, "baz": 825262476, "\U0001F621": 11426516}
+
+
+def load_iris(golden_dir):
+    """iris.data rows -> (features float32 [150, 4], label index)."""
+    import os
+    names = ["Iris-setosa", "Iris-versicolor", "Iris-virginica"]
+    feats, labels = [], []
+    with open(os.path.join(golden_dir, "iris.data")) as f:
+        for line in f:
+            parts = line.strip().split(",")
+            if len(parts) < 5:
+                continue
+            if parts[-1] not in names:
+                continue  # header row
+            feats.append([float(x) for x in parts[:4]])
+            labels.append(names.index(parts[-1]))
+    return np.asarray(feats, np.float32), np.asarray(labels)
+
+
+def load_boston(golden_dir):
+    import os
+    feats, target = [], []
+    with open(os.path.join(golden_dir, "boston_housing.data")) as f:
+        for line in f:
+            tok = line.split()
+            if not tok:
+                continue
+            feats.append([float(x) for x in tok[:-1]])
+            target.append(float(tok[-1]))
+    return np.asarray(feats, np.float32), np.asarray(target)
