@@ -1,0 +1,89 @@
+// HIP evaluator of a CatBoost tree ensemble on one MI355X (gfx950).
+// Takes the place of the reference's CUDA evaluation context
+// (catboost/libs/model/cuda/evaluator.cuh:20-97: TGPUModelData, TGPUDataInput, TCudaQuantizedData,
+// TGPUCatboostEvaluationContext) and of the host side of TGpuEvaluator
+// (catboost/libs/model/cuda/evaluator.cpp:14-416). No HIP types appear in this header.
+#pragma once
+
+#include "model.h"
+
+#include <memory>
+#include <mutex>
+
+namespace cbamd {
+
+// Where a batch of documents lives. Pointers are device pointers for the *Device calls.
+struct TFeatureBatch {
+    enum ELayout {
+        FlatRows = 0,     // Floats[doc * Stride + FlatIndex]; categorical hashes bit-cast in the same row
+        FlatColumns = 1,  // Floats[FlatIndex * Stride + doc]
+        SplitRows = 2,    // Floats[doc * Stride + Index], Cats[doc * CatStride + Index] (hashed)
+    };
+    ELayout Layout = FlatRows;
+    const float* Floats = nullptr;
+    size_t Stride = 0;
+    const int32_t* Cats = nullptr;
+    size_t CatStride = 0;
+};
+
+struct TKernelTimes {
+    float BinarizeMs = 0.f;
+    float EvalMs = 0.f;
+};
+
+class THipEvaluator {
+public:
+    // Uploads the model tables (model upload of cuda/evaluator.cpp:30-84, re-laid out as SoA).
+    THipEvaluator(const TModelTrees& trees, int deviceId);
+    ~THipEvaluator();
+    THipEvaluator(const THipEvaluator&) = delete;
+    THipEvaluator& operator=(const THipEvaluator&) = delete;
+
+    size_t GetTreeCount() const { return TreeCount; }
+    int GetApproxDimension() const { return ApproxDimension; }
+    uint32_t GetBucketCount() const { return BucketCount; }
+
+    // Bytes of the quantized buffer for docCount documents:
+    // ceil(docCount / 256) blocks x max(1, buckets) x 256 bytes.
+    size_t QuantizedBytes(size_t docCount) const;
+
+    // ---- device-resident data; `stream` is a hipStream_t (nullptr = the evaluator's own stream)
+    void QuantizeDevice(const TFeatureBatch& batch, size_t docCount, uint8_t* bins, void* stream);
+    void EvalQuantizedDevice(const uint8_t* bins, size_t docCount, size_t treeStart, size_t treeEnd,
+                             double* results, void* stream);
+    void LeafIndexesQuantizedDevice(const uint8_t* bins, size_t docCount, size_t treeStart, size_t treeEnd,
+                                    uint32_t* indexes, void* stream);
+    // bins in the reference's layout: blocks of 128 docs, [block][bucket][doc in block]
+    void ExportQuantizedDevice(const uint8_t* bins, size_t docCount, uint8_t* referenceLayout, void* stream);
+    // binarize + evaluate with a scratch bin buffer owned by the evaluator; records kernel times
+    void CalcDevice(const TFeatureBatch& batch, size_t docCount, size_t treeStart, size_t treeEnd,
+                    double* results, void* stream);
+    void Synchronize(void* stream);
+    TKernelTimes LastKernelTimes() const { return LastTimes; }
+
+    // ---- host-resident data: stage -> binarize -> evaluate -> copy back, in document chunks.
+    // rows[doc] points at rowLen floats (FlatRows / SplitRows) or columns[f] at docCount floats.
+    void CalcHostRows(const float* const* rows, size_t rowLen, bool flat, const int32_t* const* catRows,
+                      size_t catRowLen, size_t docCount, size_t treeStart, size_t treeEnd, double* results);
+    void CalcHostColumns(const float* const* columns, size_t columnCount, size_t docCount, size_t treeStart,
+                         size_t treeEnd, double* results);
+    void LeafIndexesHostRows(const float* const* rows, size_t rowLen, bool flat, const int32_t* const* catRows,
+                             size_t catRowLen, size_t docCount, size_t treeStart, size_t treeEnd, uint32_t* indexes);
+    void QuantizeHostRows(const float* const* rows, size_t rowLen, bool flat, const int32_t* const* catRows,
+                          size_t catRowLen, size_t docCount, uint8_t* referenceLayout);
+
+    struct TImpl;
+
+private:
+    std::unique_ptr<TImpl> Impl;
+    size_t TreeCount = 0;
+    int ApproxDimension = 1;
+    uint32_t BucketCount = 0;
+    TKernelTimes LastTimes;
+    std::mutex Lock;  // one batch at a time per evaluator (scratch buffers are shared)
+};
+
+// Number of HIP devices visible; throws TModelError when the runtime reports an error.
+int GetHipDeviceCount();
+
+}  // namespace cbamd

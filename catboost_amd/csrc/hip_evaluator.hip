@@ -1,0 +1,711 @@
+// Host side of the HIP evaluator: model upload, kernel launches, host staging.
+#include "hip_evaluator.h"
+#include "kernels.hip.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <limits>
+#include <string>
+#include <vector>
+
+namespace cbamd {
+
+namespace {
+
+void HipCheck(hipError_t e, const char* what) {
+    if (e != hipSuccess) {
+        throw TModelError(std::string("HIP error in ") + what + ": " + hipGetErrorString(e));
+    }
+}
+#define HIP_CHECK(expr) HipCheck((expr), #expr)
+
+template <typename T>
+class TDeviceVec {
+public:
+    TDeviceVec() = default;
+    ~TDeviceVec() { Reset(); }
+    TDeviceVec(const TDeviceVec&) = delete;
+    TDeviceVec& operator=(const TDeviceVec&) = delete;
+
+    void Reset() {
+        if (Ptr) {
+            (void)hipFree(Ptr);
+            Ptr = nullptr;
+            Cap = 0;
+        }
+    }
+    void Upload(const std::vector<T>& host) {
+        Reserve(std::max<size_t>(host.size(), 1));
+        if (!host.empty()) {
+            HIP_CHECK(hipMemcpy(Ptr, host.data(), host.size() * sizeof(T), hipMemcpyHostToDevice));
+        }
+    }
+    // grow-only
+    void Reserve(size_t count) {
+        if (count > Cap) {
+            Reset();
+            HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&Ptr), count * sizeof(T)));
+            Cap = count;
+        }
+    }
+    T* Get() const { return Ptr; }
+    size_t Capacity() const { return Cap; }
+
+private:
+    T* Ptr = nullptr;
+    size_t Cap = 0;
+};
+
+template <typename T>
+class TPinnedVec {
+public:
+    ~TPinnedVec() { Reset(); }
+    void Reset() {
+        if (Ptr) {
+            (void)hipHostFree(Ptr);
+            Ptr = nullptr;
+            Cap = 0;
+        }
+    }
+    void Reserve(size_t count) {
+        if (count > Cap) {
+            Reset();
+            HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&Ptr), count * sizeof(T), hipHostMallocDefault));
+            Cap = count;
+        }
+    }
+    T* Get() const { return Ptr; }
+
+private:
+    T* Ptr = nullptr;
+    size_t Cap = 0;
+};
+
+struct TBucketTables {
+    std::vector<uint32_t> Src;
+    TDeviceVec<uint32_t> DSrc;
+};
+
+}  // namespace
+
+int GetHipDeviceCount() {
+    int n = 0;
+    const hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) {
+        throw TModelError(std::string("HIP runtime reports no usable device: ") + hipGetErrorString(e));
+    }
+    return n;
+}
+
+struct THipEvaluator::TImpl {
+    int DeviceId = 0;
+    hipStream_t Stream = nullptr;
+    hipEvent_t Ev[3] = {nullptr, nullptr, nullptr};
+    bool Oblivious = true;
+    uint32_t RealBucketCount = 0;  // buckets of the model; the device layout uses max(1, this)
+    uint32_t LayoutBuckets = 1;
+    size_t FlatVectorSize = 0;
+    size_t MinFloatSize = 0;
+    size_t MinCatSize = 0;
+    bool HasCats = false;
+
+    // binarize tables
+    TDeviceVec<uint32_t> BucketSrcFlat, BucketSrcSplit, BucketOffset, BucketFlags, Values;
+    // tree tables
+    TDeviceVec<uint32_t> Splits, TreeStart, TreeSize, FirstLeaf, StepNodes, NodeToLeaf;
+    TDeviceVec<double> Leaves, Bias;
+    double Scale = 1.0;
+    int Dim = 1;
+    std::vector<double> HostBias;
+
+    // scratch (grow-only, guarded by THipEvaluator::Lock)
+    TDeviceVec<uint8_t> ScratchBins;
+    TDeviceVec<float> StageFloats;
+    TDeviceVec<int32_t> StageCats;
+    TDeviceVec<double> StageResults;
+    TDeviceVec<uint32_t> StageIndexes;
+    TDeviceVec<uint8_t> StageExport;
+    TPinnedVec<float> PinnedFloats;
+    TPinnedVec<int32_t> PinnedCats;
+    TPinnedVec<double> PinnedResults;
+    TPinnedVec<uint32_t> PinnedIndexes;
+    TPinnedVec<uint8_t> PinnedExport;
+
+    dev::TBinarizeTables BinarizeTables(bool flat) const {
+        dev::TBinarizeTables t;
+        t.BucketCount = LayoutBuckets;
+        t.BucketSrc = flat ? BucketSrcFlat.Get() : BucketSrcSplit.Get();
+        t.BucketOffset = BucketOffset.Get();
+        t.BucketFlags = BucketFlags.Get();
+        t.Values = Values.Get();
+        return t;
+    }
+    dev::TTreeTables TreeTables() const {
+        dev::TTreeTables t;
+        t.Splits = Splits.Get();
+        t.TreeStart = TreeStart.Get();
+        t.TreeSize = TreeSize.Get();
+        t.FirstLeaf = FirstLeaf.Get();
+        t.StepNodes = StepNodes.Get();
+        t.NodeToLeaf = NodeToLeaf.Get();
+        t.Leaves = Leaves.Get();
+        t.Bias = Bias.Get();
+        t.Scale = Scale;
+        t.Dim = Dim;
+        return t;
+    }
+    hipStream_t Pick(void* stream) const { return stream ? static_cast<hipStream_t>(stream) : Stream; }
+};
+
+THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId)
+    : Impl(new TImpl)
+{
+    const int deviceCount = GetHipDeviceCount();
+    CBAMD_ENSURE(deviceCount > 0, "no HIP device found: the HIP evaluator needs an AMD GPU");
+    CBAMD_ENSURE(deviceId >= 0 && deviceId < deviceCount, "HIP device id out of range");
+    HIP_CHECK(hipSetDevice(deviceId));
+    TImpl& m = *Impl;
+    m.DeviceId = deviceId;
+    HIP_CHECK(hipStreamCreateWithFlags(&m.Stream, hipStreamNonBlocking));
+    for (auto& e : m.Ev) {
+        HIP_CHECK(hipEventCreate(&e));
+    }
+    TreeCount = trees.GetTreeCount();
+    ApproxDimension = trees.ApproxDimension;
+    BucketCount = trees.EffectiveBinFeaturesBucketCount;
+    m.Oblivious = trees.IsOblivious();
+    m.RealBucketCount = BucketCount;
+    m.LayoutBuckets = std::max<uint32_t>(1, BucketCount);
+    m.FlatVectorSize = trees.GetFlatFeatureVectorExpectedSize();
+    m.MinFloatSize = trees.MinimalSufficientFloatFeaturesVectorSize;
+    m.MinCatSize = trees.MinimalSufficientCatFeaturesVectorSize;
+    m.HasCats = trees.UsedCatFeaturesCount > 0;
+    m.Dim = trees.ApproxDimension;
+    m.Scale = trees.Scale;
+    m.HostBias = trees.Bias;
+
+    // ---- binarize tables: one entry per bucket, float buckets first, then one-hot buckets, in
+    // the order of BinarizeFeatures (cpu/quantization.h:366-409, 54-79). Borders are sorted inside
+    // each bucket (the bin is a count, so order does not matter) and NaN borders, which never
+    // compare below anything, are dropped.
+    std::vector<uint32_t> srcFlat, srcSplit, offsets, flags, values;
+    offsets.push_back(0);
+    for (const auto& f : trees.FloatFeatures) {
+        if (!f.UsedInModel()) {
+            continue;
+        }
+        CBAMD_ENSURE(f.FlatIndex >= 0 && f.Index >= 0, "float feature without a position");
+        for (size_t begin = 0; begin < f.Borders.size(); begin += kMaxValuesPerBin) {
+            const size_t end = std::min(begin + kMaxValuesPerBin, f.Borders.size());
+            std::vector<float> b;
+            for (size_t i = begin; i < end; ++i) {
+                if (!std::isnan(f.Borders[i])) {
+                    b.push_back(f.Borders[i]);
+                }
+            }
+            std::sort(b.begin(), b.end());
+            for (float x : b) {
+                uint32_t bits;
+                std::memcpy(&bits, &x, 4);
+                values.push_back(bits);
+            }
+            offsets.push_back(static_cast<uint32_t>(values.size()));
+            srcFlat.push_back(static_cast<uint32_t>(f.FlatIndex));
+            srcSplit.push_back(static_cast<uint32_t>(f.Index));
+            const bool nanToInf = f.HasNans && f.NanValueTreatment == ENanValueTreatment::AsTrue;
+            flags.push_back(nanToInf ? dev::kBucketFlagNanToInf : 0);
+        }
+    }
+    for (const auto& oh : trees.OneHotFeatures) {
+        const TCatFeature* cat = nullptr;
+        for (const auto& c : trees.CatFeatures) {
+            if (c.Index == oh.CatFeatureIndex && c.UsedInModel) {
+                cat = &c;
+            }
+        }
+        CBAMD_ENSURE(cat != nullptr, "one-hot feature refers to an unknown or unused categorical feature");
+        CBAMD_ENSURE(cat->FlatIndex >= 0 && cat->Index >= 0, "categorical feature without a position");
+        for (size_t begin = 0; begin < oh.Values.size(); begin += kMaxValuesPerBin) {
+            const size_t end = std::min(begin + kMaxValuesPerBin, oh.Values.size());
+            for (size_t i = begin; i < end; ++i) {
+                values.push_back(static_cast<uint32_t>(oh.Values[i]));
+            }
+            offsets.push_back(static_cast<uint32_t>(values.size()));
+            srcFlat.push_back(static_cast<uint32_t>(cat->FlatIndex));
+            srcSplit.push_back(static_cast<uint32_t>(cat->Index));
+            flags.push_back(dev::kBucketFlagOneHot);
+        }
+    }
+    CBAMD_ENSURE(srcFlat.size() == BucketCount, "internal error: bucket count mismatch");
+    if (BucketCount == 0) {  // keep the device tables non-empty; the binarize kernel is skipped
+        srcFlat.push_back(0);
+        srcSplit.push_back(0);
+        offsets.push_back(0);
+        flags.push_back(0);
+    }
+    m.BucketSrcFlat.Upload(srcFlat);
+    m.BucketSrcSplit.Upload(srcSplit);
+    m.BucketOffset.Upload(offsets);
+    m.BucketFlags.Upload(flags);
+    m.Values.Upload(values);
+
+    // ---- tree tables
+    std::vector<uint32_t> splits(trees.RepackedBins.size());
+    for (size_t i = 0; i < splits.size(); ++i) {
+        const auto& rb = trees.RepackedBins[i];
+        CBAMD_ENSURE(rb.FeatureIndex < m.LayoutBuckets, "internal error: split refers to a missing bucket");
+        splits[i] = static_cast<uint32_t>(rb.FeatureIndex) | (static_cast<uint32_t>(rb.XorMask) << 16) |
+                    (static_cast<uint32_t>(rb.SplitIdx) << 24);
+    }
+    std::vector<uint32_t> treeStart(trees.TreeStartOffsets.begin(), trees.TreeStartOffsets.end());
+    std::vector<uint32_t> treeSize(trees.TreeSizes.begin(), trees.TreeSizes.end());
+    std::vector<uint32_t> firstLeaf(trees.TreeFirstLeafOffsets.size());
+    for (size_t t = 0; t < firstLeaf.size(); ++t) {
+        CBAMD_ENSURE(trees.TreeFirstLeafOffsets[t] <= std::numeric_limits<uint32_t>::max(), "model has too many leaf values");
+        firstLeaf[t] = static_cast<uint32_t>(trees.TreeFirstLeafOffsets[t]);
+    }
+    std::vector<uint32_t> steps(trees.NonSymmetricStepNodes.size());
+    for (size_t i = 0; i < steps.size(); ++i) {
+        steps[i] = static_cast<uint32_t>(trees.NonSymmetricStepNodes[i].LeftSubtreeDiff) |
+                   (static_cast<uint32_t>(trees.NonSymmetricStepNodes[i].RightSubtreeDiff) << 16);
+    }
+    m.Splits.Upload(splits);
+    m.TreeStart.Upload(treeStart);
+    m.TreeSize.Upload(treeSize);
+    m.FirstLeaf.Upload(firstLeaf);
+    m.StepNodes.Upload(steps);
+    m.NodeToLeaf.Upload(trees.NonSymmetricNodeIdToLeafId);
+    m.Leaves.Upload(trees.LeafValues);
+    m.Bias.Upload(trees.Bias);
+}
+
+THipEvaluator::~THipEvaluator() {
+    if (Impl) {
+        (void)hipSetDevice(Impl->DeviceId);
+        if (Impl->Stream) {
+            (void)hipStreamSynchronize(Impl->Stream);
+        }
+        for (auto& e : Impl->Ev) {
+            if (e) {
+                (void)hipEventDestroy(e);
+            }
+        }
+        if (Impl->Stream) {
+            (void)hipStreamDestroy(Impl->Stream);
+        }
+    }
+}
+
+size_t THipEvaluator::QuantizedBytes(size_t docCount) const {
+    const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
+    return std::max<size_t>(blocks, 1) * Impl->LayoutBuckets * dev::kDocsPerBlock;
+}
+
+void THipEvaluator::Synchronize(void* stream) {
+    HIP_CHECK(hipStreamSynchronize(Impl->Pick(stream)));
+}
+
+void THipEvaluator::QuantizeDevice(const TFeatureBatch& batch, size_t docCount, uint8_t* bins, void* stream) {
+    TImpl& m = *Impl;
+    if (docCount == 0) {
+        return;
+    }
+    hipStream_t s = m.Pick(stream);
+    const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
+    CBAMD_ENSURE(blocks <= 0x7fffffffu, "too many documents in one batch");
+    if (m.RealBucketCount == 0) {
+        HIP_CHECK(hipMemsetAsync(bins, 0, QuantizedBytes(docCount), s));
+        return;
+    }
+    CBAMD_ENSURE(bins != nullptr, "quantized buffer is null");
+    CBAMD_ENSURE(batch.Floats != nullptr || (batch.Layout == TFeatureBatch::SplitRows && m.MinFloatSize == 0),
+                 "float features pointer is null");
+    switch (batch.Layout) {
+        case TFeatureBatch::FlatRows: {
+            CBAMD_ENSURE(batch.Stride >= m.FlatVectorSize, "insufficient flat features vector size: " +
+                                                                std::to_string(batch.Stride) + " expected: " +
+                                                                std::to_string(m.FlatVectorSize));
+            const dim3 grid(static_cast<uint32_t>(blocks), (m.LayoutBuckets + dev::kBucketTile - 1) / dev::kBucketTile);
+            hipLaunchKernelGGL(dev::BinarizeRowsKernel, grid, dim3(256), 0, s, batch.Floats, batch.Stride, nullptr,
+                               size_t(0), docCount, m.BinarizeTables(true), reinterpret_cast<uint32_t*>(bins));
+            break;
+        }
+        case TFeatureBatch::SplitRows: {
+            CBAMD_ENSURE(batch.Stride >= m.MinFloatSize, "insufficient float features vector size: " +
+                                                             std::to_string(batch.Stride) + " expected: " +
+                                                             std::to_string(m.MinFloatSize));
+            if (m.HasCats) {
+                CBAMD_ENSURE(batch.Cats != nullptr, "Model has categorical features but no categorical features provided");
+                CBAMD_ENSURE(batch.CatStride >= m.MinCatSize, "insufficient cat features vector size: " +
+                                                                  std::to_string(batch.CatStride) + " expected: " +
+                                                                  std::to_string(m.MinCatSize));
+            }
+            const dim3 grid(static_cast<uint32_t>(blocks), (m.LayoutBuckets + dev::kBucketTile - 1) / dev::kBucketTile);
+            // a model with one-hot buckets always reads them from the categorical matrix here
+            hipLaunchKernelGGL(dev::BinarizeRowsKernel, grid, dim3(256), 0, s, batch.Floats, batch.Stride,
+                               m.HasCats ? batch.Cats : nullptr, batch.CatStride, docCount, m.BinarizeTables(false),
+                               reinterpret_cast<uint32_t*>(bins));
+            break;
+        }
+        case TFeatureBatch::FlatColumns: {
+            CBAMD_ENSURE(batch.Stride >= docCount, "column stride is shorter than the document count");
+            const dim3 grid(static_cast<uint32_t>(blocks), (m.LayoutBuckets + 3) / 4);
+            hipLaunchKernelGGL(dev::BinarizeColumnsKernel, grid, dim3(256), 0, s, batch.Floats, batch.Stride, docCount,
+                               m.BinarizeTables(true), reinterpret_cast<uint32_t*>(bins));
+            break;
+        }
+        default:
+            CBAMD_ENSURE(false, "unknown feature layout");
+    }
+    HIP_CHECK(hipGetLastError());
+}
+
+namespace {
+
+template <int DCHUNK>
+void LaunchEval(bool oblivious, const uint8_t* bins, size_t docCount, uint32_t buckets, const dev::TTreeTables& tt,
+                uint32_t treeBegin, uint32_t treeEnd, double* out, hipStream_t s) {
+    const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
+    if (oblivious) {
+        const uint32_t grid = static_cast<uint32_t>((blocks + 3) / 4);
+        hipLaunchKernelGGL(dev::EvalObliviousKernel<DCHUNK>, dim3(grid), dim3(256), 0, s,
+                           reinterpret_cast<const uint32_t*>(bins), docCount, buckets, tt, treeBegin, treeEnd, out);
+    } else {
+        hipLaunchKernelGGL(dev::EvalNonSymmetricKernel<DCHUNK>, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, s,
+                           bins, docCount, buckets, tt, treeBegin, treeEnd, out);
+    }
+}
+
+}  // namespace
+
+void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, size_t treeStart, size_t treeEnd,
+                                        double* results, void* stream) {
+    TImpl& m = *Impl;
+    if (docCount == 0) {
+        return;
+    }
+    hipStream_t s = m.Pick(stream);
+    CBAMD_ENSURE(results != nullptr, "results pointer is null");
+    if (TreeCount == 0) {
+        // a model without trees answers with its bias (cpu/formula_evaluator.cpp:29-41)
+        const size_t count = docCount * m.Dim;
+        hipLaunchKernelGGL(dev::FillBiasKernel, dim3(static_cast<uint32_t>((count + 255) / 256)), dim3(256), 0, s, results,
+                           count, m.Bias.Get(), m.Dim);
+        HIP_CHECK(hipGetLastError());
+        return;
+    }
+    CBAMD_ENSURE(treeStart <= treeEnd && treeEnd <= TreeCount, "tree range is out of bounds");
+    CBAMD_ENSURE(bins != nullptr, "quantized buffer is null");
+    const dev::TTreeTables tt = m.TreeTables();
+    const uint32_t tb = static_cast<uint32_t>(treeStart), te = static_cast<uint32_t>(treeEnd);
+    if (m.Dim == 1) {
+        LaunchEval<1>(m.Oblivious, bins, docCount, m.LayoutBuckets, tt, tb, te, results, s);
+    } else if (m.Dim == 2) {
+        LaunchEval<2>(m.Oblivious, bins, docCount, m.LayoutBuckets, tt, tb, te, results, s);
+    } else if (m.Dim <= 4) {
+        LaunchEval<4>(m.Oblivious, bins, docCount, m.LayoutBuckets, tt, tb, te, results, s);
+    } else if (m.Dim <= 8) {
+        LaunchEval<8>(m.Oblivious, bins, docCount, m.LayoutBuckets, tt, tb, te, results, s);
+    } else {
+        LaunchEval<16>(m.Oblivious, bins, docCount, m.LayoutBuckets, tt, tb, te, results, s);
+    }
+    HIP_CHECK(hipGetLastError());
+}
+
+void THipEvaluator::LeafIndexesQuantizedDevice(const uint8_t* bins, size_t docCount, size_t treeStart, size_t treeEnd,
+                                               uint32_t* indexes, void* stream) {
+    TImpl& m = *Impl;
+    CBAMD_ENSURE(treeStart <= treeEnd && treeEnd <= TreeCount, "tree range is out of bounds");
+    if (docCount == 0 || treeStart == treeEnd) {
+        return;
+    }
+    CBAMD_ENSURE(bins != nullptr && indexes != nullptr, "null pointer passed to leaf index calculation");
+    hipStream_t s = m.Pick(stream);
+    const size_t blocks = (docCount + 255) / 256;
+    hipLaunchKernelGGL(dev::LeafIndexesKernel, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, s, bins, docCount,
+                       m.LayoutBuckets, m.TreeTables(), m.Oblivious ? 1 : 0, static_cast<uint32_t>(treeStart),
+                       static_cast<uint32_t>(treeEnd), indexes);
+    HIP_CHECK(hipGetLastError());
+}
+
+void THipEvaluator::ExportQuantizedDevice(const uint8_t* bins, size_t docCount, uint8_t* referenceLayout, void* stream) {
+    TImpl& m = *Impl;
+    if (docCount == 0 || m.RealBucketCount == 0) {
+        return;
+    }
+    hipStream_t s = m.Pick(stream);
+    hipLaunchKernelGGL(dev::ExportBinsKernel, dim3(static_cast<uint32_t>((docCount + 255) / 256)), dim3(256), 0, s, bins,
+                       docCount, m.LayoutBuckets, referenceLayout);
+    HIP_CHECK(hipGetLastError());
+}
+
+void THipEvaluator::CalcDevice(const TFeatureBatch& batch, size_t docCount, size_t treeStart, size_t treeEnd,
+                               double* results, void* stream) {
+    std::lock_guard<std::mutex> guard(Lock);
+    TImpl& m = *Impl;
+    HIP_CHECK(hipSetDevice(m.DeviceId));
+    hipStream_t s = m.Pick(stream);
+    m.ScratchBins.Reserve(QuantizedBytes(docCount));
+    HIP_CHECK(hipEventRecord(m.Ev[0], s));
+    QuantizeDevice(batch, docCount, m.ScratchBins.Get(), s);
+    HIP_CHECK(hipEventRecord(m.Ev[1], s));
+    EvalQuantizedDevice(m.ScratchBins.Get(), docCount, treeStart, treeEnd, results, s);
+    HIP_CHECK(hipEventRecord(m.Ev[2], s));
+    HIP_CHECK(hipStreamSynchronize(s));
+    HIP_CHECK(hipEventElapsedTime(&LastTimes.BinarizeMs, m.Ev[0], m.Ev[1]));
+    HIP_CHECK(hipEventElapsedTime(&LastTimes.EvalMs, m.Ev[1], m.Ev[2]));
+}
+
+// ---------------------------------------------------------------------------- host staging ----
+
+namespace {
+
+// documents staged per round trip; bounds pinned and device staging memory
+size_t ChunkDocs(size_t rowFloats, size_t rowCats) {
+    const size_t bytesPerDoc = std::max<size_t>(1, (rowFloats + rowCats) * 4);
+    const size_t budget = size_t(512) << 20;
+    size_t docs = budget / bytesPerDoc;
+    docs = std::max<size_t>(docs, 1024);
+    docs = std::min<size_t>(docs, size_t(1) << 22);
+    return docs / dev::kDocsPerBlock * dev::kDocsPerBlock;
+}
+
+}  // namespace
+
+void THipEvaluator::CalcHostRows(const float* const* rows, size_t rowLen, bool flat, const int32_t* const* catRows,
+                                 size_t catRowLen, size_t docCount, size_t treeStart, size_t treeEnd, double* results) {
+    std::lock_guard<std::mutex> guard(Lock);
+    TImpl& m = *Impl;
+    HIP_CHECK(hipSetDevice(m.DeviceId));
+    hipStream_t s = m.Stream;
+    // only the columns the model can address are staged
+    const size_t needFloats = flat ? m.FlatVectorSize : m.MinFloatSize;
+    const size_t needCats = (!flat && m.HasCats) ? m.MinCatSize : 0;
+    CBAMD_ENSURE(needFloats == 0 || rows != nullptr, "Model has float features but no float features provided");
+    CBAMD_ENSURE(rowLen >= needFloats, (flat ? "insufficient flat features vector size: " : "insufficient float features vector size: ") +
+                                           std::to_string(rowLen) + " expected: " + std::to_string(needFloats));
+    CBAMD_ENSURE(needCats == 0 || catRows != nullptr, "Model has categorical features but no categorical features provided");
+    CBAMD_ENSURE(catRowLen >= needCats, "insufficient cat features vector size: " + std::to_string(catRowLen) +
+                                            " expected: " + std::to_string(needCats));
+    const size_t chunk = ChunkDocs(needFloats, needCats);
+    const size_t stageDocs = std::min(chunk, docCount);
+    m.PinnedFloats.Reserve(std::max<size_t>(1, stageDocs * needFloats));
+    m.StageFloats.Reserve(std::max<size_t>(1, stageDocs * needFloats));
+    if (needCats) {
+        m.PinnedCats.Reserve(stageDocs * needCats);
+        m.StageCats.Reserve(stageDocs * needCats);
+    }
+    m.PinnedResults.Reserve(std::max<size_t>(1, stageDocs * m.Dim));
+    m.StageResults.Reserve(std::max<size_t>(1, stageDocs * m.Dim));
+    m.ScratchBins.Reserve(QuantizedBytes(stageDocs));
+    LastTimes = TKernelTimes();
+    for (size_t begin = 0; begin < docCount; begin += chunk) {
+        const size_t n = std::min(chunk, docCount - begin);
+        if (needFloats) {
+            float* dst = m.PinnedFloats.Get();
+            for (size_t d = 0; d < n; ++d) {
+                std::memcpy(dst + d * needFloats, rows[begin + d], needFloats * sizeof(float));
+            }
+            HIP_CHECK(hipMemcpyAsync(m.StageFloats.Get(), dst, n * needFloats * sizeof(float), hipMemcpyHostToDevice, s));
+        }
+        if (needCats) {
+            int32_t* dst = m.PinnedCats.Get();
+            for (size_t d = 0; d < n; ++d) {
+                std::memcpy(dst + d * needCats, catRows[begin + d], needCats * sizeof(int32_t));
+            }
+            HIP_CHECK(hipMemcpyAsync(m.StageCats.Get(), dst, n * needCats * sizeof(int32_t), hipMemcpyHostToDevice, s));
+        }
+        TFeatureBatch batch;
+        batch.Layout = flat ? TFeatureBatch::FlatRows : TFeatureBatch::SplitRows;
+        batch.Floats = m.StageFloats.Get();
+        batch.Stride = needFloats;
+        batch.Cats = needCats ? m.StageCats.Get() : nullptr;
+        batch.CatStride = needCats;
+        HIP_CHECK(hipEventRecord(m.Ev[0], s));
+        QuantizeDevice(batch, n, m.ScratchBins.Get(), s);
+        HIP_CHECK(hipEventRecord(m.Ev[1], s));
+        EvalQuantizedDevice(m.ScratchBins.Get(), n, treeStart, treeEnd, m.StageResults.Get(), s);
+        HIP_CHECK(hipEventRecord(m.Ev[2], s));
+        HIP_CHECK(hipMemcpyAsync(m.PinnedResults.Get(), m.StageResults.Get(), n * m.Dim * sizeof(double),
+                                 hipMemcpyDeviceToHost, s));
+        HIP_CHECK(hipStreamSynchronize(s));
+        std::memcpy(results + begin * m.Dim, m.PinnedResults.Get(), n * m.Dim * sizeof(double));
+        float a = 0.f, b = 0.f;
+        HIP_CHECK(hipEventElapsedTime(&a, m.Ev[0], m.Ev[1]));
+        HIP_CHECK(hipEventElapsedTime(&b, m.Ev[1], m.Ev[2]));
+        LastTimes.BinarizeMs += a;
+        LastTimes.EvalMs += b;
+    }
+}
+
+void THipEvaluator::CalcHostColumns(const float* const* columns, size_t columnCount, size_t docCount, size_t treeStart,
+                                    size_t treeEnd, double* results) {
+    std::lock_guard<std::mutex> guard(Lock);
+    TImpl& m = *Impl;
+    HIP_CHECK(hipSetDevice(m.DeviceId));
+    hipStream_t s = m.Stream;
+    const size_t need = m.FlatVectorSize;
+    CBAMD_ENSURE(columnCount >= need, "Not enough features provided");
+    CBAMD_ENSURE(need == 0 || columns != nullptr, "Not enough features provided");
+    const size_t chunk = ChunkDocs(need, 0);
+    const size_t stageDocs = std::min(chunk, docCount);
+    m.PinnedFloats.Reserve(std::max<size_t>(1, stageDocs * need));
+    m.StageFloats.Reserve(std::max<size_t>(1, stageDocs * need));
+    m.PinnedResults.Reserve(std::max<size_t>(1, stageDocs * m.Dim));
+    m.StageResults.Reserve(std::max<size_t>(1, stageDocs * m.Dim));
+    m.ScratchBins.Reserve(QuantizedBytes(stageDocs));
+    LastTimes = TKernelTimes();
+    for (size_t begin = 0; begin < docCount; begin += chunk) {
+        const size_t n = std::min(chunk, docCount - begin);
+        float* dst = m.PinnedFloats.Get();
+        for (size_t f = 0; f < need; ++f) {
+            if (columns[f] != nullptr) {
+                std::memcpy(dst + f * n, columns[f] + begin, n * sizeof(float));
+            } else {
+                std::memset(dst + f * n, 0, n * sizeof(float));
+            }
+        }
+        if (need) {
+            HIP_CHECK(hipMemcpyAsync(m.StageFloats.Get(), dst, n * need * sizeof(float), hipMemcpyHostToDevice, s));
+        }
+        TFeatureBatch batch;
+        batch.Layout = TFeatureBatch::FlatColumns;
+        batch.Floats = m.StageFloats.Get();
+        batch.Stride = n;
+        HIP_CHECK(hipEventRecord(m.Ev[0], s));
+        QuantizeDevice(batch, n, m.ScratchBins.Get(), s);
+        HIP_CHECK(hipEventRecord(m.Ev[1], s));
+        EvalQuantizedDevice(m.ScratchBins.Get(), n, treeStart, treeEnd, m.StageResults.Get(), s);
+        HIP_CHECK(hipEventRecord(m.Ev[2], s));
+        HIP_CHECK(hipMemcpyAsync(m.PinnedResults.Get(), m.StageResults.Get(), n * m.Dim * sizeof(double),
+                                 hipMemcpyDeviceToHost, s));
+        HIP_CHECK(hipStreamSynchronize(s));
+        std::memcpy(results + begin * m.Dim, m.PinnedResults.Get(), n * m.Dim * sizeof(double));
+        float a = 0.f, b = 0.f;
+        HIP_CHECK(hipEventElapsedTime(&a, m.Ev[0], m.Ev[1]));
+        HIP_CHECK(hipEventElapsedTime(&b, m.Ev[1], m.Ev[2]));
+        LastTimes.BinarizeMs += a;
+        LastTimes.EvalMs += b;
+    }
+}
+
+void THipEvaluator::LeafIndexesHostRows(const float* const* rows, size_t rowLen, bool flat,
+                                        const int32_t* const* catRows, size_t catRowLen, size_t docCount,
+                                        size_t treeStart, size_t treeEnd, uint32_t* indexes) {
+    std::lock_guard<std::mutex> guard(Lock);
+    TImpl& m = *Impl;
+    HIP_CHECK(hipSetDevice(m.DeviceId));
+    hipStream_t s = m.Stream;
+    CBAMD_ENSURE(treeStart <= treeEnd && treeEnd <= TreeCount, "tree range is out of bounds");
+    const size_t treeCount = treeEnd - treeStart;
+    const size_t needFloats = flat ? m.FlatVectorSize : m.MinFloatSize;
+    const size_t needCats = (!flat && m.HasCats) ? m.MinCatSize : 0;
+    CBAMD_ENSURE(needFloats == 0 || rows != nullptr, "Model has float features but no float features provided");
+    CBAMD_ENSURE(rowLen >= needFloats, "insufficient float features vector size: " + std::to_string(rowLen) +
+                                           " expected: " + std::to_string(needFloats));
+    CBAMD_ENSURE(needCats == 0 || catRows != nullptr, "Model has categorical features but no categorical features provided");
+    CBAMD_ENSURE(catRowLen >= needCats, "insufficient cat features vector size");
+    size_t chunk = ChunkDocs(needFloats + treeCount, needCats);
+    const size_t stageDocs = std::min(chunk, docCount);
+    m.PinnedFloats.Reserve(std::max<size_t>(1, stageDocs * needFloats));
+    m.StageFloats.Reserve(std::max<size_t>(1, stageDocs * needFloats));
+    if (needCats) {
+        m.PinnedCats.Reserve(stageDocs * needCats);
+        m.StageCats.Reserve(stageDocs * needCats);
+    }
+    m.PinnedIndexes.Reserve(std::max<size_t>(1, stageDocs * treeCount));
+    m.StageIndexes.Reserve(std::max<size_t>(1, stageDocs * treeCount));
+    m.ScratchBins.Reserve(QuantizedBytes(stageDocs));
+    for (size_t begin = 0; begin < docCount; begin += chunk) {
+        const size_t n = std::min(chunk, docCount - begin);
+        if (needFloats) {
+            float* dst = m.PinnedFloats.Get();
+            for (size_t d = 0; d < n; ++d) {
+                std::memcpy(dst + d * needFloats, rows[begin + d], needFloats * sizeof(float));
+            }
+            HIP_CHECK(hipMemcpyAsync(m.StageFloats.Get(), dst, n * needFloats * sizeof(float), hipMemcpyHostToDevice, s));
+        }
+        if (needCats) {
+            int32_t* dst = m.PinnedCats.Get();
+            for (size_t d = 0; d < n; ++d) {
+                std::memcpy(dst + d * needCats, catRows[begin + d], needCats * sizeof(int32_t));
+            }
+            HIP_CHECK(hipMemcpyAsync(m.StageCats.Get(), dst, n * needCats * sizeof(int32_t), hipMemcpyHostToDevice, s));
+        }
+        TFeatureBatch batch;
+        batch.Layout = flat ? TFeatureBatch::FlatRows : TFeatureBatch::SplitRows;
+        batch.Floats = m.StageFloats.Get();
+        batch.Stride = needFloats;
+        batch.Cats = needCats ? m.StageCats.Get() : nullptr;
+        batch.CatStride = needCats;
+        QuantizeDevice(batch, n, m.ScratchBins.Get(), s);
+        LeafIndexesQuantizedDevice(m.ScratchBins.Get(), n, treeStart, treeEnd, m.StageIndexes.Get(), s);
+        if (treeCount) {
+            HIP_CHECK(hipMemcpyAsync(m.PinnedIndexes.Get(), m.StageIndexes.Get(), n * treeCount * sizeof(uint32_t),
+                                     hipMemcpyDeviceToHost, s));
+        }
+        HIP_CHECK(hipStreamSynchronize(s));
+        std::memcpy(indexes + begin * treeCount, m.PinnedIndexes.Get(), n * treeCount * sizeof(uint32_t));
+    }
+}
+
+void THipEvaluator::QuantizeHostRows(const float* const* rows, size_t rowLen, bool flat, const int32_t* const* catRows,
+                                     size_t catRowLen, size_t docCount, uint8_t* referenceLayout) {
+    std::lock_guard<std::mutex> guard(Lock);
+    TImpl& m = *Impl;
+    HIP_CHECK(hipSetDevice(m.DeviceId));
+    hipStream_t s = m.Stream;
+    const size_t needFloats = flat ? m.FlatVectorSize : m.MinFloatSize;
+    const size_t needCats = (!flat && m.HasCats) ? m.MinCatSize : 0;
+    CBAMD_ENSURE(needFloats == 0 || rows != nullptr, "Model has float features but no float features provided");
+    CBAMD_ENSURE(rowLen >= needFloats, "insufficient float features vector size: " + std::to_string(rowLen) +
+                                           " expected: " + std::to_string(needFloats));
+    CBAMD_ENSURE(needCats == 0 || catRows != nullptr, "Model has categorical features but no categorical features provided");
+    CBAMD_ENSURE(catRowLen >= needCats, "insufficient cat features vector size");
+    if (docCount == 0 || m.RealBucketCount == 0) {
+        return;
+    }
+    // chunks must end on a multiple of 128 documents so that reference blocks do not straddle chunks
+    const size_t chunk = ChunkDocs(needFloats + m.RealBucketCount / 4 + 1, needCats);
+    const size_t stageDocs = std::min(chunk, docCount);
+    m.PinnedFloats.Reserve(std::max<size_t>(1, stageDocs * needFloats));
+    m.StageFloats.Reserve(std::max<size_t>(1, stageDocs * needFloats));
+    if (needCats) {
+        m.PinnedCats.Reserve(stageDocs * needCats);
+        m.StageCats.Reserve(stageDocs * needCats);
+    }
+    m.PinnedExport.Reserve(stageDocs * m.RealBucketCount);
+    m.StageExport.Reserve(stageDocs * m.RealBucketCount);
+    m.ScratchBins.Reserve(QuantizedBytes(stageDocs));
+    for (size_t begin = 0; begin < docCount; begin += chunk) {
+        const size_t n = std::min(chunk, docCount - begin);
+        if (needFloats) {
+            float* dst = m.PinnedFloats.Get();
+            for (size_t d = 0; d < n; ++d) {
+                std::memcpy(dst + d * needFloats, rows[begin + d], needFloats * sizeof(float));
+            }
+            HIP_CHECK(hipMemcpyAsync(m.StageFloats.Get(), dst, n * needFloats * sizeof(float), hipMemcpyHostToDevice, s));
+        }
+        if (needCats) {
+            int32_t* dst = m.PinnedCats.Get();
+            for (size_t d = 0; d < n; ++d) {
+                std::memcpy(dst + d * needCats, catRows[begin + d], needCats * sizeof(int32_t));
+            }
+            HIP_CHECK(hipMemcpyAsync(m.StageCats.Get(), dst, n * needCats * sizeof(int32_t), hipMemcpyHostToDevice, s));
+        }
+        TFeatureBatch batch;
+        batch.Layout = flat ? TFeatureBatch::FlatRows : TFeatureBatch::SplitRows;
+        batch.Floats = m.StageFloats.Get();
+        batch.Stride = needFloats;
+        batch.Cats = needCats ? m.StageCats.Get() : nullptr;
+        batch.CatStride = needCats;
+        QuantizeDevice(batch, n, m.ScratchBins.Get(), s);
+        ExportQuantizedDevice(m.ScratchBins.Get(), n, m.StageExport.Get(), s);
+        HIP_CHECK(hipMemcpyAsync(m.PinnedExport.Get(), m.StageExport.Get(), n * m.RealBucketCount, hipMemcpyDeviceToHost, s));
+        HIP_CHECK(hipStreamSynchronize(s));
+        std::memcpy(referenceLayout + begin * m.RealBucketCount, m.PinnedExport.Get(), n * m.RealBucketCount);
+    }
+}
+
+}  // namespace cbamd

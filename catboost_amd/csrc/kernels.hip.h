@@ -1,0 +1,382 @@
+// Device code of the HIP evaluator (gfx950, wave64).
+//
+// Quantized layout ("bins"): documents are grouped in blocks of 256; inside a block one wave
+// lane owns the four documents {lane, lane + 64, lane + 128, lane + 192} and keeps their bins of
+// one bucket in one dword, so
+//     bins[((block * buckets + bucket) * 64 + lane) * 4 + j]  is the bin of document
+//     block * 256 + j * 64 + lane.
+// A wave reads or writes the 256 bytes of one (block, bucket) pair with a single coalesced dword
+// access per lane, and per-document results (doc = base + j * 64 + lane) are coalesced as well.
+// Bin values are those of the reference's BinarizeFeatures (cpu/quantization.h:333-529):
+// float bucket -> number of borders strictly below the value, one-hot bucket -> 1 + index of the
+// matching value (0 when none).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace cbamd::dev {
+
+constexpr int kDocsPerBlock = 256;
+constexpr int kWave = 64;
+constexpr int kBucketFlagNanToInf = 1;  // HasNans && NanValueTreatment == AsTrue
+constexpr int kBucketFlagOneHot = 2;
+constexpr int kBucketTile = 32;         // buckets binarized per workgroup
+constexpr int kMaxBucketValues = 256;   // 254 values, padded
+
+struct TBinarizeTables {
+    uint32_t BucketCount;
+    const uint32_t* BucketSrc;     // source column of the bucket in the chosen layout
+    const uint32_t* BucketOffset;  // [BucketCount + 1] offsets into Values
+    const uint32_t* BucketFlags;
+    const uint32_t* Values;        // float borders (sorted ascending) or one-hot values, as bits
+};
+
+struct TTreeTables {
+    const uint32_t* Splits;       // per tree split / node: bucket | xorMask << 16 | splitIdx << 24
+    const uint32_t* TreeStart;    // first split (oblivious) or first node (non-symmetric) of a tree
+    const uint32_t* TreeSize;     // depth (oblivious) or node count (non-symmetric)
+    const uint32_t* FirstLeaf;    // index of the tree's first value in Leaves
+    const uint32_t* StepNodes;    // non-symmetric: left diff | right diff << 16
+    const uint32_t* NodeToLeaf;   // non-symmetric: value index of a terminal node
+    const double* Leaves;
+    const double* Bias;
+    double Scale;
+    int Dim;
+};
+
+// number of sorted borders strictly below v; `borders` is padded with +inf up to 256 entries
+__device__ __forceinline__ uint32_t CountBelow(const uint32_t* borders, float v) {
+    uint32_t lo = 0;
+#pragma unroll
+    for (uint32_t step = 128; step >= 1; step >>= 1) {
+        const uint32_t mid = lo + step;
+        const float b = __uint_as_float(borders[mid - 1]);
+        lo = (b < v) ? mid : lo;
+    }
+    return lo;
+}
+
+__device__ __forceinline__ uint32_t OneHotBin(const uint32_t* values, uint32_t count, uint32_t v) {
+    uint32_t bin = 0;
+    for (uint32_t i = 0; i < count; ++i) {
+        bin |= (values[i] == v) ? (i + 1) : 0u;
+    }
+    return bin;
+}
+
+// Row-major input: floats[doc * stride + column]; hashed categorical values either bit-cast in
+// the same row (cats == nullptr) or in cats[doc * catStride + column].
+// grid = (doc blocks, ceil(buckets / kBucketTile)), block = 256 threads.
+__global__ __launch_bounds__(256) void BinarizeRowsKernel(const float* __restrict__ floats, size_t stride,
+                                                          const int32_t* __restrict__ cats, size_t catStride,
+                                                          size_t docCount, TBinarizeTables tab,
+                                                          uint32_t* __restrict__ bins) {
+    // 2 x 32 KB of LDS; the tile is rotated by the bucket index instead of padded so that both
+    // the row-wise fill and the column-wise read are bank-conflict free
+    __shared__ uint32_t sValues[kBucketTile][kMaxBucketValues];
+    __shared__ uint32_t sTile[kBucketTile][kDocsPerBlock];
+
+    const uint32_t tid = threadIdx.x;
+    const size_t block = blockIdx.x;
+    const uint32_t b0 = blockIdx.y * kBucketTile;
+    const uint32_t nb = min(static_cast<uint32_t>(kBucketTile), tab.BucketCount - b0);
+
+    for (uint32_t i = tid; i < kBucketTile * kMaxBucketValues; i += 256) {
+        const uint32_t bb = i / kMaxBucketValues, k = i % kMaxBucketValues;
+        uint32_t v = 0x7f800000u;  // +inf pads the border list
+        if (bb < nb) {
+            const uint32_t off = tab.BucketOffset[b0 + bb];
+            const uint32_t cnt = tab.BucketOffset[b0 + bb + 1] - off;
+            if (k < cnt) {
+                v = tab.Values[off + k];
+            }
+        }
+        sValues[bb][k] = v;
+    }
+    // tile load: consecutive threads take consecutive buckets of one document row
+    for (uint32_t i = tid; i < kBucketTile * kDocsPerBlock; i += 256) {
+        const uint32_t row = i / kBucketTile, bb = i % kBucketTile;
+        const size_t doc = block * kDocsPerBlock + row;
+        uint32_t v = 0;
+        if (bb < nb && doc < docCount) {
+            const uint32_t src = tab.BucketSrc[b0 + bb];
+            const bool oneHot = (tab.BucketFlags[b0 + bb] & kBucketFlagOneHot) != 0;
+            if (oneHot && cats != nullptr) {
+                v = static_cast<uint32_t>(cats[doc * catStride + src]);
+            } else {
+                v = __float_as_uint(floats[doc * stride + src]);
+            }
+        }
+        sTile[bb][(row + bb) % kDocsPerBlock] = v;
+    }
+    __syncthreads();
+
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = tid / kWave;
+    for (uint32_t bb = wave; bb < nb; bb += 256 / kWave) {
+        const uint32_t flags = tab.BucketFlags[b0 + bb];
+        const uint32_t count = tab.BucketOffset[b0 + bb + 1] - tab.BucketOffset[b0 + bb];
+        uint32_t packed = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t raw = sTile[bb][(j * kWave + lane + bb) % kDocsPerBlock];
+            uint32_t bin;
+            if (flags & kBucketFlagOneHot) {
+                bin = OneHotBin(sValues[bb], count, raw);
+            } else {
+                float v = __uint_as_float(raw);
+                if ((flags & kBucketFlagNanToInf) && isnan(v)) {
+                    v = __uint_as_float(0x7f800000u);
+                }
+                bin = CountBelow(sValues[bb], v);
+            }
+            packed |= bin << (8 * j);
+        }
+        bins[(block * tab.BucketCount + b0 + bb) * kWave + lane] = packed;
+    }
+}
+
+// Column-major input: floats[column * stride + doc] (categorical hashes bit-cast in their column).
+// grid = (doc blocks, ceil(buckets / 4)), block = 256 threads: one wave per bucket.
+__global__ __launch_bounds__(256) void BinarizeColumnsKernel(const float* __restrict__ floats, size_t stride,
+                                                             size_t docCount, TBinarizeTables tab,
+                                                             uint32_t* __restrict__ bins) {
+    __shared__ uint32_t sValues[4][kMaxBucketValues];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = tid / kWave;
+    const size_t block = blockIdx.x;
+    const uint32_t bucket = blockIdx.y * 4 + wave;
+    const bool active = bucket < tab.BucketCount;
+    uint32_t off = 0, cnt = 0, flags = 0, src = 0;
+    if (active) {
+        off = tab.BucketOffset[bucket];
+        cnt = tab.BucketOffset[bucket + 1] - off;
+        flags = tab.BucketFlags[bucket];
+        src = tab.BucketSrc[bucket];
+    }
+    for (uint32_t k = lane; k < kMaxBucketValues; k += kWave) {
+        sValues[wave][k] = (k < cnt) ? tab.Values[off + k] : 0x7f800000u;
+    }
+    __syncthreads();
+    if (!active) {
+        return;
+    }
+    uint32_t packed = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const size_t doc = block * kDocsPerBlock + j * kWave + lane;
+        uint32_t raw = 0;
+        if (doc < docCount) {
+            raw = __float_as_uint(floats[static_cast<size_t>(src) * stride + doc]);
+        }
+        uint32_t bin;
+        if (flags & kBucketFlagOneHot) {
+            bin = OneHotBin(sValues[wave], cnt, raw);
+        } else {
+            float v = __uint_as_float(raw);
+            if ((flags & kBucketFlagNanToInf) && isnan(v)) {
+                v = __uint_as_float(0x7f800000u);
+            }
+            bin = CountBelow(sValues[wave], v);
+        }
+        packed |= bin << (8 * j);
+    }
+    bins[(block * tab.BucketCount + bucket) * kWave + lane] = packed;
+}
+
+// Final value of one output cell: Scale * sum (+ Bias[k] when the range starts at tree 0),
+// as ApplyScaleAndBias (catboost/libs/model/scale_and_bias.cpp:4-50). No fused multiply-add.
+__device__ __forceinline__ double Finish(double sum, double scale, double bias, bool addBias) {
+    double r = __dmul_rn(scale, sum);
+    if (addBias) {
+        r = __dadd_rn(r, bias);
+    }
+    return r;
+}
+
+// Oblivious trees, any model: one wave per 256-document block, four documents per lane, leaf
+// sums kept in registers in fp64 and accumulated in tree order (as the CPU evaluator does).
+// DCHUNK output dimensions are accumulated per pass over the trees.
+// grid = ceil(doc blocks / 4), block = 256 threads.
+template <int DCHUNK>
+__global__ __launch_bounds__(256) void EvalObliviousKernel(const uint32_t* __restrict__ bins, size_t docCount,
+                                                           uint32_t bucketCount, TTreeTables tt, uint32_t treeBegin,
+                                                           uint32_t treeEnd, double* __restrict__ out) {
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const size_t block = static_cast<size_t>(blockIdx.x) * (256 / kWave) + threadIdx.x / kWave;
+    const size_t blockCount = (docCount + kDocsPerBlock - 1) / kDocsPerBlock;
+    if (block >= blockCount) {
+        return;
+    }
+    const uint32_t* myBins = bins + block * bucketCount * kWave + lane;
+    const int dim = tt.Dim;
+    const bool addBias = treeBegin == 0;
+    for (int d0 = 0; d0 < dim; d0 += DCHUNK) {
+        double acc[4][DCHUNK];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int k = 0; k < DCHUNK; ++k) {
+                acc[j][k] = 0.0;
+            }
+        }
+        for (uint32_t t = treeBegin; t < treeEnd; ++t) {
+            const uint32_t first = tt.TreeStart[t];
+            const uint32_t depth = tt.TreeSize[t];
+            uint32_t idx0 = 0, idx1 = 0, idx2 = 0, idx3 = 0;
+            for (uint32_t d = 0; d < depth; ++d) {
+                const uint32_t sp = tt.Splits[first + d];
+                const uint32_t w = myBins[(sp & 0xffffu) * kWave];
+                const uint32_t x = (sp >> 16) & 0xffu;
+                const uint32_t s = sp >> 24;
+                idx0 |= static_cast<uint32_t>(((w & 0xffu) ^ x) >= s) << d;
+                idx1 |= static_cast<uint32_t>((((w >> 8) & 0xffu) ^ x) >= s) << d;
+                idx2 |= static_cast<uint32_t>((((w >> 16) & 0xffu) ^ x) >= s) << d;
+                idx3 |= static_cast<uint32_t>(((w >> 24) ^ x) >= s) << d;
+            }
+            const double* leaf = tt.Leaves + tt.FirstLeaf[t] + d0;
+            const uint32_t idx[4] = {idx0, idx1, idx2, idx3};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const double* p = leaf + static_cast<size_t>(idx[j]) * dim;
+#pragma unroll
+                for (int k = 0; k < DCHUNK; ++k) {
+                    if (DCHUNK == 1 || d0 + k < dim) {
+                        acc[j][k] = __dadd_rn(acc[j][k], p[k]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const size_t doc = block * kDocsPerBlock + j * kWave + lane;
+            if (doc < docCount) {
+#pragma unroll
+                for (int k = 0; k < DCHUNK; ++k) {
+                    if (DCHUNK == 1 || d0 + k < dim) {
+                        out[doc * dim + d0 + k] = Finish(acc[j][k], tt.Scale, tt.Bias[d0 + k], addBias);
+                    }
+                }
+            }
+        }
+    }
+}
+
+__device__ __forceinline__ uint32_t BinOfDoc(const uint8_t* bins, size_t doc, uint32_t bucketCount, uint32_t bucket) {
+    const size_t block = doc / kDocsPerBlock;
+    const uint32_t r = static_cast<uint32_t>(doc % kDocsPerBlock);
+    return bins[((block * bucketCount + bucket) * kWave + (r % kWave)) * 4 + r / kWave];
+}
+
+// Walks one non-symmetric tree for one document; returns the terminal node id
+// (CalcIndexesNonSymmetric, cpu/evaluator_impl.cpp:462-493).
+__device__ __forceinline__ uint32_t WalkNonSymmetric(const uint8_t* bins, size_t doc, uint32_t bucketCount,
+                                                     const TTreeTables& tt, uint32_t tree) {
+    uint32_t node = tt.TreeStart[tree];
+    for (;;) {
+        const uint32_t sp = tt.Splits[node];
+        const uint32_t st = tt.StepNodes[node];
+        const uint32_t b = BinOfDoc(bins, doc, bucketCount, sp & 0xffffu);
+        const bool right = ((b ^ ((sp >> 16) & 0xffu)) >= (sp >> 24));
+        const uint32_t diff = right ? (st >> 16) : (st & 0xffffu);
+        if (diff == 0) {
+            return node;
+        }
+        node += diff;
+    }
+}
+
+// Non-symmetric trees: one thread per document. grid = ceil(docs / 256), block = 256.
+template <int DCHUNK>
+__global__ __launch_bounds__(256) void EvalNonSymmetricKernel(const uint8_t* __restrict__ bins, size_t docCount,
+                                                              uint32_t bucketCount, TTreeTables tt, uint32_t treeBegin,
+                                                              uint32_t treeEnd, double* __restrict__ out) {
+    const size_t doc = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (doc >= docCount) {
+        return;
+    }
+    const int dim = tt.Dim;
+    const bool addBias = treeBegin == 0;
+    for (int d0 = 0; d0 < dim; d0 += DCHUNK) {
+        double acc[DCHUNK];
+#pragma unroll
+        for (int k = 0; k < DCHUNK; ++k) {
+            acc[k] = 0.0;
+        }
+        for (uint32_t t = treeBegin; t < treeEnd; ++t) {
+            const uint32_t node = WalkNonSymmetric(bins, doc, bucketCount, tt, t);
+            const double* p = tt.Leaves + tt.NodeToLeaf[node] + d0;
+#pragma unroll
+            for (int k = 0; k < DCHUNK; ++k) {
+                if (DCHUNK == 1 || d0 + k < dim) {
+                    acc[k] = __dadd_rn(acc[k], p[k]);
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < DCHUNK; ++k) {
+            if (DCHUNK == 1 || d0 + k < dim) {
+                out[doc * dim + d0 + k] = Finish(acc[k], tt.Scale, tt.Bias[d0 + k], addBias);
+            }
+        }
+    }
+}
+
+// Leaf indexes [doc][tree - treeBegin] for both tree kinds (CalcLeafIndexesGeneric,
+// cpu/evaluator.h:174-253; non-symmetric numbering cpu/evaluator_impl.cpp:626-633).
+__global__ __launch_bounds__(256) void LeafIndexesKernel(const uint8_t* __restrict__ bins, size_t docCount,
+                                                         uint32_t bucketCount, TTreeTables tt, int oblivious,
+                                                         uint32_t treeBegin, uint32_t treeEnd,
+                                                         uint32_t* __restrict__ out) {
+    const size_t doc = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (doc >= docCount) {
+        return;
+    }
+    const size_t treeCount = treeEnd - treeBegin;
+    for (uint32_t t = treeBegin; t < treeEnd; ++t) {
+        uint32_t result;
+        if (oblivious) {
+            const uint32_t first = tt.TreeStart[t];
+            const uint32_t depth = tt.TreeSize[t];
+            uint32_t idx = 0;
+            for (uint32_t d = 0; d < depth; ++d) {
+                const uint32_t sp = tt.Splits[first + d];
+                const uint32_t b = BinOfDoc(bins, doc, bucketCount, sp & 0xffffu);
+                idx |= static_cast<uint32_t>((b ^ ((sp >> 16) & 0xffu)) >= (sp >> 24)) << d;
+            }
+            result = idx;
+        } else {
+            const uint32_t node = WalkNonSymmetric(bins, doc, bucketCount, tt, t);
+            result = (tt.NodeToLeaf[node] - tt.FirstLeaf[t]) / static_cast<uint32_t>(tt.Dim);
+        }
+        out[doc * treeCount + (t - treeBegin)] = result;
+    }
+}
+
+// Re-lays bins out as the reference does: blocks of 128 documents, [block][bucket][doc in block],
+// the last block packed with its own document count (cpu/quantization.h:357-365).
+__global__ __launch_bounds__(256) void ExportBinsKernel(const uint8_t* __restrict__ bins, size_t docCount,
+                                                        uint32_t bucketCount, uint8_t* __restrict__ out) {
+    const size_t doc = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (doc >= docCount) {
+        return;
+    }
+    const size_t refBlockStart = doc / 128 * 128;
+    const size_t inBlock = doc - refBlockStart;
+    const size_t blockDocs = min(static_cast<size_t>(128), docCount - refBlockStart);
+    for (uint32_t b = 0; b < bucketCount; ++b) {
+        out[refBlockStart * bucketCount + b * blockDocs + inBlock] = BinOfDoc(bins, doc, bucketCount, b);
+    }
+}
+
+__global__ void FillBiasKernel(double* __restrict__ out, size_t count, const double* __restrict__ bias, int dim) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < count) {
+        out[i] = bias[i % dim];
+    }
+}
+
+}  // namespace cbamd::dev

@@ -1,0 +1,163 @@
+// Host-side model of a CatBoost tree ensemble: the tables of TModelTrees plus the runtime
+// tables the evaluator needs. Mirrors catboost/libs/model/model.h:64-187 and features.h:16-160.
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+#include <map>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+namespace cbamd {
+
+// Raised for every condition the reference reports through CB_ENSURE
+// (catboost/libs/helpers/exception.h:15); the C ABI turns it into `false` + GetErrorString().
+class TModelError : public std::runtime_error {
+public:
+    explicit TModelError(const std::string& what) : std::runtime_error(what) {}
+};
+
+#define CBAMD_ENSURE(cond, msg)                                   \
+    do {                                                          \
+        if (!(cond)) {                                            \
+            throw ::cbamd::TModelError(std::string() + msg);      \
+        }                                                         \
+    } while (0)
+
+constexpr uint32_t kMaxValuesPerBin = 254;  // MAX_VALUES_PER_BIN, model.h:72
+
+enum class ENanValueTreatment : int8_t { AsIs = 0, AsFalse = 1, AsTrue = 2 };  // features.h:51-55
+
+struct TFloatFeature {  // features.h:50-94
+    bool HasNans = false;
+    int Index = -1;
+    int FlatIndex = -1;
+    std::vector<float> Borders;
+    std::string FeatureId;
+    ENanValueTreatment NanValueTreatment = ENanValueTreatment::AsIs;
+    bool UsedInModel() const { return !Borders.empty(); }
+};
+
+struct TCatFeature {  // features.h:104-140
+    int Index = -1;
+    int FlatIndex = -1;
+    std::string FeatureId;
+    bool UsedInModel = true;
+};
+
+struct TOneHotFeature {  // features.h:142-160
+    int CatFeatureIndex = -1;
+    std::vector<int> Values;
+    std::vector<std::string> StringValues;
+};
+
+struct TRepackedBin {  // model.h:64-70
+    uint16_t FeatureIndex = 0;
+    uint8_t XorMask = 0;
+    uint8_t SplitIdx = 0;
+};
+
+struct TNonSymmetricTreeStepNode {  // model.h:78-95
+    uint16_t LeftSubtreeDiff = 0xffff;
+    uint16_t RightSubtreeDiff = 0xffff;
+};
+
+enum class ESplitType : int { FloatFeature = 0, EstimatedFeature = 1, OneHotFeature = 2, OnlineCtr = 3 };  // split.h:20-25
+
+// TModelSplit restricted to the kinds this evaluator supports (split.h:27-100).
+struct TModelSplit {
+    ESplitType Type = ESplitType::FloatFeature;
+    int FeatureIndex = 0;  // float feature index / cat feature index
+    float Border = 0.f;
+    int Value = 0;
+
+    static TModelSplit Float(int feature, float border) {
+        TModelSplit s;
+        s.Type = ESplitType::FloatFeature;
+        s.FeatureIndex = feature;
+        s.Border = border;
+        return s;
+    }
+    static TModelSplit OneHot(int catFeature, int value) {
+        TModelSplit s;
+        s.Type = ESplitType::OneHotFeature;
+        s.FeatureIndex = catFeature;
+        s.Value = value;
+        return s;
+    }
+    bool operator<(const TModelSplit& o) const;
+    bool operator==(const TModelSplit& o) const;
+};
+
+struct TModelTrees {
+    // ---- serialized state (flatbuffers/model.fbs:22-46)
+    int ApproxDimension = 1;
+    std::vector<int> TreeSplits;
+    std::vector<int> TreeSizes;
+    std::vector<int> TreeStartOffsets;
+    std::vector<TCatFeature> CatFeatures;
+    std::vector<TFloatFeature> FloatFeatures;
+    std::vector<TOneHotFeature> OneHotFeatures;
+    std::vector<double> LeafValues;
+    std::vector<double> LeafWeights;
+    std::vector<TNonSymmetricTreeStepNode> NonSymmetricStepNodes;
+    std::vector<uint32_t> NonSymmetricNodeIdToLeafId;
+    double Scale = 1.0;
+    std::vector<double> Bias;  // ApproxDimension values
+    // feature kinds this evaluator refuses; only their presence is recorded
+    size_t CtrFeatureCount = 0;
+    size_t TextFeatureCount = 0;
+    size_t EstimatedFeatureCount = 0;
+    size_t EmbeddingFeatureCount = 0;
+
+    // ---- runtime state (TRuntimeData / TForApplyData, model.h:146-187)
+    std::vector<TModelSplit> BinFeatures;
+    uint32_t EffectiveBinFeaturesBucketCount = 0;
+    std::vector<TRepackedBin> RepackedBins;
+    std::vector<size_t> TreeFirstLeafOffsets;
+    size_t UsedFloatFeaturesCount = 0;
+    size_t UsedCatFeaturesCount = 0;
+    size_t MinimalSufficientFloatFeaturesVectorSize = 0;
+    size_t MinimalSufficientCatFeaturesVectorSize = 0;
+
+    bool IsOblivious() const {  // model.h:271-273
+        return NonSymmetricStepNodes.empty() && NonSymmetricNodeIdToLeafId.empty();
+    }
+    size_t GetTreeCount() const { return TreeSizes.size(); }
+    size_t GetNumFloatFeatures() const {  // model.h:494-500
+        return FloatFeatures.empty() ? 0 : static_cast<size_t>(FloatFeatures.back().Index) + 1;
+    }
+    size_t GetNumCatFeatures() const {  // model.h:502-508
+        return CatFeatures.empty() ? 0 : static_cast<size_t>(CatFeatures.back().Index) + 1;
+    }
+    size_t GetFlatFeatureVectorExpectedSize() const;  // model.h:534-541
+    bool IsIdentityScaleAndBias() const;
+    bool IsZeroBias() const;
+
+    // UpdateRuntimeData = CalcForApplyData + CalcBinFeatures (model.cpp:425-429, 471-624).
+    void UpdateRuntimeData();
+    // model.cpp:634-674
+    void ConvertObliviousToAsymmetric();
+    void SetScaleAndBias(double scale, const std::vector<double>& bias);  // model.cpp:700-709
+    // Adds the tree-start offsets that the low-level AddBinTree API derives (model.cpp:238-254).
+    void AddBinTree(const std::vector<int>& binSplits);
+};
+
+struct TFullModel {
+    TModelTrees Trees;
+    std::map<std::string, std::string> ModelInfo;
+    std::vector<std::string> ModelPartIds;
+
+    // .cbm (de)serialisation, model.cpp:1113-1228
+    void Load(const void* data, size_t size);
+    void LoadFromFile(const std::string& path);
+    std::string Save() const;
+    void SaveToFile(const std::string& path) const;
+
+    // Throws unless every feature kind in the model is one the HIP evaluator handles.
+    void EnsureSupported() const;
+    std::vector<std::string> GetUsedFeaturesNames() const;  // model.cpp:1300-1343
+};
+
+}  // namespace cbamd

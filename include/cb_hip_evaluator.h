@@ -1,0 +1,191 @@
+/*
+ * Evaluator-level C ABI of the MI355X-native CatBoost evaluator (same libcatboostmodel.so).
+ *
+ * This is the seam an in-tree backend of the reference binds: an IModelEvaluator registered for
+ * EFormulaEvaluatorType::GPU (catboost/libs/model/evaluation_interface.h:70-308,
+ * catboost/libs/model/cuda/evaluator.cpp:419) that forwards to the calls below instead of to
+ * TGPUCatboostEvaluationContext (catboost/libs/model/cuda/evaluator.cuh:80-97). Plain pointers and
+ * sizes only. None of these symbols exists in the reference's export list; they carry the CbHip
+ * prefix so the reference surface (c_api.h) stays intact.
+ *
+ * Error convention as in c_api.h: false / NULL + thread-local GetErrorString().
+ */
+#ifndef CB_HIP_EVALUATOR_H
+#define CB_HIP_EVALUATOR_H
+
+#include <stdbool.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#if defined(__cplusplus)
+extern "C" {
+#endif
+
+typedef void CbHipEvaluatorHandle;
+
+/* The tables of TModelTrees as flat arrays (catboost/libs/model/model.h:97-141 IModelTreeData,
+ * catboost/libs/model/features.h:50-160). Nothing is retained after the call returns. */
+typedef struct CbHipModelArrays {
+    int32_t ApproxDimension;
+
+    int32_t TreeCount;
+    const int32_t* TreeSizes;        /* depth (oblivious) or node count (non-symmetric) */
+    const int32_t* TreeStartOffsets;
+    int32_t TreeSplitsCount;
+    const int32_t* TreeSplits;       /* binary feature ids, CalcBinFeatures order (model.cpp:471-577) */
+
+    int32_t FloatFeatureCount;       /* in model order, sorted by FlatIndex */
+    const int32_t* FloatFeatureIndex;
+    const int32_t* FloatFeatureFlatIndex;
+    const int32_t* FloatFeatureHasNans;
+    const int32_t* FloatFeatureNanTreatment; /* 0 AsIs, 1 AsFalse, 2 AsTrue (features.h:51-55) */
+    const int32_t* FloatFeatureBorderOffsets; /* FloatFeatureCount + 1 */
+    const float* FloatFeatureBorders;
+
+    int32_t CatFeatureCount;
+    const int32_t* CatFeatureIndex;
+    const int32_t* CatFeatureFlatIndex;
+    const int32_t* CatFeatureUsed;
+
+    int32_t OneHotFeatureCount;
+    const int32_t* OneHotCatFeatureIndex;
+    const int32_t* OneHotValueOffsets; /* OneHotFeatureCount + 1 */
+    const int32_t* OneHotValues;
+
+    uint64_t LeafValuesCount;
+    const double* LeafValues;        /* [tree][leaf * ApproxDimension + k] */
+
+    int32_t StepNodeCount;           /* 0 for oblivious models */
+    const uint16_t* StepNodes;       /* pairs (LeftSubtreeDiff, RightSubtreeDiff), model.h:78-95 */
+    const uint32_t* NodeIdToLeafId;
+
+    double Scale;
+    const double* Bias;              /* ApproxDimension values */
+} CbHipModelArrays;
+
+enum ECbHipFeatureLayout {
+    CBHIP_FLAT_ROWS = 0,    /* Floats[doc * Stride + FlatIndex], cat hashes bit-cast in the row */
+    CBHIP_FLAT_COLUMNS = 1, /* Floats[FlatIndex * Stride + doc] */
+    CBHIP_SPLIT_ROWS = 2,   /* Floats[doc * Stride + Index], Cats[doc * CatStride + Index] */
+};
+
+/* A batch of documents in DEVICE memory (TGPUDataInput, cuda/evaluator.cuh:38-51). */
+typedef struct CbHipFeatures {
+    int32_t Layout;
+    const float* Floats;
+    size_t Stride;
+    const int32_t* Cats;
+    size_t CatStride;
+} CbHipFeatures;
+
+/* Model upload: validates the tables, derives buckets / repacked splits / leaf offsets and
+ * copies SoA tables to device `deviceId` (takes the place of the TGpuEvaluator constructor,
+ * cuda/evaluator.cpp:18-85). */
+CbHipEvaluatorHandle* CbHipEvaluatorCreate(const CbHipModelArrays* model, int deviceId);
+void CbHipEvaluatorDelete(CbHipEvaluatorHandle* evaluator);
+
+size_t CbHipTreeCount(CbHipEvaluatorHandle* evaluator);
+int32_t CbHipApproxDimension(CbHipEvaluatorHandle* evaluator);
+uint32_t CbHipBucketCount(CbHipEvaluatorHandle* evaluator);
+
+/* Bytes of a quantized buffer for docCount documents. */
+size_t CbHipQuantizedBytes(CbHipEvaluatorHandle* evaluator, size_t docCount);
+
+/* Binarize device-resident features into `deviceBins` (TGPUCatboostEvaluationContext::QuantizeData,
+ * cuda/evaluator.cu:379-416; IModelEvaluator::Quantize). `hipStream` is a hipStream_t or NULL for
+ * the evaluator's own stream; the call is asynchronous on that stream. */
+bool CbHipQuantize(CbHipEvaluatorHandle* evaluator, const CbHipFeatures* deviceFeatures, size_t docCount,
+                   void* deviceBins, void* hipStream);
+
+/* Evaluate trees [treeStart, treeEnd) on quantized documents into deviceResults[doc * dim + k]
+ * (EvalQuantizedData, cuda/evaluator.cu:344-377; IModelEvaluator::Calc(IQuantizedData*)).
+ * Raw formula values: Scale * sum + Bias, bias only when treeStart == 0. Asynchronous. */
+bool CbHipEvalQuantized(CbHipEvaluatorHandle* evaluator, const void* deviceBins, size_t docCount, size_t treeStart,
+                        size_t treeEnd, double* deviceResults, void* hipStream);
+
+/* Binarize + evaluate with the evaluator's own scratch bins (EvalData, cuda/evaluator.cu:418-428).
+ * Synchronises the stream before returning and records the two kernel times. */
+bool CbHipEvalData(CbHipEvaluatorHandle* evaluator, const CbHipFeatures* deviceFeatures, size_t docCount,
+                   size_t treeStart, size_t treeEnd, double* deviceResults, void* hipStream);
+
+/* Leaf indexes deviceIndexes[doc * (treeEnd - treeStart) + t] (IModelEvaluator::CalcLeafIndexes on
+ * quantized data, evaluation_interface.h:289-294; unimplemented in cuda/evaluator.cpp:337-348). */
+bool CbHipLeafIndexesQuantized(CbHipEvaluatorHandle* evaluator, const void* deviceBins, size_t docCount,
+                               size_t treeStart, size_t treeEnd, uint32_t* deviceIndexes, void* hipStream);
+
+/* Bins re-laid out as the reference's CPU quantized data: blocks of 128 documents,
+ * [block][bucket][doc in block] (cpu/quantization.h:18-52, 357-365); docCount * buckets bytes. */
+bool CbHipExportQuantized(CbHipEvaluatorHandle* evaluator, const void* deviceBins, size_t docCount,
+                          uint8_t* deviceReferenceLayout, void* hipStream);
+
+bool CbHipSynchronize(CbHipEvaluatorHandle* evaluator, void* hipStream);
+
+/* hipEvent-measured duration of the binarize and evaluate kernels of the last CbHipEvalData or
+ * host-level prediction call (summed over its chunks). */
+bool CbHipLastKernelTimes(CbHipEvaluatorHandle* evaluator, float* binarizeMs, float* evalMs);
+
+/* ---- extensions on a ModelCalcerHandle (c_api.h) ------------------------------------------ */
+
+/* The evaluator bound to a model handle (created on first use on the enabled device). Owned by
+ * the handle; invalidated by the next Load* / CbHipLoad* / CbHipBuild* call on it. */
+CbHipEvaluatorHandle* CbHipGetEvaluator(void* modelHandle);
+
+/* Install a model given as raw tables (the AddBinTree / AddLeafValue route of TModelTrees,
+ * catboost/libs/model/model.cpp:238-254). */
+bool CbHipLoadModelFromArrays(void* modelHandle, const CbHipModelArrays* model);
+
+/* A split of a tree under construction (TModelSplit, catboost/libs/model/split.h:27-100). */
+typedef struct CbHipModelSplit {
+    int32_t Type;         /* 0 float feature, 2 one-hot feature (ESplitType, split.h:20-25) */
+    int32_t FeatureIndex; /* float feature index or categorical feature index */
+    float Border;
+    int32_t Value;        /* hashed category for one-hot splits */
+} CbHipModelSplit;
+
+/* TObliviousTreeBuilder (catboost/libs/model/model_build_helper.cpp:128-204): feature descriptions
+ * come from `features` (borders ignored: only borders used by splits are kept), tree t has
+ * treeDepths[t] splits taken in order from `splits` and (1 << depth) * ApproxDimension leaf
+ * values taken in order from `leafValues` ([leaf * dim + k]). Scale and Bias of `features` apply. */
+bool CbHipBuildObliviousModel(void* modelHandle, const CbHipModelArrays* features, int32_t treeCount,
+                              const int32_t* treeDepths, const CbHipModelSplit* splits, const double* leafValues);
+
+/* TNonSymmetricTreeModelBuilder (model_build_helper.cpp:206-304). Trees arrive as node arrays:
+ * node i of tree t is a split (nodeIsSplit != 0, children nodeLeft / nodeRight as indexes into
+ * the same tree's node range, condition nodeSplits[i]) or a leaf whose ApproxDimension values
+ * start at nodeValues[nodeValueOffset[i]]. treeNodeOffsets has treeCount + 1 entries; the root
+ * of a tree is its first node. */
+bool CbHipBuildNonSymmetricModel(void* modelHandle, const CbHipModelArrays* features, int32_t treeCount,
+                                 const int32_t* treeNodeOffsets, const int32_t* nodeIsSplit,
+                                 const CbHipModelSplit* nodeSplits, const int32_t* nodeLeft, const int32_t* nodeRight,
+                                 const int64_t* nodeValueOffset, const double* nodeValues);
+
+/* TFullModel::Save (catboost/libs/model/model.cpp:1113-1163). The buffer is malloc'd. */
+bool CbHipSaveModelToFile(void* modelHandle, const char* filename);
+bool CbHipSaveModelToBuffer(void* modelHandle, void** buffer, size_t* size);
+/* TModelTrees::ConvertObliviousToAsymmetric (model.cpp:634-674) */
+bool CbHipConvertObliviousToAsymmetric(void* modelHandle);
+/* TFullModel::SetScaleAndBias (model.cpp:700-709) */
+bool CbHipSetScaleAndBias(void* modelHandle, double scale, const double* bias, size_t biasSize);
+bool CbHipSetModelInfo(void* modelHandle, const char* key, const char* value);
+
+/* Host-resident contiguous row-major matrix features[doc * stride + flat index]: one bulk copy
+ * instead of one pointer per document. */
+bool CbHipCalcFlatContiguous(void* modelHandle, const float* features, size_t docCount, size_t stride,
+                             size_t treeStart, size_t treeEnd, double* result, size_t resultSize);
+/* TFullModel::CalcLeafIndexes over flat rows (model.h:1280-1302): indexes[doc * trees + t]. */
+bool CbHipCalcLeafIndexesFlat(void* modelHandle, size_t docCount, const float** floatFeatures,
+                              size_t floatFeaturesSize, size_t treeStart, size_t treeEnd, uint32_t* indexes,
+                              size_t indexesSize);
+/* Bins of flat rows in the reference layout; binsSize must equal docCount * bucket count. */
+bool CbHipQuantizeFlat(void* modelHandle, size_t docCount, const float** floatFeatures, size_t floatFeaturesSize,
+                       uint8_t* bins, size_t binsSize);
+/* Same for split float / hashed categorical rows. */
+bool CbHipQuantizeWithHashedCatFeatures(void* modelHandle, size_t docCount, const float** floatFeatures,
+                                        size_t floatFeaturesSize, const int** catFeatures, size_t catFeaturesSize,
+                                        uint8_t* bins, size_t binsSize);
+uint32_t CbHipModelBucketCount(void* modelHandle);
+
+#if defined(__cplusplus)
+}
+#endif
+#endif

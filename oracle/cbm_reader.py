@@ -55,12 +55,13 @@ class _Table:
         p = self._indirect(slot)
         return None if p is None else _Table(self.buf, p)
 
-    def vector(self, slot, dtype):
+    def vector(self, slot, dtype, per_element=1):
+        """Vector of scalars, or of structs made of `per_element` scalars of `dtype`."""
         p = self._indirect(slot)
         if p is None:
             return np.zeros(0, dtype=dtype)
         (n,) = struct.unpack_from("<I", self.buf, p)
-        return np.frombuffer(self.buf, dtype=dtype, count=n, offset=p + 4).copy()
+        return np.frombuffer(self.buf, dtype=dtype, count=n * per_element, offset=p + 4).copy()
 
     def vector_len(self, slot):
         p = self._indirect(slot)
@@ -145,7 +146,7 @@ def read_cbm(data):
     model["ctr_feature_count"] = t.vector_len(7)
     model["leaf_values"] = t.vector(8, np.float64)
     model["leaf_weights"] = t.vector(9, np.float64)
-    model["step_nodes"] = t.vector(10, np.uint16).reshape(-1, 2)
+    model["step_nodes"] = t.vector(10, np.uint16, per_element=2).reshape(-1, 2)
     model["node_id_to_leaf_id"] = t.vector(11, np.uint32)
     model["text_feature_count"] = t.vector_len(12)
     model["estimated_feature_count"] = t.vector_len(13)

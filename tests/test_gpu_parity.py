@@ -1,0 +1,283 @@
+"""Parity of the HIP evaluator against the CPU oracle, through the C ABI. Needs an MI355X.
+
+Bar: bins and leaf indexes bit-exact; predictions within 1e-9 relative / 1e-12 absolute.
+"""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+
+import catboost_amd as cb
+from catboost_amd import synthetic as syn
+from oracle import model_builder as mb
+from oracle.cbm_reader import read_cbm, read_cbm_file
+from oracle.oracle import OracleModel, cat_feature_hash_signed
+from tests import refmodels as rm
+from tests.test_oracle import _random_flat_data, _random_oblivious
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-9, 1e-12
+
+
+def _close(got, expected):
+    np.testing.assert_allclose(got, expected, rtol=RTOL, atol=ATOL)
+
+
+def _gpu_model(model_dict):
+    m = cb.ModelCalcer()
+    m.load_from_dict(model_dict)
+    m.enable_gpu_evaluation(0)
+    return m
+
+
+def _check_flat(model_dict, x, exact=None):
+    """bins, leaf indexes and predictions of flat rows against the oracle."""
+    o = OracleModel(model_dict)
+    g = _gpu_model(model_dict)
+    np.testing.assert_array_equal(g.quantize_flat(x), o.binarize(x))
+    np.testing.assert_array_equal(g.calc_leaf_indexes_flat(x), o.leaf_indexes(x))
+    pred = g.calc_flat(x)
+    _close(pred, o.calc(x))
+    if exact is not None:
+        np.testing.assert_array_equal(pred, np.asarray(exact, np.float64))
+    return g, o
+
+
+# ------------------------------------------------------------ reference unit-test models ----
+
+def test_library_loaded_is_the_in_tree_hip_build():
+    lib = cb.load_library()
+    assert os.path.samefile(lib._name, cb.library_path())
+    assert cb.ModelCalcer().get_supported_evaluator_types() == [1]  # CBA_FET_GPU only
+
+
+@pytest.mark.parametrize("asym", [False, True])
+def test_simple_float_model(asym):
+    model = rm.simple_float_model()
+    if asym:
+        model = mb.convert_oblivious_to_asymmetric(model)
+    _check_flat(model, rm.DATA, exact=np.arange(8.0))
+
+
+@pytest.mark.parametrize("asym", [False, True])
+def test_scale_bias_two_trees(asym):
+    model = rm.simple_float_model(tree_count=2, scale=0.5, bias=[0.125])
+    if asym:
+        model = mb.convert_oblivious_to_asymmetric(model)
+    g, _ = _check_flat(model, rm.DATA, exact=0.5 * 11.0 * np.arange(8.0) + 0.125)
+    # staged ranges: bias only with tree 0 (scale_and_bias.cpp:13-24)
+    np.testing.assert_array_equal(g.calc_flat(rm.DATA, tree_start=0, tree_end=1), 0.5 * np.arange(8.0) + 0.125)
+    np.testing.assert_array_equal(g.calc_flat(rm.DATA, tree_start=1, tree_end=2), 5.0 * np.arange(8.0))
+    np.testing.assert_array_equal(g.calc_flat(rm.DATA, tree_start=1, tree_end=1), np.zeros(8))
+
+
+@pytest.mark.parametrize("asym", [False, True])
+def test_deep_tree(asym):
+    model = rm.simple_deep_tree_model(9)
+    if asym:
+        model = mb.convert_oblivious_to_asymmetric(model)
+    g, _ = _check_flat(model, rm.deep_tree_data(9), exact=np.arange(512.0))
+    np.testing.assert_array_equal(g.calc_leaf_indexes_flat(rm.deep_tree_data(9)).ravel(), np.arange(512))
+
+
+@pytest.mark.parametrize("asym", [False, True])
+def test_multi_value_model(asym):
+    model = rm.multi_value_float_model()
+    if asym:
+        model = mb.convert_oblivious_to_asymmetric(model)
+    g, _ = _check_flat(model, rm.DATA[:4], exact=[0., 10., 20., 1., 11., 21., 2., 12., 22., 3., 13., 23.])
+    np.testing.assert_array_equal(g.predict_specific_class_flat(rm.DATA[:4], 1), [10., 11., 12., 13.])
+
+
+def test_simple_asymmetric_model():
+    g, _ = _check_flat(rm.simple_asymmetric_model(), rm.DATA, exact=rm.ASYMMETRIC_PREDICTIONS)
+    np.testing.assert_array_equal(g.calc_leaf_indexes_flat(rm.DATA), rm.ASYMMETRIC_LEAF_INDEXES)
+    # built by the library's own non-symmetric builder and reloaded from its .cbm
+    ffs, heads = rm.simple_asymmetric_trees()
+    b = cb.ModelCalcer()
+    b.build_non_symmetric(ffs, [], 1, heads)
+    r = cb.ModelCalcer(buffer=b.save_to_buffer())
+    np.testing.assert_array_equal(r.calc_flat(rm.DATA), rm.ASYMMETRIC_PREDICTIONS)
+
+
+def test_zero_trees_gives_bias():
+    g = _gpu_model(rm.simple_float_model(tree_count=0, bias=[0.75]))
+    np.testing.assert_array_equal(g.calc_flat(rm.DATA), np.full(8, 0.75))
+
+
+def test_single_document_and_ragged_sizes():
+    model = rm.simple_float_model(tree_count=2)
+    o = OracleModel(model)
+    g = _gpu_model(model)
+    rng = np.random.default_rng(3)
+    for n in (1, 2, 63, 64, 65, 127, 128, 129, 255, 256, 257, 1000):
+        x = rng.normal(scale=150, size=(n, 3)).astype(np.float32)
+        np.testing.assert_array_equal(g.quantize_flat(x), o.binarize(x))
+        np.testing.assert_array_equal(g.calc_flat(x), o.calc(x))
+        np.testing.assert_array_equal(g.calc_leaf_indexes_flat(x), o.leaf_indexes(x))
+    assert g.calc_flat(np.zeros((0, 3), np.float32)).size == 0
+
+
+# ------------------------------------------------------------------- fixtures + goldens ----
+
+def test_numeric_only_fixture(golden_dir):
+    g = cb.ModelCalcer(os.path.join(golden_dir, "numeric_only_model.cbm"))
+    g.enable_gpu_evaluation(0)
+    _close(g.calc_flat(rm.NUMERIC_ONLY_ROWS), rm.NUMERIC_ONLY_EXPECTED)
+    _close(g.calc_flat_transposed(np.ascontiguousarray(rm.NUMERIC_ONLY_ROWS.T)), rm.NUMERIC_ONLY_EXPECTED)
+    _close(g.calc_flat(rm.NUMERIC_ONLY_ROWS[0]), rm.NUMERIC_ONLY_EXPECTED[:1])
+    _close(g.calc(rm.NUMERIC_ONLY_ROWS, [[] for _ in range(4)]), rm.NUMERIC_ONLY_EXPECTED)
+    _close(g.calc_single(rm.NUMERIC_ONLY_ROWS[0], []), rm.NUMERIC_ONLY_EXPECTED[:1])
+
+
+def test_rust_fixture_with_one_hot_string_cats(golden_dir):
+    g = cb.ModelCalcer(os.path.join(golden_dir, "rust_tmp_model.cbm"))
+    _close(g.calc(rm.RUST_FLOATS, rm.RUST_CATS), rm.RUST_EXPECTED)
+    hashed = np.array([[cb.string_cat_feature_hash(c) for c in row] for row in rm.RUST_CATS], np.int32)
+    _close(g.calc_hashed(rm.RUST_FLOATS, hashed), rm.RUST_EXPECTED)
+    # flat layout: the hash bit-cast into the categorical slot (flat index 2), floats at 0, 1, 3
+    flat = np.zeros((3, 4), np.float32)
+    flat[:, [0, 1, 3]] = rm.RUST_FLOATS
+    flat[:, 2] = hashed[:, 0].view(np.float32)
+    _close(g.calc_flat(flat), rm.RUST_EXPECTED)
+    o = OracleModel(read_cbm_file(os.path.join(golden_dir, "rust_tmp_model.cbm")))
+    np.testing.assert_array_equal(g.quantize_hashed(rm.RUST_FLOATS, hashed), o.binarize(rm.RUST_FLOATS, hashed, layout="split"))
+
+
+def test_querywise_fixture(golden_dir):
+    g = cb.ModelCalcer(os.path.join(golden_dir, "features_num__dataset_querywise.cbm"))
+    np.testing.assert_allclose(g.calc_flat(rm.querywise_rows()), rm.QUERYWISE_EXPECTED, rtol=1e-12, atol=1e-15)
+
+
+def test_iris_fixture(golden_dir):
+    path = os.path.join(golden_dir, "iris_model.cbm")
+    g = cb.ModelCalcer(path)
+    feats, labels = rm.load_iris(golden_dir)
+    pred = g.calc_flat(feats).reshape(-1, 3)
+    np.testing.assert_array_equal(np.argmax(pred, axis=1), labels)
+    o = OracleModel(read_cbm_file(path))
+    _close(pred.ravel(), o.calc(feats))
+    np.testing.assert_array_equal(g.calc_leaf_indexes_flat(feats), o.leaf_indexes(feats))
+    np.testing.assert_array_equal(g.quantize_flat(feats), o.binarize(feats))
+    g.set_prediction_type("Class")
+    np.testing.assert_array_equal(g.calc_flat(feats), labels.astype(np.float64))
+
+
+def test_boston_fixture(golden_dir):
+    path = os.path.join(golden_dir, "boston_housing_model.cbm")
+    g = cb.ModelCalcer(path)
+    feats, target = rm.load_boston(golden_dir)
+    pred = g.calc_flat(feats)
+    assert int(np.sum(np.abs(pred - np.log(target)) >= 0.4)) <= 7
+    _close(pred, OracleModel(read_cbm_file(path)).calc(feats))
+
+
+# ------------------------------------------------------------------------- random models ----
+
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+@pytest.mark.parametrize("dim", [1, 3, 10, 20])
+def test_random_oblivious_models(seed, dim):
+    rng = np.random.default_rng(100 * dim + seed)
+    model, cat_values = _random_oblivious(rng, dim=dim, trees=40, max_depth=8, many_borders=(seed % 2 == 0),
+                                          scale=0.5 if seed else 1.0, bias=rng.normal(size=dim) if seed else None)
+    x = _random_flat_data(rng, model, cat_values, 777)
+    g, o = _check_flat(model, x)
+    # the same model as a non-symmetric one
+    _check_flat(mb.convert_oblivious_to_asymmetric(model), x)
+    # transposed input and a tree sub-range
+    _close(g.calc_flat_transposed(np.ascontiguousarray(x.T)), o.calc(x))
+    _close(g.calc_flat(x, tree_start=3, tree_end=17), o.calc(x, tree_start=3, tree_end=17))
+    # split float / hashed categorical rows
+    ff, cf = model["float_features"], model["cat_features"]
+    floats = x[:, [f["flat_index"] for f in ff]]
+    cats = x[:, [c["flat_index"] for c in cf]].view(np.int32)
+    _close(g.calc_hashed(floats, cats), o.calc(floats, cats, layout="split"))
+
+
+def test_library_builder_matches_oracle_builder_and_roundtrips():
+    rng = np.random.default_rng(11)
+    ffs = [mb.float_feature(i, i) for i in range(5)]
+    cfs = [mb.cat_feature(0, 5)]
+    cands = [np.unique(rng.normal(size=30).astype(np.float32)) for _ in range(5)]
+    trees = []
+    for _ in range(30):
+        splits = []
+        for _ in range(int(rng.integers(1, 7))):
+            if rng.random() < 0.2:
+                splits.append(("onehot", 0, int(rng.integers(0, 5))))
+            else:
+                f = int(rng.integers(0, 5))
+                splits.append(("float", f, float(rng.choice(cands[f]))))
+        trees.append((splits, rng.normal(size=(1 << len(splits)) * 2)))
+    ref = mb.build_oblivious(ffs, cfs, 2, trees, scale=2.0, bias=[0.5, -0.5])
+    b = cb.ModelCalcer()
+    b.build_oblivious(ffs, cfs, 2, trees, scale=2.0, bias=[0.5, -0.5])
+    got = read_cbm(b.save_to_buffer())
+    for k in ("tree_splits", "tree_sizes", "tree_start_offsets", "leaf_values", "bias"):
+        np.testing.assert_array_equal(got[k], ref[k])
+    for a, c in zip(got["float_features"], ref["float_features"]):
+        np.testing.assert_array_equal(a["borders"], c["borders"])
+    x = rng.normal(size=(300, 6)).astype(np.float32)
+    x[:, 5] = rng.integers(0, 6, size=300).astype(np.int32).view(np.float32)
+    _close(b.calc_flat(x), OracleModel(ref).calc(x))
+
+
+# --------------------------------------------------------------------- the five workloads ----
+
+@pytest.mark.parametrize("name,docs", [("C1", 30000), ("C2", 20000), ("C3", 10000), ("C4", 20000), ("C5", 6000)])
+def test_workload_configs_host_path(name, docs):
+    model, info = syn.build_model(name)
+    o = OracleModel(read_cbm(model.save_to_buffer()))
+    x = syn.host_features(info, docs)
+    np.testing.assert_array_equal(model.quantize_flat(x), o.binarize(x))
+    sample = slice(0, 2000)
+    np.testing.assert_array_equal(model.calc_leaf_indexes_flat(x[sample]), o.leaf_indexes(x[sample]))
+    _close(model.calc_flat(x), o.calc(x, threads=8))
+
+
+@pytest.mark.parametrize("name,docs", [("C1", 100000), ("C2", 50000), ("C3", 20000), ("C4", 30000), ("C5", 10000)])
+def test_workload_configs_device_path(name, docs):
+    import torch
+
+    model, info = syn.build_model(name)
+    o = OracleModel(read_cbm(model.save_to_buffer()))
+    ev = model.evaluator()
+    x = syn.device_features(info, docs)
+    out = torch.zeros(docs * info["dim"], dtype=torch.float64, device="cuda:0")
+    feats = ev.features(cb.LAYOUT_FLAT_ROWS, x.data_ptr(), x.shape[1])
+    ev.eval_data(feats, docs, out.data_ptr())
+    host = x.cpu().numpy()
+    _close(out.cpu().numpy(), o.calc(host, threads=8))
+    # separate quantize + evaluate on a caller-owned buffer, and the reference-layout export
+    bins = torch.zeros(ev.quantized_bytes(docs), dtype=torch.uint8, device="cuda:0")
+    ev.quantize(feats, docs, bins.data_ptr())
+    out2 = torch.zeros_like(out)
+    ev.eval_quantized(bins.data_ptr(), docs, out2.data_ptr())
+    exported = torch.zeros(docs * ev.bucket_count, dtype=torch.uint8, device="cuda:0")
+    ev.export_quantized(bins.data_ptr(), docs, exported.data_ptr())
+    ev.synchronize()
+    assert torch.equal(out, out2)
+    np.testing.assert_array_equal(exported.cpu().numpy(), o.binarize(host))
+    binarize_ms, eval_ms = ev.last_kernel_times()
+    assert binarize_ms > 0 and eval_ms > 0
+
+
+# ----------------------------------------------------------------------------- error paths ----
+
+def test_error_paths(golden_dir):
+    g = cb.ModelCalcer(os.path.join(golden_dir, "numeric_only_model.cbm"))
+    with pytest.raises(cb.CatBoostError, match="results. size is insufficient"):
+        g.calc_flat(rm.NUMERIC_ONLY_ROWS, result_size=3)
+    with pytest.raises(cb.CatBoostError, match="insufficient"):
+        g.calc_flat(rm.NUMERIC_ONLY_ROWS[:, :2])
+    with pytest.raises(cb.CatBoostError):
+        g.enable_gpu_evaluation(99)
+    with pytest.raises(cb.CatBoostError, match="Incorrect model file descriptor"):
+        cb.ModelCalcer(os.path.join(golden_dir, "not_a_model.cbm"))
+    for name in ("categoric_only_model.cbm", "jvm_model_with_ctr.cbm", "cloudness_small.cbm"):
+        with pytest.raises(cb.CatBoostError, match="not supported"):
+            cb.ModelCalcer(os.path.join(golden_dir, name))
+    # the handle still works after failed calls
+    _close(g.calc_flat(rm.NUMERIC_ONLY_ROWS), rm.NUMERIC_ONLY_EXPECTED)
