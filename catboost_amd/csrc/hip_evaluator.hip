@@ -109,6 +109,9 @@ struct THipEvaluator::TImpl {
     size_t MinFloatSize = 0;
     size_t MinCatSize = 0;
     bool HasCats = false;
+    uint32_t MaxBucketValues = 0;  // largest number of borders / one-hot values in one bucket
+    uint32_t MaxDepth = 0;         // deepest oblivious tree
+    bool HasOneHot = false;
 
     // binarize tables
     TDeviceVec<uint32_t> BucketSrcFlat, BucketSrcSplit, BucketOffset, BucketFlags, Values;
@@ -238,6 +241,15 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId)
         }
     }
     CBAMD_ENSURE(srcFlat.size() == BucketCount, "internal error: bucket count mismatch");
+    for (size_t b = 0; b + 1 < offsets.size(); ++b) {
+        m.MaxBucketValues = std::max(m.MaxBucketValues, offsets[b + 1] - offsets[b]);
+    }
+    m.HasOneHot = !trees.OneHotFeatures.empty();
+    if (m.Oblivious) {
+        for (int d : trees.TreeSizes) {
+            m.MaxDepth = std::max<uint32_t>(m.MaxDepth, static_cast<uint32_t>(d));
+        }
+    }
     if (BucketCount == 0) {  // keep the device tables non-empty; the binarize kernel is skipped
         srcFlat.push_back(0);
         srcSplit.push_back(0);
@@ -306,6 +318,36 @@ void THipEvaluator::Synchronize(void* stream) {
     HIP_CHECK(hipStreamSynchronize(Impl->Pick(stream)));
 }
 
+namespace {
+
+constexpr uint32_t kBinarizeBlocksPerGroup = 8;
+
+template <int LOG2P>
+void LaunchBinarizeRowsP(size_t blocks, const float* floats, size_t stride, const int32_t* cats, size_t catStride,
+                         size_t docCount, const dev::TBinarizeTables& tab, uint32_t* bins, hipStream_t s) {
+    const dim3 grid(static_cast<uint32_t>((blocks + kBinarizeBlocksPerGroup - 1) / kBinarizeBlocksPerGroup),
+                    (tab.BucketCount + dev::kBucketTile - 1) / dev::kBucketTile);
+    hipLaunchKernelGGL(dev::BinarizeRowsKernel<LOG2P>, grid, dim3(256), 0, s, floats, stride, cats, catStride, docCount,
+                       tab, kBinarizeBlocksPerGroup, bins);
+}
+
+// picks the smallest LDS slot count that still exceeds the largest bucket of the model
+void LaunchBinarizeRows(uint32_t maxBucketValues, size_t blocks, const float* floats, size_t stride,
+                        const int32_t* cats, size_t catStride, size_t docCount, const dev::TBinarizeTables& tab,
+                        uint32_t* bins, hipStream_t s) {
+    if (maxBucketValues < 32) {
+        LaunchBinarizeRowsP<5>(blocks, floats, stride, cats, catStride, docCount, tab, bins, s);
+    } else if (maxBucketValues < 64) {
+        LaunchBinarizeRowsP<6>(blocks, floats, stride, cats, catStride, docCount, tab, bins, s);
+    } else if (maxBucketValues < 128) {
+        LaunchBinarizeRowsP<7>(blocks, floats, stride, cats, catStride, docCount, tab, bins, s);
+    } else {
+        LaunchBinarizeRowsP<8>(blocks, floats, stride, cats, catStride, docCount, tab, bins, s);
+    }
+}
+
+}  // namespace
+
 void THipEvaluator::QuantizeDevice(const TFeatureBatch& batch, size_t docCount, uint8_t* bins, void* stream) {
     TImpl& m = *Impl;
     if (docCount == 0) {
@@ -326,9 +368,8 @@ void THipEvaluator::QuantizeDevice(const TFeatureBatch& batch, size_t docCount, 
             CBAMD_ENSURE(batch.Stride >= m.FlatVectorSize, "insufficient flat features vector size: " +
                                                                 std::to_string(batch.Stride) + " expected: " +
                                                                 std::to_string(m.FlatVectorSize));
-            const dim3 grid(static_cast<uint32_t>(blocks), (m.LayoutBuckets + dev::kBucketTile - 1) / dev::kBucketTile);
-            hipLaunchKernelGGL(dev::BinarizeRowsKernel, grid, dim3(256), 0, s, batch.Floats, batch.Stride, nullptr,
-                               size_t(0), docCount, m.BinarizeTables(true), reinterpret_cast<uint32_t*>(bins));
+            LaunchBinarizeRows(m.MaxBucketValues, blocks, batch.Floats, batch.Stride, nullptr, 0, docCount,
+                               m.BinarizeTables(true), reinterpret_cast<uint32_t*>(bins), s);
             break;
         }
         case TFeatureBatch::SplitRows: {
@@ -341,11 +382,9 @@ void THipEvaluator::QuantizeDevice(const TFeatureBatch& batch, size_t docCount, 
                                                                   std::to_string(batch.CatStride) + " expected: " +
                                                                   std::to_string(m.MinCatSize));
             }
-            const dim3 grid(static_cast<uint32_t>(blocks), (m.LayoutBuckets + dev::kBucketTile - 1) / dev::kBucketTile);
             // a model with one-hot buckets always reads them from the categorical matrix here
-            hipLaunchKernelGGL(dev::BinarizeRowsKernel, grid, dim3(256), 0, s, batch.Floats, batch.Stride,
-                               m.HasCats ? batch.Cats : nullptr, batch.CatStride, docCount, m.BinarizeTables(false),
-                               reinterpret_cast<uint32_t*>(bins));
+            LaunchBinarizeRows(m.MaxBucketValues, blocks, batch.Floats, batch.Stride, m.HasCats ? batch.Cats : nullptr,
+                               batch.CatStride, docCount, m.BinarizeTables(false), reinterpret_cast<uint32_t*>(bins), s);
             break;
         }
         case TFeatureBatch::FlatColumns: {
@@ -362,6 +401,27 @@ void THipEvaluator::QuantizeDevice(const TFeatureBatch& batch, size_t docCount, 
 }
 
 namespace {
+
+constexpr size_t kMaxTileLdsBytes = 160 * 1024;
+
+size_t TileLdsBytes(uint32_t buckets, int dchunk) {
+    return ((static_cast<size_t>(buckets) * dev::kDocsPerBlock + 7) & ~size_t(7)) +
+           static_cast<size_t>(dev::kDocsPerBlock) * dchunk * sizeof(double);
+}
+
+template <bool SEVEN_BIT, int DCHUNK>
+void LaunchEvalTile(const uint8_t* bins, size_t docCount, uint32_t buckets, const dev::TTreeTables& tt,
+                    uint32_t treeBegin, uint32_t treeEnd, double* out, hipStream_t s) {
+    const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
+    const size_t lds = TileLdsBytes(buckets, DCHUNK);
+    auto kernel = dev::EvalObliviousTileKernel<SEVEN_BIT, DCHUNK>;
+    if (lds > 64 * 1024) {
+        HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      static_cast<int>(lds)));
+    }
+    hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(blocks)), dim3(64 * dev::kTileWaves), lds, s,
+                       reinterpret_cast<const uint32_t*>(bins), docCount, buckets, tt, treeBegin, treeEnd, out);
+}
 
 template <int DCHUNK>
 void LaunchEval(bool oblivious, const uint8_t* bins, size_t docCount, uint32_t buckets, const dev::TTreeTables& tt,
@@ -399,6 +459,27 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
     CBAMD_ENSURE(bins != nullptr, "quantized buffer is null");
     const dev::TTreeTables tt = m.TreeTables();
     const uint32_t tb = static_cast<uint32_t>(treeStart), te = static_cast<uint32_t>(treeEnd);
+    const int dchunk = m.Dim == 1 ? 1 : m.Dim == 2 ? 2 : m.Dim <= 4 ? 4 : m.Dim <= 8 ? 8 : 16;
+    if (m.Oblivious && m.MaxDepth <= 8 && TileLdsBytes(m.LayoutBuckets, dchunk) <= kMaxTileLdsBytes) {
+        // byte-parallel kernel over an LDS tile of bins; 7-bit compares when every bin fits 7 bits
+        const bool sevenBit = !m.HasOneHot && m.MaxBucketValues <= 127;
+#define CBAMD_TILE(D)                                                                                     \
+    if (sevenBit) {                                                                                       \
+        LaunchEvalTile<true, D>(bins, docCount, m.LayoutBuckets, tt, tb, te, results, s);                 \
+    } else {                                                                                              \
+        LaunchEvalTile<false, D>(bins, docCount, m.LayoutBuckets, tt, tb, te, results, s);                \
+    }
+        switch (dchunk) {
+            case 1: CBAMD_TILE(1) break;
+            case 2: CBAMD_TILE(2) break;
+            case 4: CBAMD_TILE(4) break;
+            case 8: CBAMD_TILE(8) break;
+            default: CBAMD_TILE(16) break;
+        }
+#undef CBAMD_TILE
+        HIP_CHECK(hipGetLastError());
+        return;
+    }
     if (m.Dim == 1) {
         LaunchEval<1>(m.Oblivious, bins, docCount, m.LayoutBuckets, tt, tb, te, results, s);
     } else if (m.Dim == 2) {

@@ -46,11 +46,13 @@ struct TTreeTables {
     int Dim;
 };
 
-// number of sorted borders strictly below v; `borders` is padded with +inf up to 256 entries
+// number of sorted borders strictly below v; `borders` holds 1 << LOG2P entries, the real ones
+// first and +inf after them
+template <int LOG2P>
 __device__ __forceinline__ uint32_t CountBelow(const uint32_t* borders, float v) {
     uint32_t lo = 0;
 #pragma unroll
-    for (uint32_t step = 128; step >= 1; step >>= 1) {
+    for (uint32_t step = 1u << (LOG2P - 1); step >= 1; step >>= 1) {
         const uint32_t mid = lo + step;
         const float b = __uint_as_float(borders[mid - 1]);
         lo = (b < v) ? mid : lo;
@@ -68,24 +70,34 @@ __device__ __forceinline__ uint32_t OneHotBin(const uint32_t* values, uint32_t c
 
 // Row-major input: floats[doc * stride + column]; hashed categorical values either bit-cast in
 // the same row (cats == nullptr) or in cats[doc * catStride + column].
-// grid = (doc blocks, ceil(buckets / kBucketTile)), block = 256 threads.
+// One workgroup owns kBucketTile buckets and walks `blocksPerGroup` consecutive 256-document
+// blocks: the bucket values stay in LDS (1 << LOG2P slots per bucket, every bucket of the model
+// has fewer values than that), each block's 256 x 32 feature tile is fetched with row-contiguous
+// loads into registers one block ahead, transposed through LDS (rotated by the bucket index, so
+// both the row-wise fill and the column-wise read are bank-conflict free) and binarized by a
+// branch-free binary search; a wave writes the 256 bytes of one (block, bucket) pair at once.
+// grid = (ceil(doc blocks / blocksPerGroup), ceil(buckets / kBucketTile)), block = 256 threads.
+template <int LOG2P>
 __global__ __launch_bounds__(256) void BinarizeRowsKernel(const float* __restrict__ floats, size_t stride,
                                                           const int32_t* __restrict__ cats, size_t catStride,
                                                           size_t docCount, TBinarizeTables tab,
-                                                          uint32_t* __restrict__ bins) {
-    // 2 x 32 KB of LDS; the tile is rotated by the bucket index instead of padded so that both
-    // the row-wise fill and the column-wise read are bank-conflict free
-    __shared__ uint32_t sValues[kBucketTile][kMaxBucketValues];
+                                                          uint32_t blocksPerGroup, uint32_t* __restrict__ bins) {
+    constexpr uint32_t kSlots = 1u << LOG2P;
+    constexpr int kRowsPerPass = 256 / kBucketTile;        // 8 rows per pass of 256 threads
+    constexpr int kPasses = kDocsPerBlock / kRowsPerPass;  // 32 values per thread and block
+    __shared__ uint32_t sValues[kBucketTile * kSlots];
     __shared__ uint32_t sTile[kBucketTile][kDocsPerBlock];
 
     const uint32_t tid = threadIdx.x;
-    const size_t block = blockIdx.x;
     const uint32_t b0 = blockIdx.y * kBucketTile;
     const uint32_t nb = min(static_cast<uint32_t>(kBucketTile), tab.BucketCount - b0);
+    const size_t blockCount = (docCount + kDocsPerBlock - 1) / kDocsPerBlock;
+    const size_t blockBegin = static_cast<size_t>(blockIdx.x) * blocksPerGroup;
+    const size_t blockEnd = min(blockBegin + blocksPerGroup, blockCount);
 
-    for (uint32_t i = tid; i < kBucketTile * kMaxBucketValues; i += 256) {
-        const uint32_t bb = i / kMaxBucketValues, k = i % kMaxBucketValues;
-        uint32_t v = 0x7f800000u;  // +inf pads the border list
+    for (uint32_t i = tid; i < kBucketTile * kSlots; i += 256) {
+        const uint32_t bb = i >> LOG2P, k = i & (kSlots - 1);
+        uint32_t v = 0x7f800000u;  // +inf
         if (bb < nb) {
             const uint32_t off = tab.BucketOffset[b0 + bb];
             const uint32_t cnt = tab.BucketOffset[b0 + bb + 1] - off;
@@ -93,48 +105,71 @@ __global__ __launch_bounds__(256) void BinarizeRowsKernel(const float* __restric
                 v = tab.Values[off + k];
             }
         }
-        sValues[bb][k] = v;
+        sValues[i] = v;
     }
-    // tile load: consecutive threads take consecutive buckets of one document row
-    for (uint32_t i = tid; i < kBucketTile * kDocsPerBlock; i += 256) {
-        const uint32_t row = i / kBucketTile, bb = i % kBucketTile;
-        const size_t doc = block * kDocsPerBlock + row;
-        uint32_t v = 0;
-        if (bb < nb && doc < docCount) {
-            const uint32_t src = tab.BucketSrc[b0 + bb];
-            const bool oneHot = (tab.BucketFlags[b0 + bb] & kBucketFlagOneHot) != 0;
-            if (oneHot && cats != nullptr) {
-                v = static_cast<uint32_t>(cats[doc * catStride + src]);
-            } else {
-                v = __float_as_uint(floats[doc * stride + src]);
+
+    // role of this thread while loading: bucket `myB` of rows myRow0, myRow0 + 8, ...
+    const uint32_t myB = tid % kBucketTile;
+    const uint32_t myRow0 = tid / kBucketTile;
+    const bool myActive = myB < nb;
+    uint32_t mySrc = 0;
+    bool myFromCats = false;
+    if (myActive) {
+        mySrc = tab.BucketSrc[b0 + myB];
+        myFromCats = cats != nullptr && (tab.BucketFlags[b0 + myB] & kBucketFlagOneHot) != 0;
+    }
+    uint32_t regs[kPasses];
+    auto loadBlock = [&](size_t block) {
+#pragma unroll
+        for (int i = 0; i < kPasses; ++i) {
+            const size_t doc = block * kDocsPerBlock + myRow0 + i * kRowsPerPass;
+            uint32_t v = 0;
+            if (myActive && doc < docCount) {
+                v = myFromCats ? static_cast<uint32_t>(cats[doc * catStride + mySrc])
+                               : __float_as_uint(floats[doc * stride + mySrc]);
             }
+            regs[i] = v;
         }
-        sTile[bb][(row + bb) % kDocsPerBlock] = v;
-    }
-    __syncthreads();
+    };
 
     const uint32_t lane = tid & (kWave - 1);
     const uint32_t wave = tid / kWave;
-    for (uint32_t bb = wave; bb < nb; bb += 256 / kWave) {
-        const uint32_t flags = tab.BucketFlags[b0 + bb];
-        const uint32_t count = tab.BucketOffset[b0 + bb + 1] - tab.BucketOffset[b0 + bb];
-        uint32_t packed = 0;
+    if (blockBegin < blockEnd) {
+        loadBlock(blockBegin);
+    }
+    for (size_t block = blockBegin; block < blockEnd; ++block) {
+        __syncthreads();  // the previous block's tile has been consumed (and sValues is complete)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const uint32_t raw = sTile[bb][(j * kWave + lane + bb) % kDocsPerBlock];
-            uint32_t bin;
-            if (flags & kBucketFlagOneHot) {
-                bin = OneHotBin(sValues[bb], count, raw);
-            } else {
-                float v = __uint_as_float(raw);
-                if ((flags & kBucketFlagNanToInf) && isnan(v)) {
-                    v = __uint_as_float(0x7f800000u);
-                }
-                bin = CountBelow(sValues[bb], v);
-            }
-            packed |= bin << (8 * j);
+        for (int i = 0; i < kPasses; ++i) {
+            const uint32_t row = myRow0 + i * kRowsPerPass;
+            sTile[myB][(row + myB) % kDocsPerBlock] = regs[i];
         }
-        bins[(block * tab.BucketCount + b0 + bb) * kWave + lane] = packed;
+        __syncthreads();
+        if (block + 1 < blockEnd) {
+            loadBlock(block + 1);  // in flight while this block is binarized
+        }
+        for (uint32_t bb = wave; bb < nb; bb += 256 / kWave) {
+            const uint32_t flags = tab.BucketFlags[b0 + bb];
+            const uint32_t count = tab.BucketOffset[b0 + bb + 1] - tab.BucketOffset[b0 + bb];
+            const uint32_t* values = sValues + bb * kSlots;
+            uint32_t packed = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t raw = sTile[bb][(j * kWave + lane + bb) % kDocsPerBlock];
+                uint32_t bin;
+                if (flags & kBucketFlagOneHot) {
+                    bin = OneHotBin(values, count, raw);
+                } else {
+                    float v = __uint_as_float(raw);
+                    if ((flags & kBucketFlagNanToInf) && isnan(v)) {
+                        v = __uint_as_float(0x7f800000u);
+                    }
+                    bin = CountBelow<LOG2P>(values, v);
+                }
+                packed |= bin << (8 * j);
+            }
+            bins[(block * tab.BucketCount + b0 + bb) * kWave + lane] = packed;
+        }
     }
 }
 
@@ -180,7 +215,7 @@ __global__ __launch_bounds__(256) void BinarizeColumnsKernel(const float* __rest
             if ((flags & kBucketFlagNanToInf) && isnan(v)) {
                 v = __uint_as_float(0x7f800000u);
             }
-            bin = CountBelow(sValues[wave], v);
+            bin = CountBelow<8>(sValues[wave], v);
         }
         packed |= bin << (8 * j);
     }
@@ -258,6 +293,118 @@ __global__ __launch_bounds__(256) void EvalObliviousKernel(const uint32_t* __res
                 for (int k = 0; k < DCHUNK; ++k) {
                     if (DCHUNK == 1 || d0 + k < dim) {
                         out[doc * dim + d0 + k] = Finish(acc[j][k], tt.Scale, tt.Bias[d0 + k], addBias);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// Bit 7 of every byte of the result tells whether (bin ^ xorMask) >= splitIdx for the four
+// documents packed in `a`. SEVEN_BIT: all bins and split indexes are <= 127 and there is no xor
+// mask, so adding (128 - splitIdx) to every byte carries into bit 7 exactly when bin >= splitIdx.
+// Otherwise the full 8-bit unsigned compare is evaluated as the carry out of bin + ~splitIdx + 1,
+// taken per byte: carry = (x & ns) | ((x | ns) & low), low = (x & 0x7f) + (ns & 0x7f) + 1.
+template <bool SEVEN_BIT>
+__device__ __forceinline__ uint32_t CompareBytes(uint32_t a, uint32_t sp) {
+    const uint32_t s = sp >> 24;
+    if (SEVEN_BIT) {
+        return a + (128u - s) * 0x01010101u;
+    }
+    const uint32_t x = a ^ (((sp >> 16) & 0xffu) * 0x01010101u);
+    const uint32_t ns = (~s) & 0xffu;
+    const uint32_t low = (x & 0x7f7f7f7fu) + ((ns & 0x7fu) + 1u) * 0x01010101u;
+    const uint32_t nsr = ns * 0x01010101u;
+    return (x & nsr) | ((x | nsr) & low);
+}
+
+// Oblivious trees of depth <= 8 whose bins fit an LDS tile: one workgroup of kTileWaves waves per
+// 256-document block. The block's bins (buckets x 256 bytes) are copied to LDS once; the waves
+// share the tile and split the trees among themselves (tree t goes to wave t % kTileWaves), four
+// documents per lane. A level costs one LDS dword read, the byte-parallel compare and a
+// shift-in of the four result bits; the leaf index of a tree is complete after `depth` levels
+// (first split in bit 0). Per-wave partial sums (fp64) are reduced across waves in wave order
+// through LDS. grid = doc blocks, block = 64 * kTileWaves threads,
+// dynamic LDS = buckets * 256 (rounded up to 8) + 256 * DCHUNK * 8 bytes.
+constexpr int kTileWaves = 8;
+
+template <bool SEVEN_BIT, int DCHUNK>
+__global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousTileKernel(const uint32_t* __restrict__ bins,
+                                                                           size_t docCount, uint32_t bucketCount,
+                                                                           TTreeTables tt, uint32_t treeBegin,
+                                                                           uint32_t treeEnd,
+                                                                           double* __restrict__ out) {
+    extern __shared__ uint32_t sTile[];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const size_t block = blockIdx.x;
+    const uint32_t tileDwords = bucketCount * kWave;
+    const uint32_t* src = bins + block * tileDwords;
+    for (uint32_t i = tid; i < tileDwords; i += 64 * kTileWaves) {
+        sTile[i] = src[i];
+    }
+    const int dim = tt.Dim;
+    const bool addBias = treeBegin == 0;
+    const uint32_t* myTile = sTile + lane;
+    for (int d0 = 0; d0 < dim; d0 += DCHUNK) {
+        __syncthreads();  // tile is loaded / the previous chunk's accumulator has been read
+        double acc[4][DCHUNK];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int k = 0; k < DCHUNK; ++k) {
+                acc[j][k] = 0.0;
+            }
+        }
+        for (uint32_t t = treeBegin + wave; t < treeEnd; t += kTileWaves) {
+            const uint32_t first = tt.TreeStart[t];
+            const uint32_t depth = tt.TreeSize[t];
+            uint32_t idx4 = 0;
+            for (uint32_t d = 0; d < depth; ++d) {
+                const uint32_t sp = tt.Splits[first + d];
+                const uint32_t a = myTile[(sp & 0xffffu) * kWave];
+                const uint32_t r = CompareBytes<SEVEN_BIT>(a, sp);
+                idx4 = (r & 0x80808080u) | ((idx4 >> 1) & 0x7f7f7f7fu);
+            }
+            idx4 >>= (8 - depth);
+            const double* leaf = tt.Leaves + tt.FirstLeaf[t] + d0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const double* p = leaf + static_cast<size_t>((idx4 >> (8 * j)) & 0xffu) * dim;
+#pragma unroll
+                for (int k = 0; k < DCHUNK; ++k) {
+                    if (DCHUNK == 1 || d0 + k < dim) {
+                        acc[j][k] = __dadd_rn(acc[j][k], p[k]);
+                    }
+                }
+            }
+        }
+        // waves add their partial sums in wave order into an LDS accumulator behind the tile; the
+        // last wave finishes the values and writes them out
+        double* sRed = reinterpret_cast<double*>(sTile + ((tileDwords + 1) & ~1u));
+        for (uint32_t w = 0; w + 1 < kTileWaves; ++w) {
+            if (wave == w) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                    for (int k = 0; k < DCHUNK; ++k) {
+                        double* cell = sRed + (j * kWave + lane) * DCHUNK + k;
+                        *cell = (w == 0) ? acc[j][k] : __dadd_rn(*cell, acc[j][k]);
+                    }
+                }
+            }
+            __syncthreads();
+        }
+        if (wave == kTileWaves - 1) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const size_t doc = block * kDocsPerBlock + j * kWave + lane;
+#pragma unroll
+                for (int k = 0; k < DCHUNK; ++k) {
+                    if (doc < docCount && (DCHUNK == 1 || d0 + k < dim)) {
+                        const double sum = __dadd_rn(sRed[(j * kWave + lane) * DCHUNK + k], acc[j][k]);
+                        out[doc * dim + d0 + k] = Finish(sum, tt.Scale, tt.Bias[d0 + k], addBias);
                     }
                 }
             }
