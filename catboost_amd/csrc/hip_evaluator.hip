@@ -118,6 +118,8 @@ struct THipEvaluator::TImpl {
     // tree tables
     TDeviceVec<uint32_t> Splits, TreeStart, TreeSize, FirstLeaf, StepNodes, NodeToLeaf;
     TDeviceVec<double> Leaves, Bias;
+    TDeviceVec<uint32_t> PackedTrees;  // tile kernel: 16 dwords per oblivious tree of depth <= 8
+    bool PackedSevenBit = false;
     double Scale = 1.0;
     int Dim = 1;
     std::vector<double> HostBias;
@@ -290,6 +292,28 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId)
     m.NodeToLeaf.Upload(trees.NonSymmetricNodeIdToLeafId);
     m.Leaves.Upload(trees.LeafValues);
     m.Bias.Upload(trees.Bias);
+
+    if (m.Oblivious && m.MaxDepth <= 8) {
+        // 7-bit compares need every bin and split index to fit 7 bits and no xor mask
+        m.PackedSevenBit = !m.HasOneHot && m.MaxBucketValues <= 127;
+        std::vector<uint32_t> packed(trees.GetTreeCount() * dev::kPackedTreeDwords, 0);
+        for (size_t t = 0; t < trees.GetTreeCount(); ++t) {
+            uint32_t* row = packed.data() + t * dev::kPackedTreeDwords;
+            for (int d = 0; d < 8; ++d) {
+                if (d < trees.TreeSizes[t]) {
+                    const auto& rb = trees.RepackedBins[trees.TreeStartOffsets[t] + d];
+                    row[d] = m.PackedSevenBit
+                                 ? (static_cast<uint32_t>(rb.FeatureIndex) << 8) | (128u - rb.SplitIdx)
+                                 : (static_cast<uint32_t>(rb.FeatureIndex) << 16) |
+                                       (static_cast<uint32_t>(rb.XorMask) << 8) | rb.SplitIdx;
+                } else {
+                    row[d] = m.PackedSevenBit ? 0u : 0xffu;  // a level that is false for every bin
+                }
+            }
+            row[dev::kPackedFirstLeafSlot] = firstLeaf[t];
+        }
+        m.PackedTrees.Upload(packed);
+    }
 }
 
 THipEvaluator::~THipEvaluator() {
@@ -409,18 +433,54 @@ size_t TileLdsBytes(uint32_t buckets, int dchunk) {
            static_cast<size_t>(dev::kDocsPerBlock) * dchunk * sizeof(double);
 }
 
-template <bool SEVEN_BIT, int DCHUNK>
-void LaunchEvalTile(const uint8_t* bins, size_t docCount, uint32_t buckets, const dev::TTreeTables& tt,
-                    uint32_t treeBegin, uint32_t treeEnd, double* out, hipStream_t s) {
-    const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
-    const size_t lds = TileLdsBytes(buckets, DCHUNK);
-    auto kernel = dev::EvalObliviousTileKernel<SEVEN_BIT, DCHUNK>;
+struct TTileArgs {
+    const uint8_t* Bins;
+    size_t DocCount;
+    uint32_t Buckets;
+    const uint32_t* PackedTrees;
+    const double* Leaves;
+    const double* Bias;
+    double Scale;
+    int Dim;
+    uint32_t TreeBegin, TreeEnd;
+    double* Out;
+    hipStream_t Stream;
+};
+
+template <bool SEVEN_BIT, int MAXD, int DCHUNK>
+void LaunchEvalTile(const TTileArgs& a) {
+    const size_t blocks = (a.DocCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
+    const size_t lds = TileLdsBytes(a.Buckets, DCHUNK);
+    auto kernel = dev::EvalObliviousTileKernel<SEVEN_BIT, MAXD, DCHUNK>;
     if (lds > 64 * 1024) {
         HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       static_cast<int>(lds)));
     }
-    hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(blocks)), dim3(64 * dev::kTileWaves), lds, s,
-                       reinterpret_cast<const uint32_t*>(bins), docCount, buckets, tt, treeBegin, treeEnd, out);
+    hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(blocks)), dim3(64 * dev::kTileWaves), lds, a.Stream,
+                       reinterpret_cast<const uint32_t*>(a.Bins), a.DocCount, a.Buckets, a.PackedTrees, a.Leaves, a.Bias,
+                       a.Scale, a.Dim, a.TreeBegin, a.TreeEnd, a.Out);
+}
+
+template <bool SEVEN_BIT, int MAXD>
+void LaunchEvalTileD(int dchunk, const TTileArgs& a) {
+    switch (dchunk) {
+        case 1: LaunchEvalTile<SEVEN_BIT, MAXD, 1>(a); break;
+        case 2: LaunchEvalTile<SEVEN_BIT, MAXD, 2>(a); break;
+        case 4: LaunchEvalTile<SEVEN_BIT, MAXD, 4>(a); break;
+        case 8: LaunchEvalTile<SEVEN_BIT, MAXD, 8>(a); break;
+        default: LaunchEvalTile<SEVEN_BIT, MAXD, 16>(a); break;
+    }
+}
+
+template <bool SEVEN_BIT>
+void LaunchEvalTileM(uint32_t maxDepth, int dchunk, const TTileArgs& a) {
+    if (maxDepth <= 4) {
+        LaunchEvalTileD<SEVEN_BIT, 4>(dchunk, a);
+    } else if (maxDepth <= 6) {
+        LaunchEvalTileD<SEVEN_BIT, 6>(dchunk, a);
+    } else {
+        LaunchEvalTileD<SEVEN_BIT, 8>(dchunk, a);
+    }
 }
 
 template <int DCHUNK>
@@ -461,22 +521,14 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
     const uint32_t tb = static_cast<uint32_t>(treeStart), te = static_cast<uint32_t>(treeEnd);
     const int dchunk = m.Dim == 1 ? 1 : m.Dim == 2 ? 2 : m.Dim <= 4 ? 4 : m.Dim <= 8 ? 8 : 16;
     if (m.Oblivious && m.MaxDepth <= 8 && TileLdsBytes(m.LayoutBuckets, dchunk) <= kMaxTileLdsBytes) {
-        // byte-parallel kernel over an LDS tile of bins; 7-bit compares when every bin fits 7 bits
-        const bool sevenBit = !m.HasOneHot && m.MaxBucketValues <= 127;
-#define CBAMD_TILE(D)                                                                                     \
-    if (sevenBit) {                                                                                       \
-        LaunchEvalTile<true, D>(bins, docCount, m.LayoutBuckets, tt, tb, te, results, s);                 \
-    } else {                                                                                              \
-        LaunchEvalTile<false, D>(bins, docCount, m.LayoutBuckets, tt, tb, te, results, s);                \
-    }
-        switch (dchunk) {
-            case 1: CBAMD_TILE(1) break;
-            case 2: CBAMD_TILE(2) break;
-            case 4: CBAMD_TILE(4) break;
-            case 8: CBAMD_TILE(8) break;
-            default: CBAMD_TILE(16) break;
+        // byte-parallel kernel over an LDS tile of bins
+        const TTileArgs args{bins, docCount, m.LayoutBuckets, m.PackedTrees.Get(), m.Leaves.Get(), m.Bias.Get(),
+                             m.Scale, m.Dim, tb, te, results, s};
+        if (m.PackedSevenBit) {
+            LaunchEvalTileM<true>(m.MaxDepth, dchunk, args);
+        } else {
+            LaunchEvalTileM<false>(m.MaxDepth, dchunk, args);
         }
-#undef CBAMD_TILE
         HIP_CHECK(hipGetLastError());
         return;
     }

@@ -300,40 +300,70 @@ __global__ __launch_bounds__(256) void EvalObliviousKernel(const uint32_t* __res
     }
 }
 
+// Packed tree table of the tile kernel: 16 dwords per tree. Slots 0..7 hold the tree's levels
+// (slot d = split d, unused levels padded with a split that is false for every bin), slot 8 the
+// index of the tree's first leaf value. A level is
+//   7-bit form: bucket << 8 | (128 - splitIdx)          (all bins and split indexes <= 127, no xor)
+//   8-bit form: bucket << 16 | xorMask << 8 | splitIdx
+constexpr int kPackedTreeDwords = 16;
+constexpr int kPackedFirstLeafSlot = 8;
+
 // Bit 7 of every byte of the result tells whether (bin ^ xorMask) >= splitIdx for the four
-// documents packed in `a`. SEVEN_BIT: all bins and split indexes are <= 127 and there is no xor
-// mask, so adding (128 - splitIdx) to every byte carries into bit 7 exactly when bin >= splitIdx.
-// Otherwise the full 8-bit unsigned compare is evaluated as the carry out of bin + ~splitIdx + 1,
-// taken per byte: carry = (x & ns) | ((x | ns) & low), low = (x & 0x7f) + (ns & 0x7f) + 1.
+// documents packed in `a`. 7-bit form: adding (128 - splitIdx) to every byte carries into bit 7
+// exactly when bin >= splitIdx. 8-bit form: the unsigned compare is the carry out of
+// x + ~splitIdx + 1 taken per byte, x = bin ^ xorMask:
+//   carry = (x & ns) | ((x | ns) & low), ns = ~splitIdx, low = (x & 0x7f) + (ns & 0x7f) + 1.
 template <bool SEVEN_BIT>
-__device__ __forceinline__ uint32_t CompareBytes(uint32_t a, uint32_t sp) {
-    const uint32_t s = sp >> 24;
+__device__ __forceinline__ uint32_t CompareBytes(uint32_t a, uint32_t level) {
     if (SEVEN_BIT) {
-        return a + (128u - s) * 0x01010101u;
+        return a + (level & 0xffu) * 0x01010101u;
     }
-    const uint32_t x = a ^ (((sp >> 16) & 0xffu) * 0x01010101u);
+    const uint32_t s = level & 0xffu;
+    const uint32_t x = a ^ (((level >> 8) & 0xffu) * 0x01010101u);
     const uint32_t ns = (~s) & 0xffu;
     const uint32_t low = (x & 0x7f7f7f7fu) + ((ns & 0x7fu) + 1u) * 0x01010101u;
     const uint32_t nsr = ns * 0x01010101u;
     return (x & nsr) | ((x | nsr) & low);
 }
 
-// Oblivious trees of depth <= 8 whose bins fit an LDS tile: one workgroup of kTileWaves waves per
-// 256-document block. The block's bins (buckets x 256 bytes) are copied to LDS once; the waves
-// share the tile and split the trees among themselves (tree t goes to wave t % kTileWaves), four
-// documents per lane. A level costs one LDS dword read, the byte-parallel compare and a
-// shift-in of the four result bits; the leaf index of a tree is complete after `depth` levels
-// (first split in bit 0). Per-wave partial sums (fp64) are reduced across waves in wave order
-// through LDS. grid = doc blocks, block = 64 * kTileWaves threads,
+// byte offset of a level's bucket inside the LDS tile (256 bytes per bucket)
+template <bool SEVEN_BIT>
+__device__ __forceinline__ uint32_t LevelTileOffset(uint32_t level) {
+    return SEVEN_BIT ? (level & 0xffffff00u) : ((level >> 16) << 8);
+}
+
+// Leaf indexes of one tree for the four documents of a lane, one byte each: MAXD levels, every
+// one an LDS dword read, a byte-parallel compare and a shift-in of the four result bits (the
+// first split ends up in bit 0).
+template <bool SEVEN_BIT, int MAXD>
+__device__ __forceinline__ uint32_t TreeIndexes(const uint8_t* laneTile, uint32_t packedRow) {
+    uint32_t idx4 = 0;
+#pragma unroll
+    for (int d = 0; d < MAXD; ++d) {
+        const uint32_t level = __builtin_amdgcn_readlane(packedRow, d);
+        const uint32_t a = *reinterpret_cast<const uint32_t*>(laneTile + LevelTileOffset<SEVEN_BIT>(level));
+        const uint32_t r = CompareBytes<SEVEN_BIT>(a, level);
+        idx4 = (r & 0x80808080u) | ((idx4 >> 1) & 0x7f7f7f7fu);
+    }
+    return idx4 >> (8 - MAXD);
+}
+
+// Oblivious trees of depth <= MAXD <= 8 whose bins fit an LDS tile: one workgroup of kTileWaves
+// waves per 256-document block. The block's bins (buckets x 256 bytes) are copied to LDS once;
+// the waves share the tile and split the trees among themselves (tree t goes to wave
+// t % kTileWaves), four documents per lane. A wave fetches a tree's packed row with one 64-byte
+// load (one tree ahead) and broadcasts the levels from it. Leaf values are gathered from global
+// memory (the whole table stays in L2). Per-wave partial sums (fp64) are added in wave order
+// through an LDS accumulator behind the tile, and the last wave writes the results.
+// grid = doc blocks, block = 64 * kTileWaves threads,
 // dynamic LDS = buckets * 256 (rounded up to 8) + 256 * DCHUNK * 8 bytes.
 constexpr int kTileWaves = 8;
 
-template <bool SEVEN_BIT, int DCHUNK>
-__global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousTileKernel(const uint32_t* __restrict__ bins,
-                                                                           size_t docCount, uint32_t bucketCount,
-                                                                           TTreeTables tt, uint32_t treeBegin,
-                                                                           uint32_t treeEnd,
-                                                                           double* __restrict__ out) {
+template <bool SEVEN_BIT, int MAXD, int DCHUNK>
+__global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousTileKernel(
+    const uint32_t* __restrict__ bins, size_t docCount, uint32_t bucketCount, const uint32_t* __restrict__ packedTrees,
+    const double* __restrict__ leaves, const double* __restrict__ bias, double scale, int dim, uint32_t treeBegin,
+    uint32_t treeEnd, double* __restrict__ out) {
     extern __shared__ uint32_t sTile[];
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & (kWave - 1);
@@ -344,9 +374,10 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousTileKernel(const
     for (uint32_t i = tid; i < tileDwords; i += 64 * kTileWaves) {
         sTile[i] = src[i];
     }
-    const int dim = tt.Dim;
     const bool addBias = treeBegin == 0;
-    const uint32_t* myTile = sTile + lane;
+    const uint8_t* laneTile = reinterpret_cast<const uint8_t*>(sTile) + lane * 4;
+    const uint32_t slot = lane & (kPackedTreeDwords - 1);
+    double* sRed = reinterpret_cast<double*>(sTile + ((tileDwords + 1) & ~1u));
     for (int d0 = 0; d0 < dim; d0 += DCHUNK) {
         __syncthreads();  // tile is loaded / the previous chunk's accumulator has been read
         double acc[4][DCHUNK];
@@ -357,32 +388,32 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousTileKernel(const
                 acc[j][k] = 0.0;
             }
         }
-        for (uint32_t t = treeBegin + wave; t < treeEnd; t += kTileWaves) {
-            const uint32_t first = tt.TreeStart[t];
-            const uint32_t depth = tt.TreeSize[t];
-            uint32_t idx4 = 0;
-            for (uint32_t d = 0; d < depth; ++d) {
-                const uint32_t sp = tt.Splits[first + d];
-                const uint32_t a = myTile[(sp & 0xffffu) * kWave];
-                const uint32_t r = CompareBytes<SEVEN_BIT>(a, sp);
-                idx4 = (r & 0x80808080u) | ((idx4 >> 1) & 0x7f7f7f7fu);
-            }
-            idx4 >>= (8 - depth);
-            const double* leaf = tt.Leaves + tt.FirstLeaf[t] + d0;
+        uint32_t t = treeBegin + wave;
+        uint32_t row = t < treeEnd ? packedTrees[static_cast<size_t>(t) * kPackedTreeDwords + slot] : 0;
+        while (t < treeEnd) {
+            const uint32_t tNext = t + kTileWaves;
+            const uint32_t rowNext =
+                tNext < treeEnd ? packedTrees[static_cast<size_t>(tNext) * kPackedTreeDwords + slot] : 0;
+            const uint32_t idx4 = TreeIndexes<SEVEN_BIT, MAXD>(laneTile, row);
+            const uint32_t firstLeaf = __builtin_amdgcn_readlane(row, kPackedFirstLeafSlot);
+            const double* leaf = leaves + firstLeaf + d0;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const double* p = leaf + static_cast<size_t>((idx4 >> (8 * j)) & 0xffu) * dim;
+                // DCHUNK == 1 is only instantiated for one-dimensional models
+                const uint32_t leafIdx = (idx4 >> (8 * j)) & 0xffu;
+                const uint32_t li = DCHUNK == 1 ? leafIdx : leafIdx * static_cast<uint32_t>(dim);
 #pragma unroll
                 for (int k = 0; k < DCHUNK; ++k) {
                     if (DCHUNK == 1 || d0 + k < dim) {
-                        acc[j][k] = __dadd_rn(acc[j][k], p[k]);
+                        acc[j][k] = __dadd_rn(acc[j][k], leaf[li + k]);
                     }
                 }
             }
+            t = tNext;
+            row = rowNext;
         }
-        // waves add their partial sums in wave order into an LDS accumulator behind the tile; the
-        // last wave finishes the values and writes them out
-        double* sRed = reinterpret_cast<double*>(sTile + ((tileDwords + 1) & ~1u));
+        // waves add their partial sums in wave order into the LDS accumulator; the last wave
+        // finishes the values and writes them out
         for (uint32_t w = 0; w + 1 < kTileWaves; ++w) {
             if (wave == w) {
 #pragma unroll
@@ -404,7 +435,7 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousTileKernel(const
                 for (int k = 0; k < DCHUNK; ++k) {
                     if (doc < docCount && (DCHUNK == 1 || d0 + k < dim)) {
                         const double sum = __dadd_rn(sRed[(j * kWave + lane) * DCHUNK + k], acc[j][k]);
-                        out[doc * dim + d0 + k] = Finish(sum, tt.Scale, tt.Bias[d0 + k], addBias);
+                        out[doc * dim + d0 + k] = Finish(sum, scale, bias[d0 + k], addBias);
                     }
                 }
             }
