@@ -120,6 +120,7 @@ struct THipEvaluator::TImpl {
     TDeviceVec<double> Leaves, Bias;
     TDeviceVec<uint32_t> PackedTrees;  // tile kernel: 16 dwords per oblivious tree of depth <= 8
     bool PackedSevenBit = false;
+    bool LeavesPairAligned = false;  // every tree's first leaf value sits at an even index
     double Scale = 1.0;
     int Dim = 1;
     std::vector<double> HostBias;
@@ -290,7 +291,12 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId)
     m.FirstLeaf.Upload(firstLeaf);
     m.StepNodes.Upload(steps);
     m.NodeToLeaf.Upload(trees.NonSymmetricNodeIdToLeafId);
-    m.Leaves.Upload(trees.LeafValues);
+    {
+        // the tile kernel copies (1 << 8) * dim doubles per tree: keep that much readable behind the end
+        std::vector<double> padded = trees.LeafValues;
+        padded.resize(padded.size() + 256 * static_cast<size_t>(trees.ApproxDimension), 0.0);
+        m.Leaves.Upload(padded);
+    }
     m.Bias.Upload(trees.Bias);
 
     if (m.Oblivious && m.MaxDepth <= 8) {
@@ -313,6 +319,10 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId)
             row[dev::kPackedFirstLeafSlot] = firstLeaf[t];
         }
         m.PackedTrees.Upload(packed);
+        m.LeavesPairAligned = true;
+        for (uint32_t f : firstLeaf) {
+            m.LeavesPairAligned = m.LeavesPairAligned && (f % 2 == 0);
+        }
     }
 }
 
@@ -433,6 +443,11 @@ size_t TileLdsBytes(uint32_t buckets, int dchunk) {
            static_cast<size_t>(dev::kDocsPerBlock) * dchunk * sizeof(double);
 }
 
+// LDS of the per-wave leaf regions of the tile kernel
+size_t TileLeafLdsBytes(int maxd, int dim) {
+    return static_cast<size_t>(dev::kTileWaves) * (size_t(1) << maxd) * dim * sizeof(double);
+}
+
 struct TTileArgs {
     const uint8_t* Bins;
     size_t DocCount;
@@ -445,13 +460,14 @@ struct TTileArgs {
     uint32_t TreeBegin, TreeEnd;
     double* Out;
     hipStream_t Stream;
+    bool LeavesPairAligned;
 };
 
-template <bool SEVEN_BIT, int MAXD, int DCHUNK>
-void LaunchEvalTile(const TTileArgs& a) {
+template <bool SEVEN_BIT, int MAXD, int DCHUNK, bool LEAF_LDS>
+void LaunchEvalTileL(const TTileArgs& a) {
     const size_t blocks = (a.DocCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
-    const size_t lds = TileLdsBytes(a.Buckets, DCHUNK);
-    auto kernel = dev::EvalObliviousTileKernel<SEVEN_BIT, MAXD, DCHUNK>;
+    const size_t lds = TileLdsBytes(a.Buckets, DCHUNK) + (LEAF_LDS ? TileLeafLdsBytes(MAXD, a.Dim) : 0);
+    auto kernel = dev::EvalObliviousTileKernel<SEVEN_BIT, MAXD, DCHUNK, LEAF_LDS>;
     if (lds > 64 * 1024) {
         HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       static_cast<int>(lds)));
@@ -459,6 +475,18 @@ void LaunchEvalTile(const TTileArgs& a) {
     hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(blocks)), dim3(64 * dev::kTileWaves), lds, a.Stream,
                        reinterpret_cast<const uint32_t*>(a.Bins), a.DocCount, a.Buckets, a.PackedTrees, a.Leaves, a.Bias,
                        a.Scale, a.Dim, a.TreeBegin, a.TreeEnd, a.Out);
+}
+
+template <bool SEVEN_BIT, int MAXD, int DCHUNK>
+void LaunchEvalTile(const TTileArgs& a) {
+    // leaf values go through LDS when the tile, the accumulator and the leaf regions leave room
+    // for at least two workgroups per CU
+    const size_t withLeaves = TileLdsBytes(a.Buckets, DCHUNK) + TileLeafLdsBytes(MAXD, a.Dim);
+    if (a.LeavesPairAligned && withLeaves <= 80 * 1024) {
+        LaunchEvalTileL<SEVEN_BIT, MAXD, DCHUNK, true>(a);
+    } else {
+        LaunchEvalTileL<SEVEN_BIT, MAXD, DCHUNK, false>(a);
+    }
 }
 
 template <bool SEVEN_BIT, int MAXD>
@@ -523,7 +551,7 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
     if (m.Oblivious && m.MaxDepth <= 8 && TileLdsBytes(m.LayoutBuckets, dchunk) <= kMaxTileLdsBytes) {
         // byte-parallel kernel over an LDS tile of bins
         const TTileArgs args{bins, docCount, m.LayoutBuckets, m.PackedTrees.Get(), m.Leaves.Get(), m.Bias.Get(),
-                             m.Scale, m.Dim, tb, te, results, s};
+                             m.Scale, m.Dim, tb, te, results, s, m.LeavesPairAligned};
         if (m.PackedSevenBit) {
             LaunchEvalTileM<true>(m.MaxDepth, dchunk, args);
         } else {

@@ -352,14 +352,17 @@ __device__ __forceinline__ uint32_t TreeIndexes(const uint8_t* laneTile, uint32_
 // waves per 256-document block. The block's bins (buckets x 256 bytes) are copied to LDS once;
 // the waves share the tile and split the trees among themselves (tree t goes to wave
 // t % kTileWaves), four documents per lane. A wave fetches a tree's packed row with one 64-byte
-// load (one tree ahead) and broadcasts the levels from it. Leaf values are gathered from global
-// memory (the whole table stays in L2). Per-wave partial sums (fp64) are added in wave order
-// through an LDS accumulator behind the tile, and the last wave writes the results.
-// grid = doc blocks, block = 64 * kTileWaves threads,
-// dynamic LDS = buckets * 256 (rounded up to 8) + 256 * DCHUNK * 8 bytes.
+// load (one tree ahead) and broadcasts the levels from it. Per-wave partial sums (fp64) are added
+// in wave order through an LDS accumulator behind the tile, and the last wave writes the results.
+// grid = doc blocks, block = 64 * kTileWaves threads, dynamic LDS = buckets * 256 (rounded up to
+// 8) + 256 * DCHUNK * 8 [+ kTileWaves * (1 << MAXD) * dim * 8 with LEAF_LDS] bytes.
 constexpr int kTileWaves = 8;
 
-template <bool SEVEN_BIT, int MAXD, int DCHUNK>
+// LEAF_LDS: every wave copies the leaf values of its current tree ((1 << MAXD) * dim doubles)
+// into a private LDS region with row-contiguous 16-byte loads and gathers from there; otherwise
+// leaf values are gathered straight from global memory. The leaves array must be readable for
+// (1 << MAXD) * dim doubles past the first leaf of the last tree.
+template <bool SEVEN_BIT, int MAXD, int DCHUNK, bool LEAF_LDS>
 __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousTileKernel(
     const uint32_t* __restrict__ bins, size_t docCount, uint32_t bucketCount, const uint32_t* __restrict__ packedTrees,
     const double* __restrict__ leaves, const double* __restrict__ bias, double scale, int dim, uint32_t treeBegin,
@@ -378,6 +381,9 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousTileKernel(
     const uint8_t* laneTile = reinterpret_cast<const uint8_t*>(sTile) + lane * 4;
     const uint32_t slot = lane & (kPackedTreeDwords - 1);
     double* sRed = reinterpret_cast<double*>(sTile + ((tileDwords + 1) & ~1u));
+    // per-wave leaf region behind the accumulator; treeDoubles is a multiple of 2
+    const uint32_t treeDoubles = (1u << MAXD) * static_cast<uint32_t>(dim);
+    double* sLeaf = sRed + kDocsPerBlock * DCHUNK + wave * treeDoubles;
     for (int d0 = 0; d0 < dim; d0 += DCHUNK) {
         __syncthreads();  // tile is loaded / the previous chunk's accumulator has been read
         double acc[4][DCHUNK];
@@ -388,20 +394,65 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousTileKernel(
                 acc[j][k] = 0.0;
             }
         }
+        // one-dimensional models: the leaf values of a tree are (1 << MAXD) doubles, i.e. at most two
+        // 16-byte pairs per lane, fetched one tree ahead into registers
+        constexpr uint32_t kTreePairs = (1u << MAXD) / 2;
+        double2 pref0 = {0.0, 0.0}, pref1 = {0.0, 0.0};
+#define CBAMD_FETCH_LEAVES(firstLeafValue)                                                        \
+    do {                                                                                          \
+        const double2* src2 = reinterpret_cast<const double2*>(leaves + (firstLeafValue));        \
+        if (kTreePairs >= kWave || lane < kTreePairs) {                                           \
+            pref0 = src2[lane];                                                                   \
+        }                                                                                         \
+        if (kTreePairs > kWave) {                                                                 \
+            pref1 = src2[kWave + lane];                                                           \
+        }                                                                                         \
+    } while (0)
+        // packed rows are fetched two trees ahead so that the next tree's row has arrived by the
+        // time its leaf values are requested
+#define CBAMD_FETCH_ROW(tree) \
+    ((tree) < treeEnd ? packedTrees[static_cast<size_t>(tree) * kPackedTreeDwords + slot] : 0u)
         uint32_t t = treeBegin + wave;
-        uint32_t row = t < treeEnd ? packedTrees[static_cast<size_t>(t) * kPackedTreeDwords + slot] : 0;
+        uint32_t row = CBAMD_FETCH_ROW(t);
+        uint32_t rowNext = CBAMD_FETCH_ROW(t + kTileWaves);
+        if (LEAF_LDS && DCHUNK == 1 && t < treeEnd) {
+            CBAMD_FETCH_LEAVES(__builtin_amdgcn_readlane(row, kPackedFirstLeafSlot));
+        }
         while (t < treeEnd) {
             const uint32_t tNext = t + kTileWaves;
-            const uint32_t rowNext =
-                tNext < treeEnd ? packedTrees[static_cast<size_t>(tNext) * kPackedTreeDwords + slot] : 0;
-            const uint32_t idx4 = TreeIndexes<SEVEN_BIT, MAXD>(laneTile, row);
+            const uint32_t rowNext2 = CBAMD_FETCH_ROW(tNext + kTileWaves);
             const uint32_t firstLeaf = __builtin_amdgcn_readlane(row, kPackedFirstLeafSlot);
-            const double* leaf = leaves + firstLeaf + d0;
+            const double* leaf = leaves + firstLeaf;
+            if (LEAF_LDS) {
+                // publish this tree's leaf values in the wave's region; the previous tree's gathers
+                // were issued before these stores and LDS serves one wave's requests in order
+                double2* dst2 = reinterpret_cast<double2*>(sLeaf);
+                if (DCHUNK == 1) {
+                    if (kTreePairs >= kWave || lane < kTreePairs) {
+                        dst2[lane] = pref0;
+                    }
+                    if (kTreePairs > kWave) {
+                        dst2[kWave + lane] = pref1;
+                    }
+                    if (tNext < treeEnd) {
+                        CBAMD_FETCH_LEAVES(__builtin_amdgcn_readlane(rowNext, kPackedFirstLeafSlot));
+                    }
+                } else {
+                    const double2* src2 = reinterpret_cast<const double2*>(leaf);
+                    for (uint32_t i = lane; i < treeDoubles / 2; i += kWave) {
+                        dst2[i] = src2[i];
+                    }
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                leaf = sLeaf;
+            }
+            const uint32_t idx4 = TreeIndexes<SEVEN_BIT, MAXD>(laneTile, row);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 // DCHUNK == 1 is only instantiated for one-dimensional models
                 const uint32_t leafIdx = (idx4 >> (8 * j)) & 0xffu;
-                const uint32_t li = DCHUNK == 1 ? leafIdx : leafIdx * static_cast<uint32_t>(dim);
+                const uint32_t li = (DCHUNK == 1 ? leafIdx : leafIdx * static_cast<uint32_t>(dim)) + d0;
 #pragma unroll
                 for (int k = 0; k < DCHUNK; ++k) {
                     if (DCHUNK == 1 || d0 + k < dim) {
@@ -409,9 +460,15 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousTileKernel(
                     }
                 }
             }
+            if (LEAF_LDS) {
+                __builtin_amdgcn_wave_barrier();
+            }
             t = tNext;
             row = rowNext;
+            rowNext = rowNext2;
         }
+#undef CBAMD_FETCH_ROW
+#undef CBAMD_FETCH_LEAVES
         // waves add their partial sums in wave order into the LDS accumulator; the last wave
         // finishes the values and writes them out
         for (uint32_t w = 0; w + 1 < kTileWaves; ++w) {
