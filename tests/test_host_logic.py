@@ -1,0 +1,222 @@
+"""Host-side logic of libcatboostmodel.so that needs no GPU: exported symbols, .cbm reader /
+writer, model builders, hashes, error reporting."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+import catboost_amd as cb
+from oracle import model_builder as mb
+from oracle.cbm_reader import read_cbm, read_cbm_file
+from tests import refmodels as rm
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+# export list of the reference library (catboost/libs/model_interface/calcer.exports)
+REFERENCE_EXPORTS = """GetErrorString ModelCalcerCreate ModelCalcerDelete DataWrapperCreate DataWrapperDelete
+AddFloatFeatures AddCatFeatures AddTextFeatures AddEmbeddingFeatures BuildDataProvider LoadFullModelFromFile
+LoadFullModelFromBuffer LoadFullModelZeroCopy EnableGPUEvaluation GetSupportedEvaluatorTypes SetPredictionType
+SetPredictionTypeString CalcModelPrediction CalcModelPredictionStaged CalcModelPredictionText
+CalcModelPredictionTextStaged CalcModelPredictionTextAndEmbeddings CalcModelPredictionTextAndEmbeddingsStaged
+CalcModelPredictionSingle CalcModelPredictionSingleStaged CalcModelPredictionFlat CalcModelPredictionFlatStaged
+CalcModelPredictionFlatTransposed CalcModelPredictionFlatTransposedStaged CalcModelPredictionWithHashedCatFeatures
+CalcModelPredictionWithHashedCatFeaturesAndTextFeatures
+CalcModelPredictionWithHashedCatFeaturesAndTextAndEmbeddingFeatures PredictSpecificClassFlat PredictSpecificClass
+PredictSpecificClassText PredictSpecificClassTextAndEmbeddings PredictSpecificClassSingle
+PredictSpecificClassWithHashedCatFeatures PredictSpecificClassWithHashedCatFeaturesAndTextFeatures
+PredictSpecificClassWithHashedCatFeaturesAndTextAndEmbeddingFeatures GetStringCatFeatureHash GetIntegerCatFeatureHash
+GetFloatFeaturesCount GetCatFeaturesCount GetTextFeaturesCount GetEmbeddingFeaturesCount GetTreeCount
+GetDimensionsCount GetPredictionDimensionsCount CheckModelMetadataHasKey GetModelInfoValueSize GetModelInfoValue
+GetModelUsedFeaturesNames GetCatFeatureIndices GetFloatFeatureIndices GetTextFeatureIndices
+GetEmbeddingFeatureIndices""".split()
+
+
+def _declared_functions(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b((?:CbHip|[A-Z])[A-Za-z0-9]+)\s*\(", text)) - {"CATBOOST_API"})
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(cb.library_path())
+    declared = _declared_functions("c_api.h") + _declared_functions("cb_hip_evaluator.h")
+    assert len(declared) > 80
+    for name in declared + REFERENCE_EXPORTS:
+        assert hasattr(lib, name), name
+    assert len(REFERENCE_EXPORTS) == 57
+    assert set(REFERENCE_EXPORTS) <= set(_declared_functions("c_api.h"))
+
+
+def test_hash_known_answers_through_c_api():
+    for s, expected in rm.HASH_KNOWN_ANSWERS.items():
+        assert cb.string_cat_feature_hash(s) == expected
+    for v in (0, 7, -12, 10 ** 15):
+        assert cb.integer_cat_feature_hash(v) == cb.string_cat_feature_hash(str(v))
+    # every length class of the hash (0, 1-3, 4-8, 9-16, 17-32, 33-64, >64 bytes) against the oracle's copy
+    from oracle.oracle import cat_feature_hash_signed
+    rng = np.random.default_rng(0)
+    for n in list(range(0, 70)) + [127, 128, 129, 200, 1000]:
+        s = bytes(rng.integers(1, 256, size=n, dtype=np.uint8))
+        assert cb.string_cat_feature_hash(s) == cat_feature_hash_signed(s)
+
+
+@pytest.mark.parametrize("name", ["numeric_only_model.cbm", "features_num__dataset_querywise.cbm",
+                                  "rust_tmp_model.cbm", "iris_model.cbm", "boston_housing_model.cbm"])
+def test_cbm_load_save_roundtrip(golden_dir, name):
+    path = os.path.join(golden_dir, name)
+    ref = read_cbm_file(path)
+    m = cb.ModelCalcer(path)
+    got = read_cbm(m.save_to_buffer())
+    for k in ("approx_dimension", "tree_splits", "tree_sizes", "tree_start_offsets", "leaf_values", "leaf_weights",
+              "step_nodes", "node_id_to_leaf_id", "scale", "bias", "info"):
+        np.testing.assert_array_equal(np.asarray(got[k]), np.asarray(ref[k]), err_msg=k)
+    assert len(got["float_features"]) == len(ref["float_features"])
+    for a, b in zip(got["float_features"], ref["float_features"]):
+        np.testing.assert_array_equal(a["borders"], b["borders"])
+        assert {k: a[k] for k in a if k != "borders"} == {k: b[k] for k in b if k != "borders"}
+    assert got["cat_features"] == ref["cat_features"]
+    for a, b in zip(got["one_hot_features"], ref["one_hot_features"]):
+        assert a["cat_index"] == b["cat_index"]
+        np.testing.assert_array_equal(a["values"], b["values"])
+    # the writer always stores the recomputed repacked bins (TModelTrees::FBSerialize)
+    assert got["repacked_bins_in_file"].size == got["tree_splits"].size
+    if ref["repacked_bins_in_file"].size:
+        np.testing.assert_array_equal(got["repacked_bins_in_file"], ref["repacked_bins_in_file"])
+    # a second generation is byte-identical
+    assert cb.ModelCalcer(buffer=m.save_to_buffer()).save_to_buffer() == m.save_to_buffer()
+
+
+def test_model_description_getters(golden_dir):
+    m = cb.ModelCalcer(os.path.join(golden_dir, "rust_tmp_model.cbm"))
+    assert (m.tree_count, m.dimensions_count, m.float_features_count, m.cat_features_count) == (1000, 1, 3, 1)
+    assert m.get_float_feature_indices() == [0, 1, 3] and m.get_cat_feature_indices() == [2]
+    assert m.get_used_features_names()[2] == "wind direction"
+    assert m.check_metadata_has_key("params") and not m.check_metadata_has_key("nope")
+    assert m.get_metadata_key_value("params").startswith("{")
+    assert m.prediction_dimensions_count == 1
+    iris = cb.ModelCalcer(os.path.join(golden_dir, "iris_model.cbm"))
+    assert iris.prediction_dimensions_count == 3
+    iris.set_prediction_type("Class")
+    assert iris.prediction_dimensions_count == 1
+    with pytest.raises(cb.CatBoostError):
+        iris.set_prediction_type("NoSuchType")
+
+
+def test_loader_rejects_bad_input(golden_dir):
+    with pytest.raises(cb.CatBoostError, match="Incorrect model file descriptor"):
+        cb.ModelCalcer(os.path.join(golden_dir, "not_a_model.cbm"))
+    with pytest.raises(cb.CatBoostError, match="can't open"):
+        cb.ModelCalcer(os.path.join(golden_dir, "no_such_file.cbm"))
+    data = open(os.path.join(golden_dir, "numeric_only_model.cbm"), "rb").read()
+    for cut in (3, 7, 8, 20, len(data) // 2, len(data) - 1):
+        with pytest.raises(cb.CatBoostError):
+            cb.ModelCalcer(buffer=data[:cut])
+    # flip bytes inside the flatbuffer: must fail cleanly or load, never crash
+    rng = np.random.default_rng(1)
+    for _ in range(200):
+        corrupted = bytearray(data)
+        for pos in rng.integers(8, len(data), size=4):
+            corrupted[pos] = int(rng.integers(0, 256))
+        try:
+            cb.ModelCalcer(buffer=bytes(corrupted))
+        except cb.CatBoostError:
+            pass
+    for name in ("categoric_only_model.cbm", "jvm_model_with_ctr.cbm", "cloudness_small.cbm"):
+        with pytest.raises(cb.CatBoostError, match="not supported"):
+            cb.ModelCalcer(os.path.join(golden_dir, name))
+
+
+def test_oblivious_builder_matches_oracle_builder():
+    rng = np.random.default_rng(11)
+    ffs = [mb.float_feature(i, i, has_nans=bool(i % 2), nan_treatment=i % 3) for i in range(5)]
+    cfs = [mb.cat_feature(0, 5), mb.cat_feature(1, 6)]
+    cands = [np.unique(rng.normal(size=30).astype(np.float32)) for _ in range(5)]
+    trees = []
+    for _ in range(40):
+        splits = []
+        for _ in range(int(rng.integers(0, 7))):
+            if rng.random() < 0.2:
+                splits.append(("onehot", 1, int(rng.integers(-3, 5))))
+            else:
+                f = int(rng.integers(0, 5))
+                splits.append(("float", f, float(rng.choice(cands[f]))))
+        trees.append((splits, rng.normal(size=(1 << len(splits)) * 2)))
+    ref = mb.build_oblivious(ffs, cfs, 2, trees, scale=2.0, bias=[0.5, -0.5])
+    b = cb.ModelCalcer()
+    b.build_oblivious(ffs, cfs, 2, trees, scale=2.0, bias=[0.5, -0.5])
+    got = read_cbm(b.save_to_buffer())
+    for k in ("tree_splits", "tree_sizes", "tree_start_offsets", "leaf_values", "bias", "scale"):
+        np.testing.assert_array_equal(np.asarray(got[k]), np.asarray(ref[k]), err_msg=k)
+    for a, c in zip(got["float_features"], ref["float_features"]):
+        np.testing.assert_array_equal(a["borders"], c["borders"])
+        assert (a["has_nans"], a["nan_treatment"]) == (c["has_nans"], c["nan_treatment"])
+    assert [c["used"] for c in got["cat_features"]] == [False, True]
+    np.testing.assert_array_equal(got["one_hot_features"][0]["values"], ref["one_hot_features"][0]["values"])
+    # repacked bins written by the library equal the oracle's derivation
+    from oracle.oracle import OracleModel
+    feat, xor, split = OracleModel(ref).repacked_bins()
+    packed = feat.astype(np.uint32) | (xor.astype(np.uint32) << 16) | (split.astype(np.uint32) << 24)
+    np.testing.assert_array_equal(got["repacked_bins_in_file"], packed)
+
+
+def test_non_symmetric_builder_matches_oracle_builder():
+    rng = np.random.default_rng(5)
+
+    def grow(depth):
+        if depth >= 5 or rng.random() < 0.3:
+            return mb.leaf_node([float(rng.normal()), float(rng.normal())])
+        return mb.split_node(("float", int(rng.integers(0, 4)), float(np.float32(rng.normal()))), grow(depth + 1), grow(depth + 1))
+
+    ffs = [mb.float_feature(i) for i in range(4)]
+    heads = [grow(0) for _ in range(25)]
+    ref = mb.build_non_symmetric(ffs, [], 2, heads)
+    b = cb.ModelCalcer()
+    b.build_non_symmetric(ffs, [], 2, heads)
+    got = read_cbm(b.save_to_buffer())
+    for k in ("tree_splits", "tree_sizes", "tree_start_offsets", "leaf_values", "step_nodes", "node_id_to_leaf_id"):
+        np.testing.assert_array_equal(got[k], ref[k], err_msg=k)
+
+
+def test_convert_oblivious_to_asymmetric_matches_oracle():
+    model = rm.simple_float_model(tree_count=2)
+    m = cb.ModelCalcer()
+    m.load_from_dict(model)
+    m.convert_oblivious_to_asymmetric()
+    got = read_cbm(m.save_to_buffer())
+    ref = mb.convert_oblivious_to_asymmetric(model)
+    for k in ("tree_splits", "tree_sizes", "tree_start_offsets", "leaf_values", "step_nodes", "node_id_to_leaf_id"):
+        np.testing.assert_array_equal(got[k], ref[k], err_msg=k)
+
+
+def test_invalid_tables_are_refused():
+    model = rm.simple_float_model()
+    bad = dict(model, tree_splits=np.array([300, 301, 999], np.int32))
+    with pytest.raises(cb.CatBoostError, match="out of range"):
+        cb.ModelCalcer().load_from_dict(bad)
+    bad = dict(model, leaf_values=model["leaf_values"][:5])
+    with pytest.raises(cb.CatBoostError, match="leaf values"):
+        cb.ModelCalcer().load_from_dict(bad)
+    asym = mb.convert_oblivious_to_asymmetric(model)
+    steps = asym["step_nodes"].copy()
+    steps[0] = (200, 1)
+    with pytest.raises(cb.CatBoostError, match="leaves its tree"):
+        cb.ModelCalcer().load_from_dict(dict(asym, step_nodes=steps))
+    m = cb.ModelCalcer()
+    m.load_from_dict(model)
+    with pytest.raises(cb.CatBoostError, match="bias"):
+        m.set_scale_and_bias(1.0, np.zeros(3))
+
+
+def test_prediction_without_gpu_fails_loudly():
+    import torch
+
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    m = cb.ModelCalcer()
+    m.load_from_dict(rm.simple_float_model())
+    with pytest.raises(cb.CatBoostError, match="HIP"):
+        m.calc_flat(rm.DATA)
+    with pytest.raises(cb.CatBoostError, match="HIP"):
+        m.enable_gpu_evaluation(0)
