@@ -356,19 +356,39 @@ namespace {
 
 constexpr uint32_t kBinarizeBlocksPerGroup = 8;
 
+template <int LOG2P, bool CATS_MATRIX>
+void LaunchBinarizeRowsPC(size_t blocks, const float* floats, size_t stride, const int32_t* cats, size_t catStride,
+                          size_t docCount, const dev::TBinarizeTables& tab, uint32_t* bins, hipStream_t s) {
+    const dim3 grid(static_cast<uint32_t>((blocks + kBinarizeBlocksPerGroup - 1) / kBinarizeBlocksPerGroup),
+                    (tab.BucketCount + dev::kBucketTile - 1) / dev::kBucketTile);
+    const size_t lds = (static_cast<size_t>(dev::kBucketTile) << LOG2P) * 4 +
+                       static_cast<size_t>(dev::kBucketTile) * dev::kTilePitch * 4;
+    auto kernel = dev::BinarizeRowsKernel<LOG2P, CATS_MATRIX>;
+    if (lds > 64 * 1024) {
+        HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      static_cast<int>(lds)));
+    }
+    hipLaunchKernelGGL(kernel, grid, dim3(256), lds, s, floats, static_cast<uint32_t>(stride), cats,
+                       static_cast<uint32_t>(catStride), static_cast<uint32_t>(docCount), tab, kBinarizeBlocksPerGroup,
+                       bins);
+}
+
 template <int LOG2P>
 void LaunchBinarizeRowsP(size_t blocks, const float* floats, size_t stride, const int32_t* cats, size_t catStride,
                          size_t docCount, const dev::TBinarizeTables& tab, uint32_t* bins, hipStream_t s) {
-    const dim3 grid(static_cast<uint32_t>((blocks + kBinarizeBlocksPerGroup - 1) / kBinarizeBlocksPerGroup),
-                    (tab.BucketCount + dev::kBucketTile - 1) / dev::kBucketTile);
-    hipLaunchKernelGGL(dev::BinarizeRowsKernel<LOG2P>, grid, dim3(256), 0, s, floats, stride, cats, catStride, docCount,
-                       tab, kBinarizeBlocksPerGroup, bins);
+    if (cats != nullptr) {
+        LaunchBinarizeRowsPC<LOG2P, true>(blocks, floats, stride, cats, catStride, docCount, tab, bins, s);
+    } else {
+        LaunchBinarizeRowsPC<LOG2P, false>(blocks, floats, stride, cats, catStride, docCount, tab, bins, s);
+    }
 }
 
 // picks the smallest LDS slot count that still exceeds the largest bucket of the model
 void LaunchBinarizeRows(uint32_t maxBucketValues, size_t blocks, const float* floats, size_t stride,
                         const int32_t* cats, size_t catStride, size_t docCount, const dev::TBinarizeTables& tab,
                         uint32_t* bins, hipStream_t s) {
+    CBAMD_ENSURE(docCount < (size_t(1) << 31) && stride < (size_t(1) << 31) && catStride < (size_t(1) << 31),
+                 "batch is too large for one binarize launch");
     if (maxBucketValues < 32) {
         LaunchBinarizeRowsP<5>(blocks, floats, stride, cats, catStride, docCount, tab, bins, s);
     } else if (maxBucketValues < 64) {

@@ -50,14 +50,13 @@ struct TTreeTables {
 // first and +inf after them
 template <int LOG2P>
 __device__ __forceinline__ uint32_t CountBelow(const uint32_t* borders, float v) {
-    uint32_t lo = 0;
+    const uint32_t* p = borders;
 #pragma unroll
     for (uint32_t step = 1u << (LOG2P - 1); step >= 1; step >>= 1) {
-        const uint32_t mid = lo + step;
-        const float b = __uint_as_float(borders[mid - 1]);
-        lo = (b < v) ? mid : lo;
+        const float b = __uint_as_float(p[step - 1]);
+        p = (b < v) ? p + step : p;
     }
-    return lo;
+    return static_cast<uint32_t>(p - borders);
 }
 
 __device__ __forceinline__ uint32_t OneHotBin(const uint32_t* values, uint32_t count, uint32_t v) {
@@ -68,32 +67,36 @@ __device__ __forceinline__ uint32_t OneHotBin(const uint32_t* values, uint32_t c
     return bin;
 }
 
+constexpr int kTilePitch = kDocsPerBlock + 1;  // dwords per bucket row of the transposed tile
+
 // Row-major input: floats[doc * stride + column]; hashed categorical values either bit-cast in
-// the same row (cats == nullptr) or in cats[doc * catStride + column].
+// the same row (CATS_MATRIX == false) or in cats[doc * catStride + column].
 // One workgroup owns kBucketTile buckets and walks `blocksPerGroup` consecutive 256-document
 // blocks: the bucket values stay in LDS (1 << LOG2P slots per bucket, every bucket of the model
 // has fewer values than that), each block's 256 x 32 feature tile is fetched with row-contiguous
-// loads into registers one block ahead, transposed through LDS (rotated by the bucket index, so
-// both the row-wise fill and the column-wise read are bank-conflict free) and binarized by a
+// loads into registers one block ahead, transposed through a padded LDS tile and binarized by a
 // branch-free binary search; a wave writes the 256 bytes of one (block, bucket) pair at once.
-// grid = (ceil(doc blocks / blocksPerGroup), ceil(buckets / kBucketTile)), block = 256 threads.
-template <int LOG2P>
-__global__ __launch_bounds__(256) void BinarizeRowsKernel(const float* __restrict__ floats, size_t stride,
-                                                          const int32_t* __restrict__ cats, size_t catStride,
-                                                          size_t docCount, TBinarizeTables tab,
+// Rows past the last document are read as the last document (their bins are never used).
+// grid = (ceil(doc blocks / blocksPerGroup), ceil(buckets / kBucketTile)), block = 256 threads,
+// dynamic LDS = (kBucketTile << LOG2P) * 4 + kBucketTile * kTilePitch * 4 bytes.
+template <int LOG2P, bool CATS_MATRIX>
+__global__ __launch_bounds__(256) void BinarizeRowsKernel(const float* __restrict__ floats, uint32_t stride,
+                                                          const int32_t* __restrict__ cats, uint32_t catStride,
+                                                          uint32_t docCount, TBinarizeTables tab,
                                                           uint32_t blocksPerGroup, uint32_t* __restrict__ bins) {
     constexpr uint32_t kSlots = 1u << LOG2P;
     constexpr int kRowsPerPass = 256 / kBucketTile;        // 8 rows per pass of 256 threads
     constexpr int kPasses = kDocsPerBlock / kRowsPerPass;  // 32 values per thread and block
-    __shared__ uint32_t sValues[kBucketTile * kSlots];
-    __shared__ uint32_t sTile[kBucketTile][kDocsPerBlock];
+    extern __shared__ uint32_t sBinarize[];
+    uint32_t* sValues = sBinarize;                           // [kBucketTile][kSlots]
+    uint32_t* sTile = sBinarize + kBucketTile * kSlots;      // [kBucketTile][kTilePitch]
 
     const uint32_t tid = threadIdx.x;
     const uint32_t b0 = blockIdx.y * kBucketTile;
     const uint32_t nb = min(static_cast<uint32_t>(kBucketTile), tab.BucketCount - b0);
-    const size_t blockCount = (docCount + kDocsPerBlock - 1) / kDocsPerBlock;
-    const size_t blockBegin = static_cast<size_t>(blockIdx.x) * blocksPerGroup;
-    const size_t blockEnd = min(blockBegin + blocksPerGroup, blockCount);
+    const uint32_t blockCount = (docCount + kDocsPerBlock - 1) / kDocsPerBlock;
+    const uint32_t blockBegin = blockIdx.x * blocksPerGroup;
+    const uint32_t blockEnd = min(blockBegin + blocksPerGroup, blockCount);
 
     for (uint32_t i = tid; i < kBucketTile * kSlots; i += 256) {
         const uint32_t bb = i >> LOG2P, k = i & (kSlots - 1);
@@ -108,69 +111,80 @@ __global__ __launch_bounds__(256) void BinarizeRowsKernel(const float* __restric
         sValues[i] = v;
     }
 
-    // role of this thread while loading: bucket `myB` of rows myRow0, myRow0 + 8, ...
+    // role of this thread while loading: bucket `myB` of rows myRow0, myRow0 + 8, ...; threads of
+    // buckets past the end of the model re-read the last bucket and their values are ignored
     const uint32_t myB = tid % kBucketTile;
     const uint32_t myRow0 = tid / kBucketTile;
-    const bool myActive = myB < nb;
-    uint32_t mySrc = 0;
-    bool myFromCats = false;
-    if (myActive) {
-        mySrc = tab.BucketSrc[b0 + myB];
-        myFromCats = cats != nullptr && (tab.BucketFlags[b0 + myB] & kBucketFlagOneHot) != 0;
+    const uint32_t mySrcBucket = b0 + min(myB, nb - 1);
+    const uint32_t mySrc = tab.BucketSrc[mySrcBucket];
+    const uint32_t* myBase = reinterpret_cast<const uint32_t*>(floats);
+    uint32_t myStride = stride;
+    if (CATS_MATRIX && (tab.BucketFlags[mySrcBucket] & kBucketFlagOneHot) != 0) {
+        myBase = reinterpret_cast<const uint32_t*>(cats);
+        myStride = catStride;
     }
+    uint32_t* myTileSlot = sTile + myB * kTilePitch + myRow0;
+
     uint32_t regs[kPasses];
-    auto loadBlock = [&](size_t block) {
-#pragma unroll
-        for (int i = 0; i < kPasses; ++i) {
-            const size_t doc = block * kDocsPerBlock + myRow0 + i * kRowsPerPass;
-            uint32_t v = 0;
-            if (myActive && doc < docCount) {
-                v = myFromCats ? static_cast<uint32_t>(cats[doc * catStride + mySrc])
-                               : __float_as_uint(floats[doc * stride + mySrc]);
-            }
-            regs[i] = v;
-        }
-    };
+#define CBAMD_LOAD_BLOCK(blockIndex)                                                                   \
+    do {                                                                                               \
+        const uint32_t firstDoc = (blockIndex) * kDocsPerBlock;                                        \
+        if (firstDoc + kDocsPerBlock <= docCount) {                                                    \
+            const uint32_t* rowPtr = myBase + static_cast<size_t>(firstDoc + myRow0) * myStride + mySrc; \
+            _Pragma("unroll") for (int i = 0; i < kPasses; ++i) {                                      \
+                regs[i] = rowPtr[static_cast<size_t>(i) * kRowsPerPass * myStride];                    \
+            }                                                                                          \
+        } else {                                                                                       \
+            _Pragma("unroll") for (int i = 0; i < kPasses; ++i) {                                      \
+                const uint32_t doc = min(firstDoc + myRow0 + i * kRowsPerPass, docCount - 1);          \
+                regs[i] = myBase[static_cast<size_t>(doc) * myStride + mySrc];                         \
+            }                                                                                          \
+        }                                                                                              \
+    } while (0)
 
     const uint32_t lane = tid & (kWave - 1);
-    const uint32_t wave = tid / kWave;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kWave);
     if (blockBegin < blockEnd) {
-        loadBlock(blockBegin);
+        CBAMD_LOAD_BLOCK(blockBegin);
     }
-    for (size_t block = blockBegin; block < blockEnd; ++block) {
+    for (uint32_t block = blockBegin; block < blockEnd; ++block) {
         __syncthreads();  // the previous block's tile has been consumed (and sValues is complete)
 #pragma unroll
         for (int i = 0; i < kPasses; ++i) {
-            const uint32_t row = myRow0 + i * kRowsPerPass;
-            sTile[myB][(row + myB) % kDocsPerBlock] = regs[i];
+            myTileSlot[i * kRowsPerPass] = regs[i];
         }
         __syncthreads();
         if (block + 1 < blockEnd) {
-            loadBlock(block + 1);  // in flight while this block is binarized
+            CBAMD_LOAD_BLOCK(block + 1);  // in flight while this block is binarized
         }
         for (uint32_t bb = wave; bb < nb; bb += 256 / kWave) {
             const uint32_t flags = tab.BucketFlags[b0 + bb];
-            const uint32_t count = tab.BucketOffset[b0 + bb + 1] - tab.BucketOffset[b0 + bb];
             const uint32_t* values = sValues + bb * kSlots;
+            const uint32_t* column = sTile + bb * kTilePitch + lane;
             uint32_t packed = 0;
+            if (flags & kBucketFlagOneHot) {
+                const uint32_t count = tab.BucketOffset[b0 + bb + 1] - tab.BucketOffset[b0 + bb];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint32_t raw = sTile[bb][(j * kWave + lane + bb) % kDocsPerBlock];
-                uint32_t bin;
-                if (flags & kBucketFlagOneHot) {
-                    bin = OneHotBin(values, count, raw);
-                } else {
-                    float v = __uint_as_float(raw);
-                    if ((flags & kBucketFlagNanToInf) && isnan(v)) {
-                        v = __uint_as_float(0x7f800000u);
-                    }
-                    bin = CountBelow<LOG2P>(values, v);
+                for (int j = 0; j < 4; ++j) {
+                    packed |= OneHotBin(values, count, column[j * kWave]) << (8 * j);
                 }
-                packed |= bin << (8 * j);
+            } else if (flags & kBucketFlagNanToInf) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float v = __uint_as_float(column[j * kWave]);
+                    v = isnan(v) ? __uint_as_float(0x7f800000u) : v;
+                    packed |= CountBelow<LOG2P>(values, v) << (8 * j);
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    packed |= CountBelow<LOG2P>(values, __uint_as_float(column[j * kWave])) << (8 * j);
+                }
             }
-            bins[(block * tab.BucketCount + b0 + bb) * kWave + lane] = packed;
+            bins[(static_cast<size_t>(block) * tab.BucketCount + b0 + bb) * kWave + lane] = packed;
         }
     }
+#undef CBAMD_LOAD_BLOCK
 }
 
 // Column-major input: floats[column * stride + doc] (categorical hashes bit-cast in their column).
