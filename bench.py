@@ -60,6 +60,9 @@ def main():
     ap.add_argument("--docs", type=int, default=0, help="override the document count of the workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--check-docs", type=int, default=20000)
+    ap.add_argument("--copy-probe-mib", type=int, default=0,
+                    help="also run one device-to-device copy of this many MiB (a kernel of known traffic, used to "
+                         "scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (documents would be sharded "
@@ -85,6 +88,14 @@ def main():
     out = torch.zeros(docs * dim, dtype=torch.float64, device="cuda:0")
     feats = ev.features(cb.LAYOUT_FLAT_ROWS, x.data_ptr(), x.shape[1])
     torch.cuda.synchronize()
+
+    if args.copy_probe_mib:
+        probe_src = torch.ones(args.copy_probe_mib << 18, dtype=torch.float32, device="cuda:0")
+        probe_dst = torch.empty_like(probe_src)
+        torch.cuda.synchronize()
+        probe_dst.copy_(probe_src)
+        torch.cuda.synchronize()
+        del probe_src, probe_dst
 
     for _ in range(args.warmup):
         ev.eval_data(feats, docs, out.data_ptr())

@@ -359,8 +359,10 @@ constexpr uint32_t kBinarizeBlocksPerGroup = 8;
 template <int LOG2P, bool CATS_MATRIX>
 void LaunchBinarizeRowsPC(size_t blocks, const float* floats, size_t stride, const int32_t* cats, size_t catStride,
                           size_t docCount, const dev::TBinarizeTables& tab, uint32_t* bins, hipStream_t s) {
-    const dim3 grid(static_cast<uint32_t>((blocks + kBinarizeBlocksPerGroup - 1) / kBinarizeBlocksPerGroup),
-                    (tab.BucketCount + dev::kBucketTile - 1) / dev::kBucketTile);
+    const size_t groups = (blocks + kBinarizeBlocksPerGroup - 1) / kBinarizeBlocksPerGroup;
+    const size_t tiles = (tab.BucketCount + dev::kBucketTile - 1) / dev::kBucketTile;
+    CBAMD_ENSURE(groups * tiles < (size_t(1) << 31), "batch is too large for one binarize launch");
+    const dim3 grid(static_cast<uint32_t>(groups * tiles));
     const size_t lds = (static_cast<size_t>(dev::kBucketTile) << LOG2P) * 4 +
                        static_cast<size_t>(dev::kBucketTile) * dev::kTilePitch * 4;
     auto kernel = dev::BinarizeRowsKernel<LOG2P, CATS_MATRIX>;

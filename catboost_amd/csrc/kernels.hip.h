@@ -77,7 +77,7 @@ constexpr int kTilePitch = kDocsPerBlock + 1;  // dwords per bucket row of the t
 // loads into registers one block ahead, transposed through a padded LDS tile and binarized by a
 // branch-free binary search; a wave writes the 256 bytes of one (block, bucket) pair at once.
 // Rows past the last document are read as the last document (their bins are never used).
-// grid = (ceil(doc blocks / blocksPerGroup), ceil(buckets / kBucketTile)), block = 256 threads,
+// grid = ceil(doc blocks / blocksPerGroup) * ceil(buckets / kBucketTile), block = 256 threads,
 // dynamic LDS = (kBucketTile << LOG2P) * 4 + kBucketTile * kTilePitch * 4 bytes.
 template <int LOG2P, bool CATS_MATRIX>
 __global__ __launch_bounds__(256) void BinarizeRowsKernel(const float* __restrict__ floats, uint32_t stride,
@@ -92,10 +92,13 @@ __global__ __launch_bounds__(256) void BinarizeRowsKernel(const float* __restric
     uint32_t* sTile = sBinarize + kBucketTile * kSlots;      // [kBucketTile][kTilePitch]
 
     const uint32_t tid = threadIdx.x;
-    const uint32_t b0 = blockIdx.y * kBucketTile;
+    // consecutive workgroups take the bucket tiles of one document group, so the pieces of a row
+    // are fetched close together in time
+    const uint32_t tileCount = (tab.BucketCount + kBucketTile - 1) / kBucketTile;
+    const uint32_t b0 = (blockIdx.x % tileCount) * kBucketTile;
     const uint32_t nb = min(static_cast<uint32_t>(kBucketTile), tab.BucketCount - b0);
     const uint32_t blockCount = (docCount + kDocsPerBlock - 1) / kDocsPerBlock;
-    const uint32_t blockBegin = blockIdx.x * blocksPerGroup;
+    const uint32_t blockBegin = (blockIdx.x / tileCount) * blocksPerGroup;
     const uint32_t blockEnd = min(blockBegin + blocksPerGroup, blockCount);
 
     for (uint32_t i = tid; i < kBucketTile * kSlots; i += 256) {

@@ -264,6 +264,18 @@ def test_workload_configs_device_path(name, docs):
     assert binarize_ms > 0 and eval_ms > 0
 
 
+def test_plain_c_client_of_the_c_abi(golden_dir):
+    """A C program linked against libcatboostmodel.so the way users of the reference library are."""
+    import subprocess
+
+    exe = os.path.join(os.path.dirname(__file__), "bin", "c_abi_client")
+    if not os.path.exists(exe):
+        pytest.skip("tests/bin/c_abi_client is not built (run __graft_entry__.build())")
+    out = subprocess.check_output([exe, os.path.join(golden_dir, "numeric_only_model.cbm"), "0.1", "0.3", "0.2"],
+                                  timeout=120)
+    assert abs(float(out.decode().split()[0]) - rm.NUMERIC_ONLY_EXPECTED[0]) < 1e-15
+
+
 # ----------------------------------------------------------------------------- error paths ----
 
 def test_error_paths(golden_dir):
