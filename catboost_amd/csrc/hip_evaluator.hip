@@ -501,10 +501,10 @@ void LaunchEvalTileL(const TTileArgs& a) {
 
 template <bool SEVEN_BIT, int MAXD, int DCHUNK>
 void LaunchEvalTile(const TTileArgs& a) {
-    // leaf values go through LDS when the tile, the accumulator and the leaf regions leave room
-    // for at least two workgroups per CU
+    // leaf values go through LDS whenever the tile, the accumulator and the per-wave leaf regions
+    // fit the 160 KB of a CU (gathers from global memory cost ~50 L1 accesses per wave instruction)
     const size_t withLeaves = TileLdsBytes(a.Buckets, DCHUNK) + TileLeafLdsBytes(MAXD, a.Dim);
-    if (a.LeavesPairAligned && withLeaves <= 80 * 1024) {
+    if (a.LeavesPairAligned && withLeaves <= kMaxTileLdsBytes) {
         LaunchEvalTileL<SEVEN_BIT, MAXD, DCHUNK, true>(a);
     } else {
         LaunchEvalTileL<SEVEN_BIT, MAXD, DCHUNK, false>(a);
