@@ -39,16 +39,36 @@ def _run(cmd):
     return out
 
 
+def _build_eval_reg_code_object():
+    """gen_eval_reg_kernel.py -> assembly -> gfx950 code object -> byte list included by hip_evaluator.hip"""
+    llvm = os.path.join(os.path.dirname(os.path.dirname(os.path.realpath(_hipcc()))), "llvm", "bin")
+    if not os.path.isdir(llvm):
+        llvm = "/opt/rocm/llvm/bin"
+    asm = os.path.join(OBJ_DIR, "eval_reg_kernel.s")
+    obj = os.path.join(OBJ_DIR, "eval_reg_kernel.o")
+    co = os.path.join(OBJ_DIR, "eval_reg_kernel.co")
+    _run([sys.executable, os.path.join(CSRC, "gen_eval_reg_kernel.py"), asm])
+    _run([os.path.join(llvm, "clang"), "-x", "assembler", "-target", "amdgcn-amd-amdhsa", "-mcpu=gfx950", "-c", asm,
+          "-o", obj])
+    _run([os.path.join(llvm, "ld.lld"), "-shared", "-o", co, obj])
+    with open(co, "rb") as f:
+        data = f.read()
+    with open(os.path.join(OBJ_DIR, "eval_reg_kernel_co.inc"), "w") as f:
+        for i in range(0, len(data), 32):
+            f.write(",".join(str(b) for b in data[i:i + 32]) + ",\n")
+
+
 def build(verbose=False):
     hipcc = _hipcc()
     os.makedirs(OBJ_DIR, exist_ok=True)
+    _build_eval_reg_code_object()
     jobs = []
     for src in HOST_SOURCES:
         obj = os.path.join(OBJ_DIR, src + ".o")
         jobs.append((obj, [hipcc, "-x", "c++"] + COMMON + ["-c", os.path.join(CSRC, src), "-o", obj]))
     for src in HIP_SOURCES:
         obj = os.path.join(OBJ_DIR, src + ".o")
-        jobs.append((obj, [hipcc, "-x", "hip"] + COMMON + DEVICE + ["-c", os.path.join(CSRC, src), "-o", obj]))
+        jobs.append((obj, [hipcc, "-x", "hip"] + COMMON + DEVICE + ["-I", OBJ_DIR, "-c", os.path.join(CSRC, src), "-o", obj]))
     with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(jobs))) as pool:
         for out in pool.map(lambda j: _run(j[1]), jobs):
             if verbose and out.strip():

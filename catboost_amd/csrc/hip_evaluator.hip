@@ -4,6 +4,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <limits>
 #include <string>
@@ -82,10 +83,42 @@ private:
     size_t Cap = 0;
 };
 
-struct TBucketTables {
-    std::vector<uint32_t> Src;
-    TDeviceVec<uint32_t> DSrc;
+// Code object of the register-resident evaluate kernels (assembled from the output of
+// gen_eval_reg_kernel.py at build time).
+alignas(4096) const unsigned char kEvalRegCodeObject[] = {
+#include "eval_reg_kernel_co.inc"
 };
+
+// Must match gen_eval_reg_kernel.py: kernel arguments, tree block, variants.
+struct TEvalRegArgs {
+    const void* Bins;
+    const void* Rows;
+    const void* Leaves;
+    void* Out;
+    uint32_t DocCount;
+    uint32_t BlockCount;
+    uint32_t TreeBlocks;
+    uint32_t Flags;
+    double Scale;
+    double Bias;
+    uint32_t BucketCount;
+    uint32_t Pad;
+};
+static_assert(sizeof(TEvalRegArgs) == 72, "kernel argument block of the register-resident kernels");
+
+constexpr uint32_t kRegTreeBlock = 16;
+constexpr uint32_t kRegRowDwords = 16;
+constexpr uint32_t kRegTreeLeaves = 256;
+struct TEvalRegVariant {
+    uint32_t Buckets;
+    uint32_t Waves;
+    const char* Name;
+};
+constexpr TEvalRegVariant kEvalRegVariants[] = {
+    {96, 8, "cbamd_eval_reg_b96_w8"},
+    {208, 4, "cbamd_eval_reg_b208_w4"},
+};
+constexpr size_t kEvalRegVariantCount = sizeof(kEvalRegVariants) / sizeof(kEvalRegVariants[0]);
 
 }  // namespace
 
@@ -124,6 +157,16 @@ struct THipEvaluator::TImpl {
     double Scale = 1.0;
     int Dim = 1;
     std::vector<double> HostBias;
+
+    // register-resident kernels (one-dimensional 7-bit oblivious models of depth <= 8 whose
+    // buckets fit the register file): level rows and leaf values at a fixed pitch per tree
+    bool RegKernelUsable = false;
+    hipModule_t RegModule = nullptr;
+    hipFunction_t RegFunction = nullptr;
+    uint32_t RegWaves = 0;
+    uint32_t RegTreeBlocks = 0;
+    TDeviceVec<uint32_t> RegRows;
+    TDeviceVec<double> RegLeaves;
 
     // scratch (grow-only, guarded by THipEvaluator::Lock)
     TDeviceVec<uint8_t> ScratchBins;
@@ -324,6 +367,38 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId)
             m.LeavesPairAligned = m.LeavesPairAligned && (f % 2 == 0);
         }
     }
+
+    const char* regSwitch = std::getenv("CATBOOST_AMD_REG_KERNEL");
+    const bool regEnabled = !(regSwitch && regSwitch[0] == '0');
+    const TEvalRegVariant* variant = nullptr;
+    for (size_t i = 0; i < kEvalRegVariantCount && !variant; ++i) {
+        if (m.LayoutBuckets <= kEvalRegVariants[i].Buckets) {
+            variant = &kEvalRegVariants[i];
+        }
+    }
+    if (regEnabled && variant && m.Oblivious && m.MaxDepth <= 8 && m.PackedSevenBit && m.Dim == 1 && TreeCount > 0) {
+        HIP_CHECK(hipModuleLoadData(&m.RegModule, kEvalRegCodeObject));
+        HIP_CHECK(hipModuleGetFunction(&m.RegFunction, m.RegModule, variant->Name));
+        m.RegWaves = variant->Waves;
+        m.RegTreeBlocks = static_cast<uint32_t>((TreeCount + kRegTreeBlock - 1) / kRegTreeBlock);
+        // one block of null trees behind the last one: the kernels prefetch that far
+        const size_t tableTrees = (static_cast<size_t>(m.RegTreeBlocks) + 1) * kRegTreeBlock;
+        std::vector<uint32_t> rows(tableTrees * kRegRowDwords, 0);  // (bucket 0, add 0): false for every bin
+        std::vector<double> leaves(tableTrees * kRegTreeLeaves, 0.0);
+        for (size_t t = 0; t < TreeCount; ++t) {
+            const int depth = trees.TreeSizes[t];
+            for (int d = 0; d < depth; ++d) {
+                const auto& rb = trees.RepackedBins[trees.TreeStartOffsets[t] + d];
+                rows[t * kRegRowDwords + 2 * d] = rb.FeatureIndex;
+                rows[t * kRegRowDwords + 2 * d + 1] = (128u - rb.SplitIdx) * 0x01010101u;
+            }
+            std::copy_n(trees.LeafValues.begin() + trees.TreeFirstLeafOffsets[t], size_t(1) << depth,
+                        leaves.begin() + t * kRegTreeLeaves);
+        }
+        m.RegRows.Upload(rows);
+        m.RegLeaves.Upload(leaves);
+        m.RegKernelUsable = true;
+    }
 }
 
 THipEvaluator::~THipEvaluator() {
@@ -339,6 +414,9 @@ THipEvaluator::~THipEvaluator() {
         }
         if (Impl->Stream) {
             (void)hipStreamDestroy(Impl->Stream);
+        }
+        if (Impl->RegModule) {
+            (void)hipModuleUnload(Impl->RegModule);
         }
     }
 }
@@ -569,6 +647,27 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
     CBAMD_ENSURE(bins != nullptr, "quantized buffer is null");
     const dev::TTreeTables tt = m.TreeTables();
     const uint32_t tb = static_cast<uint32_t>(treeStart), te = static_cast<uint32_t>(treeEnd);
+    if (m.RegKernelUsable && treeStart == 0 && treeEnd == TreeCount && docCount < (size_t(1) << 29)) {
+        // whole model over bins kept in registers
+        TEvalRegArgs args = {};
+        args.Bins = bins;
+        args.Rows = m.RegRows.Get();
+        args.Leaves = m.RegLeaves.Get();
+        args.Out = results;
+        args.DocCount = static_cast<uint32_t>(docCount);
+        args.BlockCount = static_cast<uint32_t>((docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock);
+        args.TreeBlocks = m.RegTreeBlocks;
+        args.Flags = 1;  // the range starts at tree 0: add the bias
+        args.Scale = m.Scale;
+        args.Bias = m.HostBias.empty() ? 0.0 : m.HostBias[0];
+        args.BucketCount = m.LayoutBuckets;
+        size_t argSize = sizeof(args);
+        void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &argSize,
+                          HIP_LAUNCH_PARAM_END};
+        const uint32_t grid = (args.BlockCount + m.RegWaves - 1) / m.RegWaves;
+        HIP_CHECK(hipModuleLaunchKernel(m.RegFunction, grid, 1, 1, 64 * m.RegWaves, 1, 1, 0, s, nullptr, config));
+        return;
+    }
     const int dchunk = m.Dim == 1 ? 1 : m.Dim == 2 ? 2 : m.Dim <= 4 ? 4 : m.Dim <= 8 ? 8 : 16;
     if (m.Oblivious && m.MaxDepth <= 8 && TileLdsBytes(m.LayoutBuckets, dchunk) <= kMaxTileLdsBytes) {
         // byte-parallel kernel over an LDS tile of bins

@@ -246,16 +246,17 @@ def test_workload_configs_device_path(name, docs):
     ev = model.evaluator()
     x = syn.device_features(info, docs)
     out = torch.zeros(docs * info["dim"], dtype=torch.float64, device="cuda:0")
+    out2 = torch.zeros_like(out)
+    bins = torch.zeros(ev.quantized_bytes(docs), dtype=torch.uint8, device="cuda:0")
+    exported = torch.zeros(docs * ev.bucket_count, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()  # the evaluator runs on its own stream: torch's fills must be done first
     feats = ev.features(cb.LAYOUT_FLAT_ROWS, x.data_ptr(), x.shape[1])
     ev.eval_data(feats, docs, out.data_ptr())
     host = x.cpu().numpy()
     _close(out.cpu().numpy(), o.calc(host, threads=8))
     # separate quantize + evaluate on a caller-owned buffer, and the reference-layout export
-    bins = torch.zeros(ev.quantized_bytes(docs), dtype=torch.uint8, device="cuda:0")
     ev.quantize(feats, docs, bins.data_ptr())
-    out2 = torch.zeros_like(out)
     ev.eval_quantized(bins.data_ptr(), docs, out2.data_ptr())
-    exported = torch.zeros(docs * ev.bucket_count, dtype=torch.uint8, device="cuda:0")
     ev.export_quantized(bins.data_ptr(), docs, exported.data_ptr())
     ev.synchronize()
     assert torch.equal(out, out2)
