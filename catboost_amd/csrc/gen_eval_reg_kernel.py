@@ -13,7 +13,7 @@ Layout of the work:
     200-register array;
   * the waves of a workgroup share the leaf values: trees go through LDS in blocks of TREE_BLOCK
     trees (256 doubles per tree), double buffered; the copy of the next block is spread over the
-    current block's trees;
+    current block's trees and goes from global memory straight into LDS (global_load_lds);
   * a tree's levels come from a table of 16 dwords per tree, (bucket, (128 - splitIdx) * 0x01010101)
     per level, read with one scalar load two trees ahead;
   * the four leaf gathers of a tree are issued behind its levels and consumed after the levels of
@@ -23,8 +23,8 @@ Layout of the work:
 
 Kernel arguments (72 bytes):
    0 bins        const uint32*   [docBlock][bucketCount][64]
-   8 rows        const uint32*   [treeBlocks * TREE_BLOCK + TREE_BLOCK][16]
-  16 leaves      const double*   [treeBlocks * TREE_BLOCK + TREE_BLOCK][256]
+   8 rows        const uint32*   [(treeBlocks + 2) * TREE_BLOCK][16]    (null trees behind the model's)
+  16 leaves      const double*   [(treeBlocks + 2) * TREE_BLOCK][256]
   24 out         double*         [docCount]
   32 docCount    uint32          36 blockCount uint32 (ceil(docCount / 256), >= 1)
   40 treeBlocks  uint32 (>= 1)   44 flags uint32 (bit 0: add the bias)
@@ -54,14 +54,23 @@ def kernel_name(buckets, waves):
 def gen_kernel(buckets, waves):
     name = kernel_name(buckets, waves)
     threads = waves * 64
-    chunks = BUF_BYTES // 16 // threads  # 16-byte pieces of a tree block per thread
-    assert chunks >= 1 and TREE_BLOCK % chunks == 0
-    period = TREE_BLOCK // chunks
-    assert period >= 2
+    row_bytes = threads * 16              # one 16-byte piece per thread
+    chunks = BUF_BYTES // row_bytes       # pieces of a tree block per thread
+    assert 1 <= chunks <= TREE_BLOCK
     vgprs = B0 + buckets
-    assert vgprs <= 256 and 4 * chunks <= buckets
+    assert vgprs <= 256
     o = []
     e = o.append
+
+    def stage(lds_offset):
+        """One piece of the leaf table, global memory -> LDS without passing through registers:
+        lane l of wave w writes 16 bytes at lds_offset + w * 1024 + l * 16 (M0 holds the wave's
+        base). M0 doubles as the VGPR index register, so its index-mode value is put back after."""
+        e("  s_add_u32 m0, s68, %d" % lds_offset)
+        e("  s_nop 0")
+        e("  global_load_lds_dwordx4 v2, s[26:27]")
+        e("  s_add_u32 s26, s26, %d" % row_bytes)
+        e("  s_addc_u32 s27, s27, 0")
 
     e(".text")
     e(".globl %s" % name)
@@ -83,20 +92,13 @@ def gen_kernel(buckets, waves):
     e("  v_readfirstlane_b32 s20, v5")           # wave of the workgroup
     e("  s_mov_b32 s22, 0x80808080")
     e("  s_mov_b32 s23, 3")
+    e("  s_lshl_b32 s68, s20, 10")               # LDS offset of the wave's part of a copied piece
     e("  s_waitcnt lgkmcnt(0)")
-    # first tree block -> buffer 0, staged through the (still unused) bins registers
+    # first tree block -> buffer 0
     e("  s_mov_b32 s26, s8")
     e("  s_mov_b32 s27, s9")
     for c in range(chunks):
-        r = B0 + 4 * c
-        e("  global_load_dwordx4 v[%d:%d], v2, s[26:27]" % (r, r + 3))
-        e("  s_add_u32 s26, s26, %d" % (threads * 16))
-        e("  s_addc_u32 s27, s27, 0")
-    e("  s_waitcnt vmcnt(0)")
-    for c in range(chunks):
-        r = B0 + 4 * c
-        e("  ds_write_b128 v2, v[%d:%d] offset:%d" % (r, r + 3, c * threads * 16))
-    e("  s_waitcnt lgkmcnt(0)")
+        stage(c * row_bytes)
     # document block of this wave; waves past the last block redo the last one and store nothing
     e("  s_mul_i32 s21, s2, %d" % waves)
     e("  s_add_u32 s21, s21, s20")
@@ -147,15 +149,15 @@ def gen_kernel(buckets, waves):
                   % (22 + j, j))
                 e("  ds_read_b64 v[%d:%d], v%d offset:%d" % (l, l + 1, 22 + j, buf * BUF_BYTES + i * TREE_BYTES))
             e("  s_load_dwordx16 s[%d:%d], s[6:7], 0x%x" % (rows, rows + 15, (buf * TREE_BLOCK + i + 2) * ROW_BYTES))
-            # copy of the next tree block into the other buffer, one piece every `period` trees
-            if i % period == 0:
-                e("  global_load_dwordx4 v[26:29], v2, s[26:27]")
-                e("  s_add_u32 s26, s26, %d" % (threads * 16))
-                e("  s_addc_u32 s27, s27, 0")
-            elif i % period == period // 2:
-                c = i // period
-                e("  s_waitcnt vmcnt(0)")
-                e("  ds_write_b128 v2, v[26:29] offset:%d" % ((1 - buf) * BUF_BYTES + c * threads * 16))
+            # copy of the next tree block into the other buffer, one piece per tree
+            if i < chunks:
+                stage((1 - buf) * BUF_BYTES + i * row_bytes)
+                e("  s_mov_b32 m0, 0x1000")      # index mode value again: src0 relative, index 0
+            if i == 0:
+                # the rows of the next tree block are pulled into the scalar cache now, so that the
+                # per-tree row loads of that block do not each wait for a miss
+                for k in range(TREE_BLOCK):
+                    e("  s_load_dword s3, s[6:7], 0x%x" % ((buf * TREE_BLOCK + TREE_BLOCK + 2 + k) * ROW_BYTES))
         # every wave is done reading this buffer and writing the other one
         e("  s_waitcnt vmcnt(0) lgkmcnt(0)")
         e("  s_barrier")
@@ -208,7 +210,7 @@ def gen_kernel(buckets, waves):
     e("  .amdhsa_system_sgpr_workgroup_id_z 0")
     e("  .amdhsa_system_vgpr_workitem_id 0")
     e("  .amdhsa_next_free_vgpr %d" % vgprs)
-    e("  .amdhsa_next_free_sgpr 68")
+    e("  .amdhsa_next_free_sgpr 69")
     e("  .amdhsa_accum_offset %d" % ((vgprs + 3) // 4 * 4))
     e("  .amdhsa_reserve_vcc 1")
     e("  .amdhsa_float_round_mode_32 0")

@@ -381,8 +381,8 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId)
         HIP_CHECK(hipModuleGetFunction(&m.RegFunction, m.RegModule, variant->Name));
         m.RegWaves = variant->Waves;
         m.RegTreeBlocks = static_cast<uint32_t>((TreeCount + kRegTreeBlock - 1) / kRegTreeBlock);
-        // one block of null trees behind the last one: the kernels prefetch that far
-        const size_t tableTrees = (static_cast<size_t>(m.RegTreeBlocks) + 1) * kRegTreeBlock;
+        // two blocks of null trees behind the last one: the kernels prefetch that far
+        const size_t tableTrees = (static_cast<size_t>(m.RegTreeBlocks) + 2) * kRegTreeBlock;
         std::vector<uint32_t> rows(tableTrees * kRegRowDwords, 0);  // (bucket 0, add 0): false for every bin
         std::vector<double> leaves(tableTrees * kRegTreeLeaves, 0.0);
         for (size_t t = 0; t < TreeCount; ++t) {
