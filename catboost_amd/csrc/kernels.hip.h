@@ -22,6 +22,7 @@ constexpr int kDocsPerBlock = 256;
 constexpr int kWave = 64;
 constexpr int kBucketFlagNanToInf = 1;  // HasNans && NanValueTreatment == AsTrue
 constexpr int kBucketFlagOneHot = 2;
+constexpr uint32_t kXcdCount = 8;       // accelerator dies of an MI355X, each with its own L2
 constexpr int kBucketTile = 32;         // buckets binarized per workgroup
 constexpr int kMaxBucketValues = 256;   // 254 values, padded
 
@@ -92,13 +93,18 @@ __global__ __launch_bounds__(256) void BinarizeRowsKernel(const float* __restric
     uint32_t* sTile = sBinarize + kBucketTile * kSlots;      // [kBucketTile][kTilePitch]
 
     const uint32_t tid = threadIdx.x;
-    // consecutive workgroups take the bucket tiles of one document group, so the pieces of a row
-    // are fetched close together in time
     const uint32_t tileCount = (tab.BucketCount + kBucketTile - 1) / kBucketTile;
-    const uint32_t b0 = (blockIdx.x % tileCount) * kBucketTile;
+    // Workgroups go round-robin to the 8 XCDs, each with an L2 of its own. The bucket tiles of one
+    // document group share cache lines (a row piece of 128 bytes is not line aligned), so they are
+    // given to workgroups of the same XCD that start one after the other: XCD x owns a contiguous
+    // range of the work list.
+    const uint32_t perXcd = gridDim.x / kXcdCount, extra = gridDim.x % kXcdCount;
+    const uint32_t xcd = blockIdx.x % kXcdCount;
+    const uint32_t work = xcd * perXcd + min(xcd, extra) + blockIdx.x / kXcdCount;
+    const uint32_t b0 = (work % tileCount) * kBucketTile;
     const uint32_t nb = min(static_cast<uint32_t>(kBucketTile), tab.BucketCount - b0);
     const uint32_t blockCount = (docCount + kDocsPerBlock - 1) / kDocsPerBlock;
-    const uint32_t blockBegin = (blockIdx.x / tileCount) * blocksPerGroup;
+    const uint32_t blockBegin = (work / tileCount) * blocksPerGroup;
     const uint32_t blockEnd = min(blockBegin + blocksPerGroup, blockCount);
 
     for (uint32_t i = tid; i < kBucketTile * kSlots; i += 256) {
