@@ -17,6 +17,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
+# HBM bytes of one step (both launches, fetched + written), from rocprofv3 FETCH_SIZE / WRITE_SIZE
+# runs scaled by a copy kernel of known size; only known for workloads that were profiled
+MEASURED_TRAFFIC_BYTES = {("C2", 4000000, 1000): 5.44e9}
 
 
 def cpu_baseline(model_bytes, info, target_seconds=12.0):
@@ -155,7 +158,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, docs, model.tree_count)),
             "algorithmic_bytes_per_doc": bytes_per_doc,
             "kernel": "binarize + evaluate (the two launches of one step)",
         },
