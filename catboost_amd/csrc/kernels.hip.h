@@ -23,7 +23,7 @@ constexpr int kWave = 64;
 constexpr int kBucketFlagNanToInf = 1;  // HasNans && NanValueTreatment == AsTrue
 constexpr int kBucketFlagOneHot = 2;
 constexpr uint32_t kXcdCount = 8;       // accelerator dies of an MI355X, each with its own L2
-constexpr int kBucketTile = 32;         // buckets binarized per workgroup
+constexpr int kBucketTile = 16;         // buckets binarized per workgroup (small: ~20 KB of LDS, 7 workgroups per CU)
 constexpr int kMaxBucketValues = 256;   // 254 values, padded
 
 struct TBinarizeTables {
@@ -74,7 +74,7 @@ constexpr int kTilePitch = kDocsPerBlock + 1;  // dwords per bucket row of the t
 // the same row (CATS_MATRIX == false) or in cats[doc * catStride + column].
 // One workgroup owns kBucketTile buckets and walks `blocksPerGroup` consecutive 256-document
 // blocks: the bucket values stay in LDS (1 << LOG2P slots per bucket, every bucket of the model
-// has fewer values than that), each block's 256 x 32 feature tile is fetched with row-contiguous
+// has fewer values than that), each block's 256 x kBucketTile feature tile is fetched with row-contiguous
 // loads into registers one block ahead, transposed through a padded LDS tile and binarized by a
 // branch-free binary search; a wave writes the 256 bytes of one (block, bucket) pair at once.
 // Rows past the last document are read as the last document (their bins are never used).
@@ -86,8 +86,8 @@ __global__ __launch_bounds__(256) void BinarizeRowsKernel(const float* __restric
                                                           uint32_t docCount, TBinarizeTables tab,
                                                           uint32_t blocksPerGroup, uint32_t* __restrict__ bins) {
     constexpr uint32_t kSlots = 1u << LOG2P;
-    constexpr int kRowsPerPass = 256 / kBucketTile;        // 8 rows per pass of 256 threads
-    constexpr int kPasses = kDocsPerBlock / kRowsPerPass;  // 32 values per thread and block
+    constexpr int kRowsPerPass = 256 / kBucketTile;        // rows per pass of 256 threads
+    constexpr int kPasses = kDocsPerBlock / kRowsPerPass;  // values per thread and block
     extern __shared__ uint32_t sBinarize[];
     uint32_t* sValues = sBinarize;                           // [kBucketTile][kSlots]
     uint32_t* sTile = sBinarize + kBucketTile * kSlots;      // [kBucketTile][kTilePitch]
