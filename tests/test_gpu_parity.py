@@ -196,6 +196,72 @@ def test_random_oblivious_models(seed, dim):
     _close(g.calc_hashed(floats, cats), o.calc(floats, cats, layout="split"))
 
 
+def _float_only_model(rng, n_float, trees, max_depth, scale=1.0, bias=None):
+    """Oblivious model over float features only (at most 40 borders each), every feature used."""
+    ffs = [mb.float_feature(i, i) for i in range(n_float)]
+    cands = [np.unique(rng.normal(size=int(rng.integers(1, 40))).astype(np.float32)) for _ in range(n_float)]
+    tree_list = []
+    order = rng.permutation(n_float)
+    next_feature = 0
+    t = 0
+    while t < trees or next_feature < n_float:
+        depth = int(rng.integers(1, max_depth + 1))
+        splits = []
+        for _ in range(depth):
+            if next_feature < n_float:
+                f = int(order[next_feature])
+                next_feature += 1
+            else:
+                f = int(rng.integers(0, n_float))
+            splits.append(("float", f, float(rng.choice(cands[f]))))
+        tree_list.append((splits, rng.normal(size=1 << depth)))
+        t += 1
+    return mb.build_oblivious(ffs, [], 1, tree_list, scale=scale, bias=bias)
+
+
+# Models of this kind (one-dimensional, float features with < 128 borders, depth <= 8, at most
+# 208 buckets) run on the register-resident kernels, which add leaf values in tree order like the
+# CPU evaluator: their predictions are compared bit for bit. 209 buckets fall back to the LDS tile
+# kernel (sums per wave, then across waves), which only meets the tolerance.
+@pytest.mark.parametrize("n_float,trees,max_depth,docs", [
+    (1, 1, 1, 1), (1, 1, 8, 255), (3, 15, 8, 256), (5, 16, 8, 257), (7, 17, 6, 2049), (20, 33, 8, 1000),
+    (96, 40, 8, 3000), (97, 40, 8, 3000), (208, 70, 8, 5000), (209, 70, 8, 1500), (50, 200, 4, 70001),
+])
+def test_register_kernel_shapes(n_float, trees, max_depth, docs):
+    rng = np.random.default_rng(1000 * n_float + trees)
+    model = _float_only_model(rng, n_float, trees, max_depth, scale=0.75, bias=[0.125])
+    x = rng.normal(size=(docs, n_float)).astype(np.float32)
+    x[rng.random(x.shape) < 0.01] = np.nan
+    o = OracleModel(model)
+    g = _gpu_model(model)
+    expected = o.calc(x)
+    got = g.calc_flat(x)
+    if n_float <= 208:
+        np.testing.assert_array_equal(got, expected)
+    else:
+        _close(got, expected)
+    np.testing.assert_array_equal(g.quantize_flat(x), o.binarize(x))
+    # a tree sub-range goes through the tile kernel
+    if len(model["tree_sizes"]) >= 3:
+        _close(g.calc_flat(x, tree_start=1, tree_end=len(model["tree_sizes"]) - 1),
+               o.calc(x, tree_start=1, tree_end=len(model["tree_sizes"]) - 1))
+
+
+def test_register_kernel_against_tile_kernel():
+    """The same model with the register-resident kernels switched off: both paths agree."""
+    rng = np.random.default_rng(5)
+    model = _float_only_model(rng, 120, 300, 8)
+    x = rng.normal(size=(20000, 120)).astype(np.float32)
+    reg = _gpu_model(model).calc_flat(x)
+    os.environ["CATBOOST_AMD_REG_KERNEL"] = "0"
+    try:
+        tile = _gpu_model(model).calc_flat(x)
+    finally:
+        del os.environ["CATBOOST_AMD_REG_KERNEL"]
+    np.testing.assert_array_equal(reg, OracleModel(model).calc(x))
+    _close(tile, reg)
+
+
 def test_library_builder_matches_oracle_builder_and_roundtrips():
     rng = np.random.default_rng(11)
     ffs = [mb.float_feature(i, i) for i in range(5)]
