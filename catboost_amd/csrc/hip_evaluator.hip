@@ -120,6 +120,116 @@ constexpr TEvalRegVariant kEvalRegVariants[] = {
 };
 constexpr size_t kEvalRegVariantCount = sizeof(kEvalRegVariants) / sizeof(kEvalRegVariants[0]);
 
+// Level-order tables of non-symmetric trees for EvalNonSymmetricTileKernel (its comment has the
+// entry format). The walk they encode is CalcIndexesNonSymmetric, cpu/evaluator_impl.cpp:462-493:
+// from a node, the chosen side's diff leads to the next node and a zero diff ends the walk at the
+// node's own leaf (NonSymmetricNodeIdToLeafId). A zero side becomes a terminal entry of its own.
+// usable = false when a tree does not fit the 16-bit offsets of an entry.
+// The compact tables (EvalNonSymmetricLdsKernel) are filled when the model is one-dimensional,
+// has no xor masks, at most 1023 buckets and no tree above dev::kNsLdsEntries entries.
+void BuildLevelOrderTrees(const TModelTrees& trees, int dim, const std::vector<uint32_t>& firstLeaf,
+                          TDeviceVec<uint32_t>* entriesOut, TDeviceVec<uint32_t>* rowsOut, bool* usable, bool* noXor,
+                          std::vector<uint32_t>* compactEntries, std::vector<uint32_t>* compactRows,
+                          std::vector<double>* valuesByEntry, bool* compactUsable) {
+    struct TItem {
+        uint32_t Node;   // model node, or the parent node of a synthetic terminal
+        bool Terminal;
+    };
+    const size_t treeCount = trees.GetTreeCount();
+    *noXor = true;
+    for (const auto& rb : trees.RepackedBins) {
+        *noXor = *noXor && rb.XorMask == 0;
+    }
+    std::vector<uint32_t> entries, rows(treeCount * 4, 0);
+    *usable = true;
+    *compactUsable = *noXor && dim == 1 && trees.EffectiveBinFeaturesBucketCount <= 1023;
+    compactRows->assign(treeCount * 4, 0);
+    for (size_t t = 0; t < treeCount && *usable; ++t) {
+        const uint32_t root = static_cast<uint32_t>(trees.TreeStartOffsets[t]);
+        const size_t firstEntry = entries.size() / 2;
+        std::vector<TItem> order = {{root, false}};
+        std::vector<uint32_t> level = {0};
+        uint32_t height = 0;
+        // first pass: breadth-first order; second pass below fills the entries
+        std::vector<std::pair<uint32_t, uint32_t>> children;  // entry index of (left, right); terminals: unused
+        for (size_t i = 0; i < order.size(); ++i) {
+            const TItem item = order[i];
+            const auto& st = trees.NonSymmetricStepNodes[item.Node];
+            const bool terminal = item.Terminal || (st.LeftSubtreeDiff == 0 && st.RightSubtreeDiff == 0);
+            order[i].Terminal = terminal;
+            if (terminal) {
+                height = std::max(height, level[i]);
+                children.emplace_back(0, 0);
+                continue;
+            }
+            uint32_t child[2];
+            const uint32_t diffs[2] = {st.LeftSubtreeDiff, st.RightSubtreeDiff};
+            for (int side = 0; side < 2; ++side) {
+                child[side] = static_cast<uint32_t>(order.size());
+                if (diffs[side] == 0) {
+                    order.push_back({item.Node, true});
+                } else {
+                    order.push_back({item.Node + diffs[side], false});
+                }
+                level.push_back(level[i] + 1);
+            }
+            children.emplace_back(child[0], child[1]);
+        }
+        if (order.size() * 8 > 0xffffu) {
+            *usable = false;
+            break;
+        }
+        for (size_t i = 0; i < order.size(); ++i) {
+            const TItem item = order[i];
+            uint32_t x, y;
+            if (item.Terminal) {
+                const uint32_t leafRel = (trees.NonSymmetricNodeIdToLeafId[item.Node] - firstLeaf[t]) / static_cast<uint32_t>(dim);
+                if (leafRel > 0xffffu) {
+                    *usable = false;
+                    break;
+                }
+                x = 0;
+                y = leafRel | (static_cast<uint32_t>(i * 8) << 16);
+            } else {
+                const auto& rb = trees.RepackedBins[item.Node];
+                x = *noXor ? (static_cast<uint32_t>(rb.FeatureIndex) << 8) | (static_cast<uint32_t>(rb.SplitIdx) << 24)
+                           : static_cast<uint32_t>(rb.FeatureIndex) | (static_cast<uint32_t>(rb.XorMask) << 16) |
+                                 (static_cast<uint32_t>(rb.SplitIdx) << 24);
+                y = (children[i].first * 8) | ((children[i].second * 8) << 16);
+            }
+            entries.push_back(x);
+            entries.push_back(y);
+        }
+        rows[t * 4 + 0] = static_cast<uint32_t>(firstEntry);
+        rows[t * 4 + 1] = height;
+        rows[t * 4 + 2] = firstLeaf[t];
+        *compactUsable = *compactUsable && *usable && order.size() <= static_cast<size_t>(dev::kNsLdsEntries);
+        if (*compactUsable) {
+            (*compactRows)[t * 4 + 0] = static_cast<uint32_t>(compactEntries->size());
+            (*compactRows)[t * 4 + 1] = height;
+            (*compactRows)[t * 4 + 2] = static_cast<uint32_t>(order.size());
+            for (size_t i = 0; i < order.size(); ++i) {
+                const TItem item = order[i];
+                if (item.Terminal) {
+                    compactEntries->push_back(255u | (static_cast<uint32_t>(i) << 18));
+                    valuesByEntry->push_back(trees.LeafValues[trees.NonSymmetricNodeIdToLeafId[item.Node]]);
+                } else {
+                    const auto& rb = trees.RepackedBins[item.Node];
+                    // the right child always follows the left one in `order`
+                    compactEntries->push_back(static_cast<uint32_t>(rb.SplitIdx) |
+                                              (static_cast<uint32_t>(rb.FeatureIndex) << 8) | (children[i].first << 18));
+                    valuesByEntry->push_back(0.0);
+                }
+            }
+        }
+    }
+    *compactUsable = *compactUsable && *usable;
+    if (*usable) {
+        entriesOut->Upload(entries);
+        rowsOut->Upload(rows);
+    }
+}
+
 }  // namespace
 
 int GetHipDeviceCount() {
@@ -157,6 +267,17 @@ struct THipEvaluator::TImpl {
     double Scale = 1.0;
     int Dim = 1;
     std::vector<double> HostBias;
+
+    // non-symmetric trees re-laid level by level for the tile kernel
+    bool NsTileUsable = false;
+    bool NsNoXor = false;
+    TDeviceVec<uint32_t> NsEntries;  // pairs of dwords
+    TDeviceVec<uint32_t> NsRows;     // 4 dwords per tree
+    bool NsLdsUsable = false;        // compact entries walked out of LDS (one-dimensional, no xor)
+    TDeviceVec<uint32_t> NsCompactEntries;
+    TDeviceVec<uint32_t> NsCompactRows;  // 8 dwords per unit of trees
+    uint32_t NsUnitCount = 0;
+    TDeviceVec<double> NsValuesByEntry;
 
     // register-resident kernels (one-dimensional 7-bit oblivious models of depth <= 8 whose
     // buckets fit the register file): level rows and leaf values at a fixed pitch per tree
@@ -365,6 +486,35 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId)
         m.LeavesPairAligned = true;
         for (uint32_t f : firstLeaf) {
             m.LeavesPairAligned = m.LeavesPairAligned && (f % 2 == 0);
+        }
+    }
+
+    if (!m.Oblivious) {
+        std::vector<uint32_t> compactEntries, compactRows;
+        std::vector<double> valuesByEntry;
+        BuildLevelOrderTrees(trees, m.Dim, firstLeaf, &m.NsEntries, &m.NsRows, &m.NsTileUsable, &m.NsNoXor,
+                             &compactEntries, &compactRows, &valuesByEntry, &m.NsLdsUsable);
+        if (m.NsLdsUsable) {
+            // units: consecutive trees, at most kNsUnitTrees of them and kNsLdsEntries entries
+            std::vector<uint32_t> units;
+            for (size_t t = 0; t < TreeCount;) {
+                const uint32_t first = compactRows[t * 4];
+                uint32_t height = 0, count = 0, n = 0;
+                uint32_t start[dev::kNsUnitTrees] = {};
+                while (t < TreeCount && n < static_cast<uint32_t>(dev::kNsUnitTrees) &&
+                       count + compactRows[t * 4 + 2] <= static_cast<uint32_t>(dev::kNsLdsEntries)) {
+                    start[n++] = count;
+                    height = std::max(height, compactRows[t * 4 + 1]);
+                    count += compactRows[t * 4 + 2];
+                    ++t;
+                }
+                const uint32_t unit[8] = {first, height, count, start[1], start[2], n, 0, 0};
+                units.insert(units.end(), unit, unit + 8);
+            }
+            m.NsUnitCount = static_cast<uint32_t>(units.size() / 8);
+            m.NsCompactEntries.Upload(compactEntries);
+            m.NsCompactRows.Upload(units);
+            m.NsValuesByEntry.Upload(valuesByEntry);
         }
     }
 
@@ -611,6 +761,39 @@ void LaunchEvalTileM(uint32_t maxDepth, int dchunk, const TTileArgs& a) {
     }
 }
 
+template <bool NO_XOR, int DCHUNK>
+void LaunchEvalNonSymmetricTileX(const uint8_t* bins, size_t docCount, uint32_t buckets, const uint2* entries,
+                                 const uint4* rows, const double* leaves, const double* bias, double scale, int dim,
+                                 uint32_t treeBegin, uint32_t treeEnd, double* out, hipStream_t s) {
+    const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
+    const size_t lds = TileLdsBytes(buckets, DCHUNK);
+    auto kernel = dev::EvalNonSymmetricTileKernel<NO_XOR, DCHUNK>;
+    if (lds > 64 * 1024) {
+        HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      static_cast<int>(lds)));
+    }
+    hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(blocks)), dim3(64 * dev::kTileWaves), lds, s,
+                       reinterpret_cast<const uint32_t*>(bins), docCount, buckets, entries, rows, leaves, bias, scale, dim,
+                       treeBegin, treeEnd, out);
+}
+
+template <typename... TArgs>
+void LaunchEvalNonSymmetricTile(bool noXor, int dchunk, TArgs... args) {
+    if (noXor) {
+        switch (dchunk) {
+            case 1: LaunchEvalNonSymmetricTileX<true, 1>(args...); break;
+            case 4: LaunchEvalNonSymmetricTileX<true, 4>(args...); break;
+            default: LaunchEvalNonSymmetricTileX<true, 16>(args...); break;
+        }
+    } else {
+        switch (dchunk) {
+            case 1: LaunchEvalNonSymmetricTileX<false, 1>(args...); break;
+            case 4: LaunchEvalNonSymmetricTileX<false, 4>(args...); break;
+            default: LaunchEvalNonSymmetricTileX<false, 16>(args...); break;
+        }
+    }
+}
+
 template <int DCHUNK>
 void LaunchEval(bool oblivious, const uint8_t* bins, size_t docCount, uint32_t buckets, const dev::TTreeTables& tt,
                 uint32_t treeBegin, uint32_t treeEnd, double* out, hipStream_t s) {
@@ -680,6 +863,32 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
         }
         HIP_CHECK(hipGetLastError());
         return;
+    }
+    if (!m.Oblivious && m.NsLdsUsable && treeStart == 0 && treeEnd == TreeCount &&
+        TileLdsBytes(m.LayoutBuckets, 1) + dev::kTileWaves * dev::kNsLdsEntries * 4 <= kMaxTileLdsBytes) {
+        const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
+        const size_t lds = TileLdsBytes(m.LayoutBuckets, 1) + dev::kTileWaves * dev::kNsLdsEntries * 4;
+        if (lds > 64 * 1024) {
+            HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(dev::EvalNonSymmetricLdsKernel),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+        }
+        hipLaunchKernelGGL(dev::EvalNonSymmetricLdsKernel, dim3(static_cast<uint32_t>(blocks)), dim3(64 * dev::kTileWaves),
+                           lds, s, reinterpret_cast<const uint32_t*>(bins), docCount, m.LayoutBuckets,
+                           m.NsCompactEntries.Get(), reinterpret_cast<const uint4*>(m.NsCompactRows.Get()),
+                           m.NsUnitCount, m.NsValuesByEntry.Get(), m.Bias.Get(), m.Scale, results);
+        HIP_CHECK(hipGetLastError());
+        return;
+    }
+    if (!m.Oblivious && m.NsTileUsable) {
+        const int nsChunk = m.Dim == 1 ? 1 : m.Dim <= 4 ? 4 : 16;
+        if (TileLdsBytes(m.LayoutBuckets, nsChunk) <= kMaxTileLdsBytes) {
+            LaunchEvalNonSymmetricTile(m.NsNoXor, nsChunk, bins, docCount, m.LayoutBuckets,
+                                       reinterpret_cast<const uint2*>(m.NsEntries.Get()),
+                                       reinterpret_cast<const uint4*>(m.NsRows.Get()), m.Leaves.Get(), m.Bias.Get(),
+                                       m.Scale, m.Dim, tb, te, results, s);
+            HIP_CHECK(hipGetLastError());
+            return;
+        }
     }
     if (m.Dim == 1) {
         LaunchEval<1>(m.Oblivious, bins, docCount, m.LayoutBuckets, tt, tb, te, results, s);

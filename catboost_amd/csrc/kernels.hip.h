@@ -583,6 +583,320 @@ __global__ __launch_bounds__(256) void EvalNonSymmetricKernel(const uint8_t* __r
     }
 }
 
+// Non-symmetric trees over an LDS tile of bins: one workgroup of kTileWaves waves per
+// 256-document block, the waves split the trees in groups of kNsGroup consecutive trees, four
+// documents per lane walk the trees of a group side by side (4 * kNsGroup independent chains).
+// The trees come re-laid level by level: an entry is 8 bytes,
+//   x: NO_XOR   bucket << 8 | splitIdx << 24          (bucket << 8 = offset of the bucket in the tile)
+//      else     bucket | xorMask << 16 | splitIdx << 24
+//   y: byte offset (entry index * 8, relative to the tree's first entry) of the left child in the
+//      low half and of the right child in the high half.
+// A terminal entry has x = 0 (true for every bin), its own offset as right child and, in the low
+// half of y, the index of its leaf relative to the tree's first leaf. All lanes take the same
+// number of steps (the height of the tallest tree of the group): a lane that has reached its leaf
+// stays there. Since
+// the lanes of a wave are always on the same level, their gathers of a step fall into the few
+// cache lines of that level.
+// treeRows: 4 dwords per tree: first entry, height, first leaf value, unused.
+// grid = doc blocks, block = 64 * kTileWaves, dynamic LDS = buckets * 256 (rounded up to 8) +
+// 256 * DCHUNK * 8 bytes.
+constexpr int kNsGroup = 4;
+
+template <bool NO_XOR, int DCHUNK>
+__global__ __launch_bounds__(64 * kTileWaves) void EvalNonSymmetricTileKernel(
+    const uint32_t* __restrict__ bins, size_t docCount, uint32_t bucketCount, const uint2* __restrict__ entries,
+    const uint4* __restrict__ treeRows, const double* __restrict__ leaves, const double* __restrict__ bias, double scale,
+    int dim, uint32_t treeBegin, uint32_t treeEnd, double* __restrict__ out) {
+    extern __shared__ uint32_t sTile[];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const size_t block = blockIdx.x;
+    const uint32_t tileDwords = bucketCount * kWave;
+    const uint32_t* src = bins + block * tileDwords;
+    for (uint32_t i = tid; i < tileDwords; i += 64 * kTileWaves) {
+        sTile[i] = src[i];
+    }
+    const bool addBias = treeBegin == 0;
+    const uint8_t* laneTile = reinterpret_cast<const uint8_t*>(sTile) + lane * 4;
+    double* sRed = reinterpret_cast<double*>(sTile + ((tileDwords + 1) & ~1u));
+    for (int d0 = 0; d0 < dim; d0 += DCHUNK) {
+        __syncthreads();  // tile is loaded / the previous chunk's accumulator has been read
+        double acc[4][DCHUNK];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int k = 0; k < DCHUNK; ++k) {
+                acc[j][k] = 0.0;
+            }
+        }
+        // a wave walks kNsGroup trees at a time (trees t0 .. t0 + kNsGroup - 1), i.e. 4 * kNsGroup
+        // independent chains per lane, to cover the latency of the entry gathers
+        for (uint32_t t0 = treeBegin + wave * kNsGroup; t0 < treeEnd; t0 += kTileWaves * kNsGroup) {
+            const char* base[kNsGroup];
+            uint32_t firstLeaf[kNsGroup];
+            uint32_t height = 0;
+#pragma unroll
+            for (int g = 0; g < kNsGroup; ++g) {
+                // trees past the end walk tree t0 again and are not added
+                const uint4 row = treeRows[t0 + g < treeEnd ? t0 + g : t0];
+                base[g] = reinterpret_cast<const char*>(entries + __builtin_amdgcn_readfirstlane(row.x));
+                height = max(height, static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(row.y)));
+                firstLeaf[g] = __builtin_amdgcn_readfirstlane(row.z);
+            }
+            uint32_t off[kNsGroup][4];
+#pragma unroll
+            for (int g = 0; g < kNsGroup; ++g) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    off[g][j] = 0;
+                }
+            }
+            for (uint32_t step = 0; step < height; ++step) {
+                uint2 node[kNsGroup][4];
+#pragma unroll
+                for (int g = 0; g < kNsGroup; ++g) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        node[g][j] = *reinterpret_cast<const uint2*>(base[g] + off[g][j]);
+                    }
+                }
+#pragma unroll
+                for (int g = 0; g < kNsGroup; ++g) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const uint32_t x = node[g][j].x;
+                        uint32_t bin;
+                        if (NO_XOR) {
+                            bin = laneTile[(x & 0xffffffu) + j];
+                        } else {
+                            bin = laneTile[((x & 0xffffu) << 8) + j] ^ ((x >> 16) & 0xffu);
+                        }
+                        const uint32_t shift = bin >= (x >> 24) ? 16u : 0u;
+                        off[g][j] = (node[g][j].y >> shift) & 0xffffu;
+                    }
+                }
+            }
+#pragma unroll
+            for (int g = 0; g < kNsGroup; ++g) {
+                if (t0 + g < treeEnd) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const uint2 last = *reinterpret_cast<const uint2*>(base[g] + off[g][j]);
+                        const uint32_t leafRel = last.y & 0xffffu;
+                        const double* p = leaves + firstLeaf[g] +
+                                          (DCHUNK == 1 ? leafRel : leafRel * static_cast<uint32_t>(dim)) + d0;
+#pragma unroll
+                        for (int k = 0; k < DCHUNK; ++k) {
+                            if (DCHUNK == 1 || d0 + k < dim) {
+                                acc[j][k] = __dadd_rn(acc[j][k], p[k]);
+                            }
+                        }
+                    }
+                }
+            }
+        }
+        // waves add their partial sums in wave order into the LDS accumulator; the last wave
+        // finishes the values and writes them out
+        for (uint32_t w = 0; w + 1 < kTileWaves; ++w) {
+            if (wave == w) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                    for (int k = 0; k < DCHUNK; ++k) {
+                        double* cell = sRed + (j * kWave + lane) * DCHUNK + k;
+                        *cell = (w == 0) ? acc[j][k] : __dadd_rn(*cell, acc[j][k]);
+                    }
+                }
+            }
+            __syncthreads();
+        }
+        if (wave == kTileWaves - 1) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const size_t doc = block * kDocsPerBlock + j * kWave + lane;
+#pragma unroll
+                for (int k = 0; k < DCHUNK; ++k) {
+                    if (doc < docCount && (DCHUNK == 1 || d0 + k < dim)) {
+                        const double sum = __dadd_rn(sRed[(j * kWave + lane) * DCHUNK + k], acc[j][k]);
+                        out[doc * dim + d0 + k] = Finish(sum, scale, bias[d0 + k], addBias);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// One-dimensional non-symmetric models without xor masks whose trees have at most kNsLdsEntries
+// entries, whole model: as EvalNonSymmetricTileKernel, but a wave walks its trees out of a copy in
+// its own LDS region (an LDS gather costs a fraction of a gather from global memory). Consecutive
+// trees are grouped into units of up to kNsUnitTrees trees and kNsLdsEntries entries; a wave takes
+// a unit at a time and walks its trees side by side (4 documents x kNsUnitTrees chains per lane).
+// A compact entry is one dword:
+//   bits 0-7 splitIdx, bits 8-17 bucket (so entry & 0x3ff00 is the bucket's offset in the tile),
+//   bits 18-31 index of the left child relative to the tree's first entry; the right child
+//   follows the left one.
+// A terminal entry has splitIdx 255 (false for every bin) and itself as left child. The next
+// unit's entries are fetched into registers while the current unit is walked. valuesByEntry holds
+// the leaf value of every terminal entry, indexed like `entries`; a unit's values are requested
+// behind its walk and added after the next unit's walk.
+// unitRows: 8 dwords per unit: first entry, height of the tallest tree, number of entries, first
+// entry of the second and of the third tree relative to the unit's, number of trees, 2 unused.
+// grid = doc blocks, block = 64 * kTileWaves, dynamic LDS = buckets * 256 (rounded up to 8) +
+// 256 * 8 + kTileWaves * kNsLdsEntries * 4 bytes.
+constexpr int kNsLdsEntries = 2048;
+constexpr int kNsUnitTrees = 3;
+
+__global__ __launch_bounds__(64 * kTileWaves) void EvalNonSymmetricLdsKernel(
+    const uint32_t* __restrict__ bins, size_t docCount, uint32_t bucketCount, const uint32_t* __restrict__ entries,
+    const uint4* __restrict__ unitRows, uint32_t unitCount, const double* __restrict__ valuesByEntry,
+    const double* __restrict__ bias, double scale, double* __restrict__ out) {
+    constexpr int kFetch = kNsLdsEntries / kWave;
+    extern __shared__ uint32_t sTile[];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const size_t block = blockIdx.x;
+    const uint32_t tileDwords = bucketCount * kWave;
+    const uint32_t* src = bins + block * tileDwords;
+    for (uint32_t i = tid; i < tileDwords; i += 64 * kTileWaves) {
+        sTile[i] = src[i];
+    }
+    const uint8_t* tileBytes = reinterpret_cast<const uint8_t*>(sTile);
+    const uint32_t laneOff = lane * 4;
+    const uint32_t redBase = (tileDwords + 1) & ~1u;
+    double* sRed = reinterpret_cast<double*>(sTile + redBase);
+    uint32_t* sEntries = sTile + redBase + 2 * kDocsPerBlock + wave * kNsLdsEntries;
+    __syncthreads();  // tile is loaded
+
+    uint32_t fetched[kFetch];
+#define CBAMD_FETCH_UNIT(rowValue)                                                   \
+    do {                                                                             \
+        const uint32_t fFirst = __builtin_amdgcn_readfirstlane((rowValue).x);        \
+        const uint32_t fCount = __builtin_amdgcn_readfirstlane((rowValue).z);        \
+        _Pragma("unroll") for (int i = 0; i < kFetch; ++i) {                         \
+            if (static_cast<uint32_t>(i) * kWave < fCount) {                         \
+                fetched[i] = entries[fFirst + min(i * kWave + lane, fCount - 1)];    \
+            }                                                                        \
+        }                                                                            \
+    } while (0)
+
+    double acc[4] = {0.0, 0.0, 0.0, 0.0};
+    double pending[kNsUnitTrees][4];
+#pragma unroll
+    for (int g = 0; g < kNsUnitTrees; ++g) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            pending[g][j] = 0.0;
+        }
+    }
+    uint32_t u = wave;
+    uint4 row = make_uint4(0, 0, 0, 0), row2 = make_uint4(0, 0, 0, 0);
+    if (u < unitCount) {
+        row = unitRows[2 * u];
+        row2 = unitRows[2 * u + 1];
+        CBAMD_FETCH_UNIT(row);
+    }
+    while (u < unitCount) {
+        const uint32_t first = __builtin_amdgcn_readfirstlane(row.x);
+        const uint32_t height = __builtin_amdgcn_readfirstlane(row.y);
+        const uint32_t count = __builtin_amdgcn_readfirstlane(row.z);
+        const uint32_t trees = __builtin_amdgcn_readfirstlane(row2.y);
+        // trees the unit does not have walk its first tree again; their values are not added
+        const uint32_t start[kNsUnitTrees] = {0u, trees > 1 ? __builtin_amdgcn_readfirstlane(row.w) : 0u,
+                                              trees > 2 ? __builtin_amdgcn_readfirstlane(row2.x) : 0u};
+        // the previous unit's reads were issued before these stores and LDS serves one wave in order
+#pragma unroll
+        for (int i = 0; i < kFetch; ++i) {
+            if (static_cast<uint32_t>(i) * kWave < count) {
+                sEntries[i * kWave + lane] = fetched[i];
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        const uint32_t uNext = u + kTileWaves;
+        uint4 rowNext = make_uint4(0, 0, 0, 0), row2Next = make_uint4(0, 0, 0, 0);
+        if (uNext < unitCount) {
+            rowNext = unitRows[2 * uNext];
+            row2Next = unitRows[2 * uNext + 1];
+            CBAMD_FETCH_UNIT(rowNext);
+        }
+        uint32_t idx[kNsUnitTrees][4];
+#pragma unroll
+        for (int g = 0; g < kNsUnitTrees; ++g) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                idx[g][j] = 0;
+            }
+        }
+        for (uint32_t step = 0; step < height; ++step) {
+#pragma unroll
+            for (int g = 0; g < kNsUnitTrees; ++g) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t e = sEntries[start[g] + idx[g][j]];
+                    const uint32_t bin = tileBytes[((e & 0x3ff00u) | laneOff) + j];
+                    idx[g][j] = (e >> 18) + (bin >= (e & 0xffu) ? 1u : 0u);
+                }
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < kNsUnitTrees; ++g) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                acc[j] = __dadd_rn(acc[j], pending[g][j]);
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < kNsUnitTrees; ++g) {
+            if (static_cast<uint32_t>(g) < trees) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    pending[g][j] = valuesByEntry[first + start[g] + idx[g][j]];
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    pending[g][j] = 0.0;
+                }
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        u = uNext;
+        row = rowNext;
+        row2 = row2Next;
+    }
+#undef CBAMD_FETCH_UNIT
+#pragma unroll
+    for (int g = 0; g < kNsUnitTrees; ++g) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            acc[j] = __dadd_rn(acc[j], pending[g][j]);
+        }
+    }
+    // waves add their partial sums in wave order into the LDS accumulator; the last wave
+    // finishes the values and writes them out
+    for (uint32_t w = 0; w + 1 < kTileWaves; ++w) {
+        if (wave == w) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                double* cell = sRed + j * kWave + lane;
+                *cell = (w == 0) ? acc[j] : __dadd_rn(*cell, acc[j]);
+            }
+        }
+        __syncthreads();
+    }
+    if (wave == kTileWaves - 1) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const size_t doc = block * kDocsPerBlock + j * kWave + lane;
+            if (doc < docCount) {
+                out[doc] = Finish(__dadd_rn(sRed[j * kWave + lane], acc[j]), scale, bias[0], true);
+            }
+        }
+    }
+}
+
 // Leaf indexes [doc][tree - treeBegin] for both tree kinds (CalcLeafIndexesGeneric,
 // cpu/evaluator.h:174-253; non-symmetric numbering cpu/evaluator_impl.cpp:626-633).
 __global__ __launch_bounds__(256) void LeafIndexesKernel(const uint8_t* __restrict__ bins, size_t docCount,
