@@ -203,21 +203,30 @@ void BuildLevelOrderTrees(const TModelTrees& trees, int dim, const std::vector<u
         rows[t * 4 + 0] = static_cast<uint32_t>(firstEntry);
         rows[t * 4 + 1] = height;
         rows[t * 4 + 2] = firstLeaf[t];
-        *compactUsable = *compactUsable && *usable && order.size() <= static_cast<size_t>(dev::kNsLdsEntries);
+        // compact layout: root at 0, entry 1 unused, so that every pair of children starts even
+        *compactUsable = *compactUsable && *usable && order.size() + 1 <= static_cast<size_t>(dev::kNsLdsEntries);
         if (*compactUsable) {
+            const auto compactIndex = [](size_t i) { return static_cast<uint32_t>(i == 0 ? 0 : i + 1); };
             (*compactRows)[t * 4 + 0] = static_cast<uint32_t>(compactEntries->size());
             (*compactRows)[t * 4 + 1] = height;
-            (*compactRows)[t * 4 + 2] = static_cast<uint32_t>(order.size());
+            (*compactRows)[t * 4 + 2] = static_cast<uint32_t>(order.size() + 1);
             for (size_t i = 0; i < order.size(); ++i) {
                 const TItem item = order[i];
+                const uint32_t self = compactIndex(i);
                 if (item.Terminal) {
-                    compactEntries->push_back(255u | (static_cast<uint32_t>(i) << 18));
+                    const bool odd = (self & 1u) != 0;
+                    compactEntries->push_back((odd ? 0u : 255u) | ((self & ~1u) << 21));
                     valuesByEntry->push_back(trees.LeafValues[trees.NonSymmetricNodeIdToLeafId[item.Node]]);
                 } else {
                     const auto& rb = trees.RepackedBins[item.Node];
                     // the right child always follows the left one in `order`
                     compactEntries->push_back(static_cast<uint32_t>(rb.SplitIdx) |
-                                              (static_cast<uint32_t>(rb.FeatureIndex) << 8) | (children[i].first << 18));
+                                              (static_cast<uint32_t>(rb.FeatureIndex) << 8) |
+                                              (compactIndex(children[i].first) << 21));
+                    valuesByEntry->push_back(0.0);
+                }
+                if (i == 0) {
+                    compactEntries->push_back(255u);  // the unused entry
                     valuesByEntry->push_back(0.0);
                 }
             }

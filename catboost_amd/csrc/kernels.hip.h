@@ -734,12 +734,15 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalNonSymmetricTileKernel(
 // a unit at a time and walks its trees side by side (4 documents x kNsUnitTrees chains per lane).
 // A compact entry is one dword:
 //   bits 0-7 splitIdx, bits 8-17 bucket (so entry & 0x3ff00 is the bucket's offset in the tile),
-//   bits 18-31 index of the left child relative to the tree's first entry; the right child
-//   follows the left one.
-// A terminal entry has splitIdx 255 (false for every bin) and itself as left child. The next
-// unit's entries are fetched into registers while the current unit is walked. valuesByEntry holds
-// the leaf value of every terminal entry, indexed like `entries`; a unit's values are requested
-// behind its walk and added after the next unit's walk.
+//   bits 21-31 index of the left child relative to the tree's first entry.
+// The two children of a node sit side by side at an even index (the root is entry 0, entry 1 is
+// unused), so one 8-byte LDS read, issued together with the read of the node's bin, brings both
+// and the compare only selects: one LDS round trip per level. A terminal entry points at its own
+// pair and compares so that it selects itself (even index: splitIdx 255, false for every bin;
+// odd index: splitIdx 0, true for every bin, which no real split has). The next unit's entries
+// are fetched into registers while the current unit is walked. valuesByEntry holds the leaf
+// value of every terminal entry, indexed like `entries`; a unit's values are requested behind
+// its walk and added after the next unit's walk.
 // unitRows: 8 dwords per unit: first entry, height of the tallest tree, number of entries, first
 // entry of the second and of the third tree relative to the unit's, number of trees, 2 unused.
 // grid = doc blocks, block = 64 * kTileWaves, dynamic LDS = buckets * 256 (rounded up to 8) +
@@ -821,23 +824,41 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalNonSymmetricLdsKernel(
             row2Next = unitRows[2 * uNext + 1];
             CBAMD_FETCH_UNIT(rowNext);
         }
+        uint32_t entry[kNsUnitTrees][4];
+#pragma unroll
+        for (int g = 0; g < kNsUnitTrees; ++g) {
+            const uint32_t rootEntry = sEntries[start[g]];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                entry[g][j] = rootEntry;
+            }
+        }
+        for (uint32_t step = 0; step < height; ++step) {
+            uint2 pair[kNsUnitTrees][4];
+            uint32_t bin[kNsUnitTrees][4];
+#pragma unroll
+            for (int g = 0; g < kNsUnitTrees; ++g) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t e = entry[g][j];
+                    pair[g][j] = *reinterpret_cast<const uint2*>(sEntries + start[g] + (e >> 21));
+                    bin[g][j] = tileBytes[((e & 0x3ff00u) | laneOff) + j];
+                }
+            }
+#pragma unroll
+            for (int g = 0; g < kNsUnitTrees; ++g) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    entry[g][j] = bin[g][j] >= (entry[g][j] & 0xffu) ? pair[g][j].y : pair[g][j].x;
+                }
+            }
+        }
         uint32_t idx[kNsUnitTrees][4];
 #pragma unroll
         for (int g = 0; g < kNsUnitTrees; ++g) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                idx[g][j] = 0;
-            }
-        }
-        for (uint32_t step = 0; step < height; ++step) {
-#pragma unroll
-            for (int g = 0; g < kNsUnitTrees; ++g) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const uint32_t e = sEntries[start[g] + idx[g][j]];
-                    const uint32_t bin = tileBytes[((e & 0x3ff00u) | laneOff) + j];
-                    idx[g][j] = (e >> 18) + (bin >= (e & 0xffu) ? 1u : 0u);
-                }
+                idx[g][j] = (entry[g][j] >> 21) + ((entry[g][j] & 0xffu) == 0 ? 1u : 0u);
             }
         }
 #pragma unroll
