@@ -120,6 +120,11 @@ constexpr TEvalRegVariant kEvalRegVariants[] = {
 };
 constexpr size_t kEvalRegVariantCount = sizeof(kEvalRegVariants) / sizeof(kEvalRegVariants[0]);
 
+// dimensions the tile kernel accumulates per pass over the trees (and the pitch of its padded leaf rows)
+int TileChunk(int dim) {
+    return dim == 1 ? 1 : dim == 2 ? 2 : dim <= 4 ? 4 : dim <= 8 ? 8 : dim <= 12 ? 12 : 16;
+}
+
 // Level-order tables of non-symmetric trees for EvalNonSymmetricTileKernel (its comment has the
 // entry format). The walk they encode is CalcIndexesNonSymmetric, cpu/evaluator_impl.cpp:462-493:
 // from a node, the chosen side's diff leads to the next node and a zero diff ends the walk at the
@@ -271,6 +276,7 @@ struct THipEvaluator::TImpl {
     TDeviceVec<uint32_t> Splits, TreeStart, TreeSize, FirstLeaf, StepNodes, NodeToLeaf;
     TDeviceVec<double> Leaves, Bias;
     TDeviceVec<uint32_t> PackedTrees;  // tile kernel: 16 dwords per oblivious tree of depth <= 8
+    TDeviceVec<double> LeavesPadded;   // tile kernel, multi-dimensional: [tree][chunk][leaf][TileChunk(dim)]
     bool PackedSevenBit = false;
     bool LeavesPairAligned = false;  // every tree's first leaf value sits at an even index
     double Scale = 1.0;
@@ -491,6 +497,28 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId)
             }
             row[dev::kPackedFirstLeafSlot] = firstLeaf[t];
         }
+        if (m.Dim > 1) {
+            const size_t pitch = static_cast<size_t>(TileChunk(m.Dim));
+            const size_t chunks = (static_cast<size_t>(m.Dim) + pitch - 1) / pitch;
+            std::vector<double> padded;
+            for (size_t t = 0; t < trees.GetTreeCount(); ++t) {
+                const size_t leafCount = size_t(1) << trees.TreeSizes[t];
+                CBAMD_ENSURE(padded.size() <= std::numeric_limits<uint32_t>::max(), "model has too many leaf values");
+                packed[t * dev::kPackedTreeDwords + dev::kPackedPaddedLeafSlot] = static_cast<uint32_t>(padded.size());
+                packed[t * dev::kPackedTreeDwords + dev::kPackedLeafCountSlot] = static_cast<uint32_t>(leafCount);
+                const double* values = trees.LeafValues.data() + trees.TreeFirstLeafOffsets[t];
+                for (size_t c = 0; c < chunks; ++c) {
+                    for (size_t leaf = 0; leaf < leafCount; ++leaf) {
+                        for (size_t k = 0; k < pitch; ++k) {
+                            const size_t d = c * pitch + k;
+                            padded.push_back(d < static_cast<size_t>(m.Dim) ? values[leaf * m.Dim + d] : 0.0);
+                        }
+                    }
+                }
+            }
+            padded.resize(padded.size() + 256 * pitch, 0.0);  // the kernel copies 256 leaves' worth per tree
+            m.LeavesPadded.Upload(padded);
+        }
         m.PackedTrees.Upload(packed);
         m.LeavesPairAligned = true;
         for (uint32_t f : firstLeaf) {
@@ -703,8 +731,8 @@ size_t TileLdsBytes(uint32_t buckets, int dchunk) {
 }
 
 // LDS of the per-wave leaf regions of the tile kernel
-size_t TileLeafLdsBytes(int maxd, int dim) {
-    return static_cast<size_t>(dev::kTileWaves) * (size_t(1) << maxd) * dim * sizeof(double);
+size_t TileLeafLdsBytes(int maxd, int dchunk) {
+    return static_cast<size_t>(dev::kTileWaves) * (size_t(1) << maxd) * dchunk * sizeof(double);
 }
 
 struct TTileArgs {
@@ -725,7 +753,7 @@ struct TTileArgs {
 template <bool SEVEN_BIT, int MAXD, int DCHUNK, bool LEAF_LDS>
 void LaunchEvalTileL(const TTileArgs& a) {
     const size_t blocks = (a.DocCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
-    const size_t lds = TileLdsBytes(a.Buckets, DCHUNK) + (LEAF_LDS ? TileLeafLdsBytes(MAXD, a.Dim) : 0);
+    const size_t lds = TileLdsBytes(a.Buckets, DCHUNK) + (LEAF_LDS ? TileLeafLdsBytes(MAXD, DCHUNK) : 0);
     auto kernel = dev::EvalObliviousTileKernel<SEVEN_BIT, MAXD, DCHUNK, LEAF_LDS>;
     if (lds > 64 * 1024) {
         HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -740,7 +768,7 @@ template <bool SEVEN_BIT, int MAXD, int DCHUNK>
 void LaunchEvalTile(const TTileArgs& a) {
     // leaf values go through LDS whenever the tile, the accumulator and the per-wave leaf regions
     // fit the 160 KB of a CU (gathers from global memory cost ~50 L1 accesses per wave instruction)
-    const size_t withLeaves = TileLdsBytes(a.Buckets, DCHUNK) + TileLeafLdsBytes(MAXD, a.Dim);
+    const size_t withLeaves = TileLdsBytes(a.Buckets, DCHUNK) + TileLeafLdsBytes(MAXD, DCHUNK);
     if (a.LeavesPairAligned && withLeaves <= kMaxTileLdsBytes) {
         LaunchEvalTileL<SEVEN_BIT, MAXD, DCHUNK, true>(a);
     } else {
@@ -755,6 +783,7 @@ void LaunchEvalTileD(int dchunk, const TTileArgs& a) {
         case 2: LaunchEvalTile<SEVEN_BIT, MAXD, 2>(a); break;
         case 4: LaunchEvalTile<SEVEN_BIT, MAXD, 4>(a); break;
         case 8: LaunchEvalTile<SEVEN_BIT, MAXD, 8>(a); break;
+        case 12: LaunchEvalTile<SEVEN_BIT, MAXD, 12>(a); break;
         default: LaunchEvalTile<SEVEN_BIT, MAXD, 16>(a); break;
     }
 }
@@ -860,11 +889,12 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
         HIP_CHECK(hipModuleLaunchKernel(m.RegFunction, grid, 1, 1, 64 * m.RegWaves, 1, 1, 0, s, nullptr, config));
         return;
     }
-    const int dchunk = m.Dim == 1 ? 1 : m.Dim == 2 ? 2 : m.Dim <= 4 ? 4 : m.Dim <= 8 ? 8 : 16;
+    const int dchunk = TileChunk(m.Dim);
     if (m.Oblivious && m.MaxDepth <= 8 && TileLdsBytes(m.LayoutBuckets, dchunk) <= kMaxTileLdsBytes) {
         // byte-parallel kernel over an LDS tile of bins
-        const TTileArgs args{bins, docCount, m.LayoutBuckets, m.PackedTrees.Get(), m.Leaves.Get(), m.Bias.Get(),
-                             m.Scale, m.Dim, tb, te, results, s, m.LeavesPairAligned};
+        const TTileArgs args{bins, docCount, m.LayoutBuckets, m.PackedTrees.Get(),
+                             m.Dim == 1 ? m.Leaves.Get() : m.LeavesPadded.Get(), m.Bias.Get(), m.Scale, m.Dim, tb, te,
+                             results, s, m.Dim == 1 ? m.LeavesPairAligned : true};
         if (m.PackedSevenBit) {
             LaunchEvalTileM<true>(m.MaxDepth, dchunk, args);
         } else {

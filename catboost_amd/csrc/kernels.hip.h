@@ -375,21 +375,37 @@ __device__ __forceinline__ uint32_t TreeIndexes(const uint8_t* laneTile, uint32_
 // waves per 256-document block. The block's bins (buckets x 256 bytes) are copied to LDS once;
 // the waves share the tile and split the trees among themselves (tree t goes to wave
 // t % kTileWaves), four documents per lane. A wave fetches a tree's packed row with one 64-byte
-// load (one tree ahead) and broadcasts the levels from it. Per-wave partial sums (fp64) are added
+// load (two trees ahead) and broadcasts the levels from it. Per-wave partial sums (fp64) are added
 // in wave order through an LDS accumulator behind the tile, and the last wave writes the results.
+//
+// Leaf values. DCHUNK == 1 (one-dimensional models): `leaves` is the model's array and slot 8 of a
+// packed row the tree's first value. DCHUNK > 1: `leaves` is a copy padded to DCHUNK values per
+// leaf, one run of (leaf count) x DCHUNK values per tree and chunk of DCHUNK dimensions (zeros
+// behind the last dimension); slot 9 is the tree's first padded value and slot 10 its leaf count.
+// A lane adds all DCHUNK values of a leaf without looking at the dimension; only the final store
+// does. LEAF_LDS: every wave copies the (1 << MAXD) * DCHUNK values of its current tree and chunk
+// into a private LDS region with row-contiguous 16-byte loads, one tree ahead through registers
+// when that takes at most 8 loads per lane, and gathers from there; otherwise the values are
+// gathered straight from global memory. `leaves` must be readable for (1 << MAXD) * DCHUNK values
+// past the first value of the last tree.
 // grid = doc blocks, block = 64 * kTileWaves threads, dynamic LDS = buckets * 256 (rounded up to
-// 8) + 256 * DCHUNK * 8 [+ kTileWaves * (1 << MAXD) * dim * 8 with LEAF_LDS] bytes.
+// 8) + 256 * DCHUNK * 8 [+ kTileWaves * (1 << MAXD) * DCHUNK * 8 with LEAF_LDS] bytes.
 constexpr int kTileWaves = 8;
+constexpr int kPackedPaddedLeafSlot = 9;
+constexpr int kPackedLeafCountSlot = 10;
 
-// LEAF_LDS: every wave copies the leaf values of its current tree ((1 << MAXD) * dim doubles)
-// into a private LDS region with row-contiguous 16-byte loads and gathers from there; otherwise
-// leaf values are gathered straight from global memory. The leaves array must be readable for
-// (1 << MAXD) * dim doubles past the first leaf of the last tree.
 template <bool SEVEN_BIT, int MAXD, int DCHUNK, bool LEAF_LDS>
-__global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousTileKernel(
+__global__ __launch_bounds__(64 * kTileWaves) __attribute__((amdgpu_waves_per_eu(2, 4))) void EvalObliviousTileKernel(
     const uint32_t* __restrict__ bins, size_t docCount, uint32_t bucketCount, const uint32_t* __restrict__ packedTrees,
     const double* __restrict__ leaves, const double* __restrict__ bias, double scale, int dim, uint32_t treeBegin,
     uint32_t treeEnd, double* __restrict__ out) {
+    static_assert(DCHUNK == 1 || DCHUNK % 2 == 0, "padded leaf rows are copied in 16-byte pairs");
+    constexpr uint32_t kTreeDoubles = (1u << MAXD) * DCHUNK;    // values of one tree and chunk in LDS
+    constexpr uint32_t kTreePairs = kTreeDoubles / 2;
+    constexpr int kPairsPerLane = static_cast<int>((kTreePairs + kWave - 1) / kWave);
+    constexpr bool kPrefetch = kPairsPerLane <= 8;  // registers of the copy that runs one tree ahead
+    constexpr int kPrefetchRegs = kPrefetch ? kPairsPerLane : 1;
+    constexpr int kFirstSlot = DCHUNK == 1 ? kPackedFirstLeafSlot : kPackedPaddedLeafSlot;
     extern __shared__ uint32_t sTile[];
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & (kWave - 1);
@@ -404,11 +420,10 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousTileKernel(
     const uint8_t* laneTile = reinterpret_cast<const uint8_t*>(sTile) + lane * 4;
     const uint32_t slot = lane & (kPackedTreeDwords - 1);
     double* sRed = reinterpret_cast<double*>(sTile + ((tileDwords + 1) & ~1u));
-    // per-wave leaf region behind the accumulator; treeDoubles is a multiple of 2
-    const uint32_t treeDoubles = (1u << MAXD) * static_cast<uint32_t>(dim);
-    double* sLeaf = sRed + kDocsPerBlock * DCHUNK + wave * treeDoubles;
+    double* sLeaf = sRed + kDocsPerBlock * DCHUNK + wave * kTreeDoubles;  // per-wave leaf region
     for (int d0 = 0; d0 < dim; d0 += DCHUNK) {
         __syncthreads();  // tile is loaded / the previous chunk's accumulator has been read
+        const uint32_t chunk = static_cast<uint32_t>(d0) / DCHUNK;
         double acc[4][DCHUNK];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -417,18 +432,22 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousTileKernel(
                 acc[j][k] = 0.0;
             }
         }
-        // one-dimensional models: the leaf values of a tree are (1 << MAXD) doubles, i.e. at most two
-        // 16-byte pairs per lane, fetched one tree ahead into registers
-        constexpr uint32_t kTreePairs = (1u << MAXD) / 2;
-        double2 pref0 = {0.0, 0.0}, pref1 = {0.0, 0.0};
-#define CBAMD_FETCH_LEAVES(firstLeafValue)                                                        \
+        double2 pref[kPrefetchRegs];
+#pragma unroll
+        for (int i = 0; i < kPrefetchRegs; ++i) {
+            pref[i] = {0.0, 0.0};
+        }
+        // first value of this chunk of the tree whose packed row is `rowValue`
+#define CBAMD_TREE_VALUES(rowValue)                                                               \
+    (leaves + __builtin_amdgcn_readlane(rowValue, kFirstSlot) +                                   \
+     (DCHUNK == 1 ? 0u : chunk * __builtin_amdgcn_readlane(rowValue, kPackedLeafCountSlot) * DCHUNK))
+#define CBAMD_FETCH_LEAVES(rowValue)                                                              \
     do {                                                                                          \
-        const double2* src2 = reinterpret_cast<const double2*>(leaves + (firstLeafValue));        \
-        if (kTreePairs >= kWave || lane < kTreePairs) {                                           \
-            pref0 = src2[lane];                                                                   \
-        }                                                                                         \
-        if (kTreePairs > kWave) {                                                                 \
-            pref1 = src2[kWave + lane];                                                           \
+        const double2* src2 = reinterpret_cast<const double2*>(CBAMD_TREE_VALUES(rowValue));     \
+        _Pragma("unroll") for (int i = 0; i < kPrefetchRegs; ++i) {                               \
+            if (static_cast<uint32_t>(i + 1) * kWave <= kTreePairs || i * kWave + lane < kTreePairs) { \
+                pref[i] = src2[i * kWave + lane];                                                 \
+            }                                                                                     \
         }                                                                                         \
     } while (0)
         // packed rows are fetched two trees ahead so that the next tree's row has arrived by the
@@ -438,31 +457,30 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousTileKernel(
         uint32_t t = treeBegin + wave;
         uint32_t row = CBAMD_FETCH_ROW(t);
         uint32_t rowNext = CBAMD_FETCH_ROW(t + kTileWaves);
-        if (LEAF_LDS && DCHUNK == 1 && t < treeEnd) {
-            CBAMD_FETCH_LEAVES(__builtin_amdgcn_readlane(row, kPackedFirstLeafSlot));
+        if (LEAF_LDS && kPrefetch && t < treeEnd) {
+            CBAMD_FETCH_LEAVES(row);
         }
         while (t < treeEnd) {
             const uint32_t tNext = t + kTileWaves;
             const uint32_t rowNext2 = CBAMD_FETCH_ROW(tNext + kTileWaves);
-            const uint32_t firstLeaf = __builtin_amdgcn_readlane(row, kPackedFirstLeafSlot);
-            const double* leaf = leaves + firstLeaf;
+            const double* leaf = CBAMD_TREE_VALUES(row);
             if (LEAF_LDS) {
                 // publish this tree's leaf values in the wave's region; the previous tree's gathers
                 // were issued before these stores and LDS serves one wave's requests in order
                 double2* dst2 = reinterpret_cast<double2*>(sLeaf);
-                if (DCHUNK == 1) {
-                    if (kTreePairs >= kWave || lane < kTreePairs) {
-                        dst2[lane] = pref0;
-                    }
-                    if (kTreePairs > kWave) {
-                        dst2[kWave + lane] = pref1;
+                if (kPrefetch) {
+#pragma unroll
+                    for (int i = 0; i < kPrefetchRegs; ++i) {
+                        if (static_cast<uint32_t>(i + 1) * kWave <= kTreePairs || i * kWave + lane < kTreePairs) {
+                            dst2[i * kWave + lane] = pref[i];
+                        }
                     }
                     if (tNext < treeEnd) {
-                        CBAMD_FETCH_LEAVES(__builtin_amdgcn_readlane(rowNext, kPackedFirstLeafSlot));
+                        CBAMD_FETCH_LEAVES(rowNext);
                     }
                 } else {
                     const double2* src2 = reinterpret_cast<const double2*>(leaf);
-                    for (uint32_t i = lane; i < treeDoubles / 2; i += kWave) {
+                    for (uint32_t i = lane; i < kTreePairs; i += kWave) {
                         dst2[i] = src2[i];
                     }
                 }
@@ -471,15 +489,32 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousTileKernel(
                 leaf = sLeaf;
             }
             const uint32_t idx4 = TreeIndexes<SEVEN_BIT, MAXD>(laneTile, row);
+            if (DCHUNK == 1) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                // DCHUNK == 1 is only instantiated for one-dimensional models
-                const uint32_t leafIdx = (idx4 >> (8 * j)) & 0xffu;
-                const uint32_t li = (DCHUNK == 1 ? leafIdx : leafIdx * static_cast<uint32_t>(dim)) + d0;
+                for (int j = 0; j < 4; ++j) {
+                    acc[j][0] = __dadd_rn(acc[j][0], leaf[(idx4 >> (8 * j)) & 0xffu]);
+                }
+            } else {
+                // the DCHUNK values of the next document's leaf are requested before the current
+                // document's are added (the scheduling fences keep the two groups apart)
+                double val[2][DCHUNK];
 #pragma unroll
                 for (int k = 0; k < DCHUNK; ++k) {
-                    if (DCHUNK == 1 || d0 + k < dim) {
-                        acc[j][k] = __dadd_rn(acc[j][k], leaf[li + k]);
+                    val[0][k] = leaf[(idx4 & 0xffu) * DCHUNK + k];
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (j < 3) {
+#pragma unroll
+                        for (int k = 0; k < DCHUNK; ++k) {
+                            val[(j + 1) & 1][k] = leaf[((idx4 >> (8 * (j + 1))) & 0xffu) * DCHUNK + k];
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int k = 0; k < DCHUNK; ++k) {
+                        acc[j][k] = __dadd_rn(acc[j][k], val[j & 1][k]);
                     }
                 }
             }
@@ -492,6 +527,7 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousTileKernel(
         }
 #undef CBAMD_FETCH_ROW
 #undef CBAMD_FETCH_LEAVES
+#undef CBAMD_TREE_VALUES
         // waves add their partial sums in wave order into the LDS accumulator; the last wave
         // finishes the values and writes them out
         for (uint32_t w = 0; w + 1 < kTileWaves; ++w) {
