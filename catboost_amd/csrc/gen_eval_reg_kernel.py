@@ -1,8 +1,8 @@
 """Writes the gfx950 assembly of the register-resident evaluate kernels.
 
-The kernels evaluate oblivious trees of depth <= 8 of a one-dimensional model whose bins and
-split indexes all fit 7 bits (no xor masks), the case of float-feature models with at most 127
-used borders per feature.
+The kernels evaluate oblivious trees of depth <= 8 of a model whose bins and split indexes all fit
+7 bits (no xor masks), the case of float-feature models with at most 127 used borders per feature.
+One launch produces PITCH consecutive dimensions of the result (1 for a one-dimensional model).
 
 Layout of the work:
   * a wave owns one block of 256 documents and keeps the block's bins in vector registers for the
@@ -12,53 +12,84 @@ Layout of the work:
     VGPR index mode (S_SET_GPR_IDX_*), the one thing the HIP compiler cannot be made to emit for a
     200-register array;
   * the waves of a workgroup share the leaf values: trees go through LDS in blocks of TREE_BLOCK
-    trees (256 doubles per tree), double buffered; the copy of the next block is spread over the
-    current block's trees and goes from global memory straight into LDS (global_load_lds);
+    trees (LEAVES rows of PITCH doubles per tree), double buffered; the copy of the next block is
+    spread over the current block's trees and goes from global memory straight into LDS
+    (global_load_lds);
   * a tree's levels come from a table of 16 dwords per tree, (bucket, (128 - splitIdx) * 0x01010101)
-    per level, read with one scalar load two trees ahead;
-  * the four leaf gathers of a tree are issued behind its levels and consumed after the levels of
-    the next tree, so their LDS latency is covered; every document's sum is accumulated in fp64 in
-    tree order, exactly like the CPU evaluator (cpu/evaluator_impl.cpp:362-460), and finished as
-    ApplyScaleAndBias does (scale_and_bias.cpp:4-50).
+    per level, read with one scalar load two trees ahead; kernels for LEAVES = 64 use the first six;
+  * the leaf gathers of a tree (four documents per lane) are issued behind its levels and consumed
+    after the levels of the next tree, so their LDS latency is covered; every sum is accumulated in
+    fp64 in tree order, exactly like the CPU evaluator (cpu/evaluator_impl.cpp:362-460), and
+    finished as ApplyScaleAndBias does (scale_and_bias.cpp:4-50).
 
-Kernel arguments (72 bytes):
+Kernel arguments (80 bytes):
    0 bins        const uint32*   [docBlock][bucketCount][64]
    8 rows        const uint32*   [(treeBlocks + 2) * TREE_BLOCK][16]    (null trees behind the model's)
-  16 leaves      const double*   [(treeBlocks + 2) * TREE_BLOCK][256]
-  24 out         double*         [docCount]
+  16 leaves      const double*   [(treeBlocks + 2) * TREE_BLOCK][LEAVES][PITCH]
+  24 out         double*         [docCount][dim]
   32 docCount    uint32          36 blockCount uint32 (ceil(docCount / 256), >= 1)
   40 treeBlocks  uint32 (>= 1)   44 flags uint32 (bit 0: add the bias)
-  48 scale       double          56 bias double
-  64 bucketCount uint32 (1 .. BUCKETS)
-grid = ceil(blockCount / WAVES) workgroups of WAVES * 64 threads, LDS = 2 * TREE_BLOCK * 2048 bytes.
+  48 scale       double          56 bias const double* (first dimension of this launch)
+  64 bucketCount uint32 (1 .. BUCKETS)                68 dim uint32
+  72 first dimension of this launch uint32            76 dimensions to store uint32 (1 .. PITCH)
+grid = ceil(blockCount / WAVES) workgroups of WAVES * 64 threads, LDS = 2 * TREE_BLOCK * LEAVES *
+PITCH * 8 bytes.
 
 Usage: gen_eval_reg_kernel.py OUT.s
 """
 import sys
 
-TREE_BLOCK = 16
-TREE_BYTES = 2048
-BUF_BYTES = TREE_BLOCK * TREE_BYTES
-LDS_BYTES = 2 * BUF_BYTES
 ROW_BYTES = 64
-B0 = 32  # first bins register
+LDS_BUFFER_LIMIT = 32 * 1024
 
-# (bins registers, waves per workgroup)
-VARIANTS = [(208, 4), (96, 8)]
+# (bins registers, waves per workgroup, PITCH, LEAVES); hip_evaluator.hip lists the same variants
+VARIANTS = [
+    (208, 4, 1, 256), (96, 8, 1, 256),
+    (192, 4, 2, 64), (160, 4, 4, 64), (128, 4, 6, 64),
+    (192, 4, 2, 256), (160, 4, 4, 256), (128, 4, 6, 256),
+]
 
 
-def kernel_name(buckets, waves):
-    return "cbamd_eval_reg_b%d_w%d" % (buckets, waves)
+def kernel_name(buckets, waves, pitch, leaves):
+    return "cbamd_eval_reg_b%d_w%d_p%d_l%d" % (buckets, waves, pitch, leaves)
 
 
-def gen_kernel(buckets, waves):
-    name = kernel_name(buckets, waves)
+def tree_block(pitch, leaves):
+    """Trees per LDS buffer: a power of two, at most 16, buffer at most LDS_BUFFER_LIMIT bytes."""
+    block = 16
+    while block > 1 and block * leaves * pitch * 8 > LDS_BUFFER_LIMIT:
+        block //= 2
+    return block
+
+
+def gen_kernel(buckets, waves, pitch, leaves):
+    name = kernel_name(buckets, waves, pitch, leaves)
+    assert pitch == 1 or pitch % 2 == 0
+    depth = {64: 6, 256: 8}[leaves]
     threads = waves * 64
     row_bytes = threads * 16              # one 16-byte piece per thread
-    chunks = BUF_BYTES // row_bytes       # pieces of a tree block per thread
-    assert 1 <= chunks <= TREE_BLOCK
-    vgprs = B0 + buckets
+    tree_bytes = leaves * pitch * 8
+    block = tree_block(pitch, leaves)
+    buf_bytes = block * tree_bytes
+    lds_bytes = 2 * buf_bytes
+    assert buf_bytes % row_bytes == 0 and lds_bytes <= 65536
+    chunks = buf_bytes // row_bytes       # pieces of a tree block per thread
+    per_tree = (chunks + block - 1) // block
+    # vector registers: v0 thread, v1 lane * 4, v2 thread * 16, v3 leaf indexes, v4/v5 scratch
+    lv0 = 6                               # leaf values in flight: 4 documents x pitch doubles
+    ac0 = lv0 + 8 * pitch                 # the sums
+    ga0 = ac0 + 8 * pitch                 # gather addresses of the four documents
+    te0 = ga0 + 4                         # two scratch registers of the epilogue
+    b0 = te0 + 2                          # the bins
+    vgprs = b0 + buckets
     assert vgprs <= 256
+
+    def lv(j, k):
+        return lv0 + 2 * (j * pitch + k)
+
+    def ac(j, k):
+        return ac0 + 2 * (j * pitch + k)
+
     o = []
     e = o.append
 
@@ -72,6 +103,12 @@ def gen_kernel(buckets, waves):
         e("  s_add_u32 s26, s26, %d" % row_bytes)
         e("  s_addc_u32 s27, s27, 0")
 
+    def add_leaf_values():
+        for j in range(4):
+            for k in range(pitch):
+                e("  v_add_f64 v[%d:%d], v[%d:%d], v[%d:%d]" % (ac(j, k), ac(j, k) + 1, ac(j, k), ac(j, k) + 1,
+                                                                 lv(j, k), lv(j, k) + 1))
+
     e(".text")
     e(".globl %s" % name)
     e(".p2align 8")
@@ -80,7 +117,7 @@ def gen_kernel(buckets, waves):
     # s[0:1] kernarg segment, s2 workgroup id, v0 thread id
     e("  s_load_dwordx8 s[4:11], s[0:1], 0x0")
     e("  s_load_dwordx8 s[12:19], s[0:1], 0x20")
-    e("  s_load_dword s29, s[0:1], 0x40")
+    e("  s_load_dwordx4 s[72:75], s[0:1], 0x40")
     e("  v_and_b32_e32 v0, 0x3ff, v0")           # work-item ids come packed; keep x
     e("  v_lshrrev_b32_e32 v5, 6, v0")
     e("  v_and_b32_e32 v1, 63, v0")
@@ -91,7 +128,9 @@ def gen_kernel(buckets, waves):
     e("  s_nop 1")
     e("  v_readfirstlane_b32 s20, v5")           # wave of the workgroup
     e("  s_mov_b32 s22, 0x80808080")
-    e("  s_mov_b32 s23, 3")
+    # byte j of the leaf indexes times s23 = offset of the document's leaf row in a tree's table
+    # (a six-level index sits in bits 2..7 of its byte)
+    e("  s_mov_b32 s23, %d" % (pitch * 8 >> (8 - depth)))
     e("  s_lshl_b32 s68, s20, 10")               # LDS offset of the wave's part of a copied piece
     e("  s_waitcnt lgkmcnt(0)")
     # first tree block -> buffer 0
@@ -104,33 +143,33 @@ def gen_kernel(buckets, waves):
     e("  s_add_u32 s21, s21, s20")
     e("  s_add_u32 s24, s13, -1")
     e("  s_min_u32 s24, s21, s24")
-    e("  s_lshl_b32 s25, s29, 8")                # bytes of bins per document block
+    e("  s_lshl_b32 s25, s72, 8")                # bytes of bins per document block
     e("  s_mul_hi_u32 s31, s24, s25")
     e("  s_mul_i32 s30, s24, s25")
     e("  s_add_u32 s64, s4, s30")
     e("  s_addc_u32 s65, s5, s31")
-    e("  s_add_u32 s28, s29, -1")
+    e("  s_add_u32 s28, s72, -1")
     for i in range(buckets):
         # registers past the model's bucket count reload the last bucket and are never indexed
         e("  s_min_u32 s24, %d, s28" % i)
         e("  s_lshl_b32 s24, s24, 8")
         e("  s_add_u32 s66, s64, s24")
         e("  s_addc_u32 s67, s65, 0")
-        e("  global_load_dword v%d, v1, s[66:67]" % (B0 + i))
+        e("  global_load_dword v%d, v1, s[66:67]" % (b0 + i))
     e("  s_load_dwordx16 s[32:47], s[6:7], 0x0")
     e("  s_load_dwordx16 s[48:63], s[6:7], 0x%x" % ROW_BYTES)
-    for r in range(6, 22):
-        e("  v_mov_b32_e32 v%d, 0" % r)          # leaf values in flight and the four sums
+    for r in range(lv0, ga0):
+        e("  v_mov_b32_e32 v%d, 0" % r)          # leaf values in flight and the sums
     e("  s_waitcnt vmcnt(0) lgkmcnt(0)")
     e("  s_barrier")
-    e("  s_set_gpr_idx_on s23, 0x1")             # src0 of VALU instructions becomes index relative
+    e("  s_set_gpr_idx_on s22, 0x1")             # src0 of VALU instructions becomes index relative
     e("%s_loop:" % name)
     for buf in range(2):
-        for i in range(TREE_BLOCK):
+        for i in range(block):
             rows = 32 if i % 2 == 0 else 48
-            for d in range(8):
+            for d in range(depth):
                 e("  s_set_gpr_idx_idx s%d" % (rows + 2 * d))
-                e("  v_add_u32_e64 v4, v%d, s%d" % (B0, rows + 2 * d + 1))
+                e("  v_add_u32_e64 v4, v%d, s%d" % (b0, rows + 2 * d + 1))
                 if d == 0:
                     e("  v_and_b32_e32 v3, s22, v4")
                 else:
@@ -139,59 +178,71 @@ def gen_kernel(buckets, waves):
             e("  s_set_gpr_idx_idx 0")
             # previous tree's leaf values have arrived (and so has the next tree's row)
             e("  s_waitcnt lgkmcnt(0)")
+            add_leaf_values()
             for j in range(4):
-                a = 14 + 2 * j
-                l = 6 + 2 * j
-                e("  v_add_f64 v[%d:%d], v[%d:%d], v[%d:%d]" % (a, a + 1, a, a + 1, l, l + 1))
-            for j in range(4):
-                l = 6 + 2 * j
-                e("  v_lshlrev_b32_sdwa v%d, s23, v3 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_%d"
-                  % (22 + j, j))
-                e("  ds_read_b64 v[%d:%d], v%d offset:%d" % (l, l + 1, 22 + j, buf * BUF_BYTES + i * TREE_BYTES))
-            e("  s_load_dwordx16 s[%d:%d], s[6:7], 0x%x" % (rows, rows + 15, (buf * TREE_BLOCK + i + 2) * ROW_BYTES))
-            # copy of the next tree block into the other buffer, one piece per tree
-            if i < chunks:
-                stage((1 - buf) * BUF_BYTES + i * row_bytes)
+                e("  v_mul_u32_u24_sdwa v%d, s23, v3 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_%d"
+                  % (ga0 + j, j))
+                tree_offset = buf * buf_bytes + i * tree_bytes
+                if pitch == 1:
+                    e("  ds_read_b64 v[%d:%d], v%d offset:%d" % (lv(j, 0), lv(j, 0) + 1, ga0 + j, tree_offset))
+                else:
+                    for k in range(0, pitch, 2):
+                        e("  ds_read_b128 v[%d:%d], v%d offset:%d" % (lv(j, k), lv(j, k) + 3, ga0 + j,
+                                                                     tree_offset + 8 * k))
+            e("  s_load_dwordx16 s[%d:%d], s[6:7], 0x%x" % (rows, rows + 15, (buf * block + i + 2) * ROW_BYTES))
+            # copy of the next tree block into the other buffer, spread over this block's trees
+            staged = False
+            for c in range(i * per_tree, min(chunks, (i + 1) * per_tree)):
+                stage((1 - buf) * buf_bytes + c * row_bytes)
+                staged = True
+            if staged:
                 e("  s_mov_b32 m0, 0x1000")      # index mode value again: src0 relative, index 0
             if i == 0:
                 # the rows of the next tree block are pulled into the scalar cache now, so that the
                 # per-tree row loads of that block do not each wait for a miss
-                for k in range(TREE_BLOCK):
-                    e("  s_load_dword s3, s[6:7], 0x%x" % ((buf * TREE_BLOCK + TREE_BLOCK + 2 + k) * ROW_BYTES))
+                for k in range(block):
+                    e("  s_load_dword s3, s[6:7], 0x%x" % ((buf * block + block + 2 + k) * ROW_BYTES))
         # every wave is done reading this buffer and writing the other one
         e("  s_waitcnt vmcnt(0) lgkmcnt(0)")
         e("  s_barrier")
         e("  s_add_u32 s14, s14, -1")
         e("  s_cmp_eq_u32 s14, 0")
         e("  s_cbranch_scc1 %s_done" % name)
-    e("  s_add_u32 s6, s6, %d" % (2 * TREE_BLOCK * ROW_BYTES))
+    e("  s_add_u32 s6, s6, %d" % (2 * block * ROW_BYTES))
     e("  s_addc_u32 s7, s7, 0")
     e("  s_branch %s_loop" % name)
     e("%s_done:" % name)
-    for j in range(4):
-        a = 14 + 2 * j
-        l = 6 + 2 * j
-        e("  v_add_f64 v[%d:%d], v[%d:%d], v[%d:%d]" % (a, a + 1, a, a + 1, l, l + 1))
+    add_leaf_values()
     e("  s_set_gpr_idx_off")
+    # scale, bias of the launch's dimensions (rows registers are free now)
+    for k in range(pitch):
+        e("  s_load_dwordx2 s[%d:%d], s[18:19], 0x%x" % (32 + 2 * k, 33 + 2 * k, 8 * k))
     for j in range(4):
-        a = 14 + 2 * j
-        e("  v_mul_f64 v[%d:%d], s[16:17], v[%d:%d]" % (a, a + 1, a, a + 1))
+        for k in range(pitch):
+            e("  v_mul_f64 v[%d:%d], s[16:17], v[%d:%d]" % (ac(j, k), ac(j, k) + 1, ac(j, k), ac(j, k) + 1))
+    e("  s_waitcnt lgkmcnt(0)")
     e("  s_bitcmp1_b32 s15, 0")
     e("  s_cbranch_scc0 %s_store" % name)
     for j in range(4):
-        a = 14 + 2 * j
-        e("  v_add_f64 v[%d:%d], v[%d:%d], s[18:19]" % (a, a + 1, a, a + 1))
+        for k in range(pitch):
+            e("  v_add_f64 v[%d:%d], v[%d:%d], s[%d:%d]" % (ac(j, k), ac(j, k) + 1, ac(j, k), ac(j, k) + 1,
+                                                             32 + 2 * k, 33 + 2 * k))
     e("%s_store:" % name)
     e("  v_and_b32_e32 v5, 63, v0")
     e("  s_lshl_b32 s24, s21, 8")
     e("  v_add_u32_e32 v5, s24, v5")
     for j in range(4):
-        a = 14 + 2 * j
-        e("  v_add_u32_e32 v30, %d, v5" % (64 * j))
-        e("  v_cmp_gt_u32_e32 vcc, s12, v30")
+        e("  v_add_u32_e32 v%d, %d, v5" % (te0, 64 * j))
+        e("  v_cmp_gt_u32_e32 vcc, s12, v%d" % te0)
         e("  s_and_saveexec_b64 s[30:31], vcc")
-        e("  v_lshlrev_b32_e32 v31, 3, v30")
-        e("  global_store_dwordx2 v31, v[%d:%d], s[10:11]" % (a, a + 1))
+        e("  v_mul_lo_u32 v%d, v%d, s73" % (te0 + 1, te0))               # document * dim
+        e("  v_add_lshl_u32 v%d, v%d, s74, 3" % (te0 + 1, te0 + 1))     # + first dimension, in bytes
+        for k in range(pitch):
+            if k > 0:
+                e("  s_cmp_gt_u32 s75, %d" % k)
+                e("  s_cbranch_scc0 %s_stored_%d" % (name, j))
+            e("  global_store_dwordx2 v%d, v[%d:%d], s[10:11] offset:%d" % (te0 + 1, ac(j, k), ac(j, k) + 1, 8 * k))
+        e("%s_stored_%d:" % (name, j))
         e("  s_mov_b64 exec, s[30:31]")
     e("  s_endpgm")
     e(".Lend_%s:" % name)
@@ -200,9 +251,9 @@ def gen_kernel(buckets, waves):
     e(".rodata")
     e(".p2align 6")
     e(".amdhsa_kernel %s" % name)
-    e("  .amdhsa_group_segment_fixed_size %d" % LDS_BYTES)
+    e("  .amdhsa_group_segment_fixed_size %d" % lds_bytes)
     e("  .amdhsa_private_segment_fixed_size 0")
-    e("  .amdhsa_kernarg_size 72")
+    e("  .amdhsa_kernarg_size 80")
     e("  .amdhsa_user_sgpr_count 2")
     e("  .amdhsa_user_sgpr_kernarg_segment_ptr 1")
     e("  .amdhsa_system_sgpr_workgroup_id_x 1")
@@ -210,7 +261,7 @@ def gen_kernel(buckets, waves):
     e("  .amdhsa_system_sgpr_workgroup_id_z 0")
     e("  .amdhsa_system_vgpr_workitem_id 0")
     e("  .amdhsa_next_free_vgpr %d" % vgprs)
-    e("  .amdhsa_next_free_sgpr 69")
+    e("  .amdhsa_next_free_sgpr 76")
     e("  .amdhsa_accum_offset %d" % ((vgprs + 3) // 4 * 4))
     e("  .amdhsa_reserve_vcc 1")
     e("  .amdhsa_float_round_mode_32 0")
@@ -232,15 +283,18 @@ def gen_kernel(buckets, waves):
       - {.offset: 40, .size: 4, .value_kind: by_value}
       - {.offset: 44, .size: 4, .value_kind: by_value}
       - {.offset: 48, .size: 8, .value_kind: by_value}
-      - {.offset: 56, .size: 8, .value_kind: by_value}
+      - {.address_space: global, .offset: 56, .size: 8, .value_kind: global_buffer}
       - {.offset: 64, .size: 4, .value_kind: by_value}
+      - {.offset: 68, .size: 4, .value_kind: by_value}
+      - {.offset: 72, .size: 4, .value_kind: by_value}
+      - {.offset: 76, .size: 4, .value_kind: by_value}
     .group_segment_fixed_size: %d
     .kernarg_segment_align: 8
-    .kernarg_segment_size: 72
+    .kernarg_segment_size: 80
     .max_flat_workgroup_size: %d
     .name: %s
     .private_segment_fixed_size: 0
-    .sgpr_count: 76
+    .sgpr_count: 84
     .sgpr_spill_count: 0
     .symbol: %s.kd
     .uniform_work_group_size: 1
@@ -248,15 +302,15 @@ def gen_kernel(buckets, waves):
     .vgpr_count: %d
     .vgpr_spill_count: 0
     .wavefront_size: 64
-""" % (LDS_BYTES, threads, name, name, vgprs)
+""" % (lds_bytes, threads, name, name, vgprs)
     return "\n".join(o), meta
 
 
 def generate():
     parts = ['.amdgcn_target "amdgcn-amd-amdhsa--gfx950"', ".amdhsa_code_object_version 6", ""]
     metas = []
-    for buckets, waves in VARIANTS:
-        text, meta = gen_kernel(buckets, waves)
+    for buckets, waves, pitch, leaves in VARIANTS:
+        text, meta = gen_kernel(buckets, waves, pitch, leaves)
         parts.append(text)
         metas.append(meta)
     parts.append(".amdgpu_metadata")

@@ -89,7 +89,7 @@ alignas(4096) const unsigned char kEvalRegCodeObject[] = {
 #include "eval_reg_kernel_co.inc"
 };
 
-// Must match gen_eval_reg_kernel.py: kernel arguments, tree block, variants.
+// Must match gen_eval_reg_kernel.py: kernel arguments, variants, trees per LDS buffer.
 struct TEvalRegArgs {
     const void* Bins;
     const void* Rows;
@@ -100,25 +100,55 @@ struct TEvalRegArgs {
     uint32_t TreeBlocks;
     uint32_t Flags;
     double Scale;
-    double Bias;
+    const double* Bias;
     uint32_t BucketCount;
-    uint32_t Pad;
+    uint32_t Dim;
+    uint32_t FirstDim;
+    uint32_t StoreDims;
 };
-static_assert(sizeof(TEvalRegArgs) == 72, "kernel argument block of the register-resident kernels");
+static_assert(sizeof(TEvalRegArgs) == 80, "kernel argument block of the register-resident kernels");
 
-constexpr uint32_t kRegTreeBlock = 16;
 constexpr uint32_t kRegRowDwords = 16;
-constexpr uint32_t kRegTreeLeaves = 256;
 struct TEvalRegVariant {
     uint32_t Buckets;
     uint32_t Waves;
+    uint32_t Pitch;   // dimensions per launch = doubles per leaf row
+    uint32_t Leaves;  // leaf rows per tree (64: trees of depth <= 6)
     const char* Name;
 };
 constexpr TEvalRegVariant kEvalRegVariants[] = {
-    {96, 8, "cbamd_eval_reg_b96_w8"},
-    {208, 4, "cbamd_eval_reg_b208_w4"},
+    {96, 8, 1, 256, "cbamd_eval_reg_b96_w8_p1_l256"},   {208, 4, 1, 256, "cbamd_eval_reg_b208_w4_p1_l256"},
+    {192, 4, 2, 64, "cbamd_eval_reg_b192_w4_p2_l64"},   {160, 4, 4, 64, "cbamd_eval_reg_b160_w4_p4_l64"},
+    {128, 4, 6, 64, "cbamd_eval_reg_b128_w4_p6_l64"},   {192, 4, 2, 256, "cbamd_eval_reg_b192_w4_p2_l256"},
+    {160, 4, 4, 256, "cbamd_eval_reg_b160_w4_p4_l256"}, {128, 4, 6, 256, "cbamd_eval_reg_b128_w4_p6_l256"},
 };
-constexpr size_t kEvalRegVariantCount = sizeof(kEvalRegVariants) / sizeof(kEvalRegVariants[0]);
+
+// trees per LDS buffer of a variant: a power of two, at most 16, buffer at most 32 KB
+uint32_t RegTreeBlock(const TEvalRegVariant& v) {
+    uint32_t block = 16;
+    while (block > 1 && block * v.Leaves * v.Pitch * 8 > 32 * 1024) {
+        block /= 2;
+    }
+    return block;
+}
+
+// The variant for a model: one-dimensional models take the smallest register file that holds
+// their buckets; others the pitch that needs the fewest launches (then the smallest such pitch).
+const TEvalRegVariant* PickRegVariant(uint32_t buckets, uint32_t dim, uint32_t maxDepth) {
+    const TEvalRegVariant* best = nullptr;
+    uint32_t bestLaunches = 0;
+    for (const auto& v : kEvalRegVariants) {
+        if (buckets > v.Buckets || (dim == 1) != (v.Pitch == 1) || v.Leaves != (dim > 1 && maxDepth <= 6 ? 64u : 256u)) {
+            continue;
+        }
+        const uint32_t launches = (dim + v.Pitch - 1) / v.Pitch;
+        if (!best || launches < bestLaunches || (launches == bestLaunches && dim > 1 && v.Pitch < best->Pitch)) {
+            best = &v;
+            bestLaunches = launches;
+        }
+    }
+    return best;
+}
 
 // dimensions the tile kernel accumulates per pass over the trees (and the pitch of its padded leaf rows)
 int TileChunk(int dim) {
@@ -300,9 +330,12 @@ struct THipEvaluator::TImpl {
     hipModule_t RegModule = nullptr;
     hipFunction_t RegFunction = nullptr;
     uint32_t RegWaves = 0;
+    uint32_t RegPitch = 1;
     uint32_t RegTreeBlocks = 0;
+    size_t RegLaunchLeaves = 0;  // doubles of the leaf table of one launch
     TDeviceVec<uint32_t> RegRows;
-    TDeviceVec<double> RegLeaves;
+    TDeviceVec<double> RegLeaves;  // [launch][tree][leaf row][pitch]
+    TDeviceVec<double> RegBias;    // the bias, readable for a whole pitch behind every dimension
 
     // scratch (grow-only, guarded by THipEvaluator::Lock)
     TDeviceVec<uint8_t> ScratchBins;
@@ -557,21 +590,24 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId)
 
     const char* regSwitch = std::getenv("CATBOOST_AMD_REG_KERNEL");
     const bool regEnabled = !(regSwitch && regSwitch[0] == '0');
-    const TEvalRegVariant* variant = nullptr;
-    for (size_t i = 0; i < kEvalRegVariantCount && !variant; ++i) {
-        if (m.LayoutBuckets <= kEvalRegVariants[i].Buckets) {
-            variant = &kEvalRegVariants[i];
-        }
-    }
-    if (regEnabled && variant && m.Oblivious && m.MaxDepth <= 8 && m.PackedSevenBit && m.Dim == 1 && TreeCount > 0) {
+    const TEvalRegVariant* variant =
+        m.Oblivious && m.MaxDepth <= 8 && m.PackedSevenBit && TreeCount > 0
+            ? PickRegVariant(m.LayoutBuckets, static_cast<uint32_t>(m.Dim), m.MaxDepth)
+            : nullptr;
+    if (regEnabled && variant) {
         HIP_CHECK(hipModuleLoadData(&m.RegModule, kEvalRegCodeObject));
         HIP_CHECK(hipModuleGetFunction(&m.RegFunction, m.RegModule, variant->Name));
+        const uint32_t block = RegTreeBlock(*variant);
+        const size_t pitch = variant->Pitch, rowsPerTree = variant->Leaves;
         m.RegWaves = variant->Waves;
-        m.RegTreeBlocks = static_cast<uint32_t>((TreeCount + kRegTreeBlock - 1) / kRegTreeBlock);
+        m.RegPitch = variant->Pitch;
+        m.RegTreeBlocks = static_cast<uint32_t>((TreeCount + block - 1) / block);
         // two blocks of null trees behind the last one: the kernels prefetch that far
-        const size_t tableTrees = (static_cast<size_t>(m.RegTreeBlocks) + 2) * kRegTreeBlock;
+        const size_t tableTrees = (static_cast<size_t>(m.RegTreeBlocks) + 2) * block;
+        const size_t launches = (static_cast<size_t>(m.Dim) + pitch - 1) / pitch;
+        m.RegLaunchLeaves = tableTrees * rowsPerTree * pitch;
         std::vector<uint32_t> rows(tableTrees * kRegRowDwords, 0);  // (bucket 0, add 0): false for every bin
-        std::vector<double> leaves(tableTrees * kRegTreeLeaves, 0.0);
+        std::vector<double> leaves(launches * m.RegLaunchLeaves, 0.0);
         for (size_t t = 0; t < TreeCount; ++t) {
             const int depth = trees.TreeSizes[t];
             for (int d = 0; d < depth; ++d) {
@@ -579,11 +615,21 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId)
                 rows[t * kRegRowDwords + 2 * d] = rb.FeatureIndex;
                 rows[t * kRegRowDwords + 2 * d + 1] = (128u - rb.SplitIdx) * 0x01010101u;
             }
-            std::copy_n(trees.LeafValues.begin() + trees.TreeFirstLeafOffsets[t], size_t(1) << depth,
-                        leaves.begin() + t * kRegTreeLeaves);
+            const double* values = trees.LeafValues.data() + trees.TreeFirstLeafOffsets[t];
+            for (size_t launch = 0; launch < launches; ++launch) {
+                double* table = leaves.data() + launch * m.RegLaunchLeaves + t * rowsPerTree * pitch;
+                for (size_t leaf = 0; leaf < (size_t(1) << depth); ++leaf) {
+                    for (size_t k = 0; k < pitch && launch * pitch + k < static_cast<size_t>(m.Dim); ++k) {
+                        table[leaf * pitch + k] = values[leaf * m.Dim + launch * pitch + k];
+                    }
+                }
+            }
         }
+        std::vector<double> biasPadded(static_cast<size_t>(m.Dim) + pitch, 0.0);
+        std::copy(m.HostBias.begin(), m.HostBias.end(), biasPadded.begin());
         m.RegRows.Upload(rows);
         m.RegLeaves.Upload(leaves);
+        m.RegBias.Upload(biasPadded);
         m.RegKernelUsable = true;
     }
 }
@@ -868,25 +914,30 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
     CBAMD_ENSURE(bins != nullptr, "quantized buffer is null");
     const dev::TTreeTables tt = m.TreeTables();
     const uint32_t tb = static_cast<uint32_t>(treeStart), te = static_cast<uint32_t>(treeEnd);
-    if (m.RegKernelUsable && treeStart == 0 && treeEnd == TreeCount && docCount < (size_t(1) << 29)) {
-        // whole model over bins kept in registers
+    if (m.RegKernelUsable && treeStart == 0 && treeEnd == TreeCount && docCount * m.Dim < (size_t(1) << 29)) {
+        // whole model over bins kept in registers, RegPitch dimensions per launch
         TEvalRegArgs args = {};
         args.Bins = bins;
         args.Rows = m.RegRows.Get();
-        args.Leaves = m.RegLeaves.Get();
         args.Out = results;
         args.DocCount = static_cast<uint32_t>(docCount);
         args.BlockCount = static_cast<uint32_t>((docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock);
         args.TreeBlocks = m.RegTreeBlocks;
         args.Flags = 1;  // the range starts at tree 0: add the bias
         args.Scale = m.Scale;
-        args.Bias = m.HostBias.empty() ? 0.0 : m.HostBias[0];
         args.BucketCount = m.LayoutBuckets;
-        size_t argSize = sizeof(args);
-        void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &argSize,
-                          HIP_LAUNCH_PARAM_END};
+        args.Dim = static_cast<uint32_t>(m.Dim);
         const uint32_t grid = (args.BlockCount + m.RegWaves - 1) / m.RegWaves;
-        HIP_CHECK(hipModuleLaunchKernel(m.RegFunction, grid, 1, 1, 64 * m.RegWaves, 1, 1, 0, s, nullptr, config));
+        for (uint32_t first = 0, launch = 0; first < args.Dim; first += m.RegPitch, ++launch) {
+            args.Leaves = m.RegLeaves.Get() + launch * m.RegLaunchLeaves;
+            args.Bias = m.RegBias.Get() + first;
+            args.FirstDim = first;
+            args.StoreDims = std::min(m.RegPitch, args.Dim - first);
+            size_t argSize = sizeof(args);
+            void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &argSize,
+                              HIP_LAUNCH_PARAM_END};
+            HIP_CHECK(hipModuleLaunchKernel(m.RegFunction, grid, 1, 1, 64 * m.RegWaves, 1, 1, 0, s, nullptr, config));
+        }
         return;
     }
     const int dchunk = TileChunk(m.Dim);

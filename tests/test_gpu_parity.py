@@ -196,7 +196,7 @@ def test_random_oblivious_models(seed, dim):
     _close(g.calc_hashed(floats, cats), o.calc(floats, cats, layout="split"))
 
 
-def _float_only_model(rng, n_float, trees, max_depth, scale=1.0, bias=None):
+def _float_only_model(rng, n_float, trees, max_depth, scale=1.0, bias=None, dim=1):
     """Oblivious model over float features only (at most 40 borders each), every feature used."""
     ffs = [mb.float_feature(i, i) for i in range(n_float)]
     cands = [np.unique(rng.normal(size=int(rng.integers(1, 40))).astype(np.float32)) for _ in range(n_float)]
@@ -214,9 +214,9 @@ def _float_only_model(rng, n_float, trees, max_depth, scale=1.0, bias=None):
             else:
                 f = int(rng.integers(0, n_float))
             splits.append(("float", f, float(rng.choice(cands[f]))))
-        tree_list.append((splits, rng.normal(size=1 << depth)))
+        tree_list.append((splits, rng.normal(size=(1 << depth) * dim)))
         t += 1
-    return mb.build_oblivious(ffs, [], 1, tree_list, scale=scale, bias=bias)
+    return mb.build_oblivious(ffs, [], dim, tree_list, scale=scale, bias=bias)
 
 
 # Models of this kind (one-dimensional, float features with < 128 borders, depth <= 8, at most
@@ -245,6 +245,23 @@ def test_register_kernel_shapes(n_float, trees, max_depth, docs):
     if len(model["tree_sizes"]) >= 3:
         _close(g.calc_flat(x, tree_start=1, tree_end=len(model["tree_sizes"]) - 1),
                o.calc(x, tree_start=1, tree_end=len(model["tree_sizes"]) - 1))
+
+
+@pytest.mark.parametrize("dim,max_depth,n_float,trees,docs", [
+    (2, 6, 10, 20, 1000), (3, 6, 30, 33, 3000), (5, 8, 12, 9, 700), (6, 6, 128, 50, 2500), (7, 8, 100, 21, 1300),
+    (10, 6, 100, 100, 5000), (13, 8, 60, 18, 900), (20, 6, 40, 30, 2049), (4, 6, 160, 60, 600), (2, 8, 192, 70, 600),
+])
+def test_register_kernel_multi_dimensional(dim, max_depth, n_float, trees, docs):
+    """Multi-dimensional float-only models: several launches of a register-resident kernel, each
+    adding its dimensions in tree order like the CPU evaluator, hence bit for bit."""
+    rng = np.random.default_rng(77 * dim + trees)
+    model = _float_only_model(rng, n_float, trees, max_depth, scale=1.25, bias=list(rng.normal(size=dim)), dim=dim)
+    x = rng.normal(size=(docs, n_float)).astype(np.float32)
+    o = OracleModel(model)
+    g = _gpu_model(model)
+    np.testing.assert_array_equal(g.calc_flat(x), o.calc(x))
+    _close(g.calc_flat(x, tree_start=1, tree_end=len(model["tree_sizes"])),
+           o.calc(x, tree_start=1, tree_end=len(model["tree_sizes"])))
 
 
 def test_register_kernel_against_tile_kernel():
