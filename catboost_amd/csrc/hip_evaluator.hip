@@ -150,6 +150,26 @@ const TEvalRegVariant* PickRegVariant(uint32_t buckets, uint32_t dim, uint32_t m
     return best;
 }
 
+// log2 of the LDS slots per bucket of the row binarize kernel: the smallest count that still
+// exceeds the largest bucket of the model
+int BinarizeLog2Slots(uint32_t maxBucketValues) {
+    return maxBucketValues < 32 ? 5 : maxBucketValues < 64 ? 6 : maxBucketValues < 128 ? 7 : 8;
+}
+
+// Host twin of dev::GridCell: the same two roundings and the same truncation.
+uint32_t GridCell(float v, float lo, float scale) {
+    volatile float d = v - lo;
+    volatile float t = d * scale;
+    const float tt = t;
+    if (!(tt > 0.0f)) {
+        return 0;
+    }
+    if (tt >= 4294967296.0f) {
+        return dev::kLutCells - 1;
+    }
+    return std::min<uint32_t>(static_cast<uint32_t>(tt), dev::kLutCells - 1);
+}
+
 // dimensions the tile kernel accumulates per pass over the trees (and the pitch of its padded leaf rows)
 int TileChunk(int dim) {
     return dim == 1 ? 1 : dim == 2 ? 2 : dim <= 4 ? 4 : dim <= 8 ? 8 : dim <= 12 ? 12 : 16;
@@ -302,6 +322,8 @@ struct THipEvaluator::TImpl {
 
     // binarize tables
     TDeviceVec<uint32_t> BucketSrcFlat, BucketSrcSplit, BucketOffset, BucketFlags, Values;
+    TDeviceVec<uint32_t> BucketGrid;  // 4 dwords per bucket: lowest border, cells per unit, search steps, 0
+    TDeviceVec<uint32_t> BucketLut;   // kLutCells bytes per bucket
     // tree tables
     TDeviceVec<uint32_t> Splits, TreeStart, TreeSize, FirstLeaf, StepNodes, NodeToLeaf;
     TDeviceVec<double> Leaves, Bias;
@@ -357,6 +379,8 @@ struct THipEvaluator::TImpl {
         t.BucketOffset = BucketOffset.Get();
         t.BucketFlags = BucketFlags.Get();
         t.Values = Values.Get();
+        t.Grid = reinterpret_cast<const uint4*>(BucketGrid.Get());
+        t.Lut = BucketLut.Get();
         return t;
     }
     dev::TTreeTables TreeTables() const {
@@ -470,6 +494,53 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId)
         srcSplit.push_back(0);
         offsets.push_back(0);
         flags.push_back(0);
+    }
+    // grid and search window of every float bucket (dev::CountBelowInCell)
+    {
+        const uint32_t slots = 1u << BinarizeLog2Slots(m.MaxBucketValues);
+        const size_t bucketRows = offsets.size() - 1;
+        std::vector<uint32_t> grid(bucketRows * 4, 0), lut(bucketRows * (dev::kLutCells / 4), 0);
+        for (size_t b = 0; b < bucketRows; ++b) {
+            const uint32_t n = offsets[b + 1] - offsets[b];
+            if ((flags[b] & dev::kBucketFlagOneHot) || n == 0) {
+                continue;
+            }
+            std::vector<float> borders(n);
+            std::memcpy(borders.data(), values.data() + offsets[b], n * sizeof(float));
+            float lo = borders.front(), scale = 0.0f;
+            const float span = borders.back() - lo;
+            if (std::isfinite(lo) && std::isfinite(span) && span > 0.0f) {
+                scale = static_cast<float>(dev::kLutCells) / span;
+                if (!std::isfinite(scale)) {
+                    scale = 0.0f;
+                }
+            } else {
+                lo = 0.0f;
+            }
+            // start[c] = borders in cells below c; the tallest cell decides the number of steps
+            std::vector<uint32_t> population(dev::kLutCells, 0);
+            for (float x : borders) {
+                ++population[GridCell(x, lo, scale)];
+            }
+            const uint32_t tallest = *std::max_element(population.begin(), population.end());
+            uint32_t steps = 0;
+            while ((1u << steps) - 1 < tallest) {
+                ++steps;
+            }
+            CBAMD_ENSURE((1u << steps) <= slots, "internal error: search window exceeds the bucket's slots");
+            uint8_t* cells = reinterpret_cast<uint8_t*>(lut.data() + b * (dev::kLutCells / 4));
+            uint32_t start = 0;
+            for (int c = 0; c < dev::kLutCells; ++c) {
+                // a lower start only adds borders known to be below the value; it keeps the window inside the slots
+                cells[c] = static_cast<uint8_t>(std::min(start, slots - (1u << steps)));
+                start += population[c];
+            }
+            std::memcpy(&grid[b * 4 + 0], &lo, 4);
+            std::memcpy(&grid[b * 4 + 1], &scale, 4);
+            grid[b * 4 + 2] = steps;
+        }
+        m.BucketGrid.Upload(grid);
+        m.BucketLut.Upload(lut);
     }
     m.BucketSrcFlat.Upload(srcFlat);
     m.BucketSrcSplit.Upload(srcSplit);
@@ -675,6 +746,7 @@ void LaunchBinarizeRowsPC(size_t blocks, const float* floats, size_t stride, con
     CBAMD_ENSURE(groups * tiles < (size_t(1) << 31), "batch is too large for one binarize launch");
     const dim3 grid(static_cast<uint32_t>(groups * tiles));
     const size_t lds = (static_cast<size_t>(dev::kBucketTile) << LOG2P) * 4 +
+                       static_cast<size_t>(dev::kBucketTile) * dev::kLutCells +
                        static_cast<size_t>(dev::kBucketTile) * dev::kTilePitch * 4;
     auto kernel = dev::BinarizeRowsKernel<LOG2P, CATS_MATRIX>;
     if (lds > 64 * 1024) {
@@ -702,11 +774,12 @@ void LaunchBinarizeRows(uint32_t maxBucketValues, size_t blocks, const float* fl
                         uint32_t* bins, hipStream_t s) {
     CBAMD_ENSURE(docCount < (size_t(1) << 31) && stride < (size_t(1) << 31) && catStride < (size_t(1) << 31),
                  "batch is too large for one binarize launch");
-    if (maxBucketValues < 32) {
+    const int log2Slots = BinarizeLog2Slots(maxBucketValues);
+    if (log2Slots == 5) {
         LaunchBinarizeRowsP<5>(blocks, floats, stride, cats, catStride, docCount, tab, bins, s);
-    } else if (maxBucketValues < 64) {
+    } else if (log2Slots == 6) {
         LaunchBinarizeRowsP<6>(blocks, floats, stride, cats, catStride, docCount, tab, bins, s);
-    } else if (maxBucketValues < 128) {
+    } else if (log2Slots == 7) {
         LaunchBinarizeRowsP<7>(blocks, floats, stride, cats, catStride, docCount, tab, bins, s);
     } else {
         LaunchBinarizeRowsP<8>(blocks, floats, stride, cats, catStride, docCount, tab, bins, s);

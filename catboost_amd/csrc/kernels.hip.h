@@ -32,6 +32,10 @@ struct TBinarizeTables {
     const uint32_t* BucketOffset;  // [BucketCount + 1] offsets into Values
     const uint32_t* BucketFlags;
     const uint32_t* Values;        // float borders (sorted ascending) or one-hot values, as bits
+    // float buckets, row binarize kernel: a uniform grid of kLutCells cells over the bucket's borders
+    // gives the search a start and a short window instead of the whole border array
+    const uint4* Grid;             // per bucket: lowest border, cells per unit (both fp32 bits), search steps, 0
+    const uint32_t* Lut;           // per bucket kLutCells bytes: first border the search looks at, per cell
 };
 
 struct TTreeTables {
@@ -60,6 +64,32 @@ __device__ __forceinline__ uint32_t CountBelow(const uint32_t* borders, float v)
     return static_cast<uint32_t>(p - borders);
 }
 
+constexpr int kLutCells = 256;
+
+// Cell of a value in a bucket's grid: (v - lo) * scale, truncated, negative and NaN to 0, at most
+// kLutCells - 1. Subtract and multiply are separate roundings, and the host computes the borders'
+// cells with the very same operations (GridCell in hip_evaluator.hip), so cell(b) <= cell(v)
+// whenever b <= v: every border in a lower cell is below v, every border in a higher cell above.
+__device__ __forceinline__ uint32_t GridCell(float v, float lo, float scale) {
+    const float t = __fmul_rn(__fsub_rn(v, lo), scale);
+    uint32_t c;
+    asm("v_cvt_u32_f32 %0, %1" : "=v"(c) : "v"(t));  // saturating, NaN -> 0
+    return min(c, static_cast<uint32_t>(kLutCells - 1));
+}
+
+// Number of borders strictly below v, searching only the window the value's cell points at:
+// `lut[cell]` borders are known to be below v, the next 2 * topStep - 1 entries hold every border of
+// the cell (and then higher ones or the +inf padding, which never count).
+__device__ __forceinline__ uint32_t CountBelowInCell(const uint32_t* borders, const uint8_t* lut, float lo, float scale,
+                                                     uint32_t topStep, float v) {
+    const uint32_t* p = borders + lut[GridCell(v, lo, scale)];
+    for (uint32_t step = topStep; step >= 1; step >>= 1) {
+        const float b = __uint_as_float(p[step - 1]);
+        p = (b < v) ? p + step : p;
+    }
+    return static_cast<uint32_t>(p - borders);
+}
+
 __device__ __forceinline__ uint32_t OneHotBin(const uint32_t* values, uint32_t count, uint32_t v) {
     uint32_t bin = 0;
     for (uint32_t i = 0; i < count; ++i) {
@@ -79,7 +109,7 @@ constexpr int kTilePitch = kDocsPerBlock + 1;  // dwords per bucket row of the t
 // branch-free binary search; a wave writes the 256 bytes of one (block, bucket) pair at once.
 // Rows past the last document are read as the last document (their bins are never used).
 // grid = ceil(doc blocks / blocksPerGroup) * ceil(buckets / kBucketTile), block = 256 threads,
-// dynamic LDS = (kBucketTile << LOG2P) * 4 + kBucketTile * kTilePitch * 4 bytes.
+// dynamic LDS = (kBucketTile << LOG2P) * 4 + kBucketTile * kLutCells + kBucketTile * kTilePitch * 4 bytes.
 template <int LOG2P, bool CATS_MATRIX>
 __global__ __launch_bounds__(256) void BinarizeRowsKernel(const float* __restrict__ floats, uint32_t stride,
                                                           const int32_t* __restrict__ cats, uint32_t catStride,
@@ -90,7 +120,8 @@ __global__ __launch_bounds__(256) void BinarizeRowsKernel(const float* __restric
     constexpr int kPasses = kDocsPerBlock / kRowsPerPass;  // values per thread and block
     extern __shared__ uint32_t sBinarize[];
     uint32_t* sValues = sBinarize;                           // [kBucketTile][kSlots]
-    uint32_t* sTile = sBinarize + kBucketTile * kSlots;      // [kBucketTile][kTilePitch]
+    uint32_t* sLut = sBinarize + kBucketTile * kSlots;       // [kBucketTile][kLutCells / 4]
+    uint32_t* sTile = sLut + kBucketTile * (kLutCells / 4);  // [kBucketTile][kTilePitch]
 
     const uint32_t tid = threadIdx.x;
     const uint32_t tileCount = (tab.BucketCount + kBucketTile - 1) / kBucketTile;
@@ -118,6 +149,10 @@ __global__ __launch_bounds__(256) void BinarizeRowsKernel(const float* __restric
             }
         }
         sValues[i] = v;
+    }
+    for (uint32_t i = tid; i < kBucketTile * (kLutCells / 4); i += 256) {
+        const uint32_t bb = i / (kLutCells / 4);
+        sLut[i] = bb < nb ? tab.Lut[static_cast<size_t>(b0) * (kLutCells / 4) + i] : 0u;
     }
 
     // role of this thread while loading: bucket `myB` of rows myRow0, myRow0 + 8, ...; threads of
@@ -153,6 +188,20 @@ __global__ __launch_bounds__(256) void BinarizeRowsKernel(const float* __restric
 
     const uint32_t lane = tid & (kWave - 1);
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    // the buckets this wave binarizes in every block (wave, wave + 4, ...) and their grids
+    constexpr int kBucketsPerWave = kBucketTile / (256 / kWave);
+    uint32_t myFlags[kBucketsPerWave], myTopStep[kBucketsPerWave];
+    float myLo[kBucketsPerWave], myScale[kBucketsPerWave];
+#pragma unroll
+    for (int k = 0; k < kBucketsPerWave; ++k) {
+        const uint32_t bucket = b0 + min(wave + k * (256 / kWave), nb - 1);
+        const uint4 grid = tab.Grid[bucket];
+        myFlags[k] = __builtin_amdgcn_readfirstlane(tab.BucketFlags[bucket]);
+        myLo[k] = __uint_as_float(__builtin_amdgcn_readfirstlane(grid.x));
+        myScale[k] = __uint_as_float(__builtin_amdgcn_readfirstlane(grid.y));
+        const uint32_t steps = __builtin_amdgcn_readfirstlane(grid.z);
+        myTopStep[k] = steps ? 1u << (steps - 1) : 0u;
+    }
     if (blockBegin < blockEnd) {
         CBAMD_LOAD_BLOCK(blockBegin);
     }
@@ -166,28 +215,31 @@ __global__ __launch_bounds__(256) void BinarizeRowsKernel(const float* __restric
         if (block + 1 < blockEnd) {
             CBAMD_LOAD_BLOCK(block + 1);  // in flight while this block is binarized
         }
-        for (uint32_t bb = wave; bb < nb; bb += 256 / kWave) {
-            const uint32_t flags = tab.BucketFlags[b0 + bb];
+#pragma unroll
+        for (int k = 0; k < kBucketsPerWave; ++k) {
+            const uint32_t bb = wave + k * (256 / kWave);
+            if (bb >= nb) {
+                break;
+            }
             const uint32_t* values = sValues + bb * kSlots;
             const uint32_t* column = sTile + bb * kTilePitch + lane;
             uint32_t packed = 0;
-            if (flags & kBucketFlagOneHot) {
+            if (myFlags[k] & kBucketFlagOneHot) {
                 const uint32_t count = tab.BucketOffset[b0 + bb + 1] - tab.BucketOffset[b0 + bb];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     packed |= OneHotBin(values, count, column[j * kWave]) << (8 * j);
                 }
-            } else if (flags & kBucketFlagNanToInf) {
+            } else {
+                const uint8_t* lut = reinterpret_cast<const uint8_t*>(sLut + bb * (kLutCells / 4));
+                const bool nanToInf = (myFlags[k] & kBucketFlagNanToInf) != 0;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     float v = __uint_as_float(column[j * kWave]);
-                    v = isnan(v) ? __uint_as_float(0x7f800000u) : v;
-                    packed |= CountBelow<LOG2P>(values, v) << (8 * j);
-                }
-            } else {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    packed |= CountBelow<LOG2P>(values, __uint_as_float(column[j * kWave])) << (8 * j);
+                    if (nanToInf) {
+                        v = isnan(v) ? __uint_as_float(0x7f800000u) : v;
+                    }
+                    packed |= CountBelowInCell(values, lut, myLo[k], myScale[k], myTopStep[k], v) << (8 * j);
                 }
             }
             bins[(static_cast<size_t>(block) * tab.BucketCount + b0 + bb) * kWave + lane] = packed;
