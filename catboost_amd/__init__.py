@@ -198,12 +198,9 @@ def integer_cat_feature_hash(v):
 def _row_pointers(matrix, ctype):
     """Array of per-row pointers into a C-contiguous 2-D numpy array."""
     n = matrix.shape[0]
-    ptrs = (ctypes.POINTER(ctype) * max(n, 1))()
-    base = matrix.ctypes.data
-    stride = matrix.strides[0]
-    for i in range(n):
-        ptrs[i] = ctypes.cast(base + i * stride, ctypes.POINTER(ctype))
-    return ptrs
+    addresses = matrix.ctypes.data + np.arange(max(n, 1), dtype=np.uint64) * np.uint64(matrix.strides[0])
+    # the ctypes array shares (and keeps alive) the numpy buffer of addresses
+    return (ctypes.POINTER(ctype) * max(n, 1)).from_buffer(addresses)
 
 
 def model_arrays(float_features=(), cat_features=(), one_hot_features=(), approx_dimension=1, tree_sizes=(),

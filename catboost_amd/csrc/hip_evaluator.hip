@@ -8,6 +8,7 @@
 #include <cstring>
 #include <limits>
 #include <string>
+#include <thread>
 #include <vector>
 
 namespace cbamd {
@@ -369,6 +370,15 @@ struct THipEvaluator::TImpl {
     TPinnedVec<float> PinnedFloats;
     TPinnedVec<int32_t> PinnedCats;
     TPinnedVec<double> PinnedResults;
+    // second slot of the row staging pipeline (CalcHostRows) and the events of both slots:
+    // binarize start, binarize end, evaluate end, results on the host
+    TPinnedVec<float> PinnedFloats2;
+    TPinnedVec<int32_t> PinnedCats2;
+    TPinnedVec<double> PinnedResults2;
+    TDeviceVec<float> StageFloats2;
+    TDeviceVec<int32_t> StageCats2;
+    TDeviceVec<double> StageResults2;
+    hipEvent_t SlotEv[2][4] = {{nullptr, nullptr, nullptr, nullptr}, {nullptr, nullptr, nullptr, nullptr}};
     TPinnedVec<uint32_t> PinnedIndexes;
     TPinnedVec<uint8_t> PinnedExport;
 
@@ -412,6 +422,11 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId)
     HIP_CHECK(hipStreamCreateWithFlags(&m.Stream, hipStreamNonBlocking));
     for (auto& e : m.Ev) {
         HIP_CHECK(hipEventCreate(&e));
+    }
+    for (auto& slot : m.SlotEv) {
+        for (auto& e : slot) {
+            HIP_CHECK(hipEventCreate(&e));
+        }
     }
     TreeCount = trees.GetTreeCount();
     ApproxDimension = trees.ApproxDimension;
@@ -714,6 +729,13 @@ THipEvaluator::~THipEvaluator() {
         for (auto& e : Impl->Ev) {
             if (e) {
                 (void)hipEventDestroy(e);
+            }
+        }
+        for (auto& slot : Impl->SlotEv) {
+            for (auto& e : slot) {
+                if (e) {
+                    (void)hipEventDestroy(e);
+                }
             }
         }
         if (Impl->Stream) {
@@ -1127,6 +1149,50 @@ size_t ChunkDocs(size_t rowFloats, size_t rowCats) {
 
 }  // namespace
 
+namespace {
+
+// Copies `count` rows of `rowLen` elements each, given by pointer, into a dense matrix; large
+// batches are split over a few threads (the copy is what bounds the pointer-per-row entry points).
+template <typename T>
+void GatherRows(const T* const* rows, size_t count, size_t rowLen, T* dst) {
+    const size_t bytes = count * rowLen * sizeof(T);
+    size_t threads = std::min<size_t>(std::max(1u, std::thread::hardware_concurrency()), 16);
+    threads = std::min(threads, bytes / (size_t(4) << 20) + 1);
+    const auto copy = [=](size_t begin, size_t end) {
+        for (size_t d = begin; d < end; ++d) {
+            std::memcpy(dst + d * rowLen, rows[d], rowLen * sizeof(T));
+        }
+    };
+    if (threads <= 1) {
+        copy(0, count);
+        return;
+    }
+    std::vector<std::thread> pool;
+    const size_t per = (count + threads - 1) / threads;
+    for (size_t t = 1; t < threads; ++t) {
+        pool.emplace_back(copy, std::min(count, t * per), std::min(count, (t + 1) * per));
+    }
+    copy(0, std::min(count, per));
+    for (auto& th : pool) {
+        th.join();
+    }
+}
+
+// documents per slot of the row staging pipeline: small enough that gathering the next slot on
+// the host overlaps the transfer and the kernels of the current one
+size_t PipelineDocs(size_t rowFloats, size_t rowCats) {
+    const size_t bytesPerDoc = std::max<size_t>(1, (rowFloats + rowCats) * 4);
+    size_t docs = (size_t(64) << 20) / bytesPerDoc;
+    docs = std::max<size_t>(docs, 4096);
+    docs = std::min<size_t>(docs, size_t(1) << 20);
+    return docs / dev::kDocsPerBlock * dev::kDocsPerBlock;
+}
+
+}  // namespace
+
+// Rows by pointer (the reference API's float** / hashed int**): two slots of pinned and device
+// staging memory; while the GPU copies in, binarizes, evaluates and copies out slot k, the host
+// gathers the rows of slot k + 1.
 void THipEvaluator::CalcHostRows(const float* const* rows, size_t rowLen, bool flat, const int32_t* const* catRows,
                                  size_t catRowLen, size_t docCount, size_t treeStart, size_t treeEnd, double* results) {
     std::lock_guard<std::mutex> guard(Lock);
@@ -1142,54 +1208,80 @@ void THipEvaluator::CalcHostRows(const float* const* rows, size_t rowLen, bool f
     CBAMD_ENSURE(needCats == 0 || catRows != nullptr, "Model has categorical features but no categorical features provided");
     CBAMD_ENSURE(catRowLen >= needCats, "insufficient cat features vector size: " + std::to_string(catRowLen) +
                                             " expected: " + std::to_string(needCats));
-    const size_t chunk = ChunkDocs(needFloats, needCats);
+    const size_t chunk = PipelineDocs(needFloats, needCats);
     const size_t stageDocs = std::min(chunk, docCount);
-    m.PinnedFloats.Reserve(std::max<size_t>(1, stageDocs * needFloats));
-    m.StageFloats.Reserve(std::max<size_t>(1, stageDocs * needFloats));
-    if (needCats) {
-        m.PinnedCats.Reserve(stageDocs * needCats);
-        m.StageCats.Reserve(stageDocs * needCats);
+    const bool twoSlots = docCount > chunk;
+    TPinnedVec<float>* pinnedFloats[2] = {&m.PinnedFloats, &m.PinnedFloats2};
+    TPinnedVec<int32_t>* pinnedCats[2] = {&m.PinnedCats, &m.PinnedCats2};
+    TPinnedVec<double>* pinnedResults[2] = {&m.PinnedResults, &m.PinnedResults2};
+    TDeviceVec<float>* stageFloats[2] = {&m.StageFloats, &m.StageFloats2};
+    TDeviceVec<int32_t>* stageCats[2] = {&m.StageCats, &m.StageCats2};
+    TDeviceVec<double>* stageResults[2] = {&m.StageResults, &m.StageResults2};
+    for (int slot = 0; slot < (twoSlots ? 2 : 1); ++slot) {
+        pinnedFloats[slot]->Reserve(std::max<size_t>(1, stageDocs * needFloats));
+        stageFloats[slot]->Reserve(std::max<size_t>(1, stageDocs * needFloats));
+        if (needCats) {
+            pinnedCats[slot]->Reserve(stageDocs * needCats);
+            stageCats[slot]->Reserve(stageDocs * needCats);
+        }
+        pinnedResults[slot]->Reserve(std::max<size_t>(1, stageDocs * m.Dim));
+        stageResults[slot]->Reserve(std::max<size_t>(1, stageDocs * m.Dim));
     }
-    m.PinnedResults.Reserve(std::max<size_t>(1, stageDocs * m.Dim));
-    m.StageResults.Reserve(std::max<size_t>(1, stageDocs * m.Dim));
     m.ScratchBins.Reserve(QuantizedBytes(stageDocs));
     LastTimes = TKernelTimes();
-    for (size_t begin = 0; begin < docCount; begin += chunk) {
+    // takes the results of the chunk that went through `slot` and adds its kernel times
+    const auto collect = [&](int slot, size_t begin, size_t n) {
+        HIP_CHECK(hipEventSynchronize(m.SlotEv[slot][3]));
+        std::memcpy(results + begin * m.Dim, pinnedResults[slot]->Get(), n * m.Dim * sizeof(double));
+        float a = 0.f, b = 0.f;
+        HIP_CHECK(hipEventElapsedTime(&a, m.SlotEv[slot][0], m.SlotEv[slot][1]));
+        HIP_CHECK(hipEventElapsedTime(&b, m.SlotEv[slot][1], m.SlotEv[slot][2]));
+        LastTimes.BinarizeMs += a;
+        LastTimes.EvalMs += b;
+    };
+    size_t pendingBegin[2] = {0, 0}, pendingDocs[2] = {0, 0};
+    size_t index = 0;
+    for (size_t begin = 0; begin < docCount; begin += chunk, ++index) {
+        const int slot = static_cast<int>(index & 1);
         const size_t n = std::min(chunk, docCount - begin);
+        if (pendingDocs[slot]) {  // the slot's previous chunk must be out before its buffers are reused
+            collect(slot, pendingBegin[slot], pendingDocs[slot]);
+            pendingDocs[slot] = 0;
+        }
         if (needFloats) {
-            float* dst = m.PinnedFloats.Get();
-            for (size_t d = 0; d < n; ++d) {
-                std::memcpy(dst + d * needFloats, rows[begin + d], needFloats * sizeof(float));
-            }
-            HIP_CHECK(hipMemcpyAsync(m.StageFloats.Get(), dst, n * needFloats * sizeof(float), hipMemcpyHostToDevice, s));
+            GatherRows(rows + begin, n, needFloats, pinnedFloats[slot]->Get());
+            HIP_CHECK(hipMemcpyAsync(stageFloats[slot]->Get(), pinnedFloats[slot]->Get(), n * needFloats * sizeof(float),
+                                     hipMemcpyHostToDevice, s));
         }
         if (needCats) {
-            int32_t* dst = m.PinnedCats.Get();
-            for (size_t d = 0; d < n; ++d) {
-                std::memcpy(dst + d * needCats, catRows[begin + d], needCats * sizeof(int32_t));
-            }
-            HIP_CHECK(hipMemcpyAsync(m.StageCats.Get(), dst, n * needCats * sizeof(int32_t), hipMemcpyHostToDevice, s));
+            GatherRows(catRows + begin, n, needCats, pinnedCats[slot]->Get());
+            HIP_CHECK(hipMemcpyAsync(stageCats[slot]->Get(), pinnedCats[slot]->Get(), n * needCats * sizeof(int32_t),
+                                     hipMemcpyHostToDevice, s));
         }
         TFeatureBatch batch;
         batch.Layout = flat ? TFeatureBatch::FlatRows : TFeatureBatch::SplitRows;
-        batch.Floats = m.StageFloats.Get();
+        batch.Floats = stageFloats[slot]->Get();
         batch.Stride = needFloats;
-        batch.Cats = needCats ? m.StageCats.Get() : nullptr;
+        batch.Cats = needCats ? stageCats[slot]->Get() : nullptr;
         batch.CatStride = needCats;
-        HIP_CHECK(hipEventRecord(m.Ev[0], s));
+        HIP_CHECK(hipEventRecord(m.SlotEv[slot][0], s));
         QuantizeDevice(batch, n, m.ScratchBins.Get(), s);
-        HIP_CHECK(hipEventRecord(m.Ev[1], s));
-        EvalQuantizedDevice(m.ScratchBins.Get(), n, treeStart, treeEnd, m.StageResults.Get(), s);
-        HIP_CHECK(hipEventRecord(m.Ev[2], s));
-        HIP_CHECK(hipMemcpyAsync(m.PinnedResults.Get(), m.StageResults.Get(), n * m.Dim * sizeof(double),
+        HIP_CHECK(hipEventRecord(m.SlotEv[slot][1], s));
+        EvalQuantizedDevice(m.ScratchBins.Get(), n, treeStart, treeEnd, stageResults[slot]->Get(), s);
+        HIP_CHECK(hipEventRecord(m.SlotEv[slot][2], s));
+        HIP_CHECK(hipMemcpyAsync(pinnedResults[slot]->Get(), stageResults[slot]->Get(), n * m.Dim * sizeof(double),
                                  hipMemcpyDeviceToHost, s));
-        HIP_CHECK(hipStreamSynchronize(s));
-        std::memcpy(results + begin * m.Dim, m.PinnedResults.Get(), n * m.Dim * sizeof(double));
-        float a = 0.f, b = 0.f;
-        HIP_CHECK(hipEventElapsedTime(&a, m.Ev[0], m.Ev[1]));
-        HIP_CHECK(hipEventElapsedTime(&b, m.Ev[1], m.Ev[2]));
-        LastTimes.BinarizeMs += a;
-        LastTimes.EvalMs += b;
+        HIP_CHECK(hipEventRecord(m.SlotEv[slot][3], s));
+        pendingBegin[slot] = begin;
+        pendingDocs[slot] = n;
+    }
+    // the (up to) two chunks still in flight, older first
+    for (size_t k = 0; k < 2; ++k) {
+        const int slot = static_cast<int>((index + k) & 1);
+        if (pendingDocs[slot]) {
+            collect(slot, pendingBegin[slot], pendingDocs[slot]);
+            pendingDocs[slot] = 0;
+        }
     }
 }
 
