@@ -171,6 +171,14 @@ uint32_t GridCell(float v, float lo, float scale) {
     return std::min<uint32_t>(static_cast<uint32_t>(tt), dev::kLutCells - 1);
 }
 
+constexpr size_t kMaxTileLdsBytes = 160 * 1024;
+
+// LDS of the tile kernel without leaf regions: the bins of 256 documents and the accumulator
+size_t TileLdsBytes(uint32_t buckets, int dchunk) {
+    return ((static_cast<size_t>(buckets) * dev::kDocsPerBlock + 7) & ~size_t(7)) +
+           static_cast<size_t>(dev::kDocsPerBlock) * dchunk * sizeof(double);
+}
+
 // dimensions the tile kernel accumulates per pass over the trees (and the pitch of its padded leaf rows)
 int TileChunk(int dim) {
     return dim == 1 ? 1 : dim == 2 ? 2 : dim <= 4 ? 4 : dim <= 8 ? 8 : dim <= 12 ? 12 : 16;
@@ -329,6 +337,8 @@ struct THipEvaluator::TImpl {
     TDeviceVec<uint32_t> Splits, TreeStart, TreeSize, FirstLeaf, StepNodes, NodeToLeaf;
     TDeviceVec<double> Leaves, Bias;
     TDeviceVec<uint32_t> PackedTrees;  // tile kernel: 16 dwords per oblivious tree of depth <= 8
+    TDeviceVec<uint32_t> PackedMixed;  // half-tile kernel: packed rows in the form chosen per tree
+    TDeviceVec<double> HalfTileLeaves; // half-tile kernel: 64 or 256 leaf values per tree at a fixed pitch
     TDeviceVec<double> LeavesPadded;   // tile kernel, multi-dimensional: [tree][chunk][leaf][TileChunk(dim)]
     bool PackedSevenBit = false;
     bool LeavesPairAligned = false;  // every tree's first leaf value sits at an even index
@@ -639,6 +649,45 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId)
             m.LeavesPadded.Upload(padded);
         }
         m.PackedTrees.Upload(packed);
+        if (m.Dim == 1) {
+            // per-tree form: 7-bit when the tree has no one-hot split and every float bin fits 7 bits
+            uint32_t maxFloatValues = 0;
+            for (size_t b = 0; b + 1 < offsets.size(); ++b) {
+                if (!(flags[b] & dev::kBucketFlagOneHot)) {
+                    maxFloatValues = std::max(maxFloatValues, offsets[b + 1] - offsets[b]);
+                }
+            }
+            std::vector<uint32_t> mixed(packed.size(), 0);
+            for (size_t t = 0; t < trees.GetTreeCount(); ++t) {
+                bool sevenBit = maxFloatValues <= 127;
+                for (int d = 0; d < trees.TreeSizes[t]; ++d) {
+                    sevenBit = sevenBit && trees.RepackedBins[trees.TreeStartOffsets[t] + d].XorMask == 0;
+                }
+                uint32_t* row = mixed.data() + t * dev::kPackedTreeDwords;
+                for (int d = 0; d < 8; ++d) {
+                    if (d < trees.TreeSizes[t]) {
+                        const auto& rb = trees.RepackedBins[trees.TreeStartOffsets[t] + d];
+                        row[d] = sevenBit ? (static_cast<uint32_t>(rb.FeatureIndex) << 8) | (128u - rb.SplitIdx)
+                                          : (static_cast<uint32_t>(rb.FeatureIndex) << 16) |
+                                                (static_cast<uint32_t>(rb.XorMask) << 8) | rb.SplitIdx;
+                    } else {
+                        row[d] = sevenBit ? 0u : 0xffu;
+                    }
+                }
+                row[dev::kPackedFirstLeafSlot] = firstLeaf[t];
+                row[dev::kPackedFormSlot] = sevenBit ? 0u : 1u;
+            }
+            m.PackedMixed.Upload(mixed);
+            if (TileLdsBytes(m.LayoutBuckets, 1) > kMaxTileLdsBytes) {
+                const size_t pitch = m.MaxDepth <= 6 ? 64 : 256;
+                std::vector<double> fixed(trees.GetTreeCount() * pitch, 0.0);
+                for (size_t t = 0; t < trees.GetTreeCount(); ++t) {
+                    std::copy_n(trees.LeafValues.begin() + trees.TreeFirstLeafOffsets[t], size_t(1) << trees.TreeSizes[t],
+                                fixed.begin() + t * pitch);
+                }
+                m.HalfTileLeaves.Upload(fixed);
+            }
+        }
         m.LeavesPairAligned = true;
         for (uint32_t f : firstLeaf) {
             m.LeavesPairAligned = m.LeavesPairAligned && (f % 2 == 0);
@@ -864,11 +913,11 @@ void THipEvaluator::QuantizeDevice(const TFeatureBatch& batch, size_t docCount, 
 
 namespace {
 
-constexpr size_t kMaxTileLdsBytes = 160 * 1024;
 
-size_t TileLdsBytes(uint32_t buckets, int dchunk) {
-    return ((static_cast<size_t>(buckets) * dev::kDocsPerBlock + 7) & ~size_t(7)) +
-           static_cast<size_t>(dev::kDocsPerBlock) * dchunk * sizeof(double);
+// LDS of the half-tile kernel: 128 documents' bins, the accumulator, the per-wave leaf regions
+size_t HalfTileLdsBytes(uint32_t buckets, int maxd) {
+    return ((static_cast<size_t>(buckets) * 128 + 7) & ~size_t(7)) + 128 * sizeof(double) +
+           static_cast<size_t>(dev::kTileWaves) * (size_t(1) << maxd) * sizeof(double);
 }
 
 // LDS of the per-wave leaf regions of the tile kernel
@@ -1045,6 +1094,29 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
             LaunchEvalTileM<true>(m.MaxDepth, dchunk, args);
         } else {
             LaunchEvalTileM<false>(m.MaxDepth, dchunk, args);
+        }
+        HIP_CHECK(hipGetLastError());
+        return;
+    }
+    if (m.Oblivious && m.MaxDepth <= 8 && m.Dim == 1 && m.HalfTileLeaves.Get() != nullptr &&
+        HalfTileLdsBytes(m.LayoutBuckets, 8) <= kMaxTileLdsBytes) {
+        // the bins of a block exceed the 256-document tile: half blocks
+        const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
+        const int maxd = m.MaxDepth <= 6 ? 6 : 8;
+        const size_t lds = HalfTileLdsBytes(m.LayoutBuckets, maxd);
+        const auto launch = [&](auto kernel) {
+            if (lds > 64 * 1024) {
+                HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+            }
+            hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(2 * blocks)), dim3(64 * dev::kTileWaves), lds, s,
+                               reinterpret_cast<const uint16_t*>(bins), docCount, m.LayoutBuckets, m.PackedMixed.Get(),
+                               m.HalfTileLeaves.Get(), m.Bias.Get(), m.Scale, tb, te, results);
+        };
+        if (maxd == 6) {
+            launch(dev::EvalObliviousHalfTileKernel<6>);
+        } else {
+            launch(dev::EvalObliviousHalfTileKernel<8>);
         }
         HIP_CHECK(hipGetLastError());
         return;

@@ -611,6 +611,141 @@ __global__ __launch_bounds__(64 * kTileWaves) __attribute__((amdgpu_waves_per_eu
     }
 }
 
+// One-dimensional oblivious models whose bins do not fit the 256-document tile (more than ~600
+// buckets): the same scheme on half a block. A workgroup copies the bins of 128 documents
+// (buckets x 128 bytes, two documents per lane: documents (2 * half + j) * 64 + lane of the block)
+// and its waves split the trees; everything else is EvalObliviousTileKernel with DCHUNK == 1 and
+// leaf values through LDS. `leaves` holds (1 << MAXD) values per tree at a fixed pitch.
+// The packed rows come in the form chosen per tree (slot kPackedFormSlot): the 7-bit form when
+// the tree has no one-hot split and all float bins of the model fit 7 bits, else the 8-bit form;
+// a model with a few one-hot splits pays the longer compare only in the trees that have them.
+// grid = 2 * doc blocks, block = 64 * kTileWaves threads, dynamic LDS = buckets * 128 (rounded up
+// to 8) + 128 * 8 + kTileWaves * (1 << MAXD) * 8 bytes.
+constexpr int kPackedFormSlot = 11;  // mixed table: 0 = 7-bit form, 1 = 8-bit form
+
+template <bool SEVEN_BIT, int MAXD>
+__device__ __forceinline__ uint32_t TreeIndexesPair(const uint8_t* laneTile, uint32_t packedRow) {
+    uint32_t idx2 = 0;
+#pragma unroll
+    for (int d = 0; d < MAXD; ++d) {
+        const uint32_t level = __builtin_amdgcn_readlane(packedRow, d);
+        const uint32_t a = *reinterpret_cast<const uint16_t*>(laneTile + (LevelTileOffset<SEVEN_BIT>(level) >> 1));
+        const uint32_t r = CompareBytes<SEVEN_BIT>(a, level);
+        idx2 = (r & 0x8080u) | ((idx2 >> 1) & 0x7f7fu);
+    }
+    return idx2 >> (8 - MAXD);
+}
+
+template <int MAXD>
+__global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousHalfTileKernel(
+    const uint16_t* __restrict__ bins, size_t docCount, uint32_t bucketCount, const uint32_t* __restrict__ packedMixed,
+    const double* __restrict__ leaves, const double* __restrict__ bias, double scale, uint32_t treeBegin,
+    uint32_t treeEnd, double* __restrict__ out) {
+    constexpr uint32_t kTreePairs = (1u << MAXD) / 2;
+    constexpr int kPrefetchRegs = static_cast<int>((kTreePairs + kWave - 1) / kWave);
+    extern __shared__ uint32_t sTile[];
+    uint16_t* sTile16 = reinterpret_cast<uint16_t*>(sTile);
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const size_t block = blockIdx.x >> 1;
+    const uint32_t half = blockIdx.x & 1;
+    const uint32_t tileWords = bucketCount * kWave;
+    const uint16_t* src = bins + block * tileWords * 2 + half;
+    for (uint32_t i = tid; i < tileWords; i += 64 * kTileWaves) {
+        sTile16[i] = src[2 * i];
+    }
+    const bool addBias = treeBegin == 0;
+    const uint8_t* laneTile = reinterpret_cast<const uint8_t*>(sTile) + lane * 2;
+    const uint32_t slot = lane & (kPackedTreeDwords - 1);
+    double* sRed = reinterpret_cast<double*>(sTile + ((tileWords / 2 + 1) & ~1u));
+    double* sLeaf = sRed + 2 * kWave + wave * (1u << MAXD);  // per-wave leaf region
+    __syncthreads();  // tile is loaded
+    double acc[2] = {0.0, 0.0};
+    // A wave has only one partner on its SIMD here (the tile leaves room for one workgroup per CU),
+    // so what it needs from global memory is requested kAhead of its trees ahead: the packed row
+    // and the leaf values ((1 << MAXD) doubles per tree at a fixed pitch) of tree t + kAhead * 8
+    // go into the registers that tree t has just given up.
+    constexpr int kAhead = 4;
+    uint32_t rows[kAhead];
+    double2 pref[kAhead][kPrefetchRegs];
+#define CBAMD_FETCH_TREE(k, tree)                                                                 \
+    do {                                                                                          \
+        const uint32_t fetchTree = (tree);                                                        \
+        rows[k] = 0u;                                                                             \
+        if (fetchTree < treeEnd) {                                                                \
+            rows[k] = packedMixed[static_cast<size_t>(fetchTree) * kPackedTreeDwords + slot];     \
+            const double2* src2 = reinterpret_cast<const double2*>(leaves) + static_cast<size_t>(fetchTree) * kTreePairs; \
+            _Pragma("unroll") for (int i = 0; i < kPrefetchRegs; ++i) {                           \
+                if (static_cast<uint32_t>(i + 1) * kWave <= kTreePairs || i * kWave + lane < kTreePairs) { \
+                    pref[k][i] = src2[i * kWave + lane];                                          \
+                }                                                                                 \
+            }                                                                                     \
+        }                                                                                         \
+    } while (0)
+    uint32_t t = treeBegin + wave;
+#pragma unroll
+    for (int k = 0; k < kAhead; ++k) {
+#pragma unroll
+        for (int i = 0; i < kPrefetchRegs; ++i) {
+            pref[k][i] = {0.0, 0.0};
+        }
+        CBAMD_FETCH_TREE(k, t + k * kTileWaves);
+    }
+    while (t < treeEnd) {
+#pragma unroll
+        for (int k = 0; k < kAhead; ++k) {
+            if (t < treeEnd) {
+                // publish this tree's leaf values in the wave's region; the previous tree's gathers
+                // were issued before these stores and LDS serves one wave's requests in order
+                double2* dst2 = reinterpret_cast<double2*>(sLeaf);
+#pragma unroll
+                for (int i = 0; i < kPrefetchRegs; ++i) {
+                    if (static_cast<uint32_t>(i + 1) * kWave <= kTreePairs || i * kWave + lane < kTreePairs) {
+                        dst2[i * kWave + lane] = pref[k][i];
+                    }
+                }
+                const uint32_t row = rows[k];
+                CBAMD_FETCH_TREE(k, t + kAhead * kTileWaves);
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                uint32_t idx2;
+                if (__builtin_amdgcn_readlane(row, kPackedFormSlot) != 0) {
+                    idx2 = TreeIndexesPair<false, MAXD>(laneTile, row);
+                } else {
+                    idx2 = TreeIndexesPair<true, MAXD>(laneTile, row);
+                }
+                acc[0] = __dadd_rn(acc[0], sLeaf[idx2 & 0xffu]);
+                acc[1] = __dadd_rn(acc[1], sLeaf[(idx2 >> 8) & 0xffu]);
+                __builtin_amdgcn_wave_barrier();
+                t += kTileWaves;
+            }
+        }
+    }
+#undef CBAMD_FETCH_TREE
+    // waves add their partial sums in wave order into the LDS accumulator; the last wave
+    // finishes the values and writes them out
+    for (uint32_t w = 0; w + 1 < kTileWaves; ++w) {
+        if (wave == w) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                double* cell = sRed + j * kWave + lane;
+                *cell = (w == 0) ? acc[j] : __dadd_rn(*cell, acc[j]);
+            }
+        }
+        __syncthreads();
+    }
+    if (wave == kTileWaves - 1) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const size_t doc = block * kDocsPerBlock + (2 * half + j) * kWave + lane;
+            if (doc < docCount) {
+                out[doc] = Finish(__dadd_rn(sRed[j * kWave + lane], acc[j]), scale, bias[0], addBias);
+            }
+        }
+    }
+}
+
 __device__ __forceinline__ uint32_t BinOfDoc(const uint8_t* bins, size_t doc, uint32_t bucketCount, uint32_t bucket) {
     const size_t block = doc / kDocsPerBlock;
     const uint32_t r = static_cast<uint32_t>(doc % kDocsPerBlock);
