@@ -377,3 +377,58 @@ def test_error_paths(golden_dir):
             cb.ModelCalcer(os.path.join(golden_dir, name))
     # the handle still works after failed calls
     _close(g.calc_flat(rm.NUMERIC_ONLY_ROWS), rm.NUMERIC_ONLY_EXPECTED)
+
+
+# --------------------------------------------------- full workload size, properties ----
+
+def test_c2_full_size_properties():
+    """C2 at its full 4M documents on the device path. The oracle checks a sample; the rest is
+    covered by properties that hold at any size: a prediction does not depend on where its
+    document sits in the batch (bit for bit on the register-resident kernels), quantize +
+    evaluate equals the one-call path, and tree sub-ranges add up to the whole model."""
+    import torch
+
+    docs = 4_000_000
+    model, info = syn.build_model("C2")
+    ev = model.evaluator()
+    x = syn.device_features(info, docs)
+    out = torch.zeros(docs, dtype=torch.float64, device="cuda:0")
+    torch.cuda.synchronize()
+    feats = ev.features(cb.LAYOUT_FLAT_ROWS, x.data_ptr(), x.shape[1])
+    ev.eval_data(feats, docs, out.data_ptr())
+    ev.synchronize()
+    # sample against the oracle
+    rng = np.random.default_rng(3)
+    sample = np.sort(rng.choice(docs, 4000, replace=False))
+    sample_t = torch.from_numpy(sample).to("cuda:0")
+    o = OracleModel(read_cbm(model.save_to_buffer()))
+    np.testing.assert_array_equal(out[sample_t].cpu().numpy(), o.calc(x[sample_t].cpu().numpy()))
+    # position independence: the batch reversed block-wise with a ragged tail
+    keep = docs - 12345
+    perm = torch.arange(keep - 1, -1, -1, device="cuda:0")
+    xp = x[perm].contiguous()
+    outp = torch.zeros(keep, dtype=torch.float64, device="cuda:0")
+    torch.cuda.synchronize()
+    ev.eval_data(ev.features(cb.LAYOUT_FLAT_ROWS, xp.data_ptr(), xp.shape[1]), keep, outp.data_ptr())
+    ev.synchronize()
+    assert torch.equal(outp, out[perm])
+    del xp, outp, perm
+    # quantize into a caller-owned buffer, evaluate from it
+    bins = torch.zeros(ev.quantized_bytes(docs), dtype=torch.uint8, device="cuda:0")
+    out2 = torch.zeros_like(out)
+    torch.cuda.synchronize()
+    ev.quantize(feats, docs, bins.data_ptr())
+    ev.eval_quantized(bins.data_ptr(), docs, out2.data_ptr())
+    ev.synchronize()
+    assert torch.equal(out, out2)
+    # tree sub-ranges (tile kernel) add up to the whole model (scale 1, bias 0 in this workload)
+    trees = model.tree_count
+    parts = torch.zeros_like(out)
+    part = torch.zeros_like(out)
+    torch.cuda.synchronize()
+    for begin, end in ((0, 300), (300, 301), (301, trees)):
+        ev.eval_quantized(bins.data_ptr(), docs, part.data_ptr(), tree_start=begin, tree_end=end)
+        ev.synchronize()
+        parts += part
+    torch.cuda.synchronize()
+    assert torch.allclose(parts, out, rtol=RTOL, atol=ATOL)
