@@ -1,8 +1,10 @@
 """Writes the gfx950 assembly of the register-resident evaluate kernels.
 
-The kernels evaluate oblivious trees of depth <= 8 of a model whose bins and split indexes all fit
-7 bits (no xor masks), the case of float-feature models with at most 127 used borders per feature.
-One launch produces PITCH consecutive dimensions of the result (1 for a one-dimensional model).
+The kernels evaluate oblivious trees of depth <= 8. The plain variants take models whose bins and
+split indexes all fit 7 bits (no xor masks), the case of float-feature models with at most 127
+used borders per feature; the "_m" (mixed) variants take any bins and xor masks (one-hot splits)
+and choose the compare per tree. One launch produces PITCH consecutive dimensions of the result
+(1 for a one-dimensional model).
 
 Layout of the work:
   * a wave owns one block of 256 documents and keeps the block's bins in vector registers for the
@@ -16,7 +18,12 @@ Layout of the work:
     spread over the current block's trees and goes from global memory straight into LDS
     (global_load_lds);
   * a tree's levels come from a table of 16 dwords per tree, (bucket, (128 - splitIdx) * 0x01010101)
-    per level, read with one scalar load two trees ahead; kernels for LEAVES = 64 use the first six;
+    per level, read with one scalar load two trees ahead; kernels for LEAVES = 64 use the first six.
+    Mixed variants: 32 dwords per tree. Bit 31 of the first dword clear: the 7-bit form above (the
+    tree has no xor mask and all bins of its buckets fit 7 bits). Set: 4 dwords per level, bucket,
+    xorMask, splitIdx & 0x7f (both times 0x01010101) and 0x80808080 if splitIdx < 128 else 0; the
+    unsigned byte compare (bin ^ xorMask) >= splitIdx is then bit 7 of
+    majority(x, (x | 0x80) - (splitIdx & 0x7f), splitIdx < 128) taken per byte, x = bin ^ xorMask;
   * the leaf gathers of a tree (four documents per lane) are issued behind its levels and consumed
     after the levels of the next tree, so their LDS latency is covered; every sum is accumulated in
     fp64 in tree order, exactly like the CPU evaluator (cpu/evaluator_impl.cpp:362-460), and
@@ -24,7 +31,7 @@ Layout of the work:
 
 Kernel arguments (80 bytes):
    0 bins        const uint32*   [docBlock][bucketCount][64]
-   8 rows        const uint32*   [(treeBlocks + 2) * TREE_BLOCK][16]    (null trees behind the model's)
+   8 rows        const uint32*   [(treeBlocks + 2) * TREE_BLOCK][16 or 32]  (null trees behind the model's)
   16 leaves      const double*   [(treeBlocks + 2) * TREE_BLOCK][LEAVES][PITCH]
   24 out         double*         [docCount][dim]
   32 docCount    uint32          36 blockCount uint32 (ceil(docCount / 256), >= 1)
@@ -39,19 +46,20 @@ Usage: gen_eval_reg_kernel.py OUT.s
 """
 import sys
 
-ROW_BYTES = 64
 LDS_BUFFER_LIMIT = 32 * 1024
 
-# (bins registers, waves per workgroup, PITCH, LEAVES); hip_evaluator.hip lists the same variants
-VARIANTS = [
+# (bins registers, waves per workgroup, PITCH, LEAVES), each in a plain and a mixed form;
+# hip_evaluator.hip lists the same variants
+SHAPES = [
     (208, 4, 1, 256), (96, 8, 1, 256),
     (192, 4, 2, 64), (160, 4, 4, 64), (128, 4, 6, 64),
     (192, 4, 2, 256), (160, 4, 4, 256), (128, 4, 6, 256),
 ]
+VARIANTS = [shape + (mixed,) for mixed in (False, True) for shape in SHAPES]
 
 
-def kernel_name(buckets, waves, pitch, leaves):
-    return "cbamd_eval_reg_b%d_w%d_p%d_l%d" % (buckets, waves, pitch, leaves)
+def kernel_name(buckets, waves, pitch, leaves, mixed):
+    return "cbamd_eval_reg_b%d_w%d_p%d_l%d%s" % (buckets, waves, pitch, leaves, "_m" if mixed else "")
 
 
 def tree_block(pitch, leaves):
@@ -62,12 +70,15 @@ def tree_block(pitch, leaves):
     return block
 
 
-def gen_kernel(buckets, waves, pitch, leaves):
-    name = kernel_name(buckets, waves, pitch, leaves)
+def gen_kernel(buckets, waves, pitch, leaves, mixed):
+    name = kernel_name(buckets, waves, pitch, leaves, mixed)
+    row_dwords = 32 if mixed else 16      # level table of a tree
+    tree_row_bytes = row_dwords * 4
+    rows_a, rows_b = 32, 32 + row_dwords  # the two sets of scalar registers holding level tables
     assert pitch == 1 or pitch % 2 == 0
     depth = {64: 6, 256: 8}[leaves]
     threads = waves * 64
-    row_bytes = threads * 16              # one 16-byte piece per thread
+    row_bytes = threads * 16              # one 16-byte piece per thread of a leaf table copy
     tree_bytes = leaves * pitch * 8
     block = tree_block(pitch, leaves)
     buf_bytes = block * tree_bytes
@@ -97,7 +108,7 @@ def gen_kernel(buckets, waves, pitch, leaves):
         """One piece of the leaf table, global memory -> LDS without passing through registers:
         lane l of wave w writes 16 bytes at lds_offset + w * 1024 + l * 16 (M0 holds the wave's
         base). M0 doubles as the VGPR index register, so its index-mode value is put back after."""
-        e("  s_add_u32 m0, s68, %d" % lds_offset)
+        e("  s_add_u32 m0, s100, %d" % lds_offset)
         e("  s_nop 0")
         e("  global_load_lds_dwordx4 v2, s[26:27]")
         e("  s_add_u32 s26, s26, %d" % row_bytes)
@@ -109,6 +120,36 @@ def gen_kernel(buckets, waves, pitch, leaves):
                 e("  v_add_f64 v[%d:%d], v[%d:%d], v[%d:%d]" % (ac(j, k), ac(j, k) + 1, ac(j, k), ac(j, k) + 1,
                                                                  lv(j, k), lv(j, k) + 1))
 
+    def load_rows(regs, tree):
+        """Level table of tree `tree` (counted from the table position in s[6:7]) -> registers."""
+        for part in range(row_dwords // 16):
+            e("  s_load_dwordx16 s[%d:%d], s[6:7], 0x%x" % (regs + 16 * part, regs + 16 * part + 15,
+                                                            tree * tree_row_bytes + 64 * part))
+
+    def levels_seven_bit(rows):
+        for d in range(depth):
+            e("  s_set_gpr_idx_idx s%d" % (rows + 2 * d))
+            e("  v_add_u32_e64 v4, v%d, s%d" % (b0, rows + 2 * d + 1))
+            if d == 0:
+                e("  v_and_b32_e32 v3, s22, v4")
+            else:
+                e("  v_lshrrev_b32_e32 v3, 1, v3")
+                e("  v_bfi_b32 v3, s22, v4, v3")
+
+    def levels_eight_bit(rows):
+        for d in range(depth):
+            level = rows + 4 * d
+            e("  s_set_gpr_idx_idx s%d" % level)                      # index = bits 0..7 of the bucket dword
+            e("  v_xor_b32_e64 v4, v%d, s%d" % (b0, level + 1))       # x = bin ^ xorMask
+            e("  v_or_b32_e32 v5, s22, v4")
+            e("  v_subrev_u32_e32 v5, s%d, v5" % (level + 2))         # (x | 0x80) - (splitIdx & 0x7f), per byte
+            e("  v_bitop3_b32 v4, s%d, v4, v5 bitop3:0xe8" % (level + 3))  # majority
+            if d == 0:
+                e("  v_and_b32_e32 v3, s22, v4")
+            else:
+                e("  v_lshrrev_b32_e32 v3, 1, v3")
+                e("  v_bfi_b32 v3, s22, v4, v3")
+
     e(".text")
     e(".globl %s" % name)
     e(".p2align 8")
@@ -117,7 +158,7 @@ def gen_kernel(buckets, waves, pitch, leaves):
     # s[0:1] kernarg segment, s2 workgroup id, v0 thread id
     e("  s_load_dwordx8 s[4:11], s[0:1], 0x0")
     e("  s_load_dwordx8 s[12:19], s[0:1], 0x20")
-    e("  s_load_dwordx4 s[72:75], s[0:1], 0x40")
+    e("  s_load_dwordx4 s[96:99], s[0:1], 0x40")
     e("  v_and_b32_e32 v0, 0x3ff, v0")           # work-item ids come packed; keep x
     e("  v_lshrrev_b32_e32 v5, 6, v0")
     e("  v_and_b32_e32 v1, 63, v0")
@@ -131,7 +172,7 @@ def gen_kernel(buckets, waves, pitch, leaves):
     # byte j of the leaf indexes times s23 = offset of the document's leaf row in a tree's table
     # (a six-level index sits in bits 2..7 of its byte)
     e("  s_mov_b32 s23, %d" % (pitch * 8 >> (8 - depth)))
-    e("  s_lshl_b32 s68, s20, 10")               # LDS offset of the wave's part of a copied piece
+    e("  s_lshl_b32 s100, s20, 10")              # LDS offset of the wave's part of a copied piece
     e("  s_waitcnt lgkmcnt(0)")
     # first tree block -> buffer 0
     e("  s_mov_b32 s26, s8")
@@ -143,21 +184,22 @@ def gen_kernel(buckets, waves, pitch, leaves):
     e("  s_add_u32 s21, s21, s20")
     e("  s_add_u32 s24, s13, -1")
     e("  s_min_u32 s24, s21, s24")
-    e("  s_lshl_b32 s25, s72, 8")                # bytes of bins per document block
+    # (the level table registers are free until the first tables are loaded)
+    e("  s_lshl_b32 s25, s96, 8")                # bytes of bins per document block
     e("  s_mul_hi_u32 s31, s24, s25")
     e("  s_mul_i32 s30, s24, s25")
-    e("  s_add_u32 s64, s4, s30")
-    e("  s_addc_u32 s65, s5, s31")
-    e("  s_add_u32 s28, s72, -1")
+    e("  s_add_u32 s32, s4, s30")
+    e("  s_addc_u32 s33, s5, s31")
+    e("  s_add_u32 s28, s96, -1")
     for i in range(buckets):
         # registers past the model's bucket count reload the last bucket and are never indexed
         e("  s_min_u32 s24, %d, s28" % i)
         e("  s_lshl_b32 s24, s24, 8")
-        e("  s_add_u32 s66, s64, s24")
-        e("  s_addc_u32 s67, s65, 0")
-        e("  global_load_dword v%d, v1, s[66:67]" % (b0 + i))
-    e("  s_load_dwordx16 s[32:47], s[6:7], 0x0")
-    e("  s_load_dwordx16 s[48:63], s[6:7], 0x%x" % ROW_BYTES)
+        e("  s_add_u32 s34, s32, s24")
+        e("  s_addc_u32 s35, s33, 0")
+        e("  global_load_dword v%d, v1, s[34:35]" % (b0 + i))
+    load_rows(rows_a, 0)
+    load_rows(rows_b, 1)
     for r in range(lv0, ga0):
         e("  v_mov_b32_e32 v%d, 0" % r)          # leaf values in flight and the sums
     e("  s_waitcnt vmcnt(0) lgkmcnt(0)")
@@ -166,15 +208,18 @@ def gen_kernel(buckets, waves, pitch, leaves):
     e("%s_loop:" % name)
     for buf in range(2):
         for i in range(block):
-            rows = 32 if i % 2 == 0 else 48
-            for d in range(depth):
-                e("  s_set_gpr_idx_idx s%d" % (rows + 2 * d))
-                e("  v_add_u32_e64 v4, v%d, s%d" % (b0, rows + 2 * d + 1))
-                if d == 0:
-                    e("  v_and_b32_e32 v3, s22, v4")
-                else:
-                    e("  v_lshrrev_b32_e32 v3, 1, v3")
-                    e("  v_bfi_b32 v3, s22, v4, v3")
+            rows = rows_a if i % 2 == 0 else rows_b
+            if mixed:
+                label = "%s_t%d_%d" % (name, buf, i)
+                e("  s_bitcmp1_b32 s%d, 31" % rows)
+                e("  s_cbranch_scc1 %s_x" % label)
+                levels_seven_bit(rows)
+                e("  s_branch %s_j" % label)
+                e("%s_x:" % label)
+                levels_eight_bit(rows)
+                e("%s_j:" % label)
+            else:
+                levels_seven_bit(rows)
             e("  s_set_gpr_idx_idx 0")
             # previous tree's leaf values have arrived (and so has the next tree's row)
             e("  s_waitcnt lgkmcnt(0)")
@@ -189,7 +234,7 @@ def gen_kernel(buckets, waves, pitch, leaves):
                     for k in range(0, pitch, 2):
                         e("  ds_read_b128 v[%d:%d], v%d offset:%d" % (lv(j, k), lv(j, k) + 3, ga0 + j,
                                                                      tree_offset + 8 * k))
-            e("  s_load_dwordx16 s[%d:%d], s[6:7], 0x%x" % (rows, rows + 15, (buf * block + i + 2) * ROW_BYTES))
+            load_rows(rows, buf * block + i + 2)
             # copy of the next tree block into the other buffer, spread over this block's trees
             staged = False
             for c in range(i * per_tree, min(chunks, (i + 1) * per_tree)):
@@ -200,15 +245,15 @@ def gen_kernel(buckets, waves, pitch, leaves):
             if i == 0:
                 # the rows of the next tree block are pulled into the scalar cache now, so that the
                 # per-tree row loads of that block do not each wait for a miss
-                for k in range(block):
-                    e("  s_load_dword s3, s[6:7], 0x%x" % ((buf * block + block + 2 + k) * ROW_BYTES))
+                for k in range(block * tree_row_bytes // 64):
+                    e("  s_load_dword s3, s[6:7], 0x%x" % ((buf * block + block + 2) * tree_row_bytes + 64 * k))
         # every wave is done reading this buffer and writing the other one
         e("  s_waitcnt vmcnt(0) lgkmcnt(0)")
         e("  s_barrier")
         e("  s_add_u32 s14, s14, -1")
         e("  s_cmp_eq_u32 s14, 0")
         e("  s_cbranch_scc1 %s_done" % name)
-    e("  s_add_u32 s6, s6, %d" % (2 * block * ROW_BYTES))
+    e("  s_add_u32 s6, s6, %d" % (2 * block * tree_row_bytes))
     e("  s_addc_u32 s7, s7, 0")
     e("  s_branch %s_loop" % name)
     e("%s_done:" % name)
@@ -235,11 +280,11 @@ def gen_kernel(buckets, waves, pitch, leaves):
         e("  v_add_u32_e32 v%d, %d, v5" % (te0, 64 * j))
         e("  v_cmp_gt_u32_e32 vcc, s12, v%d" % te0)
         e("  s_and_saveexec_b64 s[30:31], vcc")
-        e("  v_mul_lo_u32 v%d, v%d, s73" % (te0 + 1, te0))               # document * dim
-        e("  v_add_lshl_u32 v%d, v%d, s74, 3" % (te0 + 1, te0 + 1))     # + first dimension, in bytes
+        e("  v_mul_lo_u32 v%d, v%d, s97" % (te0 + 1, te0))               # document * dim
+        e("  v_add_lshl_u32 v%d, v%d, s98, 3" % (te0 + 1, te0 + 1))     # + first dimension, in bytes
         for k in range(pitch):
             if k > 0:
-                e("  s_cmp_gt_u32 s75, %d" % k)
+                e("  s_cmp_gt_u32 s99, %d" % k)
                 e("  s_cbranch_scc0 %s_stored_%d" % (name, j))
             e("  global_store_dwordx2 v%d, v[%d:%d], s[10:11] offset:%d" % (te0 + 1, ac(j, k), ac(j, k) + 1, 8 * k))
         e("%s_stored_%d:" % (name, j))
@@ -261,7 +306,7 @@ def gen_kernel(buckets, waves, pitch, leaves):
     e("  .amdhsa_system_sgpr_workgroup_id_z 0")
     e("  .amdhsa_system_vgpr_workitem_id 0")
     e("  .amdhsa_next_free_vgpr %d" % vgprs)
-    e("  .amdhsa_next_free_sgpr 76")
+    e("  .amdhsa_next_free_sgpr 101")
     e("  .amdhsa_accum_offset %d" % ((vgprs + 3) // 4 * 4))
     e("  .amdhsa_reserve_vcc 1")
     e("  .amdhsa_float_round_mode_32 0")
@@ -294,7 +339,7 @@ def gen_kernel(buckets, waves, pitch, leaves):
     .max_flat_workgroup_size: %d
     .name: %s
     .private_segment_fixed_size: 0
-    .sgpr_count: 84
+    .sgpr_count: 108
     .sgpr_spill_count: 0
     .symbol: %s.kd
     .uniform_work_group_size: 1
@@ -309,8 +354,8 @@ def gen_kernel(buckets, waves, pitch, leaves):
 def generate():
     parts = ['.amdgcn_target "amdgcn-amd-amdhsa--gfx950"', ".amdhsa_code_object_version 6", ""]
     metas = []
-    for buckets, waves, pitch, leaves in VARIANTS:
-        text, meta = gen_kernel(buckets, waves, pitch, leaves)
+    for buckets, waves, pitch, leaves, mixed in VARIANTS:
+        text, meta = gen_kernel(buckets, waves, pitch, leaves, mixed)
         parts.append(text)
         metas.append(meta)
     parts.append(".amdgpu_metadata")

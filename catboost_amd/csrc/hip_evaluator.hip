@@ -109,19 +109,31 @@ struct TEvalRegArgs {
 };
 static_assert(sizeof(TEvalRegArgs) == 80, "kernel argument block of the register-resident kernels");
 
-constexpr uint32_t kRegRowDwords = 16;
 struct TEvalRegVariant {
     uint32_t Buckets;
     uint32_t Waves;
     uint32_t Pitch;   // dimensions per launch = doubles per leaf row
     uint32_t Leaves;  // leaf rows per tree (64: trees of depth <= 6)
+    bool Mixed;       // 32-dword level tables, compare form chosen per tree
     const char* Name;
 };
 constexpr TEvalRegVariant kEvalRegVariants[] = {
-    {96, 8, 1, 256, "cbamd_eval_reg_b96_w8_p1_l256"},   {208, 4, 1, 256, "cbamd_eval_reg_b208_w4_p1_l256"},
-    {192, 4, 2, 64, "cbamd_eval_reg_b192_w4_p2_l64"},   {160, 4, 4, 64, "cbamd_eval_reg_b160_w4_p4_l64"},
-    {128, 4, 6, 64, "cbamd_eval_reg_b128_w4_p6_l64"},   {192, 4, 2, 256, "cbamd_eval_reg_b192_w4_p2_l256"},
-    {160, 4, 4, 256, "cbamd_eval_reg_b160_w4_p4_l256"}, {128, 4, 6, 256, "cbamd_eval_reg_b128_w4_p6_l256"},
+    {96, 8, 1, 256, false, "cbamd_eval_reg_b96_w8_p1_l256"},
+    {208, 4, 1, 256, false, "cbamd_eval_reg_b208_w4_p1_l256"},
+    {192, 4, 2, 64, false, "cbamd_eval_reg_b192_w4_p2_l64"},
+    {160, 4, 4, 64, false, "cbamd_eval_reg_b160_w4_p4_l64"},
+    {128, 4, 6, 64, false, "cbamd_eval_reg_b128_w4_p6_l64"},
+    {192, 4, 2, 256, false, "cbamd_eval_reg_b192_w4_p2_l256"},
+    {160, 4, 4, 256, false, "cbamd_eval_reg_b160_w4_p4_l256"},
+    {128, 4, 6, 256, false, "cbamd_eval_reg_b128_w4_p6_l256"},
+    {96, 8, 1, 256, true, "cbamd_eval_reg_b96_w8_p1_l256_m"},
+    {208, 4, 1, 256, true, "cbamd_eval_reg_b208_w4_p1_l256_m"},
+    {192, 4, 2, 64, true, "cbamd_eval_reg_b192_w4_p2_l64_m"},
+    {160, 4, 4, 64, true, "cbamd_eval_reg_b160_w4_p4_l64_m"},
+    {128, 4, 6, 64, true, "cbamd_eval_reg_b128_w4_p6_l64_m"},
+    {192, 4, 2, 256, true, "cbamd_eval_reg_b192_w4_p2_l256_m"},
+    {160, 4, 4, 256, true, "cbamd_eval_reg_b160_w4_p4_l256_m"},
+    {128, 4, 6, 256, true, "cbamd_eval_reg_b128_w4_p6_l256_m"},
 };
 
 // trees per LDS buffer of a variant: a power of two, at most 16, buffer at most 32 KB
@@ -135,11 +147,13 @@ uint32_t RegTreeBlock(const TEvalRegVariant& v) {
 
 // The variant for a model: one-dimensional models take the smallest register file that holds
 // their buckets; others the pitch that needs the fewest launches (then the smallest such pitch).
-const TEvalRegVariant* PickRegVariant(uint32_t buckets, uint32_t dim, uint32_t maxDepth) {
+// mixed: the model has one-hot splits or bins above 127.
+const TEvalRegVariant* PickRegVariant(uint32_t buckets, uint32_t dim, uint32_t maxDepth, bool mixed) {
     const TEvalRegVariant* best = nullptr;
     uint32_t bestLaunches = 0;
     for (const auto& v : kEvalRegVariants) {
-        if (buckets > v.Buckets || (dim == 1) != (v.Pitch == 1) || v.Leaves != (dim > 1 && maxDepth <= 6 ? 64u : 256u)) {
+        if (buckets > v.Buckets || (dim == 1) != (v.Pitch == 1) || v.Leaves != (dim > 1 && maxDepth <= 6 ? 64u : 256u) ||
+            v.Mixed != mixed) {
             continue;
         }
         const uint32_t launches = (dim + v.Pitch - 1) / v.Pitch;
@@ -726,14 +740,15 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId)
     const char* regSwitch = std::getenv("CATBOOST_AMD_REG_KERNEL");
     const bool regEnabled = !(regSwitch && regSwitch[0] == '0');
     const TEvalRegVariant* variant =
-        m.Oblivious && m.MaxDepth <= 8 && m.PackedSevenBit && TreeCount > 0
-            ? PickRegVariant(m.LayoutBuckets, static_cast<uint32_t>(m.Dim), m.MaxDepth)
+        m.Oblivious && m.MaxDepth <= 8 && TreeCount > 0
+            ? PickRegVariant(m.LayoutBuckets, static_cast<uint32_t>(m.Dim), m.MaxDepth, !m.PackedSevenBit)
             : nullptr;
     if (regEnabled && variant) {
         HIP_CHECK(hipModuleLoadData(&m.RegModule, kEvalRegCodeObject));
         HIP_CHECK(hipModuleGetFunction(&m.RegFunction, m.RegModule, variant->Name));
         const uint32_t block = RegTreeBlock(*variant);
         const size_t pitch = variant->Pitch, rowsPerTree = variant->Leaves;
+        const size_t rowDwords = variant->Mixed ? 32 : 16;
         m.RegWaves = variant->Waves;
         m.RegPitch = variant->Pitch;
         m.RegTreeBlocks = static_cast<uint32_t>((TreeCount + block - 1) / block);
@@ -741,14 +756,47 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId)
         const size_t tableTrees = (static_cast<size_t>(m.RegTreeBlocks) + 2) * block;
         const size_t launches = (static_cast<size_t>(m.Dim) + pitch - 1) / pitch;
         m.RegLaunchLeaves = tableTrees * rowsPerTree * pitch;
-        std::vector<uint32_t> rows(tableTrees * kRegRowDwords, 0);  // (bucket 0, add 0): false for every bin
+        std::vector<uint32_t> rows(tableTrees * rowDwords, 0);  // 7-bit form (bucket 0, add 0): false for every bin
         std::vector<double> leaves(launches * m.RegLaunchLeaves, 0.0);
         for (size_t t = 0; t < TreeCount; ++t) {
             const int depth = trees.TreeSizes[t];
+            // 7-bit form: no xor mask in the tree and every bin of its buckets below 128
+            bool sevenBit = true;
             for (int d = 0; d < depth; ++d) {
                 const auto& rb = trees.RepackedBins[trees.TreeStartOffsets[t] + d];
-                rows[t * kRegRowDwords + 2 * d] = rb.FeatureIndex;
-                rows[t * kRegRowDwords + 2 * d + 1] = (128u - rb.SplitIdx) * 0x01010101u;
+                sevenBit = sevenBit && rb.XorMask == 0 && offsets[rb.FeatureIndex + 1] - offsets[rb.FeatureIndex] <= 127;
+            }
+            CBAMD_ENSURE(sevenBit || variant->Mixed, "internal error: tree needs the 8-bit compare");
+            // a mixed model's bucket 0 may hold bins above 127, which the 7-bit padding level
+            // (bucket 0, add 0) would take for true: a tree without levels goes the 8-bit way and
+            // the padding levels of the others use the tree's own first bucket
+            sevenBit = sevenBit && (depth > 0 || !variant->Mixed);
+            uint32_t* row = rows.data() + t * rowDwords;
+            if (sevenBit) {
+                for (int d = 0; d < depth; ++d) {
+                    const auto& rb = trees.RepackedBins[trees.TreeStartOffsets[t] + d];
+                    row[2 * d] = rb.FeatureIndex;
+                    row[2 * d + 1] = (128u - rb.SplitIdx) * 0x01010101u;
+                }
+                for (int d = depth; d < 8 && depth > 0; ++d) {
+                    row[2 * d] = row[0];
+                }
+            } else {
+                for (int d = 0; d < 8; ++d) {
+                    // levels past the tree's depth: splitIdx 255, false for every bin (bins are at most 254)
+                    uint32_t bucket = 0, xorMask = 0, splitIdx = 255;
+                    if (d < depth) {
+                        const auto& rb = trees.RepackedBins[trees.TreeStartOffsets[t] + d];
+                        bucket = rb.FeatureIndex;
+                        xorMask = rb.XorMask;
+                        splitIdx = rb.SplitIdx;
+                    }
+                    row[4 * d] = bucket;
+                    row[4 * d + 1] = xorMask * 0x01010101u;
+                    row[4 * d + 2] = (splitIdx & 0x7fu) * 0x01010101u;
+                    row[4 * d + 3] = splitIdx < 128 ? 0x80808080u : 0u;
+                }
+                row[0] |= 0x80000000u;
             }
             const double* values = trees.LeafValues.data() + trees.TreeFirstLeafOffsets[t];
             for (size_t launch = 0; launch < launches; ++launch) {

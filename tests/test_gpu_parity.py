@@ -184,6 +184,9 @@ def test_random_oblivious_models(seed, dim):
                                           scale=0.5 if seed else 1.0, bias=rng.normal(size=dim) if seed else None)
     x = _random_flat_data(rng, model, cat_values, 777)
     g, o = _check_flat(model, x)
+    # one-hot splits and features with more than 127 borders: the mixed register-resident kernels,
+    # which add in tree order like the CPU evaluator
+    np.testing.assert_array_equal(g.calc_flat(x), o.calc(x))
     # the same model as a non-symmetric one
     _check_flat(mb.convert_oblivious_to_asymmetric(model), x)
     # transposed input and a tree sub-range
