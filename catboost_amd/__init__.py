@@ -162,6 +162,8 @@ def load_library():
         "CbHipQuantizeFlat": (ctypes.c_bool, [vp, sz, c_float_pp, sz, vp, sz]),
         "CbHipQuantizeWithHashedCatFeatures": (ctypes.c_bool, [vp, sz, c_float_pp, sz, c_int_pp, sz, vp, sz]),
         "CbHipModelBucketCount": (ctypes.c_uint32, [vp]),
+        "CbHipFastExpInplace": (None, [vp, sz]),
+        "CbHipApplyPredictionType": (ctypes.c_bool, [ctypes.c_int, sz, sz, vp, vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)
@@ -201,6 +203,28 @@ def _row_pointers(matrix, ctype):
     addresses = matrix.ctypes.data + np.arange(max(n, 1), dtype=np.uint64) * np.uint64(matrix.strides[0])
     # the ctypes array shares (and keeps alive) the numpy buffer of addresses
     return (ctypes.POINTER(ctype) * max(n, 1)).from_buffer(addresses)
+
+
+def fast_exp(values, chunk=None):
+    """The reference's exponent (CbHipFastExpInplace) over runs of `chunk` values (default: all at once)."""
+    lib = load_library()
+    x = np.array(values, dtype=np.float64).ravel()
+    chunk = len(x) if chunk is None else chunk
+    for begin in range(0, len(x), max(chunk, 1)):
+        part = np.ascontiguousarray(x[begin:begin + chunk])
+        lib.CbHipFastExpInplace(part.ctypes.data, len(part))
+        x[begin:begin + chunk] = part
+    return x
+
+
+def apply_prediction_type(raw, dim, prediction_type):
+    """Raw formula values [doc * dim + k] -> prediction type (an APT_* constant), on the host."""
+    lib = load_library()
+    raw = np.ascontiguousarray(np.asarray(raw, dtype=np.float64).ravel())
+    docs = len(raw) // dim
+    out = np.zeros(docs if prediction_type == APT_CLASS else docs * dim)
+    _check(lib.CbHipApplyPredictionType(prediction_type, dim, docs, raw.ctypes.data, out.ctypes.data))
+    return out
 
 
 def model_arrays(float_features=(), cat_features=(), one_hot_features=(), approx_dimension=1, tree_sizes=(),

@@ -6,6 +6,7 @@
 #include "../../include/cb_hip_evaluator.h"
 
 #include "cat_hash.h"
+#include "fast_exp.h"
 #include "hip_evaluator.h"
 #include "model.h"
 #include "model_builder.h"
@@ -84,71 +85,79 @@ void CheckResultSize(const TModelHandle& h, size_t docCount, size_t resultSize) 
     }
 }
 
-// Turns raw formula values into the requested prediction type on the host
-// (TEvalResultProcessor::PostprocessBlock, eval_processing.h:174-240).
+// Turns raw formula values into the requested prediction type on the host, block by block like
+// TEvalResultProcessor::PostprocessBlock (eval_processing.h:174-240; blocks of min(128, docCount)
+// documents, cpu/formula_evaluator.cpp:27), with the reference's exponent (fast_exp.h).
 void PostProcess(EApiPredictionType type, size_t dim, size_t docCount, const double* raw, double* out) {
-    if (dim == 1) {
-        for (size_t i = 0; i < docCount; ++i) {
-            const double v = raw[i];
+    const size_t block = std::min<size_t>(128, docCount);
+    for (size_t begin = 0; begin < docCount; begin += block) {
+        const size_t n = std::min(block, docCount - begin);
+        const double* r = raw + begin * dim;
+        if (type == APT_CLASS) {
+            double* o = out + begin;
+            for (size_t i = 0; i < n; ++i) {
+                // one dimension: the raw value against the border 0 (the CPU evaluator never passes a
+                // probability border); otherwise the first largest dimension
+                o[i] = dim == 1 ? static_cast<double>(r[i] > 0.0)
+                                : static_cast<double>(std::max_element(r + i * dim, r + (i + 1) * dim) - (r + i * dim));
+            }
+            continue;
+        }
+        double* o = out + begin * dim;
+        std::copy(r, r + n * dim, o);
+        const auto sigmoid = [](double* v, size_t count) {  // CalcSigmoid, eval_processing.h:92-99
+            for (size_t i = 0; i < count; ++i) {
+                v[i] = -v[i];
+            }
+            FastExpInplace(v, count);
+            for (size_t i = 0; i < count; ++i) {
+                v[i] = 1. / (1. + v[i]);
+            }
+        };
+        if (dim == 1) {
             switch (type) {
                 case APT_PROBABILITY:
-                    out[i] = 1.0 / (1.0 + std::exp(-v));
+                    sigmoid(o, n);
                     break;
                 case APT_EXPONENT:
-                    out[i] = std::exp(v);
-                    break;
-                case APT_CLASS:
-                    out[i] = v > 0.0 ? 1.0 : 0.0;
+                    FastExpInplace(o, n);
                     break;
                 default:
                     CBAMD_ENSURE(false, "unsupported prediction type");
             }
+            continue;
         }
-        return;
-    }
-    for (size_t i = 0; i < docCount; ++i) {
-        const double* r = raw + i * dim;
         switch (type) {
-            case APT_RMSE_WITH_UNCERTAINTY: {
-                double* o = out + i * dim;
-                for (size_t k = 0; k < dim; ++k) {
-                    o[k] = r[k];
-                }
-                o[1] = std::exp(2.0 * r[1]);
-                break;
-            }
-            case APT_PROBABILITY: {
-                double* o = out + i * dim;
-                const double mx = *std::max_element(r, r + dim);
-                double sum = 0;
-                for (size_t k = 0; k < dim; ++k) {
-                    o[k] = std::exp(r[k] - mx);
-                    sum += o[k];
-                }
-                for (size_t k = 0; k < dim; ++k) {
-                    o[k] /= sum;
+            case APT_RMSE_WITH_UNCERTAINTY:  // CalcSquaredExponentInplace on the second value of a document
+                for (size_t i = 1; i < n * dim; i += dim) {
+                    o[i] *= 2.0f;
+                    FastExpInplace(o + i, 1);
                 }
                 break;
-            }
-            case APT_MULTI_PROBABILITY: {
-                double* o = out + i * dim;
-                for (size_t k = 0; k < dim; ++k) {
-                    o[k] = 1.0 / (1.0 + std::exp(-r[k]));
+            case APT_PROBABILITY:  // CalcSoftmax per document, eval_processing.h:15-27
+                for (size_t i = 0; i < n; ++i) {
+                    double* v = o + i * dim;
+                    const double top = *std::max_element(v, v + dim);
+                    for (size_t k = 0; k < dim; ++k) {
+                        v[k] = v[k] - top;
+                    }
+                    FastExpInplace(v, dim);
+                    double sum = 0;
+                    for (size_t k = 0; k < dim; ++k) {
+                        sum += v[k];
+                    }
+                    for (size_t k = 0; k < dim; ++k) {
+                        v[k] /= sum;
+                    }
                 }
                 break;
-            }
-            case APT_CLASS:
-                out[i] = static_cast<double>(std::max_element(r, r + dim) - r);
+            case APT_MULTI_PROBABILITY:
+                sigmoid(o, n * dim);
                 break;
-            case APT_EXPONENT: {
-                double* o = out + i * dim;
-                for (size_t k = 0; k < dim; ++k) {
-                    o[k] = std::exp(r[k]);
-                }
-                break;
-            }
             default:
-                CBAMD_ENSURE(false, "unsupported prediction type");
+                // the reference's switch has no other case for several dimensions and leaves the raw
+                // values in place (a debug-only assert)
+                break;
         }
     }
 }
@@ -1018,6 +1027,22 @@ bool CbHipQuantizeWithHashedCatFeatures(void* modelHandle, size_t docCount, cons
 
 uint32_t CbHipModelBucketCount(void* modelHandle) {
     return static_cast<TModelHandle*>(modelHandle)->Model.Trees.EffectiveBinFeaturesBucketCount;
+}
+
+void CbHipFastExpInplace(double* values, size_t count) {
+    FastExpInplace(values, count);
+}
+
+bool CbHipApplyPredictionType(int predictionType, size_t dim, size_t docCount, const double* raw, double* result) {
+    return Guard([&] {
+        CBAMD_ENSURE(dim >= 1 && (docCount == 0 || (raw != nullptr && result != nullptr)), "invalid arguments");
+        const auto type = static_cast<EApiPredictionType>(predictionType);
+        if (type == APT_RAW_FORMULA_VAL) {
+            std::copy(raw, raw + docCount * dim, result);
+        } else {
+            PostProcess(type, dim, docCount, raw, result);
+        }
+    });
 }
 
 }  // extern "C"

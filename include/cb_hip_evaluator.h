@@ -185,6 +185,16 @@ bool CbHipQuantizeWithHashedCatFeatures(void* modelHandle, size_t docCount, cons
                                         uint8_t* bins, size_t binsSize);
 uint32_t CbHipModelBucketCount(void* modelHandle);
 
+/* ---- prediction types (host side; no GPU involved) ------------------------------------- */
+
+/* values[i] = exp(values[i]) as NCB::FastExpWithInfInplace computes it on an AVX2 host
+ * (catboost/libs/helpers/math_utils.cpp:14-27, contrib/libs/fmath/fmath.hpp:565-648). */
+void CbHipFastExpInplace(double* values, size_t count);
+/* Raw formula values raw[doc * dim + k] -> the prediction type, block by block like
+ * TEvalResultProcessor::PostprocessBlock (catboost/libs/model/eval_processing.h:174-240).
+ * `result` holds docCount values for APT_CLASS, docCount * dim otherwise. */
+bool CbHipApplyPredictionType(int predictionType, size_t dim, size_t docCount, const double* raw, double* result);
+
 #if defined(__cplusplus)
 }
 #endif

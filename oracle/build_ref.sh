@@ -24,3 +24,6 @@ fi
 g++ -std=c++17 -O2 -w -I "$OUT/gen" -I "$R" -I "$FB/include" -I "$R/catboost/libs/standalone_evaluator" \
   -include cstring "$HERE/ref_main.cpp" "$R/catboost/libs/standalone_evaluator/evaluator.cpp" -o "$OUT/standalone_eval"
 echo "built $OUT/standalone_eval"
+# the exponent of the prediction types (fmath::expd_v, AVX2 path as on the hosts this runs on)
+g++ -std=c++17 -O2 -mavx2 -w -I "$R" "$HERE/ref_fmath_main.cpp" -o "$OUT/fmath_exp"
+echo "built $OUT/fmath_exp"

@@ -727,3 +727,169 @@ void cbo_calc_bruteforce(const cbo_model* m, const cbo_features* f, size_t n_doc
         }
     }
 }
+
+/* ---- prediction types ---------------------------------------------------------------- */
+
+/* fmath's table-based exponent, double precision: ExpdVar (fmath.hpp:150-185). The table and the
+ * scale come from the C library's pow / log exactly as the reference computes them at start-up. */
+#define CBO_EXPD_SBIT 11
+static uint64_t g_expd_tbl[1 << CBO_EXPD_SBIT];
+static double g_expd_a, g_expd_ra;
+static pthread_once_t g_expd_once = PTHREAD_ONCE_INIT;
+
+static void expd_init(void) {
+    const int s = 1 << CBO_EXPD_SBIT;
+    g_expd_a = s / log(2.0);
+    g_expd_ra = 1 / g_expd_a;
+    for (int i = 0; i < s; i++) {
+        const double d = pow(2.0, i * (1.0 / s));
+        uint64_t bits;
+        memcpy(&bits, &d, 8);
+        g_expd_tbl[i] = bits & ((1ULL << 52) - 1);
+    }
+}
+
+/* One value through the arithmetic both paths share (fmath.hpp:587-600 / :484-495): every
+ * multiply, add and subtract is a separate rounding. `di` is the integer the table index and the
+ * exponent are taken from: all 64 bits of d on the vector path, its sign-extended low half on the
+ * scalar path (only bits 0..22 matter). */
+static double expd_core(double x, uint64_t (*index_bits)(double)) {
+    const double b = (double)(3ULL << 51);
+    const uint64_t adj = (1ULL << (CBO_EXPD_SBIT + 10)) - (1ULL << CBO_EXPD_SBIT);
+    const double C1 = 1.0, C2 = 0.16666666685227835064, C3 = 3.0000000027955394;
+    double d = x * g_expd_a;
+    d = d + b;
+    const uint64_t di = index_bits(d);
+    const uint64_t iax = g_expd_tbl[di & ((1u << CBO_EXPD_SBIT) - 1)];
+    double t = d - b;
+    t = t * g_expd_ra;
+    t = t - x;
+    const uint64_t u = (((di + adj) >> CBO_EXPD_SBIT) << 52) | iax;
+    double y = C3 - t;
+    const double tt = t * t;
+    y = y * tt;
+    y = y * C2;
+    y = y - t;
+    y = y + C1;
+    double scale;
+    memcpy(&scale, &u, 8);
+    return y * scale;
+}
+
+static uint64_t expd_bits_all(double d) {
+    uint64_t bits;
+    memcpy(&bits, &d, 8);
+    return bits;
+}
+
+static uint64_t expd_bits_low(double d) {
+    uint64_t bits;
+    memcpy(&bits, &d, 8);
+    return (uint64_t)(int64_t)(int32_t)(uint32_t)bits;
+}
+
+void cbo_fast_exp_inplace(double* x, size_t n) {
+    pthread_once(&g_expd_once, expd_init);
+    const size_t vec = n & ~(size_t)3;
+    for (size_t i = 0; i < vec; i++) {
+        /* _mm256_min_pd / _mm256_max_pd hand back their second operand unless the compare holds,
+         * so a NaN becomes the upper clamp */
+        double v = x[i];
+        v = (v < 709.78272569338397) ? v : 709.78272569338397;
+        v = (v > -708.39641853226408) ? v : -708.39641853226408;
+        x[i] = expd_core(v, expd_bits_all);
+    }
+    for (size_t i = vec; i < n; i++) {
+        const double v = x[i];
+        if (v <= -708.39641853226408) {
+            x[i] = 0;
+        } else if (v >= 709.78271289338397) {
+            x[i] = INFINITY;
+        } else {
+            x[i] = expd_core(v, expd_bits_low);
+        }
+    }
+}
+
+int cbo_apply_prediction_type(int type, size_t dim, size_t n_docs, const double* raw, double* out) {
+    const size_t block = n_docs < 128 ? n_docs : 128;
+    if (type == CBO_RAW) {
+        memcpy(out, raw, n_docs * dim * sizeof(double));
+        return 0;
+    }
+    for (size_t begin = 0; begin < n_docs; begin += block) {
+        const size_t n = n_docs - begin < block ? n_docs - begin : block;
+        const double* r = raw + begin * dim;
+        if (type == CBO_CLASS) {
+            double* o = out + begin;
+            for (size_t i = 0; i < n; i++) {
+                if (dim == 1) {
+                    o[i] = r[i] > 0.0;
+                } else {
+                    size_t best = 0;  /* first maximum, as MaxElement */
+                    for (size_t k = 1; k < dim; k++) {
+                        if (r[i * dim + best] < r[i * dim + k]) {
+                            best = k;
+                        }
+                    }
+                    o[i] = (double)best;
+                }
+            }
+            continue;
+        }
+        double* o = out + begin * dim;
+        memcpy(o, r, n * dim * sizeof(double));
+        if (dim == 1) {
+            if (type == CBO_PROBABILITY) {           /* CalcSigmoid over the block */
+                for (size_t i = 0; i < n; i++) {
+                    o[i] = -o[i];
+                }
+                cbo_fast_exp_inplace(o, n);
+                for (size_t i = 0; i < n; i++) {
+                    o[i] = 1. / (1. + o[i]);
+                }
+            } else if (type == CBO_EXPONENT) {
+                cbo_fast_exp_inplace(o, n);
+            } else {
+                return -1;
+            }
+        } else if (type == CBO_RMSE_WITH_UNCERTAINTY) {  /* exp(2 x) of the second value of a document */
+            for (size_t i = 1; i < n * dim; i += dim) {
+                o[i] *= 2.0f;
+                cbo_fast_exp_inplace(o + i, 1);
+            }
+        } else if (type == CBO_PROBABILITY) {            /* CalcSoftmax per document */
+            for (size_t i = 0; i < n; i++) {
+                double* v = o + i * dim;
+                double mx = v[0];
+                for (size_t k = 1; k < dim; k++) {
+                    if (mx < v[k]) {
+                        mx = v[k];
+                    }
+                }
+                for (size_t k = 0; k < dim; k++) {
+                    v[k] = v[k] - mx;
+                }
+                cbo_fast_exp_inplace(v, dim);
+                double sum = 0;
+                for (size_t k = 0; k < dim; k++) {
+                    sum += v[k];
+                }
+                for (size_t k = 0; k < dim; k++) {
+                    v[k] /= sum;
+                }
+            }
+        } else if (type == CBO_MULTI_PROBABILITY) {      /* CalcSigmoid over the block's values */
+            for (size_t i = 0; i < n * dim; i++) {
+                o[i] = -o[i];
+            }
+            cbo_fast_exp_inplace(o, n * dim);
+            for (size_t i = 0; i < n * dim; i++) {
+                o[i] = 1. / (1. + o[i]);
+            }
+        } else {
+            return -1;
+        }
+    }
+    return 0;
+}

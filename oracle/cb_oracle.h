@@ -120,6 +120,19 @@ uint32_t cbo_cat_feature_hash(const char* s, size_t len);
 /* GetIntegerCatFeatureHash (catboost/libs/model_interface/c_api.cpp:944-949). */
 int32_t cbo_integer_cat_feature_hash(long long v);
 
+/* The exponent of the prediction types: NCB::FastExpWithInfInplace on an AVX2 host
+ * (catboost/libs/helpers/math_utils.cpp:14-27) = fmath::expd_v (contrib/libs/fmath/fmath.hpp:565-648):
+ * the first n & ~3 values take the vector path, the rest fmath::expd (:474-512). */
+void cbo_fast_exp_inplace(double* x, size_t n);
+
+/* TEvalResultProcessor::PostprocessBlock over blocks of min(128, n_docs) documents
+ * (catboost/libs/model/eval_processing.h:174-240, cpu/formula_evaluator.cpp:27). raw[doc * dim + k]
+ * -> out; out holds n_docs values for CBO_CLASS, n_docs * dim otherwise. Returns 0, or -1 for a
+ * prediction type the dimension does not support. */
+enum { CBO_RAW = 0, CBO_EXPONENT = 1, CBO_RMSE_WITH_UNCERTAINTY = 2, CBO_PROBABILITY = 3, CBO_CLASS = 4,
+       CBO_MULTI_PROBABILITY = 5 };
+int cbo_apply_prediction_type(int type, size_t dim, size_t n_docs, const double* raw, double* out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -95,6 +95,10 @@ def _load():
         lib.cbo_cat_feature_hash.argtypes = [ctypes.c_char_p, ctypes.c_size_t]
         lib.cbo_integer_cat_feature_hash.restype = ctypes.c_int32
         lib.cbo_integer_cat_feature_hash.argtypes = [ctypes.c_longlong]
+        lib.cbo_fast_exp_inplace.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
+        lib.cbo_apply_prediction_type.restype = ctypes.c_int
+        lib.cbo_apply_prediction_type.argtypes = [ctypes.c_int, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_void_p,
+                                                  ctypes.c_void_p]
         _lib = lib
     return _lib
 
@@ -121,6 +125,32 @@ def integer_cat_feature_hash(v):
 
 def _p(a):
     return a.ctypes.data_as(ctypes.c_void_p)
+
+
+PREDICTION_TYPES = {"RawFormulaVal": 0, "Exponent": 1, "RMSEWithUncertainty": 2, "Probability": 3, "Class": 4,
+                    "MultiProbability": 5}
+
+
+def fast_exp(values, chunk=None):
+    """The reference's exponent applied to runs of `chunk` values (default: all at once)."""
+    x = np.array(values, dtype=np.float64).ravel()
+    chunk = len(x) if chunk is None else chunk
+    for begin in range(0, len(x), max(chunk, 1)):
+        part = np.ascontiguousarray(x[begin:begin + chunk])
+        _load().cbo_fast_exp_inplace(_p(part), len(part))
+        x[begin:begin + chunk] = part
+    return x
+
+
+def apply_prediction_type(raw, dim, prediction_type):
+    """Raw formula values [doc * dim + k] -> the prediction type, as TEvalResultProcessor does."""
+    raw = np.ascontiguousarray(np.asarray(raw, dtype=np.float64).ravel())
+    docs = len(raw) // dim
+    kind = PREDICTION_TYPES[prediction_type]
+    out = np.zeros(docs if prediction_type == "Class" else docs * dim)
+    if _load().cbo_apply_prediction_type(kind, dim, docs, _p(raw), _p(out)) != 0:
+        raise ValueError("unsupported prediction type %s for dimension %d" % (prediction_type, dim))
+    return out
 
 
 class OracleModel:

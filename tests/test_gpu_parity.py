@@ -163,6 +163,36 @@ def test_iris_fixture(golden_dir):
     np.testing.assert_array_equal(g.quantize_flat(feats), o.binarize(feats))
     g.set_prediction_type("Class")
     np.testing.assert_array_equal(g.calc_flat(feats), labels.astype(np.float64))
+    # the other prediction types of a multi-class model: the oracle's result processor on the
+    # library's own raw values, bit for bit
+    from oracle.oracle import apply_prediction_type
+    for name in ("Probability", "MultiProbability"):
+        g.set_prediction_type(name)
+        np.testing.assert_array_equal(g.calc_flat(feats), apply_prediction_type(pred.ravel(), 3, name))
+    g.set_prediction_type("Probability")
+    np.testing.assert_allclose(g.calc_flat(feats).reshape(-1, 3).sum(axis=1), 1.0, atol=1e-12)
+
+
+def test_prediction_types_of_the_reference_unit_test():
+    """TestFlatCalcMultiValMultiProba (formula_evaluator_ut.cpp:148-165) through the C API, and the
+    one-dimensional types on the two-tree model with scale and bias."""
+    from oracle.oracle import apply_prediction_type
+    g = _gpu_model(rm.multi_value_float_model())
+    raw = np.array([0., 10., 20., 1., 11., 21., 2., 12., 22., 3., 13., 23.])
+    g.set_prediction_type("MultiProbability")
+    probs = g.calc_flat(rm.DATA[:4])
+    np.testing.assert_allclose(probs, 1 / (1 + np.exp(-raw)), atol=1e-6)
+    np.testing.assert_array_equal(probs, apply_prediction_type(raw, 3, "MultiProbability"))
+    rng = np.random.default_rng(12)
+    model, cat_values = _random_oblivious(rng, dim=1, trees=30, max_depth=6, scale=0.5, bias=[0.25])
+    x = _random_flat_data(rng, model, cat_values, 1000)
+    g = _gpu_model(model)
+    raw = g.calc_flat(x)
+    for name in ("Probability", "Exponent", "Class"):
+        g.set_prediction_type(name)
+        np.testing.assert_array_equal(g.calc_flat(x), apply_prediction_type(raw, 1, name))
+    g.set_prediction_type("Probability")
+    np.testing.assert_allclose(g.calc_flat(x), 1 / (1 + np.exp(-raw)), rtol=1e-12)
 
 
 def test_boston_fixture(golden_dir):

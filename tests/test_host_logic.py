@@ -220,3 +220,27 @@ def test_prediction_without_gpu_fails_loudly():
         m.calc_flat(rm.DATA)
     with pytest.raises(cb.CatBoostError, match="HIP"):
         m.enable_gpu_evaluation(0)
+
+
+# --------------------------------------------------------------- prediction types ----
+
+def test_library_exponent_matches_reference_fmath(golden_dir):
+    """CbHipFastExpInplace against the vectors of the reference's fmath::expd_v, bit for bit."""
+    g = np.load(os.path.join(golden_dir, "fmath_exp_vectors.npz"))
+    for chunk in (1, 3, 4, 10, 128):
+        np.testing.assert_array_equal(cb.fast_exp(g["x"], chunk).view(np.uint64), g["chunk_%d" % chunk].view(np.uint64))
+
+
+def test_library_prediction_types_match_the_oracle():
+    from oracle.oracle import PREDICTION_TYPES, apply_prediction_type
+
+    rng = np.random.default_rng(8)
+    cases = ((1, ("Probability", "Exponent", "Class", "RawFormulaVal")), (2, ("RMSEWithUncertainty", "Probability")),
+             (3, ("Probability", "Class", "MultiProbability")), (10, ("Probability", "Class")))
+    for dim, types in cases:
+        for docs in (1, 5, 128, 129, 1000):
+            raw = rng.normal(0, 5, size=docs * dim)
+            raw[rng.random(raw.shape) < 0.01] = 800.0  # beyond the exponent's clamp
+            for name in types:
+                got = cb.apply_prediction_type(raw, dim, PREDICTION_TYPES[name])
+                np.testing.assert_array_equal(got.view(np.uint64), apply_prediction_type(raw, dim, name).view(np.uint64))

@@ -361,3 +361,53 @@ def test_last_block_is_packed_with_its_own_doc_count():
     dm = o.binarize_doc_major(x)
     np.testing.assert_array_equal(first.T, dm[:128])
     np.testing.assert_array_equal(tail.T, dm[128:])
+
+
+# --------------------------------------------------------------- prediction types ----
+
+def test_fast_exp_matches_reference_fmath(golden_dir):
+    """The exponent restatement against the reference's own fmath::expd_v (built from the reference
+    tree by oracle/build_ref.sh; vectors by tests/golden/make_fmath_vectors.py): bit for bit,
+    for every run length the result processor uses, clamps, infinities and NaN included."""
+    from oracle.oracle import fast_exp
+
+    g = np.load(os.path.join(golden_dir, "fmath_exp_vectors.npz"))
+    x = g["x"]
+    for chunk in (1, 3, 4, 10, 128):
+        np.testing.assert_array_equal(fast_exp(x, chunk).view(np.uint64), g["chunk_%d" % chunk].view(np.uint64))
+
+
+def test_fast_exp_is_an_exponent():
+    """Independent of the vectors: a relative error of a few 1e-16 against libm over the range
+    raw formula values live in, exact at 0, monotone."""
+    from oracle.oracle import fast_exp
+
+    x = np.linspace(-50.0, 50.0, 200001)
+    y = fast_exp(x)
+    assert np.max(np.abs(y / np.exp(x) - 1.0)) < 1e-14
+    assert fast_exp([0.0, 0.0, 0.0, 0.0, 0.0])[0] == 1.0 and fast_exp([0.0])[0] == 1.0
+    assert np.all(np.diff(y) >= 0)
+
+
+def test_prediction_types_closed_forms():
+    """TestFlatCalcMultiValMultiProba (formula_evaluator_ut.cpp:148-165): sigmoid of the raw values
+    within 1e-6; softmax sums to one and keeps the order; Class is the arg max / the sign."""
+    from oracle.oracle import apply_prediction_type
+
+    raw = np.array([0., 10., 20., 1., 11., 21., 2., 12., 22., 3., 13., 23.])
+    np.testing.assert_allclose(apply_prediction_type(raw, 3, "MultiProbability"), 1 / (1 + np.exp(-raw)), atol=1e-6)
+    rng = np.random.default_rng(5)
+    raw = rng.normal(0, 4, size=(333, 7))
+    p = apply_prediction_type(raw, 7, "Probability").reshape(333, 7)
+    np.testing.assert_allclose(p.sum(axis=1), 1.0, atol=1e-12)
+    np.testing.assert_allclose(p, np.exp(raw - raw.max(axis=1, keepdims=True)) /
+                               np.exp(raw - raw.max(axis=1, keepdims=True)).sum(axis=1, keepdims=True), rtol=1e-12)
+    np.testing.assert_array_equal(apply_prediction_type(raw, 7, "Class"), raw.argmax(axis=1))
+    one = rng.normal(0, 4, size=1000)
+    np.testing.assert_allclose(apply_prediction_type(one, 1, "Probability"), 1 / (1 + np.exp(-one)), rtol=1e-12)
+    np.testing.assert_allclose(apply_prediction_type(one, 1, "Exponent"), np.exp(one), rtol=1e-12)
+    np.testing.assert_array_equal(apply_prediction_type(one, 1, "Class"), one > 0)
+    two = rng.normal(0, 1, size=(50, 2))
+    u = apply_prediction_type(two, 2, "RMSEWithUncertainty").reshape(50, 2)
+    np.testing.assert_array_equal(u[:, 0], two[:, 0])
+    np.testing.assert_allclose(u[:, 1], np.exp(2 * two[:, 1]), rtol=1e-12)
