@@ -11,8 +11,12 @@
  *   block driver         catboost/libs/model/cpu/formula_evaluator.cpp:10-81, cpu/evaluator.h:95-155
  *   scale and bias       catboost/libs/model/scale_and_bias.cpp:4-50
  *   cat feature hash     catboost/libs/cat_feature/cat_feature.cpp:6-8, util/digest/city.cpp:58-200
+ *   prediction types     catboost/libs/model/eval_processing.h:15-99, 174-240,
+ *                        contrib/libs/fmath/fmath.hpp:150-185, 474-512, 565-648 (the exponent)
  *
- * Pinned by (see tests/test_oracle_*.py): the reference unit-test closed forms
+ * Pinned by (see tests/test_oracle.py, tests/test_ref_vectors.py): the reference's own
+ * standalone evaluator and its own fmath exponent, both built from the reference tree by
+ * oracle/build_ref.sh (vectors under tests/golden/), the reference unit-test closed forms
  * (catboost/libs/model/ut/formula_evaluator_ut.cpp:76-146, 284-307), the .cbm fixtures with
  * golden predictions of the JVM / Rust / .NET binding tests, the JVM hash known answers, the
  * numpy searchsorted invariant for binarize, the oblivious -> non-symmetric equivalence and the
