@@ -43,6 +43,16 @@ def cpu_baseline(model_bytes, info, target_seconds=12.0):
         oracle.calc(x, threads=threads)
     elapsed = time.perf_counter() - t0
     total = docs * repeats
+    # one thread, on a smaller sample (about 3 s)
+    single_docs = min(docs, 20_000)
+    t0 = time.perf_counter()
+    oracle.calc(x[:single_docs], threads=1)
+    single_probe = time.perf_counter() - t0
+    single_repeats = int(max(1, min(50, round(3.0 / max(single_probe, 1e-6)))))
+    t0 = time.perf_counter()
+    for _ in range(single_repeats):
+        oracle.calc(x[:single_docs], threads=1)
+    single_elapsed = time.perf_counter() - t0
     return {
         "value": total / elapsed,
         "unit": "docs/sec",
@@ -51,6 +61,7 @@ def cpu_baseline(model_bytes, info, target_seconds=12.0):
         "sample": "%d docs of the same workload evaluated %d times, %d threads over 128-doc blocks, %.1f s" % (
             docs, repeats, threads, elapsed),
         "tree_evals_per_sec": total * oracle.tree_count / elapsed,
+        "single_thread_docs_per_sec": single_docs * single_repeats / single_elapsed,
     }
 
 
