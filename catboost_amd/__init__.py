@@ -460,9 +460,8 @@ class ModelCalcer:
         offsets, is_split, splits, left, right, voff, values = [0], [], [], [], [], [], []
         for head in tree_heads:
             base = len(is_split)
-            stack = [(head, None, None)]
-            # pre-order numbering so that children follow their parent
-            def add(node):
+
+            def add(node):  # pre-order numbering, children follow their parent
                 i = len(is_split) - base
                 if node[0] == "split":
                     is_split.append(1)
@@ -482,7 +481,7 @@ class ModelCalcer:
                     v = node[1]
                     values.extend([float(v)] if np.isscalar(v) else [float(x) for x in v])
                 return i
-            del stack
+
             add(head)
             offsets.append(len(is_split))
         self.build_non_symmetric_packed(float_features, cat_features, approx_dimension, offsets, is_split,

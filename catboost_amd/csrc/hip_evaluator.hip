@@ -119,6 +119,7 @@ struct TEvalRegVariant {
 };
 constexpr TEvalRegVariant kEvalRegVariants[] = {
     {96, 8, 1, 256, false, "cbamd_eval_reg_b96_w8_p1_l256"},
+    {200, 4, 1, 256, false, "cbamd_eval_reg_b200_w4_p1_l256"},
     {208, 4, 1, 256, false, "cbamd_eval_reg_b208_w4_p1_l256"},
     {192, 4, 2, 64, false, "cbamd_eval_reg_b192_w4_p2_l64"},
     {160, 4, 4, 64, false, "cbamd_eval_reg_b160_w4_p4_l64"},
@@ -127,6 +128,7 @@ constexpr TEvalRegVariant kEvalRegVariants[] = {
     {160, 4, 4, 256, false, "cbamd_eval_reg_b160_w4_p4_l256"},
     {128, 4, 6, 256, false, "cbamd_eval_reg_b128_w4_p6_l256"},
     {96, 8, 1, 256, true, "cbamd_eval_reg_b96_w8_p1_l256_m"},
+    {200, 4, 1, 256, true, "cbamd_eval_reg_b200_w4_p1_l256_m"},
     {208, 4, 1, 256, true, "cbamd_eval_reg_b208_w4_p1_l256_m"},
     {192, 4, 2, 64, true, "cbamd_eval_reg_b192_w4_p2_l64_m"},
     {160, 4, 4, 64, true, "cbamd_eval_reg_b160_w4_p4_l64_m"},

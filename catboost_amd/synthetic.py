@@ -185,9 +185,3 @@ def device_features(info, doc_count, seed=1, device="cuda:0"):
             ids = torch.randint(0, len(hashes), (e - b,), device=device, generator=gen)
             part[:, nf + c] = table[ids].view(torch.float32)
     return x
-
-
-def algorithmic_bytes_per_doc(model, info):
-    """4 bytes per used float feature + 4 per used categorical feature + 8 per output value."""
-    used_floats = len(set(model.get_float_feature_indices()))  # all described floats; trimmed below
-    return 4 * info["floats"] + 4 * len(info["cat_hashes"]) + 8 * info["dim"] if used_floats >= 0 else 0
