@@ -44,7 +44,7 @@ struct TModelHandle {
         std::lock_guard<std::mutex> g(EvaluatorLock);
         if (!Evaluator) {
             Model.EnsureSupported();
-            Evaluator.reset(new THipEvaluator(Model.Trees, DeviceId));
+            Evaluator.reset(new THipEvaluator(Model.Trees, DeviceId, &Model.CtrTables));
         }
         return *Evaluator;
     }

@@ -22,6 +22,90 @@ enum ETreesSlot {
     TS_RepackedBins, TS_EmbeddingFeatures
 };
 
+// TModelCtrBase / TFeatureCombination, ctr_data.fbs:15-19 and features.fbs:71-75
+// (TModelCtrBase::FBDeserialize, TFeatureCombination::FBDeserialize, online_ctr.cpp:17-26, 72-95)
+TModelCtrBase ReadCtrBase(const fb::TTable& t) {
+    TModelCtrBase base;
+    if (!t.Valid()) {
+        return base;
+    }
+    const fb::TTable proj = t.Table(0);
+    if (proj.Valid()) {
+        base.Projection.CatFeatures = proj.Vector<int>(0);
+        static_assert(sizeof(TFloatSplit) == 8 && sizeof(TOneHotSplit) == 8, "splits are two 4-byte fields");
+        base.Projection.BinFeatures = proj.Vector<TFloatSplit>(1);
+        base.Projection.OneHotFeatures = proj.Vector<TOneHotSplit>(2);
+    }
+    const int8_t type = t.Scalar<int8_t>(1, 0);
+    CBAMD_ENSURE(type >= 0 && type <= 5, "unknown CTR type in model");
+    base.CtrType = static_cast<ECtrType>(type);
+    base.TargetBorderClassifierIdx = t.Scalar<int32_t>(2, 0);
+    return base;
+}
+
+// TCtrFeature / TModelCtr, ctr_data.fbs:21-33 (TModelCtr::FBDeserialize, online_ctr.cpp:41-48)
+TCtrFeature ReadCtrFeature(const fb::TTable& t) {
+    TCtrFeature f;
+    const fb::TTable ctr = t.Table(0);
+    CBAMD_ENSURE(ctr.Valid(), "CTR feature without a CTR description");
+    f.Ctr.Base = ReadCtrBase(ctr.Table(0));
+    f.Ctr.TargetBorderIdx = ctr.Scalar<int32_t>(1, 0);
+    f.Ctr.PriorNum = ctr.Scalar<float>(2, 0.f);
+    f.Ctr.PriorDenom = ctr.Scalar<float>(3, 1.f);
+    f.Ctr.Shift = ctr.Scalar<float>(4, 0.f);
+    f.Ctr.Scale = ctr.Scalar<float>(5, 1.f);
+    f.Borders = t.Vector<float>(1);
+    return f;
+}
+
+// LoadSize of util/ysaveload.h:277-296: u32, or 0xffffffff followed by a u64
+uint64_t ReadSize(const uint8_t* p, size_t size, size_t* pos) {
+    CBAMD_ENSURE(*pos + 4 <= size, "Failed to read model part: file is truncated");
+    uint32_t s32;
+    std::memcpy(&s32, p + *pos, 4);
+    *pos += 4;
+    if (s32 != 0xffffffffu) {
+        return s32;
+    }
+    CBAMD_ENSURE(*pos + 8 <= size, "Failed to read model part: file is truncated");
+    uint64_t s64;
+    std::memcpy(&s64, p + *pos, 8);
+    *pos += 8;
+    return s64;
+}
+
+// TCtrData::Load (ctr_data.cpp:24-34): a count, then per table a size and a flatbuffer whose
+// root is TCtrValueTable (ctr_data.fbs:35-41; TCtrValueTable::LoadSolid, ctr_value_table.cpp:57-71)
+void ReadStaticCtrProvider(const uint8_t* p, size_t size, size_t* pos, std::vector<TCtrValueTable>* tables) {
+    const uint64_t count = ReadSize(p, size, pos);
+    tables->clear();
+    for (uint64_t i = 0; i < count; ++i) {
+        const uint64_t len = ReadSize(p, size, pos);
+        CBAMD_ENSURE(len >= 8 && len <= size - *pos, "Failed to read CTR value table: file is truncated");
+        fb::TReader reader(p + *pos, static_cast<size_t>(len));
+        const fb::TTable t = fb::GetRoot(reader);
+        TCtrValueTable table;
+        table.ModelCtrBase = ReadCtrBase(t.Table(0));
+        table.IndexHashRaw = t.Vector<uint8_t>(1);
+        table.CTRBlob = t.Vector<uint8_t>(2);
+        table.CounterDenominator = t.Scalar<int32_t>(3, 0);
+        table.TargetClassesCount = t.Scalar<int32_t>(4, 0);
+        *pos += static_cast<size_t>(len);
+        // a later table with the same key replaces an earlier one, as the hash map insert does
+        bool replaced = false;
+        for (auto& old : *tables) {
+            if (old.ModelCtrBase == table.ModelCtrBase) {
+                old = std::move(table);
+                replaced = true;
+                break;
+            }
+        }
+        if (!replaced) {
+            tables->push_back(std::move(table));
+        }
+    }
+}
+
 void ReadTrees(const fb::TTable& t, TModelTrees* trees) {
     *trees = TModelTrees();
     trees->ApproxDimension = t.Scalar<int32_t>(TS_ApproxDimension, 0);
@@ -56,7 +140,9 @@ void ReadTrees(const fb::TTable& t, TModelTrees* trees) {
         f.StringValues = c.Strings(2);
         trees->OneHotFeatures.push_back(std::move(f));
     }
-    trees->CtrFeatureCount = t.VectorLen(TS_CtrFeatures);
+    for (const auto& c : t.Tables(TS_CtrFeatures)) {
+        trees->CtrFeatures.push_back(ReadCtrFeature(c));
+    }
     trees->TextFeatureCount = t.VectorLen(TS_TextFeatures);
     trees->EstimatedFeatureCount = t.VectorLen(TS_EstimatedFeatures);
     trees->EmbeddingFeatureCount = t.VectorLen(TS_EmbeddingFeatures);
@@ -192,9 +278,13 @@ void TFullModel::Load(const void* data, size_t size) {
     } else {
         Trees = TModelTrees();
     }
+    CtrTables.clear();
+    size_t partPos = pos + static_cast<size_t>(coreSize);
     for (const auto& part : ModelPartIds) {
-        // model.cpp:1201-1226 knows static ctr / text / embedding parts; this evaluator has none of them
-        CBAMD_ENSURE(false, "Model part '" + part + "' (CTR, text or embedding data) is not supported by the HIP evaluator");
+        // model.cpp:1201-1226 knows static ctr / text / embedding parts; this evaluator reads the first kind
+        CBAMD_ENSURE(part == "static_provider_v1",
+                     "Model part '" + std::string(part.c_str()) + "' (text or embedding data) is not supported by the HIP evaluator");
+        ReadStaticCtrProvider(p, size, &partPos, &CtrTables);
     }
     EnsureSupported();
     Trees.UpdateRuntimeData();
@@ -208,6 +298,8 @@ void TFullModel::LoadFromFile(const std::string& path) {
 }
 
 std::string TFullModel::Save() const {
+    CBAMD_ENSURE(Trees.CtrFeatures.empty() && CtrTables.empty(),
+                 "Saving a model with CTR features is not supported by the HIP evaluator library");
     fb::TWriter w;
     // TModelCore
     fb::TWriter::TTableBuilder coreB;

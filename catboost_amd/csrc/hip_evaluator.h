@@ -34,7 +34,8 @@ struct TKernelTimes {
 class THipEvaluator {
 public:
     // Uploads the model tables (model upload of cuda/evaluator.cpp:30-84, re-laid out as SoA).
-    THipEvaluator(const TModelTrees& trees, int deviceId);
+    // `ctrTables`: the tables of the model's static CTR provider; needed when the model has CTR features.
+    THipEvaluator(const TModelTrees& trees, int deviceId, const std::vector<TCtrValueTable>* ctrTables = nullptr);
     ~THipEvaluator();
     THipEvaluator(const THipEvaluator&) = delete;
     THipEvaluator& operator=(const THipEvaluator&) = delete;

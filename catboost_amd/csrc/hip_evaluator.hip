@@ -319,6 +319,199 @@ void BuildLevelOrderTrees(const TModelTrees& trees, int dim, const std::vector<u
     }
 }
 
+// Device tables of the model's CTR features (TStaticCtrProvider, catboost/libs/model/static_ctr_provider.cpp):
+// per feature a descriptor and its projection (SetupBinFeatureIndexes, :142-178, resolved to bucket
+// numbers and input columns), all index buckets and all rows. Every row index and class index the kernel
+// can reach is checked here, so a damaged model fails at load instead of reading out of bounds.
+// Appends one bucket entry per 254 borders of a CTR feature to the binarize bucket tables.
+void BuildCtrTables(const TModelTrees& trees, const std::vector<TCtrValueTable>& tables, std::vector<uint32_t>* srcFlat,
+                    std::vector<uint32_t>* srcSplit, std::vector<uint32_t>* offsets, std::vector<uint32_t>* flags,
+                    std::vector<uint32_t>* values, TDeviceVec<uint32_t>* featuresOut, TDeviceVec<uint32_t>* itemsOut,
+                    TDeviceVec<uint32_t>* indexOut, TDeviceVec<uint32_t>* blobOut) {
+    static_assert(sizeof(dev::TCtrFeatureDev) == 64 && sizeof(dev::TCtrItemDev) == 16, "device CTR records changed size");
+    std::vector<dev::TCtrFeatureDev> features;
+    std::vector<dev::TCtrItemDev> items;
+    std::vector<uint32_t> index, blob;
+    std::vector<uint32_t> tableIndexBegin(tables.size(), 0), tableBlobBegin(tables.size(), 0), tableRows(tables.size(), 0);
+    std::vector<bool> tableUploaded(tables.size(), false);
+
+    // first bucket of every used float feature and of every one-hot feature
+    std::vector<uint32_t> floatFirstBucket(trees.FloatFeatures.size(), 0), oneHotFirstBucket(trees.OneHotFeatures.size(), 0);
+    uint32_t bucket = 0;
+    for (size_t i = 0; i < trees.FloatFeatures.size(); ++i) {
+        floatFirstBucket[i] = bucket;
+        bucket += static_cast<uint32_t>((trees.FloatFeatures[i].Borders.size() + kMaxValuesPerBin - 1) / kMaxValuesPerBin);
+    }
+    for (size_t i = 0; i < trees.OneHotFeatures.size(); ++i) {
+        oneHotFirstBucket[i] = bucket;
+        bucket += static_cast<uint32_t>((trees.OneHotFeatures[i].Values.size() + kMaxValuesPerBin - 1) / kMaxValuesPerBin);
+    }
+
+    for (const auto& feature : trees.CtrFeatures) {
+        const TModelCtr& ctr = feature.Ctr;
+        size_t t = 0;
+        while (t < tables.size() && !(tables[t].ModelCtrBase == ctr.Base)) {
+            ++t;
+        }
+        CBAMD_ENSURE(t < tables.size(), "Model has a CTR feature without its table of learned statistics");
+        const TCtrValueTable& table = tables[t];
+        const size_t bucketCount = table.IndexHashRaw.size() / 12;
+        CBAMD_ENSURE(table.IndexHashRaw.size() % 12 == 0 && bucketCount > 0 && (bucketCount & (bucketCount - 1)) == 0 &&
+                         bucketCount <= (size_t(1) << 31),
+                     "Dense hash view must have 2^k buckets");
+        // bytes of one row and the class indexes the CTR reads (static_ctr_provider.cpp:52-126)
+        size_t rowBytes = 0;
+        switch (ctr.Base.CtrType) {
+            case ECtrType::BinarizedTargetMeanValue:
+            case ECtrType::FloatTargetMeanValue:
+                rowBytes = 8;
+                break;
+            case ECtrType::Counter:
+            case ECtrType::FeatureFreq:
+                rowBytes = 4;
+                break;
+            case ECtrType::Buckets:
+                CBAMD_ENSURE(table.TargetClassesCount > 0 && ctr.TargetBorderIdx >= 0 &&
+                                 ctr.TargetBorderIdx < table.TargetClassesCount,
+                             "CTR target border index out of range");
+                rowBytes = 4 * static_cast<size_t>(table.TargetClassesCount);
+                break;
+            case ECtrType::Borders:
+                if (table.TargetClassesCount > 2) {
+                    CBAMD_ENSURE(ctr.TargetBorderIdx >= 0 && ctr.TargetBorderIdx < table.TargetClassesCount,
+                                 "CTR target border index out of range");
+                    rowBytes = 4 * static_cast<size_t>(table.TargetClassesCount);
+                } else {
+                    rowBytes = 8;
+                }
+                break;
+        }
+        if (!tableUploaded[t]) {
+            tableUploaded[t] = true;
+            tableIndexBegin[t] = static_cast<uint32_t>(index.size() / 3);
+            tableBlobBegin[t] = static_cast<uint32_t>(blob.size());
+            bool hasEmpty = false;
+            uint32_t maxRow = 0;
+            bool anyRow = false;
+            for (size_t b = 0; b < bucketCount; ++b) {
+                uint32_t w[3];
+                std::memcpy(w, table.IndexHashRaw.data() + 12 * b, 12);
+                index.insert(index.end(), w, w + 3);
+                if ((w[0] & w[1]) == 0xffffffffu) {
+                    hasEmpty = true;
+                } else {
+                    maxRow = std::max(maxRow, w[2]);
+                    anyRow = true;
+                }
+            }
+            CBAMD_ENSURE(hasEmpty, "CTR index hash table has no empty bucket");
+            tableRows[t] = anyRow ? maxRow + 1 : 0;
+            blob.resize(blob.size() + (table.CTRBlob.size() + 3) / 4, 0);
+            if (!table.CTRBlob.empty()) {
+                std::memcpy(blob.data() + tableBlobBegin[t], table.CTRBlob.data(), table.CTRBlob.size());
+            }
+            CBAMD_ENSURE(index.size() / 3 < (size_t(1) << 32) && blob.size() < (size_t(1) << 32), "CTR tables are too large");
+        }
+        CBAMD_ENSURE(static_cast<size_t>(tableRows[t]) * rowBytes <= table.CTRBlob.size(),
+                     "CTR value table is shorter than its index");
+
+        dev::TCtrFeatureDev f{};
+        f.ItemBegin = static_cast<uint32_t>(items.size());
+        for (int catIndex : ctr.Base.Projection.CatFeatures) {
+            const TCatFeature* cat = nullptr;
+            for (const auto& c : trees.CatFeatures) {
+                if (c.Index == catIndex && c.UsedInModel) {
+                    cat = &c;
+                }
+            }
+            CBAMD_ENSURE(cat != nullptr && cat->FlatIndex >= 0 && cat->Index >= 0,
+                         "CTR projection refers to an unknown or unused categorical feature");
+            items.push_back({dev::kCtrItemCat, static_cast<uint32_t>(cat->FlatIndex), static_cast<uint32_t>(cat->Index), 0});
+        }
+        for (const auto& split : ctr.Base.Projection.BinFeatures) {
+            bool found = false;
+            for (size_t i = 0; i < trees.FloatFeatures.size() && !found; ++i) {
+                const auto& ff = trees.FloatFeatures[i];
+                if (ff.Index != split.FloatFeature) {
+                    continue;
+                }
+                for (size_t b = 0; b < ff.Borders.size(); ++b) {
+                    if (ff.Borders[b] == split.Split) {
+                        const uint32_t at = floatFirstBucket[i] + static_cast<uint32_t>(b / kMaxValuesPerBin);
+                        items.push_back({dev::kCtrItemBinGe, at, at, static_cast<uint32_t>(b % kMaxValuesPerBin) + 1});
+                        found = true;
+                        break;
+                    }
+                }
+            }
+            CBAMD_ENSURE(found, "CTR projection refers to a float split the model does not have");
+        }
+        for (const auto& split : ctr.Base.Projection.OneHotFeatures) {
+            bool found = false;
+            for (size_t i = 0; i < trees.OneHotFeatures.size() && !found; ++i) {
+                const auto& oh = trees.OneHotFeatures[i];
+                if (oh.CatFeatureIndex != split.CatFeatureIdx) {
+                    continue;
+                }
+                for (size_t v = 0; v < oh.Values.size(); ++v) {
+                    if (oh.Values[v] == split.Value) {
+                        const uint32_t at = oneHotFirstBucket[i] + static_cast<uint32_t>(v / kMaxValuesPerBin);
+                        items.push_back({dev::kCtrItemBinEq, at, at, static_cast<uint32_t>(v % kMaxValuesPerBin) + 1});
+                        found = true;
+                        break;
+                    }
+                }
+            }
+            CBAMD_ENSURE(found, "CTR projection refers to a one-hot split the model does not have");
+        }
+        f.ItemEnd = static_cast<uint32_t>(items.size());
+        f.HashBuckets = tableIndexBegin[t];
+        f.HashMask = static_cast<uint32_t>(bucketCount - 1);
+        f.BlobOffset = tableBlobBegin[t];
+        f.Type = static_cast<uint32_t>(ctr.Base.CtrType);
+        f.TargetBorderIdx = ctr.TargetBorderIdx;
+        f.TargetClassesCount = table.TargetClassesCount;
+        f.CounterDenominator = table.CounterDenominator;
+        f.PriorNum = ctr.PriorNum;
+        f.PriorDenom = ctr.PriorDenom;
+        f.Shift = ctr.Shift;
+        f.Scale = ctr.Scale;
+        f.FirstBucket = static_cast<uint32_t>(srcFlat->size());
+        for (size_t begin = 0; begin < feature.Borders.size(); begin += kMaxValuesPerBin) {
+            const size_t end = std::min(begin + kMaxValuesPerBin, feature.Borders.size());
+            std::vector<float> b;
+            for (size_t i = begin; i < end; ++i) {
+                if (!std::isnan(feature.Borders[i])) {
+                    b.push_back(feature.Borders[i]);
+                }
+            }
+            std::sort(b.begin(), b.end());
+            for (float x : b) {
+                uint32_t bits;
+                std::memcpy(&bits, &x, 4);
+                values->push_back(bits);
+            }
+            offsets->push_back(static_cast<uint32_t>(values->size()));
+            srcFlat->push_back(0);
+            srcSplit->push_back(0);
+            flags->push_back(dev::kBucketFlagCtr);
+        }
+        f.BucketCount = static_cast<uint32_t>(srcFlat->size()) - f.FirstBucket;
+        features.push_back(f);
+    }
+    std::vector<uint32_t> raw(features.size() * (sizeof(dev::TCtrFeatureDev) / 4));
+    std::memcpy(raw.data(), features.data(), raw.size() * 4);
+    featuresOut->Upload(raw);
+    raw.assign(std::max<size_t>(items.size(), 1) * (sizeof(dev::TCtrItemDev) / 4), 0);
+    std::memcpy(raw.data(), items.data(), items.size() * sizeof(dev::TCtrItemDev));
+    itemsOut->Upload(raw);
+    indexOut->Upload(index);
+    if (blob.empty()) {
+        blob.push_back(0);
+    }
+    blobOut->Upload(blob);
+}
+
 }  // namespace
 
 int GetHipDeviceCount() {
@@ -337,6 +530,8 @@ struct THipEvaluator::TImpl {
     bool Oblivious = true;
     uint32_t RealBucketCount = 0;  // buckets of the model; the device layout uses max(1, this)
     uint32_t LayoutBuckets = 1;
+    uint32_t BinarizeBuckets = 0;  // float and one-hot buckets: what the binarize kernels fill
+    uint32_t CtrCount = 0;         // CTR features; their buckets follow and CtrBinarizeKernel fills them
     size_t FlatVectorSize = 0;
     size_t MinFloatSize = 0;
     size_t MinCatSize = 0;
@@ -349,6 +544,8 @@ struct THipEvaluator::TImpl {
     TDeviceVec<uint32_t> BucketSrcFlat, BucketSrcSplit, BucketOffset, BucketFlags, Values;
     TDeviceVec<uint32_t> BucketGrid;  // 4 dwords per bucket: lowest border, cells per unit, search steps, 0
     TDeviceVec<uint32_t> BucketLut;   // kLutCells bytes per bucket
+    // CTR tables: feature descriptors, projection items, the index buckets and the rows of all tables
+    TDeviceVec<uint32_t> CtrFeatures, CtrItems, CtrIndexBuckets, CtrBlob;
     // tree tables
     TDeviceVec<uint32_t> Splits, TreeStart, TreeSize, FirstLeaf, StepNodes, NodeToLeaf;
     TDeviceVec<double> Leaves, Bias;
@@ -410,13 +607,22 @@ struct THipEvaluator::TImpl {
 
     dev::TBinarizeTables BinarizeTables(bool flat) const {
         dev::TBinarizeTables t;
-        t.BucketCount = LayoutBuckets;
+        t.BucketCount = BinarizeBuckets;
+        t.BucketPitch = LayoutBuckets;
         t.BucketSrc = flat ? BucketSrcFlat.Get() : BucketSrcSplit.Get();
         t.BucketOffset = BucketOffset.Get();
         t.BucketFlags = BucketFlags.Get();
         t.Values = Values.Get();
         t.Grid = reinterpret_cast<const uint4*>(BucketGrid.Get());
         t.Lut = BucketLut.Get();
+        return t;
+    }
+    dev::TCtrTablesDev CtrTables() const {
+        dev::TCtrTablesDev t;
+        t.Features = reinterpret_cast<const dev::TCtrFeatureDev*>(CtrFeatures.Get());
+        t.Items = reinterpret_cast<const dev::TCtrItemDev*>(CtrItems.Get());
+        t.IndexBuckets = CtrIndexBuckets.Get();
+        t.Blob = CtrBlob.Get();
         return t;
     }
     dev::TTreeTables TreeTables() const {
@@ -436,7 +642,7 @@ struct THipEvaluator::TImpl {
     hipStream_t Pick(void* stream) const { return stream ? static_cast<hipStream_t>(stream) : Stream; }
 };
 
-THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId)
+THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::vector<TCtrValueTable>* ctrTables)
     : Impl(new TImpl)
 {
     const int deviceCount = GetHipDeviceCount();
@@ -519,6 +725,14 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId)
             srcSplit.push_back(static_cast<uint32_t>(cat->Index));
             flags.push_back(dev::kBucketFlagOneHot);
         }
+    }
+    m.BinarizeBuckets = static_cast<uint32_t>(srcFlat.size());
+    CBAMD_ENSURE(m.BinarizeBuckets == trees.CtrFirstBucket, "internal error: bucket count mismatch");
+    if (!trees.CtrFeatures.empty()) {
+        CBAMD_ENSURE(ctrTables != nullptr, "Model has CTR features but no tables of learned statistics");
+        BuildCtrTables(trees, *ctrTables, &srcFlat, &srcSplit, &offsets, &flags, &values, &m.CtrFeatures, &m.CtrItems,
+                       &m.CtrIndexBuckets, &m.CtrBlob);
+        m.CtrCount = static_cast<uint32_t>(trees.CtrFeatures.size());
     }
     CBAMD_ENSURE(srcFlat.size() == BucketCount, "internal error: bucket count mismatch");
     for (size_t b = 0; b + 1 < offsets.size(); ++b) {
@@ -895,6 +1109,9 @@ void LaunchBinarizeRows(uint32_t maxBucketValues, size_t blocks, const float* fl
                         uint32_t* bins, hipStream_t s) {
     CBAMD_ENSURE(docCount < (size_t(1) << 31) && stride < (size_t(1) << 31) && catStride < (size_t(1) << 31),
                  "batch is too large for one binarize launch");
+    if (tab.BucketCount == 0) {
+        return;  // a model of CTR features only
+    }
     const int log2Slots = BinarizeLog2Slots(maxBucketValues);
     if (log2Slots == 5) {
         LaunchBinarizeRowsP<5>(blocks, floats, stride, cats, catStride, docCount, tab, bins, s);
@@ -950,15 +1167,40 @@ void THipEvaluator::QuantizeDevice(const TFeatureBatch& batch, size_t docCount, 
         }
         case TFeatureBatch::FlatColumns: {
             CBAMD_ENSURE(batch.Stride >= docCount, "column stride is shorter than the document count");
-            const dim3 grid(static_cast<uint32_t>(blocks), (m.LayoutBuckets + 3) / 4);
-            hipLaunchKernelGGL(dev::BinarizeColumnsKernel, grid, dim3(256), 0, s, batch.Floats, batch.Stride, docCount,
-                               m.BinarizeTables(true), reinterpret_cast<uint32_t*>(bins));
+            if (m.BinarizeBuckets > 0) {
+                const dim3 grid(static_cast<uint32_t>(blocks), (m.BinarizeBuckets + 3) / 4);
+                hipLaunchKernelGGL(dev::BinarizeColumnsKernel, grid, dim3(256), 0, s, batch.Floats, batch.Stride, docCount,
+                                   m.BinarizeTables(true), reinterpret_cast<uint32_t*>(bins));
+            }
             break;
         }
         default:
             CBAMD_ENSURE(false, "unknown feature layout");
     }
     HIP_CHECK(hipGetLastError());
+    if (m.CtrCount > 0) {
+        // the CTR features read the bins written above and the hashed categorical values
+        dev::TCatSource cats;
+        cats.SplitColumns = batch.Layout == TFeatureBatch::SplitRows ? 1u : 0u;
+        if (batch.Layout == TFeatureBatch::SplitRows) {
+            cats.Base = reinterpret_cast<const uint32_t*>(batch.Cats);
+            cats.DocStride = batch.CatStride;
+            cats.ColumnStride = 1;
+        } else if (batch.Layout == TFeatureBatch::FlatRows) {
+            cats.Base = reinterpret_cast<const uint32_t*>(batch.Floats);
+            cats.DocStride = batch.Stride;
+            cats.ColumnStride = 1;
+        } else {
+            cats.Base = reinterpret_cast<const uint32_t*>(batch.Floats);
+            cats.DocStride = 1;
+            cats.ColumnStride = batch.Stride;
+        }
+        CBAMD_ENSURE(m.CtrCount <= 65535, "too many CTR features for one launch");
+        const dim3 grid(static_cast<uint32_t>(blocks), m.CtrCount);
+        hipLaunchKernelGGL(dev::CtrBinarizeKernel, grid, dim3(64), 0, s, cats, static_cast<uint32_t>(docCount), m.CtrTables(),
+                           m.BinarizeTables(batch.Layout != TFeatureBatch::SplitRows), reinterpret_cast<uint32_t*>(bins));
+        HIP_CHECK(hipGetLastError());
+    }
 }
 
 namespace {

@@ -26,8 +26,11 @@ constexpr uint32_t kXcdCount = 8;       // accelerator dies of an MI355X, each w
 constexpr int kBucketTile = 16;         // buckets binarized per workgroup (small: ~20 KB of LDS, 7 workgroups per CU)
 constexpr int kMaxBucketValues = 256;   // 254 values, padded
 
+constexpr int kBucketFlagCtr = 4;        // bucket of a CTR feature: filled by CtrBinarizeKernel
+
 struct TBinarizeTables {
-    uint32_t BucketCount;
+    uint32_t BucketCount;          // buckets the binarize kernels fill: float and one-hot features
+    uint32_t BucketPitch;          // buckets per document block in `bins` (those and the CTR buckets)
     const uint32_t* BucketSrc;     // source column of the bucket in the chosen layout
     const uint32_t* BucketOffset;  // [BucketCount + 1] offsets into Values
     const uint32_t* BucketFlags;
@@ -242,7 +245,7 @@ __global__ __launch_bounds__(256) void BinarizeRowsKernel(const float* __restric
                     packed |= CountBelowInCell(values, lut, myLo[k], myScale[k], myTopStep[k], v) << (8 * j);
                 }
             }
-            bins[(static_cast<size_t>(block) * tab.BucketCount + b0 + bb) * kWave + lane] = packed;
+            bins[(static_cast<size_t>(block) * tab.BucketPitch + b0 + bb) * kWave + lane] = packed;
         }
     }
 #undef CBAMD_LOAD_BLOCK
@@ -294,7 +297,180 @@ __global__ __launch_bounds__(256) void BinarizeColumnsKernel(const float* __rest
         }
         packed |= bin << (8 * j);
     }
-    bins[(block * tab.BucketCount + bucket) * kWave + lane] = packed;
+    bins[(block * tab.BucketPitch + bucket) * kWave + lane] = packed;
+}
+
+// ---- CTR (target statistics) features -------------------------------------------------------
+// What TStaticCtrProvider::CalcCtrs (catboost/libs/model/static_ctr_provider.cpp:14-131) and the
+// binarization of its results (cpu/quantization.h:304-325) do per block, done per document here.
+
+struct TCtrFeatureDev {
+    uint32_t ItemBegin, ItemEnd;  // the projection: entries of TCtrTablesDev::Items
+    uint32_t HashBuckets;         // first 12-byte bucket of the CTR's table in IndexBuckets
+    uint32_t HashMask;            // buckets of the table - 1
+    uint32_t BlobOffset;          // first dword of the table's rows in Blob
+    uint32_t Type;                // ECtrType
+    int32_t TargetBorderIdx;
+    int32_t TargetClassesCount;
+    int32_t CounterDenominator;
+    float PriorNum, PriorDenom, Shift, Scale;
+    uint32_t FirstBucket, BucketCount;  // where the binarized CTR goes
+    uint32_t Pad;
+};
+
+constexpr uint32_t kCtrItemCat = 0;       // hashed categorical value of column SrcFlat / SrcSplit
+constexpr uint32_t kCtrItemBinGe = 1;     // float split: bin of bucket SrcFlat >= Value
+constexpr uint32_t kCtrItemBinEq = 2;     // one-hot split: bin of bucket SrcFlat == Value
+
+struct TCtrItemDev {
+    uint32_t Kind, SrcFlat, SrcSplit, Value;
+};
+
+struct TCtrTablesDev {
+    const TCtrFeatureDev* Features;
+    const TCtrItemDev* Items;
+    const uint32_t* IndexBuckets;  // {hash low, hash high, row} per bucket (helpers/dense_hash_view.h:12-26)
+    const uint32_t* Blob;
+};
+
+// hashed categorical values of a batch: Base[doc * DocStride + column * ColumnStride]
+struct TCatSource {
+    const uint32_t* Base;
+    size_t DocStride, ColumnStride;
+    uint32_t SplitColumns;  // columns are categorical feature indexes (not flat feature indexes)
+};
+
+__device__ __forceinline__ uint64_t CtrCalcHash(uint64_t a, uint64_t b) {  // catboost/libs/model/hash.h:11-14
+    constexpr uint64_t kMagicMult = 0x4906ba494954cb65ull;
+    return kMagicMult * (a + kMagicMult * b);
+}
+
+// TModelCtr::Calc, online_ctr.h:290-293: two roundings each for the quotient and the affine map
+__device__ __forceinline__ float CtrCalc(const TCtrFeatureDev& f, float countInClass, float totalCount) {
+    const float ctr = __fdiv_rn(__fadd_rn(countInClass, f.PriorNum), __fadd_rn(totalCount, f.PriorDenom));
+    return __fmul_rn(__fadd_rn(ctr, f.Shift), f.Scale);
+}
+
+constexpr uint32_t kCtrNotFound = 0xffffffffu;
+
+// TDenseIndexHashView::GetIndex, helpers/dense_hash_view.h:46-56; the probe sequence ends at the first
+// empty bucket, and after one pass over the table at the latest
+__device__ __forceinline__ uint32_t CtrTableRow(const TCtrTablesDev& ctr, const TCtrFeatureDev& f, uint64_t hash) {
+    const uint32_t lo = static_cast<uint32_t>(hash), hi = static_cast<uint32_t>(hash >> 32);
+    uint32_t zz = lo & f.HashMask;
+    for (uint32_t probes = 0; probes <= f.HashMask; ++probes) {
+        const uint32_t* bucket = ctr.IndexBuckets + 3 * (static_cast<size_t>(f.HashBuckets) + zz);
+        const uint32_t blo = bucket[0], bhi = bucket[1];
+        if ((blo & bhi) == 0xffffffffu) {
+            return kCtrNotFound;
+        }
+        if (blo == lo && bhi == hi) {
+            return bucket[2];
+        }
+        zz = (zz + 1) & f.HashMask;
+    }
+    return kCtrNotFound;
+}
+
+// static_ctr_provider.cpp:52-126, one branch per CTR type
+__device__ __forceinline__ float CtrValue(const TCtrTablesDev& ctr, const TCtrFeatureDev& f, uint32_t row) {
+    const uint32_t* blob = ctr.Blob + f.BlobOffset;
+    if (f.Type == 2 || f.Type == 3) {  // mean of the target: {float Sum; int Count}
+        if (row == kCtrNotFound) {
+            return CtrCalc(f, 0.f, 0.f);
+        }
+        return CtrCalc(f, __uint_as_float(blob[2 * static_cast<size_t>(row)]),
+                       static_cast<float>(static_cast<int32_t>(blob[2 * static_cast<size_t>(row) + 1])));
+    }
+    if (f.Type == 4 || f.Type == 5) {  // Counter, FeatureFreq
+        const float denominator = static_cast<float>(f.CounterDenominator);
+        if (row == kCtrNotFound) {
+            return CtrCalc(f, 0.f, denominator);
+        }
+        return CtrCalc(f, static_cast<float>(static_cast<int32_t>(blob[row])), denominator);
+    }
+    const int32_t classes = f.TargetClassesCount;
+    if (f.Type == 1) {  // Buckets
+        if (row == kCtrNotFound) {
+            return CtrCalc(f, 0.f, 0.f);
+        }
+        const uint32_t* history = blob + static_cast<size_t>(row) * classes;
+        int32_t total = 0;
+        for (int32_t c = 0; c < classes; ++c) {
+            total += static_cast<int32_t>(history[c]);
+        }
+        return CtrCalc(f, static_cast<float>(static_cast<int32_t>(history[f.TargetBorderIdx])), static_cast<float>(total));
+    }
+    // Borders
+    if (classes > 2) {
+        int32_t good = 0, total = 0;
+        if (row != kCtrNotFound) {
+            const uint32_t* history = blob + static_cast<size_t>(row) * classes;
+            for (int32_t c = 0; c < f.TargetBorderIdx + 1; ++c) {
+                total += static_cast<int32_t>(history[c]);
+            }
+            for (int32_t c = f.TargetBorderIdx + 1; c < classes; ++c) {
+                good += static_cast<int32_t>(history[c]);
+            }
+            total += good;
+        }
+        return CtrCalc(f, static_cast<float>(good), static_cast<float>(total));
+    }
+    if (row == kCtrNotFound) {
+        return CtrCalc(f, 0.f, 0.f);
+    }
+    const int32_t n0 = static_cast<int32_t>(blob[2 * static_cast<size_t>(row)]);
+    const int32_t n1 = static_cast<int32_t>(blob[2 * static_cast<size_t>(row) + 1]);
+    return CtrCalc(f, static_cast<float>(n1), static_cast<float>(n0 + n1));
+}
+
+// grid = (document blocks, CTR features), one wave per workgroup: lane l computes the CTR of documents
+// l, l + 64, l + 128, l + 192 of the block from the block's float / one-hot bins (already written)
+// and the hashed categorical values, and writes the bins of the CTR's buckets.
+__global__ __launch_bounds__(64) void CtrBinarizeKernel(TCatSource cats, uint32_t docCount, TCtrTablesDev ctr,
+                                                        TBinarizeTables tab, uint32_t* __restrict__ bins) {
+    const uint32_t block = blockIdx.x, lane = threadIdx.x;
+    const TCtrFeatureDev f = ctr.Features[blockIdx.y];
+    uint64_t hash[4] = {0, 0, 0, 0};
+    for (uint32_t i = f.ItemBegin; i < f.ItemEnd; ++i) {
+        const TCtrItemDev item = ctr.Items[i];
+        if (item.Kind == kCtrItemCat) {
+            const size_t column = cats.SplitColumns ? item.SrcSplit : item.SrcFlat;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const size_t doc = min(block * kDocsPerBlock + j * kWave + lane, docCount - 1);
+                const int32_t v = static_cast<int32_t>(cats.Base[doc * cats.DocStride + column * cats.ColumnStride]);
+                hash[j] = CtrCalcHash(hash[j], static_cast<uint64_t>(static_cast<int64_t>(v)));
+            }
+        } else {
+            const uint32_t word = bins[(static_cast<size_t>(block) * tab.BucketPitch + item.SrcFlat) * kWave + lane];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t bin = (word >> (8 * j)) & 0xffu;
+                const bool holds = item.Kind == kCtrItemBinGe ? bin >= item.Value : bin == item.Value;
+                hash[j] = CtrCalcHash(hash[j], holds ? 1u : 0u);
+            }
+        }
+    }
+    float value[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        value[j] = CtrValue(ctr, f, CtrTableRow(ctr, f, hash[j]));
+    }
+    for (uint32_t k = 0; k < f.BucketCount; ++k) {
+        const uint32_t bucket = f.FirstBucket + k;
+        const uint32_t begin = tab.BucketOffset[bucket], end = tab.BucketOffset[bucket + 1];
+        uint32_t count[4] = {0, 0, 0, 0};
+        for (uint32_t b = begin; b < end; ++b) {
+            const float border = __uint_as_float(tab.Values[b]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                count[j] += value[j] > border ? 1u : 0u;
+            }
+        }
+        bins[(static_cast<size_t>(block) * tab.BucketPitch + bucket) * kWave + lane] =
+            count[0] | (count[1] << 8) | (count[2] << 16) | (count[3] << 24);
+    }
 }
 
 // Final value of one output cell: Scale * sum (+ Bias[k] when the range starts at tree 0),

@@ -14,7 +14,7 @@ bool TModelSplit::operator<(const TModelSplit& o) const {
     if (Type != o.Type) {
         return static_cast<int>(Type) < static_cast<int>(o.Type);
     }
-    if (Type == ESplitType::FloatFeature) {
+    if (Type == ESplitType::FloatFeature || Type == ESplitType::OnlineCtr) {
         return std::tie(FeatureIndex, Border) < std::tie(o.FeatureIndex, o.Border);
     }
     return std::tie(FeatureIndex, Value) < std::tie(o.FeatureIndex, o.Value);
@@ -24,7 +24,7 @@ bool TModelSplit::operator==(const TModelSplit& o) const {
     if (Type != o.Type) {
         return false;
     }
-    if (Type == ESplitType::FloatFeature) {
+    if (Type == ESplitType::FloatFeature || Type == ESplitType::OnlineCtr) {
         return FeatureIndex == o.FeatureIndex && Border == o.Border;
     }
     return FeatureIndex == o.FeatureIndex && Value == o.Value;
@@ -133,6 +133,16 @@ void TModelTrees::UpdateRuntimeData() {
                                 static_cast<uint32_t>(valueId % kMaxValuesPerBin) + 1});
         }
         buckets += static_cast<uint32_t>((oh.Values.size() + kMaxValuesPerBin - 1) / kMaxValuesPerBin);
+    }
+    CtrFirstBucket = buckets;
+    for (size_t i = 0; i < CtrFeatures.size(); ++i) {
+        const auto& borders = CtrFeatures[i].Borders;
+        for (size_t borderId = 0; borderId < borders.size(); ++borderId) {
+            BinFeatures.push_back(TModelSplit::Ctr(static_cast<int>(i), borders[borderId]));
+            splitIds.push_back({buckets + static_cast<uint32_t>(borderId / kMaxValuesPerBin),
+                                static_cast<uint32_t>(borderId % kMaxValuesPerBin) + 1});
+        }
+        buckets += static_cast<uint32_t>((borders.size() + kMaxValuesPerBin - 1) / kMaxValuesPerBin);
     }
     EffectiveBinFeaturesBucketCount = buckets;
 
@@ -243,11 +253,31 @@ void TModelTrees::ConvertObliviousToAsymmetric() {
 }
 
 void TFullModel::EnsureSupported() const {
-    CBAMD_ENSURE(Trees.CtrFeatureCount == 0 && ModelPartIds.empty(),
-                 "Model contains CTR (target statistics) features or extra model parts, HIP evaluation impossible");
+    for (const auto& part : ModelPartIds) {
+        CBAMD_ENSURE(part == "static_provider_v1",
+                     "Model part '" + std::string(part.c_str()) + "' (text or embedding data) is not supported by the HIP evaluator");
+    }
+    // every CTR of the model needs its table of learned statistics (ICtrProvider::HasNeededCtrs,
+    // static_ctr_provider.cpp:133-140) and refers to features the model has
+    for (const auto& feature : Trees.CtrFeatures) {
+        const TCtrValueTable* table = FindCtrTable(feature.Ctr.Base);
+        CBAMD_ENSURE(table != nullptr, "Model has a CTR feature without its table of learned statistics");
+        CBAMD_ENSURE(table->IndexHashRaw.size() % 12 == 0 && table->IndexHashRaw.size() >= 12 &&
+                         ((table->IndexHashRaw.size() / 12) & (table->IndexHashRaw.size() / 12 - 1)) == 0,
+                     "Dense hash view must have 2^k buckets");
+    }
     CBAMD_ENSURE(Trees.TextFeatureCount == 0 && Trees.EstimatedFeatureCount == 0,
                  "Model contains text features, HIP evaluation impossible");
     CBAMD_ENSURE(Trees.EmbeddingFeatureCount == 0, "Model contains embedding features, HIP evaluation impossible");
+}
+
+const TCtrValueTable* TFullModel::FindCtrTable(const TModelCtrBase& base) const {
+    for (const auto& table : CtrTables) {
+        if (table.ModelCtrBase == base) {
+            return &table;
+        }
+    }
+    return nullptr;
 }
 
 std::vector<std::string> TFullModel::GetUsedFeaturesNames() const {

@@ -52,6 +52,81 @@ struct TOneHotFeature {  // features.h:142-160
     std::vector<std::string> StringValues;
 };
 
+enum class ECtrType : int8_t {  // flatbuffers/ctr_data.fbs:5-12
+    Borders = 0,
+    Buckets = 1,
+    BinarizedTargetMeanValue = 2,
+    FloatTargetMeanValue = 3,
+    Counter = 4,
+    FeatureFreq = 5
+};
+
+struct TFloatSplit {  // online_ctr.h:32-64
+    int FloatFeature = 0;
+    float Split = 0.f;
+    bool operator==(const TFloatSplit& o) const { return FloatFeature == o.FloatFeature && Split == o.Split; }
+    bool operator<(const TFloatSplit& o) const {
+        return FloatFeature != o.FloatFeature ? FloatFeature < o.FloatFeature : Split < o.Split;
+    }
+};
+
+struct TOneHotSplit {  // online_ctr.h:66-98
+    int CatFeatureIdx = 0;
+    int Value = 0;
+    bool operator==(const TOneHotSplit& o) const { return CatFeatureIdx == o.CatFeatureIdx && Value == o.Value; }
+    bool operator<(const TOneHotSplit& o) const {
+        return CatFeatureIdx != o.CatFeatureIdx ? CatFeatureIdx < o.CatFeatureIdx : Value < o.Value;
+    }
+};
+
+// The features a CTR is computed over (online_ctr.h:108-170).
+struct TFeatureCombination {
+    std::vector<int> CatFeatures;
+    std::vector<TFloatSplit> BinFeatures;
+    std::vector<TOneHotSplit> OneHotFeatures;
+    bool operator==(const TFeatureCombination& o) const {
+        return CatFeatures == o.CatFeatures && BinFeatures == o.BinFeatures && OneHotFeatures == o.OneHotFeatures;
+    }
+};
+
+struct TModelCtrBase {  // online_ctr.h:178-258: identifies a table of learned statistics
+    TFeatureCombination Projection;
+    ECtrType CtrType = ECtrType::Borders;
+    int TargetBorderClassifierIdx = 0;
+    bool operator==(const TModelCtrBase& o) const {
+        return Projection == o.Projection && CtrType == o.CtrType &&
+               TargetBorderClassifierIdx == o.TargetBorderClassifierIdx;
+    }
+};
+
+struct TModelCtr {  // online_ctr.h:260-316
+    TModelCtrBase Base;
+    int TargetBorderIdx = 0;
+    float PriorNum = 0.f;
+    float PriorDenom = 1.f;
+    float Shift = 0.f;
+    float Scale = 1.f;
+    float Calc(float countInClass, float totalCount) const {  // online_ctr.h:290-293
+        const float ctr = (countInClass + PriorNum) / (totalCount + PriorDenom);
+        return (ctr + Shift) * Scale;
+    }
+};
+
+struct TCtrFeature {  // features.h:306-323
+    TModelCtr Ctr;
+    std::vector<float> Borders;
+};
+
+// One table of learned statistics (ctr_value_table.h:17-109): an open-addressing index
+// hash -> row (12-byte buckets {u64 hash, u32 row}, helpers/dense_hash_view.h:12-66) and the rows.
+struct TCtrValueTable {
+    TModelCtrBase ModelCtrBase;
+    std::vector<uint8_t> IndexHashRaw;
+    std::vector<uint8_t> CTRBlob;
+    int CounterDenominator = 0;
+    int TargetClassesCount = 0;
+};
+
 struct TRepackedBin {  // model.h:64-70
     uint16_t FeatureIndex = 0;
     uint8_t XorMask = 0;
@@ -68,7 +143,7 @@ enum class ESplitType : int { FloatFeature = 0, EstimatedFeature = 1, OneHotFeat
 // TModelSplit restricted to the kinds this evaluator supports (split.h:27-100).
 struct TModelSplit {
     ESplitType Type = ESplitType::FloatFeature;
-    int FeatureIndex = 0;  // float feature index / cat feature index
+    int FeatureIndex = 0;  // float feature index / cat feature index / position in CtrFeatures
     float Border = 0.f;
     int Value = 0;
 
@@ -86,6 +161,13 @@ struct TModelSplit {
         s.Value = value;
         return s;
     }
+    static TModelSplit Ctr(int ctrFeature, float border) {
+        TModelSplit s;
+        s.Type = ESplitType::OnlineCtr;
+        s.FeatureIndex = ctrFeature;
+        s.Border = border;
+        return s;
+    }
     bool operator<(const TModelSplit& o) const;
     bool operator==(const TModelSplit& o) const;
 };
@@ -99,6 +181,7 @@ struct TModelTrees {
     std::vector<TCatFeature> CatFeatures;
     std::vector<TFloatFeature> FloatFeatures;
     std::vector<TOneHotFeature> OneHotFeatures;
+    std::vector<TCtrFeature> CtrFeatures;
     std::vector<double> LeafValues;
     std::vector<double> LeafWeights;
     std::vector<TNonSymmetricTreeStepNode> NonSymmetricStepNodes;
@@ -106,7 +189,6 @@ struct TModelTrees {
     double Scale = 1.0;
     std::vector<double> Bias;  // ApproxDimension values
     // feature kinds this evaluator refuses; only their presence is recorded
-    size_t CtrFeatureCount = 0;
     size_t TextFeatureCount = 0;
     size_t EstimatedFeatureCount = 0;
     size_t EmbeddingFeatureCount = 0;
@@ -114,6 +196,7 @@ struct TModelTrees {
     // ---- runtime state (TRuntimeData / TForApplyData, model.h:146-187)
     std::vector<TModelSplit> BinFeatures;
     uint32_t EffectiveBinFeaturesBucketCount = 0;
+    uint32_t CtrFirstBucket = 0;  // buckets of float and one-hot features come first, CTR buckets after them
     std::vector<TRepackedBin> RepackedBins;
     std::vector<size_t> TreeFirstLeafOffsets;
     size_t UsedFloatFeaturesCount = 0;
@@ -148,6 +231,9 @@ struct TFullModel {
     TModelTrees Trees;
     std::map<std::string, std::string> ModelInfo;
     std::vector<std::string> ModelPartIds;
+    // the tables of the static CTR provider (model part "static_provider_v1", static_ctr_provider.h:14-88)
+    std::vector<TCtrValueTable> CtrTables;
+    const TCtrValueTable* FindCtrTable(const TModelCtrBase& base) const;
 
     // .cbm (de)serialisation, model.cpp:1113-1228
     void Load(const void* data, size_t size);

@@ -184,10 +184,18 @@ typedef struct { uint16_t feature_index; uint8_t xor_mask; uint8_t split_idx; } 
 /* one entry per binary feature (TModelSplit), in CalcBinFeatures order */
 typedef struct {
     int32_t is_onehot;
-    int32_t feature;   /* index into float features / one-hot features of the model */
+    int32_t is_ctr;
+    int32_t feature;   /* index into float features / one-hot features / CTR features of the model */
     float border;
     int32_t value;
 } cbo_bin_feature;
+
+/* a bin of the quantized block that a CTR projection looks at (TBinFeatureIndexValue, ctr_provider.h:80-92) */
+typedef struct {
+    uint32_t bin_index;
+    int32_t check_value_equal;
+    uint8_t value;
+} cbo_bin_index_value;
 
 struct cbo_model {
     int32_t approx_dim, n_trees, n_tree_splits, n_float, n_cat, n_onehot, n_step_nodes;
@@ -213,6 +221,18 @@ struct cbo_model {
     size_t min_float_size, min_cat_size, flat_expected;
     int32_t* oh_packed_cat; /* per one-hot feature: packed index among used cat features */
     int32_t has_onehot;
+    /* CTR features and their tables */
+    int32_t n_ctr, n_ctr_tables;
+    int32_t *ctr_border_offsets, *ctr_cat_offsets, *ctr_cats, *ctr_float_offsets, *ctr_float_feature;
+    int32_t *ctr_onehot_offsets, *ctr_onehot_cat, *ctr_onehot_value, *ctr_type, *ctr_target_border_idx, *ctr_table;
+    float *ctr_borders, *ctr_float_border, *ctr_prior_num, *ctr_prior_denom, *ctr_shift, *ctr_scale;
+    uint64_t *table_bucket_offsets, *table_blob_offsets;
+    uint8_t *table_buckets, *table_blobs;
+    int32_t *table_counter_denominator, *table_target_classes_count;
+    /* derived, TStaticCtrProvider::SetupBinFeatureIndexes (static_ctr_provider.cpp:142-178) */
+    int32_t* ctr_packed_cats;             /* per projection cat feature: row of the transposed hashes */
+    cbo_bin_index_value* ctr_bin_indexes; /* per projection float split, then per one-hot split */
+    int32_t *ctr_float_raw, *ctr_onehot_raw; /* position of the split's feature in the model's lists */
 };
 
 static void* dup_mem(const void* p, size_t n) {
@@ -230,6 +250,13 @@ void cbo_model_free(cbo_model* m) {
     free(m->oh_cat_index); free(m->oh_value_offsets); free(m->oh_values);
     free(m->leaf_values); free(m->step_nodes); free(m->node_id_to_leaf_id); free(m->bias);
     free(m->bin_features); free(m->repacked); free(m->first_leaf_offsets); free(m->oh_packed_cat);
+    free(m->ctr_border_offsets); free(m->ctr_cat_offsets); free(m->ctr_cats); free(m->ctr_float_offsets);
+    free(m->ctr_float_feature); free(m->ctr_onehot_offsets); free(m->ctr_onehot_cat); free(m->ctr_onehot_value);
+    free(m->ctr_type); free(m->ctr_target_border_idx); free(m->ctr_table); free(m->ctr_borders);
+    free(m->ctr_float_border); free(m->ctr_prior_num); free(m->ctr_prior_denom); free(m->ctr_shift);
+    free(m->ctr_scale); free(m->table_bucket_offsets); free(m->table_blob_offsets); free(m->table_buckets);
+    free(m->table_blobs); free(m->table_counter_denominator); free(m->table_target_classes_count);
+    free(m->ctr_packed_cats); free(m->ctr_bin_indexes); free(m->ctr_float_raw); free(m->ctr_onehot_raw);
     free(m);
 }
 
@@ -268,6 +295,37 @@ cbo_model* cbo_model_create(const cbo_model_desc* d, char* err, size_t err_len) 
     m->node_id_to_leaf_id = dup_mem(d->node_id_to_leaf_id, sizeof(uint32_t) * d->n_step_nodes);
     m->bias = dup_mem(d->bias, sizeof(double) * d->approx_dim);
     m->has_onehot = d->n_onehot > 0;
+    m->n_ctr = d->n_ctr;
+    m->n_ctr_tables = d->n_ctr_tables;
+    int32_t n_ctr_borders = 0;
+    if (d->n_ctr > 0) {
+        const int n = d->n_ctr;
+        m->ctr_border_offsets = dup_mem(d->ctr_border_offsets, sizeof(int32_t) * (n + 1));
+        m->ctr_cat_offsets = dup_mem(d->ctr_cat_offsets, sizeof(int32_t) * (n + 1));
+        m->ctr_float_offsets = dup_mem(d->ctr_float_offsets, sizeof(int32_t) * (n + 1));
+        m->ctr_onehot_offsets = dup_mem(d->ctr_onehot_offsets, sizeof(int32_t) * (n + 1));
+        n_ctr_borders = d->ctr_border_offsets[n];
+        m->ctr_borders = dup_mem(d->ctr_borders, sizeof(float) * n_ctr_borders);
+        m->ctr_cats = dup_mem(d->ctr_cats, sizeof(int32_t) * d->ctr_cat_offsets[n]);
+        m->ctr_float_feature = dup_mem(d->ctr_float_feature, sizeof(int32_t) * d->ctr_float_offsets[n]);
+        m->ctr_float_border = dup_mem(d->ctr_float_border, sizeof(float) * d->ctr_float_offsets[n]);
+        m->ctr_onehot_cat = dup_mem(d->ctr_onehot_cat, sizeof(int32_t) * d->ctr_onehot_offsets[n]);
+        m->ctr_onehot_value = dup_mem(d->ctr_onehot_value, sizeof(int32_t) * d->ctr_onehot_offsets[n]);
+        m->ctr_type = dup_mem(d->ctr_type, sizeof(int32_t) * n);
+        m->ctr_target_border_idx = dup_mem(d->ctr_target_border_idx, sizeof(int32_t) * n);
+        m->ctr_prior_num = dup_mem(d->ctr_prior_num, sizeof(float) * n);
+        m->ctr_prior_denom = dup_mem(d->ctr_prior_denom, sizeof(float) * n);
+        m->ctr_shift = dup_mem(d->ctr_shift, sizeof(float) * n);
+        m->ctr_scale = dup_mem(d->ctr_scale, sizeof(float) * n);
+        m->ctr_table = dup_mem(d->ctr_table, sizeof(int32_t) * n);
+        const int nt = d->n_ctr_tables;
+        m->table_bucket_offsets = dup_mem(d->table_bucket_offsets, sizeof(uint64_t) * (nt + 1));
+        m->table_blob_offsets = dup_mem(d->table_blob_offsets, sizeof(uint64_t) * (nt + 1));
+        m->table_buckets = dup_mem(d->table_buckets, 12 * (size_t)d->table_bucket_offsets[nt]);
+        m->table_blobs = dup_mem(d->table_blobs, (size_t)d->table_blob_offsets[nt]);
+        m->table_counter_denominator = dup_mem(d->table_counter_denominator, sizeof(int32_t) * nt);
+        m->table_target_classes_count = dup_mem(d->table_target_classes_count, sizeof(int32_t) * nt);
+    }
     /* IsOblivious, model.h:271-273 */
     m->oblivious = (d->n_step_nodes == 0);
 
@@ -294,7 +352,7 @@ cbo_model* cbo_model_create(const cbo_model_desc* d, char* err, size_t err_len) 
         m->flat_expected = (size_t)(m->ff_flat_index[m->n_float - 1] + 1);
 
     /* CalcBinFeatures, model.cpp:471-577 */
-    int32_t total = n_borders + n_values;
+    int32_t total = n_borders + n_values + n_ctr_borders;
     m->bin_features = (cbo_bin_feature*)calloc(total ? total : 1, sizeof(cbo_bin_feature));
     uint32_t* split_bucket = (uint32_t*)calloc(total ? total : 1, sizeof(uint32_t));
     uint32_t* split_idx = (uint32_t*)calloc(total ? total : 1, sizeof(uint32_t));
@@ -321,6 +379,18 @@ cbo_model* cbo_model_create(const cbo_model_desc* d, char* err, size_t err_len) 
             m->bin_features[nb].value = m->oh_values[m->oh_value_offsets[i] + v];
             split_bucket[nb] = buckets + v / CBO_MAX_VALUES_PER_BIN;
             split_idx[nb] = (v % CBO_MAX_VALUES_PER_BIN) + 1;
+            ++nb;
+        }
+        buckets += (cnt + CBO_MAX_VALUES_PER_BIN - 1) / CBO_MAX_VALUES_PER_BIN;
+    }
+    for (int i = 0; i < m->n_ctr; ++i) {
+        int32_t cnt = m->ctr_border_offsets[i + 1] - m->ctr_border_offsets[i];
+        for (int b = 0; b < cnt; ++b) {
+            m->bin_features[nb].is_ctr = 1;
+            m->bin_features[nb].feature = i;
+            m->bin_features[nb].border = m->ctr_borders[m->ctr_border_offsets[i] + b];
+            split_bucket[nb] = buckets + b / CBO_MAX_VALUES_PER_BIN;
+            split_idx[nb] = (b % CBO_MAX_VALUES_PER_BIN) + 1;
             ++nb;
         }
         buckets += (cnt + CBO_MAX_VALUES_PER_BIN - 1) / CBO_MAX_VALUES_PER_BIN;
@@ -390,6 +460,81 @@ cbo_model* cbo_model_create(const cbo_model_desc* d, char* err, size_t err_len) 
         if (found < 0) FAIL("one-hot feature refers to an unused categorical feature");
         m->oh_packed_cat[i] = found;
     }
+
+    /* TStaticCtrProvider::SetupBinFeatureIndexes, static_ctr_provider.cpp:142-178: where a projection's
+     * splits sit in the quantized block, and which row of the transposed hashes a cat feature is */
+    if (m->n_ctr > 0) {
+        const int n = m->n_ctr;
+        const int32_t nc = m->ctr_cat_offsets[n], nf = m->ctr_float_offsets[n], no = m->ctr_onehot_offsets[n];
+        m->ctr_packed_cats = (int32_t*)calloc(nc ? nc : 1, sizeof(int32_t));
+        m->ctr_bin_indexes = (cbo_bin_index_value*)calloc((nf + no) ? (nf + no) : 1, sizeof(cbo_bin_index_value));
+        m->ctr_float_raw = (int32_t*)calloc(nf ? nf : 1, sizeof(int32_t));
+        m->ctr_onehot_raw = (int32_t*)calloc(no ? no : 1, sizeof(int32_t));
+        for (int i = 0; i < nc; ++i) {
+            int32_t packed = 0, found = -1;
+            for (int c = 0; c < m->n_cat; ++c) {
+                if (!m->cf_used[c]) continue;
+                if (m->cf_index[c] == m->ctr_cats[i]) found = packed;
+                ++packed;
+            }
+            if (found < 0) FAIL("CTR projection refers to an unused categorical feature");
+            m->ctr_packed_cats[i] = found;
+        }
+        for (int i = 0; i < nf; ++i) {
+            uint32_t current = 0;
+            int found = 0;
+            for (int ff = 0; ff < m->n_float && !found; ++ff) {
+                const int32_t b0 = m->ff_border_offsets[ff], b1 = m->ff_border_offsets[ff + 1];
+                if (b1 == b0) continue;
+                if (m->ff_index[ff] == m->ctr_float_feature[i]) {
+                    for (int32_t b = b0; b < b1; ++b) {
+                        if (m->ff_borders[b] == m->ctr_float_border[i]) {
+                            m->ctr_bin_indexes[i].bin_index = current + (uint32_t)(b - b0) / CBO_MAX_VALUES_PER_BIN;
+                            m->ctr_bin_indexes[i].check_value_equal = 0;
+                            m->ctr_bin_indexes[i].value = (uint8_t)((b - b0) % CBO_MAX_VALUES_PER_BIN + 1);
+                            m->ctr_float_raw[i] = ff;
+                            found = 1;
+                            break;
+                        }
+                    }
+                }
+                current += (uint32_t)(b1 - b0 + CBO_MAX_VALUES_PER_BIN - 1) / CBO_MAX_VALUES_PER_BIN;
+            }
+            if (!found) FAIL("CTR projection refers to a float split the model does not have");
+        }
+        uint32_t float_buckets = 0;
+        for (int ff = 0; ff < m->n_float; ++ff)
+            float_buckets += (uint32_t)(m->ff_border_offsets[ff + 1] - m->ff_border_offsets[ff] + CBO_MAX_VALUES_PER_BIN - 1) /
+                             CBO_MAX_VALUES_PER_BIN;
+        for (int i = 0; i < no; ++i) {
+            uint32_t current = float_buckets;
+            int found = 0;
+            for (int oh = 0; oh < m->n_onehot && !found; ++oh) {
+                const int32_t v0 = m->oh_value_offsets[oh], v1 = m->oh_value_offsets[oh + 1];
+                if (m->oh_cat_index[oh] == m->ctr_onehot_cat[i]) {
+                    for (int32_t v = v0; v < v1; ++v) {
+                        if (m->oh_values[v] == m->ctr_onehot_value[i]) {
+                            m->ctr_bin_indexes[nf + i].bin_index = current + (uint32_t)(v - v0) / CBO_MAX_VALUES_PER_BIN;
+                            m->ctr_bin_indexes[nf + i].check_value_equal = 1;
+                            m->ctr_bin_indexes[nf + i].value = (uint8_t)((v - v0) % CBO_MAX_VALUES_PER_BIN + 1);
+                            m->ctr_onehot_raw[i] = oh;
+                            found = 1;
+                            break;
+                        }
+                    }
+                }
+                current += (uint32_t)(v1 - v0 + CBO_MAX_VALUES_PER_BIN - 1) / CBO_MAX_VALUES_PER_BIN;
+            }
+            if (!found) FAIL("CTR projection refers to a one-hot split the model does not have");
+        }
+        for (int i = 0; i < n; ++i) {
+            const int32_t t = m->ctr_table[i];
+            if (t < 0 || t >= m->n_ctr_tables) FAIL("CTR feature without a value table");
+            const uint64_t buckets_in_table = m->table_bucket_offsets[t + 1] - m->table_bucket_offsets[t];
+            if (buckets_in_table == 0 || (buckets_in_table & (buckets_in_table - 1)) != 0)
+                FAIL("dense hash view must have 2^k buckets");
+        }
+    }
     return m;
 }
 
@@ -430,6 +575,117 @@ static inline uint32_t get_cat(const cbo_model* m, const cbo_features* f, int ca
         case 0: v = f->floats[doc * f->stride + (size_t)m->cf_flat_index[cat]]; memcpy(&u, &v, 4); return u;
         case 1: v = f->floats[(size_t)m->cf_flat_index[cat] * f->stride + doc]; memcpy(&u, &v, 4); return u;
         default: return (uint32_t)f->cats[doc * f->cat_stride + (size_t)m->cf_index[cat]];
+    }
+}
+
+/* -------------------------------------------------------------------------- CTRs -------- */
+
+/* CalcHash, catboost/libs/model/hash.h:11-14 */
+static inline uint64_t ctr_calc_hash(uint64_t a, uint64_t b) {
+    const uint64_t magic = 0x4906ba494954cb65ULL;
+    return magic * (a + magic * b);
+}
+
+/* TDenseIndexHashView::GetIndex, catboost/libs/helpers/dense_hash_view.h:46-56 */
+#define CBO_NOT_FOUND 0xffffffffu
+static uint32_t ctr_table_index(const cbo_model* m, int table, uint64_t hash) {
+    const uint8_t* buckets = m->table_buckets + 12 * (size_t)m->table_bucket_offsets[table];
+    const uint64_t mask = m->table_bucket_offsets[table + 1] - m->table_bucket_offsets[table] - 1;
+    for (uint64_t zz = hash & mask;; zz = (zz + 1) & mask) {
+        uint64_t h;
+        memcpy(&h, buckets + 12 * zz, 8);
+        if (h == 0xffffffffffffffffULL) return CBO_NOT_FOUND;
+        if (h == hash) {
+            uint32_t v;
+            memcpy(&v, buckets + 12 * zz + 8, 4);
+            return v;
+        }
+    }
+}
+
+/* TModelCtr::Calc, online_ctr.h:290-293 */
+static inline float ctr_calc(const cbo_model* m, int ctr, float count_in_class, float total_count) {
+    float v = (count_in_class + m->ctr_prior_num[ctr]) / (total_count + m->ctr_prior_denom[ctr]);
+    return (v + m->ctr_shift[ctr]) * m->ctr_scale[ctr];
+}
+
+/* The value of CTR `ctr` for a row of its table (or CBO_NOT_FOUND): the per-type branches of
+ * TStaticCtrProvider::CalcCtrs, static_ctr_provider.cpp:52-126. */
+static float ctr_value(const cbo_model* m, int ctr, uint32_t row) {
+    const int table = m->ctr_table[ctr];
+    const uint8_t* blob = m->table_blobs + m->table_blob_offsets[table];
+    const int type = m->ctr_type[ctr];
+    if (type == 2 || type == 3) { /* BinarizedTargetMeanValue, FloatTargetMeanValue: {float Sum; int Count} */
+        if (row == CBO_NOT_FOUND) return ctr_calc(m, ctr, 0.f, 0.f);
+        float sum;
+        int32_t count;
+        memcpy(&sum, blob + 8 * (size_t)row, 4);
+        memcpy(&count, blob + 8 * (size_t)row + 4, 4);
+        return ctr_calc(m, ctr, sum, (float)count);
+    }
+    const int32_t* ints = (const int32_t*)blob;
+    if (type == 4 || type == 5) { /* Counter, FeatureFreq */
+        const int32_t denominator = m->table_counter_denominator[table];
+        if (row == CBO_NOT_FOUND) return ctr_calc(m, ctr, 0.f, (float)denominator);
+        return ctr_calc(m, ctr, (float)ints[row], (float)denominator);
+    }
+    const int32_t classes = m->table_target_classes_count[table];
+    const int32_t target_border = m->ctr_target_border_idx[ctr];
+    if (type == 1) { /* Buckets */
+        if (row == CBO_NOT_FOUND) return ctr_calc(m, ctr, 0.f, 0.f);
+        const int32_t* history = ints + (size_t)row * (size_t)classes;
+        int32_t good = history[target_border], total = 0;
+        for (int32_t c = 0; c < classes; ++c) total += history[c];
+        return ctr_calc(m, ctr, (float)good, (float)total);
+    }
+    /* Borders */
+    if (classes > 2) {
+        int32_t good = 0, total = 0;
+        if (row != CBO_NOT_FOUND) {
+            const int32_t* history = ints + (size_t)row * (size_t)classes;
+            for (int32_t c = 0; c < target_border + 1; ++c) total += history[c];
+            for (int32_t c = target_border + 1; c < classes; ++c) good += history[c];
+            total += good;
+        }
+        return ctr_calc(m, ctr, (float)good, (float)total);
+    }
+    if (row == CBO_NOT_FOUND) return ctr_calc(m, ctr, 0.f, 0.f);
+    const int32_t* history = ints + 2 * (size_t)row;
+    return ctr_calc(m, ctr, (float)history[1], (float)(history[0] + history[1]));
+}
+
+/* CalcCtrs over one quantized block (static_ctr_provider.cpp:14-131, CalcHashes of ctr_provider.h:94-123):
+ * bins = [bucket][doc_count] of the float and one-hot features, hashes = [used cat][doc_count];
+ * ctrs = [ctr][doc_count]. Consecutive CTRs with one projection share their hashes in the reference; the
+ * hash does not depend on that, so every CTR computes its own here. */
+static void calc_ctrs_block(const cbo_model* m, const uint8_t* bins, const uint32_t* transposed_hash,
+                            size_t doc_count, float* ctrs) {
+    uint64_t hashes[CBO_BLOCK];
+    const int32_t nf_all = m->ctr_float_offsets[m->n_ctr];
+    for (int ctr = 0; ctr < m->n_ctr; ++ctr) {
+        for (size_t d = 0; d < doc_count; ++d) hashes[d] = 0;
+        for (int32_t i = m->ctr_cat_offsets[ctr]; i < m->ctr_cat_offsets[ctr + 1]; ++i) {
+            const uint32_t* vals = transposed_hash + (size_t)m->ctr_packed_cats[i] * doc_count;
+            for (size_t d = 0; d < doc_count; ++d)
+                hashes[d] = ctr_calc_hash(hashes[d], (uint64_t)(int64_t)(int32_t)vals[d]);
+        }
+        for (int pass = 0; pass < 2; ++pass) {
+            const int32_t b = pass == 0 ? m->ctr_float_offsets[ctr] : nf_all + m->ctr_onehot_offsets[ctr];
+            const int32_t e = pass == 0 ? m->ctr_float_offsets[ctr + 1] : nf_all + m->ctr_onehot_offsets[ctr + 1];
+            for (int32_t i = b; i < e; ++i) {
+                const cbo_bin_index_value* bi = &m->ctr_bin_indexes[i];
+                const uint8_t* col = bins + (size_t)bi->bin_index * doc_count;
+                if (!bi->check_value_equal) {
+                    for (size_t d = 0; d < doc_count; ++d)
+                        hashes[d] = ctr_calc_hash(hashes[d], (uint64_t)(col[d] >= bi->value));
+                } else {
+                    for (size_t d = 0; d < doc_count; ++d)
+                        hashes[d] = ctr_calc_hash(hashes[d], (uint64_t)(col[d] == bi->value));
+                }
+            }
+        }
+        for (size_t d = 0; d < doc_count; ++d)
+            ctrs[(size_t)ctr * doc_count + d] = ctr_value(m, ctr, ctr_table_index(m, m->ctr_table[ctr], hashes[d]));
     }
 }
 
@@ -486,7 +742,41 @@ static void binarize_block(const cbo_model* m, const cbo_features* f, size_t sta
             }
             out += doc_count * (size_t)((v1 - v0 + CBO_MAX_VALUES_PER_BIN - 1) / CBO_MAX_VALUES_PER_BIN);
         }
+        if (m->n_ctr > 0) {
+            /* quantization.h:304-325: CTR values of the block, binarized like float features without
+             * a NaN policy */
+            float* ctrs = (float*)malloc(sizeof(float) * (size_t)m->n_ctr * doc_count);
+            calc_ctrs_block(m, result, transposed_hash, doc_count, ctrs);
+            for (int i = 0; i < m->n_ctr; ++i) {
+                const float* v = ctrs + (size_t)i * doc_count;
+                const int32_t b0 = m->ctr_border_offsets[i], b1 = m->ctr_border_offsets[i + 1];
+                for (int32_t bs = b0; bs < b1; bs += CBO_MAX_VALUES_PER_BIN) {
+                    const int32_t be = (bs + CBO_MAX_VALUES_PER_BIN < b1) ? bs + CBO_MAX_VALUES_PER_BIN : b1;
+                    for (int32_t b = bs; b < be; ++b) {
+                        const float border = m->ctr_borders[b];
+                        for (size_t d = 0; d < doc_count; ++d) out[d] += (uint8_t)(v[d] > border);
+                    }
+                    out += doc_count;
+                }
+            }
+            free(ctrs);
+        }
     }
+}
+
+void cbo_calc_ctrs(const cbo_model* m, const cbo_features* f, size_t n_docs, float* out) {
+    if (m->n_ctr == 0) return;
+    uint8_t* bins = (uint8_t*)malloc((size_t)(m->bucket_count ? m->bucket_count : 1) * CBO_BLOCK);
+    uint32_t* th = (uint32_t*)malloc(sizeof(uint32_t) * CBO_BLOCK * (size_t)(m->used_cat ? m->used_cat : 1));
+    float* ctrs = (float*)malloc(sizeof(float) * (size_t)m->n_ctr * CBO_BLOCK);
+    for (size_t start = 0; start < n_docs; start += CBO_BLOCK) {
+        const size_t dc = n_docs - start < CBO_BLOCK ? n_docs - start : CBO_BLOCK;
+        binarize_block(m, f, start, dc, bins, th);
+        calc_ctrs_block(m, bins, th, dc, ctrs);
+        for (int i = 0; i < m->n_ctr; ++i)
+            for (size_t d = 0; d < dc; ++d) out[(size_t)i * n_docs + start + d] = ctrs[(size_t)i * dc + d];
+    }
+    free(bins); free(th); free(ctrs);
 }
 
 void cbo_binarize(const cbo_model* m, const cbo_features* f, size_t n_docs, uint8_t* bins) {
@@ -678,8 +968,36 @@ void cbo_calc_mt(const cbo_model* m, const cbo_features* f, size_t n_docs,
 /* Truth value of binary feature `bf` for one doc straight from its definition:
  * float split  <=> value > border after the NaN policy of quantization.h:375-409,
  * one-hot split <=> hashed value == Value (split.h:17-19). */
+static float raw_float(const cbo_model* m, const cbo_features* f, int feature, size_t doc) {
+    float v = get_float(m, f, feature, doc);
+    if (isnan(v) && m->ff_has_nans[feature] && m->ff_nan_treatment[feature] != CBO_NAN_AS_IS)
+        v = (m->ff_nan_treatment[feature] == CBO_NAN_AS_FALSE) ? -INFINITY : INFINITY;
+    return v;
+}
+
+/* CTR of one document from the raw features: the projection's hash folds the categorical hashes, then
+ * "value > border" per float split and "hash == value" per one-hot split (ctr_provider.h:64-78 with the
+ * bins replaced by what they stand for). */
+static float raw_ctr(const cbo_model* m, const cbo_features* f, int ctr, size_t doc) {
+    uint64_t h = 0;
+    for (int32_t i = m->ctr_cat_offsets[ctr]; i < m->ctr_cat_offsets[ctr + 1]; ++i) {
+        for (int c = 0; c < m->n_cat; ++c)
+            if (m->cf_index[c] == m->ctr_cats[i])
+                h = ctr_calc_hash(h, (uint64_t)(int64_t)(int32_t)get_cat(m, f, c, doc));
+    }
+    for (int32_t i = m->ctr_float_offsets[ctr]; i < m->ctr_float_offsets[ctr + 1]; ++i)
+        h = ctr_calc_hash(h, (uint64_t)(raw_float(m, f, m->ctr_float_raw[i], doc) > m->ctr_float_border[i]));
+    for (int32_t i = m->ctr_onehot_offsets[ctr]; i < m->ctr_onehot_offsets[ctr + 1]; ++i) {
+        for (int c = 0; c < m->n_cat; ++c)
+            if (m->cf_index[c] == m->ctr_onehot_cat[i])
+                h = ctr_calc_hash(h, (uint64_t)((int32_t)get_cat(m, f, c, doc) == m->ctr_onehot_value[i]));
+    }
+    return ctr_value(m, ctr, ctr_table_index(m, m->ctr_table[ctr], h));
+}
+
 static int raw_condition(const cbo_model* m, const cbo_features* f, int bf, size_t doc) {
     const cbo_bin_feature* b = &m->bin_features[bf];
+    if (b->is_ctr) return raw_ctr(m, f, b->feature, doc) > b->border;
     if (!b->is_onehot) {
         float v = get_float(m, f, b->feature, doc);
         if (isnan(v) && m->ff_has_nans[b->feature] && m->ff_nan_treatment[b->feature] != CBO_NAN_AS_IS)

@@ -62,6 +62,36 @@ typedef struct cbo_model_desc {
 
     double scale;
     const double* bias; /* approx_dim values */
+
+    /* CTR features in model order (features.h:306-323, online_ctr.h:108-316); n_ctr = 0 without them.
+     * A projection = categorical features (by feature Index), float splits (feature Index, border)
+     * and one-hot splits (cat feature Index, value). */
+    int32_t n_ctr;
+    const int32_t* ctr_border_offsets; /* n_ctr + 1 */
+    const float* ctr_borders;
+    const int32_t* ctr_cat_offsets; /* n_ctr + 1 */
+    const int32_t* ctr_cats;
+    const int32_t* ctr_float_offsets; /* n_ctr + 1 */
+    const int32_t* ctr_float_feature;
+    const float* ctr_float_border;
+    const int32_t* ctr_onehot_offsets; /* n_ctr + 1 */
+    const int32_t* ctr_onehot_cat;
+    const int32_t* ctr_onehot_value;
+    const int32_t* ctr_type; /* ECtrType, ctr_data.fbs:5-12 */
+    const int32_t* ctr_target_border_idx;
+    const float* ctr_prior_num;
+    const float* ctr_prior_denom;
+    const float* ctr_shift;
+    const float* ctr_scale;
+    const int32_t* ctr_table; /* value table of the CTR's base */
+    /* value tables of the static CTR provider (ctr_value_table.h:17-109) */
+    int32_t n_ctr_tables;
+    const uint64_t* table_bucket_offsets; /* n_ctr_tables + 1, counted in 12-byte buckets */
+    const uint8_t* table_buckets;         /* {u64 hash, u32 row} packed, dense_hash_view.h:12-26 */
+    const uint64_t* table_blob_offsets;   /* n_ctr_tables + 1, in bytes */
+    const uint8_t* table_blobs;
+    const int32_t* table_counter_denominator;
+    const int32_t* table_target_classes_count;
 } cbo_model_desc;
 
 typedef struct cbo_model cbo_model;
@@ -113,6 +143,10 @@ void cbo_calc_leaf_indexes(const cbo_model* m, const cbo_features* f, size_t n_d
  * raw (feature, border) / (cat feature, value) definition, one doc at a time. */
 void cbo_calc_bruteforce(const cbo_model* m, const cbo_features* f, size_t n_docs,
                          size_t tree_start, size_t tree_end, double* out, uint32_t* leaf_indexes);
+
+/* CTR values of the model's CTR features, out[ctr * n_docs + doc], computed per document from the
+ * raw features (TStaticCtrProvider::CalcCtrs, static_ctr_provider.cpp:14-131). */
+void cbo_calc_ctrs(const cbo_model* m, const cbo_features* f, size_t n_docs, float* out);
 
 /* CalcCatFeatureHash (catboost/libs/cat_feature/cat_feature.cpp:6-8). */
 uint64_t cbo_city_hash64(const char* s, size_t len);

@@ -96,6 +96,57 @@ class _Table:
         return out
 
 
+def _read_ctr_base(t):
+    """TModelCtrBase (ctr_data.fbs:15-19) with its TFeatureCombination (features.fbs:71-75)."""
+    base = {"cat_features": np.zeros(0, np.int32), "float_splits": [], "one_hot_splits": [],
+            "ctr_type": 0, "target_border_classifier_idx": 0}
+    if t is None:
+        return base
+    proj = t.table(0)
+    if proj is not None:
+        base["cat_features"] = proj.vector(0, np.int32)
+        raw = proj.vector(1, np.uint32, per_element=2).reshape(-1, 2)
+        base["float_splits"] = [(int(np.int32(r[0])), np.array([r[1]], np.uint32).view(np.float32)[0]) for r in raw]
+        raw = proj.vector(2, np.int32, per_element=2).reshape(-1, 2)
+        base["one_hot_splits"] = [(int(r[0]), int(r[1])) for r in raw]
+    base["ctr_type"] = t.scalar(1, "b", 0)
+    base["target_border_classifier_idx"] = t.scalar(2, "i", 0)
+    return base
+
+
+def ctr_base_key(base):
+    """Hashable identity of a TModelCtrBase (its operator==, online_ctr.h:182-186)."""
+    return (tuple(int(c) for c in base["cat_features"]),
+            tuple((f, np.float32(b).tobytes()) for f, b in base["float_splits"]),
+            tuple(base["one_hot_splits"]), int(base["ctr_type"]), int(base["target_border_classifier_idx"]))
+
+
+def _read_size(data, pos):
+    """LoadSize, util/ysaveload.h:277-296."""
+    (n,) = struct.unpack_from("<I", data, pos)
+    pos += 4
+    if n == 0xFFFFFFFF:
+        (n,) = struct.unpack_from("<Q", data, pos)
+        pos += 8
+    return n, pos
+
+
+def _read_static_ctr_provider(data, pos):
+    """TCtrData::Load (ctr_data.cpp:24-34): count, then (size, flatbuffer TCtrValueTable) per table."""
+    count, pos = _read_size(data, pos)
+    tables = []
+    for _ in range(count):
+        n, pos = _read_size(data, pos)
+        buf = data[pos:pos + n]
+        pos += n
+        (root,) = struct.unpack_from("<I", buf, 0)
+        t = _Table(buf, root)
+        tables.append({"base": _read_ctr_base(t.table(0)), "index_hash_raw": t.vector(1, np.uint8),
+                       "ctr_blob": t.vector(2, np.uint8), "counter_denominator": t.scalar(3, "i", 0),
+                       "target_classes_count": t.scalar(4, "i", 0)})
+    return tables, pos
+
+
 def read_cbm(data):
     """Parses .cbm bytes into a dict of numpy arrays (keys follow the flatbuffer field names)."""
     data = memoryview(bytes(data))
@@ -144,6 +195,14 @@ def read_cbm(data):
     model["float_features"] = floats
     model["one_hot_features"] = onehots
     model["ctr_feature_count"] = t.vector_len(7)
+    ctrs = []
+    for c in t.tables(7):  # TCtrFeature / TModelCtr, ctr_data.fbs:21-33
+        mc_ctr = c.table(0)
+        ctrs.append({"base": _read_ctr_base(mc_ctr.table(0)), "target_border_idx": mc_ctr.scalar(1, "i", 0),
+                     "prior_num": mc_ctr.scalar(2, "f", 0.0), "prior_denom": mc_ctr.scalar(3, "f", 1.0),
+                     "shift": mc_ctr.scalar(4, "f", 0.0), "scale": mc_ctr.scalar(5, "f", 1.0),
+                     "borders": c.vector(1, np.float32)})
+    model["ctr_features"] = ctrs
     model["leaf_values"] = t.vector(8, np.float64)
     model["leaf_weights"] = t.vector(9, np.float64)
     model["step_nodes"] = t.vector(10, np.uint16, per_element=2).reshape(-1, 2)
@@ -162,6 +221,14 @@ def read_cbm(data):
         model["bias"] = np.full(dim, bias, dtype=np.float64)
     model["repacked_bins_in_file"] = t.vector(17, np.uint32)
     model["embedding_feature_count"] = t.vector_len(18)
+    # trailing model parts, model.cpp:1201-1226; only the static CTR provider is read
+    model["ctr_tables"] = []
+    part_pos = pos + size
+    for part in parts:
+        if part != "static_provider_v1":
+            break
+        tables, part_pos = _read_static_ctr_provider(data, part_pos)
+        model["ctr_tables"] = tables
     return model
 
 

@@ -53,6 +53,31 @@ class _Desc(ctypes.Structure):
         ("node_id_to_leaf_id", ctypes.c_void_p),
         ("scale", ctypes.c_double),
         ("bias", ctypes.c_void_p),
+        ("n_ctr", ctypes.c_int32),
+        ("ctr_border_offsets", ctypes.c_void_p),
+        ("ctr_borders", ctypes.c_void_p),
+        ("ctr_cat_offsets", ctypes.c_void_p),
+        ("ctr_cats", ctypes.c_void_p),
+        ("ctr_float_offsets", ctypes.c_void_p),
+        ("ctr_float_feature", ctypes.c_void_p),
+        ("ctr_float_border", ctypes.c_void_p),
+        ("ctr_onehot_offsets", ctypes.c_void_p),
+        ("ctr_onehot_cat", ctypes.c_void_p),
+        ("ctr_onehot_value", ctypes.c_void_p),
+        ("ctr_type", ctypes.c_void_p),
+        ("ctr_target_border_idx", ctypes.c_void_p),
+        ("ctr_prior_num", ctypes.c_void_p),
+        ("ctr_prior_denom", ctypes.c_void_p),
+        ("ctr_shift", ctypes.c_void_p),
+        ("ctr_scale", ctypes.c_void_p),
+        ("ctr_table", ctypes.c_void_p),
+        ("n_ctr_tables", ctypes.c_int32),
+        ("table_bucket_offsets", ctypes.c_void_p),
+        ("table_buckets", ctypes.c_void_p),
+        ("table_blob_offsets", ctypes.c_void_p),
+        ("table_blobs", ctypes.c_void_p),
+        ("table_counter_denominator", ctypes.c_void_p),
+        ("table_target_classes_count", ctypes.c_void_p),
     ]
 
 
@@ -86,6 +111,7 @@ def _load():
         lib.cbo_binarize.argtypes = [ctypes.c_void_p, ctypes.POINTER(_Features), ctypes.c_size_t, ctypes.c_void_p]
         lib.cbo_calc.argtypes = [ctypes.c_void_p, ctypes.POINTER(_Features), ctypes.c_size_t,
                                  ctypes.c_size_t, ctypes.c_size_t, ctypes.c_void_p]
+        lib.cbo_calc_ctrs.argtypes = [ctypes.c_void_p, ctypes.POINTER(_Features), ctypes.c_size_t, ctypes.c_void_p]
         lib.cbo_calc_mt.argtypes = lib.cbo_calc.argtypes + [ctypes.c_int]
         lib.cbo_calc_leaf_indexes.argtypes = lib.cbo_calc.argtypes
         lib.cbo_calc_bruteforce.argtypes = lib.cbo_calc.argtypes + [ctypes.c_void_p]
@@ -208,6 +234,51 @@ class OracleModel:
         d.node_id_to_leaf_id = _p(arr(model["node_id_to_leaf_id"], np.uint32))
         d.scale = float(model["scale"])
         d.bias = _p(arr(model["bias"], np.float64))
+        ctrs = model.get("ctr_features", [])
+        tables = model.get("ctr_tables", [])
+        d.n_ctr = len(ctrs)
+        d.n_ctr_tables = len(tables)
+        if ctrs:
+            from .cbm_reader import ctr_base_key
+            table_of = {ctr_base_key(t["base"]): i for i, t in enumerate(tables)}
+
+            def offsets(lengths):
+                return np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+
+            def concat(parts, dtype):
+                parts = [np.asarray(p, dtype=dtype).ravel() for p in parts]
+                return np.concatenate(parts) if parts else np.zeros(0, dtype)
+
+            d.ctr_border_offsets = _p(arr(offsets([len(c["borders"]) for c in ctrs]), np.int32))
+            d.ctr_borders = _p(arr(concat([c["borders"] for c in ctrs], np.float32), np.float32))
+            d.ctr_cat_offsets = _p(arr(offsets([len(c["base"]["cat_features"]) for c in ctrs]), np.int32))
+            d.ctr_cats = _p(arr(concat([c["base"]["cat_features"] for c in ctrs], np.int32), np.int32))
+            d.ctr_float_offsets = _p(arr(offsets([len(c["base"]["float_splits"]) for c in ctrs]), np.int32))
+            d.ctr_float_feature = _p(arr(concat([[f for f, _ in c["base"]["float_splits"]] for c in ctrs], np.int32),
+                                         np.int32))
+            d.ctr_float_border = _p(arr(concat([[b for _, b in c["base"]["float_splits"]] for c in ctrs], np.float32),
+                                        np.float32))
+            d.ctr_onehot_offsets = _p(arr(offsets([len(c["base"]["one_hot_splits"]) for c in ctrs]), np.int32))
+            d.ctr_onehot_cat = _p(arr(concat([[f for f, _ in c["base"]["one_hot_splits"]] for c in ctrs], np.int32),
+                                      np.int32))
+            d.ctr_onehot_value = _p(arr(concat([[v for _, v in c["base"]["one_hot_splits"]] for c in ctrs], np.int32),
+                                        np.int32))
+            d.ctr_type = _p(arr([c["base"]["ctr_type"] for c in ctrs], np.int32))
+            d.ctr_target_border_idx = _p(arr([c["target_border_idx"] for c in ctrs], np.int32))
+            d.ctr_prior_num = _p(arr([c["prior_num"] for c in ctrs], np.float32))
+            d.ctr_prior_denom = _p(arr([c["prior_denom"] for c in ctrs], np.float32))
+            d.ctr_shift = _p(arr([c["shift"] for c in ctrs], np.float32))
+            d.ctr_scale = _p(arr([c["scale"] for c in ctrs], np.float32))
+            d.ctr_table = _p(arr([table_of.get(ctr_base_key(c["base"]), -1) for c in ctrs], np.int32))
+            bucket_off = np.concatenate([[0], np.cumsum([len(t["index_hash_raw"]) // 12 for t in tables])])
+            blob_off = np.concatenate([[0], np.cumsum([len(t["ctr_blob"]) for t in tables])])
+            d.table_bucket_offsets = _p(arr(bucket_off, np.uint64))
+            d.table_buckets = _p(arr(concat([t["index_hash_raw"] for t in tables], np.uint8), np.uint8))
+            d.table_blob_offsets = _p(arr(blob_off, np.uint64))
+            d.table_blobs = _p(arr(concat([t["ctr_blob"] for t in tables], np.uint8), np.uint8))
+            d.table_counter_denominator = _p(arr([t["counter_denominator"] for t in tables], np.int32))
+            d.table_target_classes_count = _p(arr([t["target_classes_count"] for t in tables], np.int32))
+        self.ctr_count = len(ctrs)
         err = ctypes.create_string_buffer(512)
         self._h = lib.cbo_model_create(ctypes.byref(d), err, 512)
         if not self._h:
@@ -279,6 +350,13 @@ class OracleModel:
         else:
             self._lib.cbo_calc(self._h, ctypes.byref(f), n, tree_start, tree_end, _p(out))
         return out
+
+    def ctrs(self, floats, cats=None, layout="flat"):
+        """CTR values, one row per CTR feature of the model."""
+        f, n = self._features(floats, cats, layout)
+        out = np.zeros(max(self.ctr_count * n, 1), dtype=np.float32)
+        self._lib.cbo_calc_ctrs(self._h, ctypes.byref(f), n, _p(out))
+        return out[:self.ctr_count * n].reshape(self.ctr_count, n)
 
     def binarize(self, floats, cats=None, layout="flat"):
         """Bins in the reference layout: [block of 128][bucket][doc in block], flattened."""

@@ -152,3 +152,108 @@ def load_boston(golden_dir):
             feats.append([float(x) for x in tok[:-1]])
             target.append(float(tok[-1]))
     return np.asarray(feats, np.float32), np.asarray(target)
+
+
+# ---- models with CTR (target statistics) features ------------------------------------------
+# categoric_only_model.cbm, CatBoostModelTest.java:528-547 (three categorical features, strings)
+JVM_CATEGORIC_ONLY_CATS = [["a", "d", "g"], ["b", "e", "h"], ["c", "f", "k"]]
+JVM_CATEGORIC_ONLY_EXPECTED = np.array([0.04146251510837989, 0.015486266021159064, 0.04146251510837989])
+# model.cbm of the JVM tests (here jvm_model_with_ctr.cbm), CatBoostModelTest.java:720-743
+JVM_CTR_FLOATS = np.array([[0.5, 1.5], [0.7, 6.4], [-2.0, -1.0]], np.float32)
+JVM_CTR_CATS = JVM_CATEGORIC_ONLY_CATS
+JVM_CTR_EXPECTED = np.array([0.04666924366060905, 0.026244613740247648, 0.03094452158737013])
+# features_num_cat__dataset_adult.cbm, rust-package/src/model.rs:459-499 (tolerance there: 1e-6)
+RUST_ADULT_FLOATS = np.array([[44.0, 403782.0, 11.0, 0.0, 0.0, 45.0], [19.0, 208874.0, 10.0, 0.0, 0.0, 40.0],
+                              [27.0, 158647.0, 10.0, 0.0, 0.0, 40.0], [18.0, 115258.0, 6.0, 0.0, 0.0, 40.0]], np.float32)
+RUST_ADULT_CATS = [["0", "n", "1", "Private", "Assoc-voc", "Divorced", "Sales", "Not-in-family", "White", "Male",
+                    "United-States"]] * 4
+RUST_ADULT_EXPECTED = np.array([0.9876043724015489, 0.9869589576174197, 0.997648058191363, 1.0147797830459155])
+# node-package/test_data/adult.cbm (here node_adult.cbm), node-package/bindings/tests/model.ts:67-96:
+# predictions printed with two decimals
+NODE_ADULT_FLOATS = np.array([[40., 85019., 16., 0., 0., 45.], [28., 85019., 13., 0., 0., 13.]], np.float32)
+NODE_ADULT_CATS = [["Private", "Doctorate", "Married-civ-spouce", "Prof-specialty", "Husband", "Asian-Pac-Islander",
+                    "Male", "nan"],
+                   ["Self-emp-not-inc", "Bachelors", "Married-civ-spouce", "Exec-managerial", "Husband", "White", "Male",
+                    "United-States"]]
+NODE_ADULT_EXPECTED_2DP = ["1.54", "-1.17"]
+
+
+def mushrooms(golden_dir):
+    """mushrooms.csv of the .NET tests (CatBoostModelEvaluatorTest.cs:101-127): label, then 22 categorical
+    features; the model's raw prediction is positive exactly for label "p"."""
+    import os
+    labels, rows = [], []
+    with open(os.path.join(golden_dir, "mushrooms.csv")) as f:
+        for line in f:
+            parts = line.strip().split(",")
+            if len(parts) == 23:
+                labels.append(parts[0])
+                rows.append(parts[1:])
+    return labels, rows
+
+
+CTR_FIXTURES = ["categoric_only_model.cbm", "jvm_model_with_ctr.cbm", "features_num_cat__dataset_adult.cbm",
+                "node_adult.cbm", "mushroom_model.cbm", "cloudness_small.cbm"]
+
+
+def random_ctr_inputs(model, docs, seed, known_cats=None):
+    """Random documents for a model dict with CTR features: floats around the model's borders and
+    categorical hashes drawn from the hashes the CTR tables know (plus unknown ones)."""
+    rng = np.random.default_rng(seed)
+    ffs, cfs = model["float_features"], model["cat_features"]
+    n_float = max([f["index"] for f in ffs], default=-1) + 1
+    n_cat = max([c["index"] for c in cfs], default=-1) + 1
+    floats = rng.normal(size=(docs, n_float)).astype(np.float32)
+    for f in ffs:
+        b = np.asarray(f["borders"], np.float32)
+        if b.size:
+            pick = b[rng.integers(0, b.size, size=docs)]
+            jitter = rng.choice(np.array([-1.0, 0.0, 1.0], np.float32), size=docs) * np.abs(pick) * 1e-3
+            floats[:, f["index"]] = pick + jitter.astype(np.float32)
+    cats = rng.integers(-2 ** 31, 2 ** 31, size=(docs, n_cat), dtype=np.int64).astype(np.int32)
+    if known_cats is not None:
+        for c in cfs:
+            pool = known_cats.get(c["index"])
+            if pool is not None and len(pool):
+                use = rng.random(docs) < 0.9
+                cats[use, c["index"]] = np.asarray(pool, np.int32)[rng.integers(0, len(pool), size=int(use.sum()))]
+    return floats, cats
+
+
+def known_cat_hashes(model):
+    """Per categorical feature index: hashed values its single-feature CTR tables have rows for. A table
+    key of such a projection is MAGIC * (0 + MAGIC * (u64)(i32)hash) (catboost/libs/model/hash.h:11-14);
+    MAGIC is odd, so the key is inverted modulo 2^64."""
+    magic = 0x4906ba494954cb65
+    inv = pow(magic, -1, 1 << 64)
+    inv2 = (inv * inv) % (1 << 64)
+    out = {}
+    for table in model.get("ctr_tables", []):
+        base = table["base"]
+        if len(base["cat_features"]) != 1 or base["float_splits"] or base["one_hot_splits"]:
+            continue
+        raw = np.asarray(table["index_hash_raw"], np.uint8).reshape(-1, 12)
+        keys = raw[:, :8].copy().view(np.uint64).ravel()
+        values = []
+        for key in keys:
+            if int(key) == 0xFFFFFFFFFFFFFFFF:
+                continue
+            v = (int(key) * inv2) % (1 << 64)
+            if v >= 1 << 63:
+                v -= 1 << 64
+            if -2 ** 31 <= v < 2 ** 31:
+                values.append(v)
+        out.setdefault(int(base["cat_features"][0]), set()).update(values)
+    return {k: sorted(v) for k, v in out.items()}
+
+
+def flat_rows(model, floats, cats):
+    """[doc][flat feature index] rows from split float / hashed categorical matrices (hashes bit-cast)."""
+    ffs, cfs = model["float_features"], model["cat_features"]
+    width = max([f["flat_index"] for f in ffs] + [c["flat_index"] for c in cfs], default=-1) + 1
+    flat = np.zeros((floats.shape[0] if floats.size or not len(cats) else cats.shape[0], width), np.float32)
+    for f in ffs:
+        flat[:, f["flat_index"]] = floats[:, f["index"]]
+    for c in cfs:
+        flat[:, c["flat_index"]] = np.ascontiguousarray(cats[:, c["index"]]).view(np.float32)
+    return flat

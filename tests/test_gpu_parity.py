@@ -146,6 +146,98 @@ def test_rust_fixture_with_one_hot_string_cats(golden_dir):
     np.testing.assert_array_equal(g.quantize_hashed(rm.RUST_FLOATS, hashed), o.binarize(rm.RUST_FLOATS, hashed, layout="split"))
 
 
+# -------------------------------------------------------- CTR (target statistics) features ----
+
+def _hashed(rows):
+    return np.array([[cb.string_cat_feature_hash(c) for c in row] for row in rows], np.int32)
+
+
+def test_ctr_goldens_of_the_jvm_tests(golden_dir):
+    # CatBoostModelTest.java:457-470, 528-547, 586-601, 720-743; the reference's CUDA evaluator refuses
+    # both models (cuda/evaluator.cpp:22-28)
+    g = cb.ModelCalcer(os.path.join(golden_dir, "categoric_only_model.cbm"))
+    none = np.zeros((3, 0), np.float32)
+    _close(g.calc(none, rm.JVM_CATEGORIC_ONLY_CATS), rm.JVM_CATEGORIC_ONLY_EXPECTED)
+    _close(g.calc_single(none[0], rm.JVM_CATEGORIC_ONLY_CATS[0]), rm.JVM_CATEGORIC_ONLY_EXPECTED[:1])
+    _close(g.calc_hashed(none, _hashed(rm.JVM_CATEGORIC_ONLY_CATS)), rm.JVM_CATEGORIC_ONLY_EXPECTED)
+    with pytest.raises(cb.CatBoostError):
+        g.calc(none, [row[:2] for row in rm.JVM_CATEGORIC_ONLY_CATS])  # :508-524, too few categorical features
+    g = cb.ModelCalcer(os.path.join(golden_dir, "jvm_model_with_ctr.cbm"))
+    _close(g.calc(rm.JVM_CTR_FLOATS, rm.JVM_CTR_CATS), rm.JVM_CTR_EXPECTED)
+    _close(g.calc_single(rm.JVM_CTR_FLOATS[0], rm.JVM_CTR_CATS[0]), rm.JVM_CTR_EXPECTED[:1])
+
+
+def test_ctr_goldens_of_the_rust_and_node_tests(golden_dir):
+    g = cb.ModelCalcer(os.path.join(golden_dir, "features_num_cat__dataset_adult.cbm"))
+    _close(g.calc(rm.RUST_ADULT_FLOATS, rm.RUST_ADULT_CATS), rm.RUST_ADULT_EXPECTED)
+    g = cb.ModelCalcer(os.path.join(golden_dir, "node_adult.cbm"))
+    assert ["%.2f" % v for v in g.calc(rm.NODE_ADULT_FLOATS, rm.NODE_ADULT_CATS)] == rm.NODE_ADULT_EXPECTED_2DP
+
+
+def test_ctr_mushroom_labels(golden_dir):
+    # CatBoostModelEvaluatorTest.cs:101-127
+    g = cb.ModelCalcer(os.path.join(golden_dir, "mushroom_model.cbm"))
+    labels, rows = rm.mushrooms(golden_dir)
+    pred = g.calc(np.zeros((len(rows), 0), np.float32), rows)
+    np.testing.assert_array_equal(pred > 0, np.array(labels) == "p")
+    o = OracleModel(read_cbm_file(os.path.join(golden_dir, "mushroom_model.cbm")))
+    _close(pred, o.calc(np.zeros((len(rows), 0), np.float32), _hashed(rows), layout="split"))
+
+
+@pytest.mark.parametrize("name", rm.CTR_FIXTURES)
+@pytest.mark.parametrize("docs", [1, 257, 5000])
+def test_ctr_models_against_the_oracle(golden_dir, name, docs):
+    """Random documents (known and unknown categories, floats on and around the borders) through the
+    hashed, flat and transposed host entry points: bins bit-exact, predictions within the bar."""
+    path = os.path.join(golden_dir, name)
+    m = read_cbm_file(path)
+    o = OracleModel(m)
+    g = cb.ModelCalcer(path)
+    floats, cats = rm.random_ctr_inputs(m, docs, 100 + docs, rm.known_cat_hashes(m))
+    expected = o.calc(floats, cats, layout="split")
+    np.testing.assert_array_equal(g.quantize_hashed(floats, cats), o.binarize(floats, cats, layout="split"))
+    _close(g.calc_hashed(floats, cats), expected)
+    flat = rm.flat_rows(m, floats, cats)
+    np.testing.assert_array_equal(g.quantize_flat(flat), o.binarize(flat))
+    _close(g.calc_flat(flat), expected)
+    _close(g.calc_flat_transposed(np.ascontiguousarray(flat.T)), expected)
+    np.testing.assert_array_equal(g.calc_leaf_indexes_flat(flat), o.leaf_indexes(flat))
+    half = o.tree_count // 2
+    _close(g.calc_flat(flat, tree_start=half, tree_end=o.tree_count),
+           o.calc(flat, tree_start=half, tree_end=o.tree_count))
+
+
+def test_ctr_model_on_the_device_path(golden_dir):
+    """The device entry points (features already in HBM) on the adult model, 200 000 documents."""
+    import torch
+
+    path = os.path.join(golden_dir, "features_num_cat__dataset_adult.cbm")
+    m = read_cbm_file(path)
+    o = OracleModel(m)
+    g = cb.ModelCalcer(path)
+    ev = g.evaluator()
+    docs = 200_000
+    floats, cats = rm.random_ctr_inputs(m, docs, 5, rm.known_cat_hashes(m))
+    flat = rm.flat_rows(m, floats, cats)
+    x = torch.from_numpy(flat).to("cuda:0")
+    f = torch.from_numpy(floats).to("cuda:0")
+    c = torch.from_numpy(cats).to("cuda:0")
+    out = torch.zeros(docs, dtype=torch.float64, device="cuda:0")
+    out2 = torch.zeros_like(out)
+    bins = torch.zeros(ev.quantized_bytes(docs), dtype=torch.uint8, device="cuda:0")
+    exported = torch.zeros(docs * ev.bucket_count, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    ev.eval_data(ev.features(cb.LAYOUT_FLAT_ROWS, x.data_ptr(), x.shape[1]), docs, out.data_ptr())
+    split = ev.features(cb.LAYOUT_SPLIT_ROWS, f.data_ptr(), f.shape[1], c.data_ptr(), c.shape[1])
+    ev.quantize(split, docs, bins.data_ptr())
+    ev.eval_quantized(bins.data_ptr(), docs, out2.data_ptr())
+    ev.export_quantized(bins.data_ptr(), docs, exported.data_ptr())
+    ev.synchronize()
+    assert torch.equal(out, out2)
+    _close(out.cpu().numpy(), o.calc(flat, threads=8))
+    np.testing.assert_array_equal(exported.cpu().numpy(), o.binarize(flat))
+
+
 def test_querywise_fixture(golden_dir):
     g = cb.ModelCalcer(os.path.join(golden_dir, "features_num__dataset_querywise.cbm"))
     np.testing.assert_allclose(g.calc_flat(rm.querywise_rows()), rm.QUERYWISE_EXPECTED, rtol=1e-12, atol=1e-15)
@@ -405,9 +497,8 @@ def test_error_paths(golden_dir):
         g.enable_gpu_evaluation(99)
     with pytest.raises(cb.CatBoostError, match="Incorrect model file descriptor"):
         cb.ModelCalcer(os.path.join(golden_dir, "not_a_model.cbm"))
-    for name in ("categoric_only_model.cbm", "jvm_model_with_ctr.cbm", "cloudness_small.cbm"):
-        with pytest.raises(cb.CatBoostError, match="not supported"):
-            cb.ModelCalcer(os.path.join(golden_dir, name))
+    with pytest.raises(cb.CatBoostError, match="not supported"):
+        cb.ModelCalcer(os.path.join(golden_dir, "jvm_model_with_text_features.cbm"))
     # the handle still works after failed calls
     _close(g.calc_flat(rm.NUMERIC_ONLY_ROWS), rm.NUMERIC_ONLY_EXPECTED)
 

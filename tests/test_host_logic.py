@@ -123,9 +123,41 @@ def test_loader_rejects_bad_input(golden_dir):
             cb.ModelCalcer(buffer=bytes(corrupted))
         except cb.CatBoostError:
             pass
-    for name in ("categoric_only_model.cbm", "jvm_model_with_ctr.cbm", "cloudness_small.cbm"):
-        with pytest.raises(cb.CatBoostError, match="not supported"):
-            cb.ModelCalcer(os.path.join(golden_dir, name))
+    # text features stay out of reach: the model part that carries their dictionaries is refused
+    with pytest.raises(cb.CatBoostError, match="not supported"):
+        cb.ModelCalcer(os.path.join(golden_dir, "jvm_model_with_text_features.cbm"))
+
+
+def test_loader_reads_ctr_models(golden_dir):
+    """Models with CTR features and the tables of their static CTR provider load; the counts are those
+    the reference's binding tests expect (node-package/bindings/tests/model.ts:329-343)."""
+    adult = cb.ModelCalcer(os.path.join(golden_dir, "node_adult.cbm"))
+    assert adult.float_features_count == 6 and adult.cat_features_count == 8
+    for name in rm.CTR_FIXTURES:
+        m = cb.ModelCalcer(os.path.join(golden_dir, name))
+        expected = read_cbm_file(os.path.join(golden_dir, name))
+        borders = sum(len(f["borders"]) for f in expected["float_features"])
+        buckets = sum((len(f["borders"]) + 253) // 254 for f in expected["float_features"]) + \
+            sum((len(o["values"]) + 253) // 254 for o in expected["one_hot_features"]) + \
+            sum((len(c["borders"]) + 253) // 254 for c in expected["ctr_features"])
+        assert m.bucket_count == buckets and m.tree_count == len(expected["tree_sizes"]) and borders >= 0
+        with pytest.raises(cb.CatBoostError, match="CTR"):
+            m.save_to_buffer()
+    # a damaged CTR part fails cleanly (or loads), and never crashes
+    data = open(os.path.join(golden_dir, "jvm_model_with_ctr.cbm"), "rb").read()
+    core = int.from_bytes(data[4:8], "little")
+    for cut in (8 + core, 8 + core + 3, 8 + core + 4, 8 + core + 9, len(data) - 1):
+        with pytest.raises(cb.CatBoostError):
+            cb.ModelCalcer(buffer=data[:cut])
+    rng = np.random.default_rng(2)
+    for _ in range(300):
+        corrupted = bytearray(data)
+        for pos in rng.integers(8 + core, len(data), size=3):
+            corrupted[pos] = int(rng.integers(0, 256))
+        try:
+            cb.ModelCalcer(buffer=bytes(corrupted))
+        except cb.CatBoostError:
+            pass
 
 
 def test_oblivious_builder_matches_oracle_builder():

@@ -215,10 +215,66 @@ def test_boston_fixture(golden_dir):
     assert int(np.sum(np.abs(pred - np.log(target)) >= 0.4)) <= 7
 
 
-@pytest.mark.parametrize("name", ["categoric_only_model.cbm", "jvm_model_with_ctr.cbm", "cloudness_small.cbm"])
+@pytest.mark.parametrize("name", rm.CTR_FIXTURES)
 def test_ctr_fixtures_are_recognised(golden_dir, name):
     m = read_cbm_file(os.path.join(golden_dir, name))
     assert m["ctr_feature_count"] > 0 and "static_provider_v1" in m["model_part_ids"]
+    assert len(m["ctr_features"]) == m["ctr_feature_count"] and len(m["ctr_tables"]) > 0
+
+
+def _hashed(rows):
+    return np.array([[cat_feature_hash_signed(s) for s in r] for r in rows], np.int32)
+
+
+def test_ctr_goldens_of_the_jvm_tests(golden_dir):
+    # CatBoostModelTest.java:457-470, 528-547 (categorical features only) and :586-601, 720-743
+    o = OracleModel(read_cbm_file(os.path.join(golden_dir, "categoric_only_model.cbm")))
+    cats = _hashed(rm.JVM_CATEGORIC_ONLY_CATS)
+    np.testing.assert_array_equal(o.calc(np.zeros((3, 0), np.float32), cats, layout="split"),
+                                  rm.JVM_CATEGORIC_ONLY_EXPECTED)
+    o = OracleModel(read_cbm_file(os.path.join(golden_dir, "jvm_model_with_ctr.cbm")))
+    np.testing.assert_array_equal(o.calc(rm.JVM_CTR_FLOATS, _hashed(rm.JVM_CTR_CATS), layout="split"),
+                                  rm.JVM_CTR_EXPECTED)
+
+
+def test_ctr_goldens_of_the_rust_and_node_tests(golden_dir):
+    # rust-package/src/model.rs:459-499: 26 CTRs of kinds Borders and Counter plus a one-hot feature
+    o = OracleModel(read_cbm_file(os.path.join(golden_dir, "features_num_cat__dataset_adult.cbm")))
+    pred = o.calc(rm.RUST_ADULT_FLOATS, _hashed(rm.RUST_ADULT_CATS), layout="split")
+    np.testing.assert_allclose(pred, rm.RUST_ADULT_EXPECTED, rtol=0, atol=1e-15)
+    # node-package/bindings/tests/model.ts:67-96
+    o = OracleModel(read_cbm_file(os.path.join(golden_dir, "node_adult.cbm")))
+    pred = o.calc(rm.NODE_ADULT_FLOATS, _hashed(rm.NODE_ADULT_CATS), layout="split")
+    assert ["%.2f" % v for v in pred] == rm.NODE_ADULT_EXPECTED_2DP
+
+
+def test_ctr_mushroom_labels(golden_dir):
+    # CatBoostModelEvaluatorTest.cs:101-127: 159 CTRs over one to four categorical features, some with a
+    # one-hot split in the projection; every one of the 8124 rows must get its label
+    o = OracleModel(read_cbm_file(os.path.join(golden_dir, "mushroom_model.cbm")))
+    labels, rows = rm.mushrooms(golden_dir)
+    assert len(rows) == 8124
+    pred = o.calc(np.zeros((len(rows), 0), np.float32), _hashed(rows), layout="split")
+    np.testing.assert_array_equal(pred > 0, np.array(labels) == "p")
+
+
+@pytest.mark.parametrize("name", rm.CTR_FIXTURES)
+def test_ctr_models_against_the_raw_definition(golden_dir, name):
+    """The block-wise path (bins of the projection's splits, transposed hashes) against a per-document
+    evaluation from the raw features, in all three input layouts."""
+    m = read_cbm_file(os.path.join(golden_dir, name))
+    o = OracleModel(m)
+    floats, cats = rm.random_ctr_inputs(m, 1500, 7, rm.known_cat_hashes(m))
+    pred = o.calc(floats, cats, layout="split")
+    bf, bf_idx = o.bruteforce(floats, cats, layout="split")
+    np.testing.assert_array_equal(pred, bf)
+    np.testing.assert_array_equal(o.leaf_indexes(floats, cats, layout="split"), bf_idx)
+    flat = rm.flat_rows(m, floats, cats)
+    np.testing.assert_array_equal(o.calc(flat), pred)
+    np.testing.assert_array_equal(o.calc(np.ascontiguousarray(flat.T), layout="transposed"), pred)
+    # known and unknown categories both occur
+    ctrs = o.ctrs(floats, cats, layout="split")
+    assert all(len(np.unique(row)) > 1 for row in ctrs)
 
 
 def test_not_a_model_is_rejected(golden_dir):
