@@ -66,8 +66,8 @@ CATBOOST_API ModelCalcerHandle* ModelCalcerCreate(void);            /* c_api.h:6
 CATBOOST_API void ModelCalcerDelete(ModelCalcerHandle* modelHandle); /* c_api.h:74 */
 CATBOOST_API const char* GetErrorString(void);                      /* c_api.h:84 */
 
-/* ---- model loading: .cbm files / buffers ("CBM1" + flatbuffer). Models with CTR, text or
- * embedding features are refused with an error. */
+/* ---- model loading: .cbm files / buffers ("CBM1" + flatbuffer + the tables of the static CTR
+ * provider). Models with text or embedding features are refused with an error. */
 CATBOOST_API bool LoadFullModelFromFile(ModelCalcerHandle* modelHandle, const char* filename); /* c_api.h:92 */
 CATBOOST_API bool LoadFullModelFromBuffer(ModelCalcerHandle* modelHandle, const void* binaryBuffer, size_t binaryBufferSize); /* c_api.h:103 */
 /* The tables are copied to the GPU, so nothing points into the caller's buffer after return. */

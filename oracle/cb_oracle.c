@@ -13,6 +13,9 @@
  *   cat feature hash     catboost/libs/cat_feature/cat_feature.cpp:6-8, util/digest/city.cpp:58-200
  *   prediction types     catboost/libs/model/eval_processing.h:15-99, 174-240,
  *                        contrib/libs/fmath/fmath.hpp:150-185, 474-512, 565-648 (the exponent)
+ *   CTR features         catboost/libs/model/static_ctr_provider.cpp:14-178, ctr_provider.h:64-123,
+ *                        online_ctr.h:290-293, hash.h:11-14, catboost/libs/helpers/dense_hash_view.h:46-56,
+ *                        cpu/quantization.h:263-327
  *
  * Pinned by (see tests/test_oracle.py, tests/test_ref_vectors.py): the reference's own
  * standalone evaluator and its own fmath exponent, both built from the reference tree by
@@ -20,10 +23,16 @@
  * (catboost/libs/model/ut/formula_evaluator_ut.cpp:76-146, 284-307), the .cbm fixtures with
  * golden predictions of the JVM / Rust / .NET binding tests, the JVM hash known answers, the
  * numpy searchsorted invariant for binarize, the oblivious -> non-symmetric equivalence and the
- * raw-split brute force below.
+ * raw-split brute force below. CTR features: the golden predictions of the JVM, Rust and node
+ * binding tests for models with CTRs of kinds Borders and Counter (reproduced to the last bit) and
+ * the .NET mushroom test (8124 labels; projections of up to four categorical features, some with
+ * a one-hot split).
  * Parity unpinned (followed by reading only, cross-checked by the brute force): the NaN gating
  * "HasNans && treatment != AsIs", >254-border buckets combined with one-hot XorMask, and the
- * leaf numbering of non-symmetric multi-dimensional models.
+ * leaf numbering of non-symmetric multi-dimensional models; for CTRs the kinds Buckets,
+ * BinarizedTargetMeanValue, FloatTargetMeanValue and FeatureFreq, float splits inside a projection
+ * and the Borders branch for more than two target classes (the cloudness fixture has such CTRs
+ * but no reference output): no fixture with reference outputs covers them.
  */
 #include "cb_oracle.h"
 
