@@ -146,6 +146,7 @@ def load_library():
         "CbHipEvalData": (ctypes.c_bool, [vp, ctypes.POINTER(DeviceFeatures), sz, sz, sz, vp, vp]),
         "CbHipLeafIndexesQuantized": (ctypes.c_bool, [vp, vp, sz, sz, sz, vp, vp]),
         "CbHipExportQuantized": (ctypes.c_bool, [vp, vp, sz, vp, vp]),
+        "CbHipApplyPredictionTypeDevice": (ctypes.c_bool, [vp, ctypes.c_int, sz, vp, vp, vp]),
         "CbHipSynchronize": (ctypes.c_bool, [vp, vp]),
         "CbHipLastKernelTimes": (ctypes.c_bool, [vp, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float)]),
         "CbHipGetEvaluator": (vp, [vp]),
@@ -369,6 +370,11 @@ class DeviceEvaluator:
 
     def export_quantized(self, bins_ptr, doc_count, out_ptr, stream=None):
         _check(self._lib.CbHipExportQuantized(self._h, bins_ptr, doc_count, out_ptr, stream))
+
+    def apply_prediction_type(self, prediction_type, doc_count, raw_ptr, result_ptr, stream=None):
+        """Raw formula values on the device -> a prediction type (an APT_* constant)."""
+        kind = int(prediction_type)
+        _check(self._lib.CbHipApplyPredictionTypeDevice(self._h, kind, doc_count, raw_ptr, result_ptr, stream))
 
     def synchronize(self, stream=None):
         _check(self._lib.CbHipSynchronize(self._h, stream))

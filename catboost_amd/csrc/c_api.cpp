@@ -162,26 +162,20 @@ void PostProcess(EApiPredictionType type, size_t dim, size_t docCount, const dou
     }
 }
 
-// Runs `rawCalc(double* raw)` and applies the prediction type of the handle.
+// Runs `calc(double* result, int predictionType)`: the evaluator applies the handle's prediction type on
+// the device before it copies the results back.
 template <typename F>
-void CalcWithPredictionType(TModelHandle& h, size_t docCount, double* result, size_t resultSize, F&& rawCalc) {
+void CalcWithPredictionType(TModelHandle& h, size_t docCount, double* result, size_t resultSize, F&& calc) {
     CheckResultSize(h, docCount, resultSize);
-    const size_t dim = static_cast<size_t>(h.Model.Trees.ApproxDimension);
-    if (h.PredictionType == APT_RAW_FORMULA_VAL) {
-        rawCalc(result);
-        return;
-    }
-    std::vector<double> raw(docCount * dim);
-    rawCalc(raw.data());
-    PostProcess(h.PredictionType, dim, docCount, raw.data(), result);
+    calc(result, static_cast<int>(h.PredictionType));
 }
 
 void CalcFlatImpl(void* modelHandle, size_t docCount, size_t treeStart, size_t treeEnd, const float** floatFeatures,
                   size_t floatFeaturesSize, double* result, size_t resultSize) {
     TModelHandle& h = *H(modelHandle);
-    CalcWithPredictionType(h, docCount, result, resultSize, [&](double* raw) {
+    CalcWithPredictionType(h, docCount, result, resultSize, [&](double* out, int predictionType) {
         h.GetEvaluator().CalcHostRows(floatFeatures, floatFeaturesSize, /*flat*/ true, nullptr, 0, docCount, treeStart,
-                                      treeEnd, raw);
+                                      treeEnd, out, predictionType);
     });
 }
 
@@ -190,10 +184,10 @@ void CalcHashedImpl(void* modelHandle, size_t docCount, size_t treeStart, size_t
                     size_t resultSize) {
     TModelHandle& h = *H(modelHandle);
     static_assert(sizeof(int) == sizeof(int32_t), "int must be 32 bits");
-    CalcWithPredictionType(h, docCount, result, resultSize, [&](double* raw) {
+    CalcWithPredictionType(h, docCount, result, resultSize, [&](double* out, int predictionType) {
         h.GetEvaluator().CalcHostRows(floatFeaturesSize ? floatFeatures : nullptr, floatFeaturesSize, /*flat*/ false,
                                       catFeaturesSize ? reinterpret_cast<const int32_t* const*>(catFeatures) : nullptr,
-                                      catFeaturesSize, docCount, treeStart, treeEnd, raw);
+                                      catFeaturesSize, docCount, treeStart, treeEnd, out, predictionType);
     });
 }
 
@@ -470,8 +464,9 @@ bool CalcModelPredictionFlatTransposedStaged(ModelCalcerHandle* modelHandle, siz
                                              double* result, size_t resultSize) {
     return Guard([&] {
         TModelHandle& h = *H(modelHandle);
-        CalcWithPredictionType(h, docCount, result, resultSize, [&](double* raw) {
-            h.GetEvaluator().CalcHostColumns(floatFeatures, floatFeaturesSize, docCount, treeStart, treeEnd, raw);
+        CalcWithPredictionType(h, docCount, result, resultSize, [&](double* out, int predictionType) {
+            h.GetEvaluator().CalcHostColumns(floatFeatures, floatFeaturesSize, docCount, treeStart, treeEnd, out,
+                                             predictionType);
         });
     });
 }
@@ -829,6 +824,13 @@ bool CbHipExportQuantized(CbHipEvaluatorHandle* evaluator, const void* deviceBin
     return Guard([&] {
         E(evaluator)->ExportQuantizedDevice(static_cast<const uint8_t*>(deviceBins), docCount, deviceReferenceLayout,
                                             hipStream);
+    });
+}
+
+bool CbHipApplyPredictionTypeDevice(CbHipEvaluatorHandle* evaluator, int predictionType, size_t docCount,
+                                    const double* deviceRaw, double* deviceResult, void* hipStream) {
+    return Guard([&] {
+        E(evaluator)->ApplyPredictionTypeDevice(predictionType, 0, docCount, docCount, deviceRaw, deviceResult, hipStream);
     });
 }
 

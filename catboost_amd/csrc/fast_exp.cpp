@@ -68,6 +68,12 @@ inline double RoundedArgument(const TExpTable& c, double x) {
 
 }  // namespace
 
+TFastExpConstants FastExpConstants() {
+    const TExpTable& c = Table();
+    static_assert(sizeof(unsigned long long) == sizeof(uint64_t), "64-bit table entries");
+    return {reinterpret_cast<const unsigned long long*>(c.Mantissa), c.Scale, c.InvScale};
+}
+
 void FastExpInplace(double* x, size_t count) {
     const TExpTable& c = Table();
     const size_t vectorCount = count & ~size_t(3);

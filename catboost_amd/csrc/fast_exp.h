@@ -14,4 +14,13 @@ namespace cbamd {
 // fmath::expd (:474-512: 0 below the lower bound, +inf above the upper one).
 void FastExpInplace(double* x, size_t count);
 
+// The constants behind it, for the device version of the same arithmetic: 2048 mantissas of
+// 2^(i / 2048), then 2048 / ln 2 and its reciprocal.
+struct TFastExpConstants {
+    const unsigned long long* Mantissa;
+    double Scale;
+    double InvScale;
+};
+TFastExpConstants FastExpConstants();
+
 }  // namespace cbamd

@@ -56,6 +56,11 @@ public:
                                     uint32_t* indexes, void* stream);
     // bins in the reference's layout: blocks of 128 docs, [block][bucket][doc in block]
     void ExportQuantizedDevice(const uint8_t* bins, size_t docCount, uint8_t* referenceLayout, void* stream);
+    // raw[doc * dim + k] of documents [firstDoc, firstDoc + docCount) of a batch of totalDocs -> the
+    // prediction type (EApiPredictionType), as TEvalResultProcessor::PostprocessBlock does block by block
+    // (catboost/libs/model/eval_processing.h:174-240); result: one value per document for Class, dim otherwise
+    void ApplyPredictionTypeDevice(int predictionType, size_t firstDoc, size_t totalDocs, size_t docCount,
+                                   const double* raw, double* result, void* stream);
     // binarize + evaluate with a scratch bin buffer owned by the evaluator; records kernel times
     void CalcDevice(const TFeatureBatch& batch, size_t docCount, size_t treeStart, size_t treeEnd,
                     double* results, void* stream);
@@ -64,10 +69,13 @@ public:
 
     // ---- host-resident data: stage -> binarize -> evaluate -> copy back, in document chunks.
     // rows[doc] points at rowLen floats (FlatRows / SplitRows) or columns[f] at docCount floats.
+    // `predictionType` (EApiPredictionType) is applied on the device before the results are copied back;
+    // `results` then holds one value per document for Class, dim values otherwise.
     void CalcHostRows(const float* const* rows, size_t rowLen, bool flat, const int32_t* const* catRows,
-                      size_t catRowLen, size_t docCount, size_t treeStart, size_t treeEnd, double* results);
+                      size_t catRowLen, size_t docCount, size_t treeStart, size_t treeEnd, double* results,
+                      int predictionType = 0);
     void CalcHostColumns(const float* const* columns, size_t columnCount, size_t docCount, size_t treeStart,
-                         size_t treeEnd, double* results);
+                         size_t treeEnd, double* results, int predictionType = 0);
     void LeafIndexesHostRows(const float* const* rows, size_t rowLen, bool flat, const int32_t* const* catRows,
                              size_t catRowLen, size_t docCount, size_t treeStart, size_t treeEnd, uint32_t* indexes);
     void QuantizeHostRows(const float* const* rows, size_t rowLen, bool flat, const int32_t* const* catRows,

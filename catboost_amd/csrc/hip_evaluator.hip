@@ -1,5 +1,6 @@
 // Host side of the HIP evaluator: model upload, kernel launches, host staging.
 #include "hip_evaluator.h"
+#include "fast_exp.h"
 #include "kernels.hip.h"
 
 #include <algorithm>
@@ -544,6 +545,7 @@ struct THipEvaluator::TImpl {
     TDeviceVec<uint32_t> BucketSrcFlat, BucketSrcSplit, BucketOffset, BucketFlags, Values;
     TDeviceVec<uint32_t> BucketGrid;  // 4 dwords per bucket: lowest border, cells per unit, search steps, 0
     TDeviceVec<uint32_t> BucketLut;   // kLutCells bytes per bucket
+    TDeviceVec<unsigned long long> ExpMantissa;  // the table of the prediction types' exponent
     // CTR tables: feature descriptors, projection items, the index buckets and the rows of all tables
     TDeviceVec<uint32_t> CtrFeatures, CtrItems, CtrIndexBuckets, CtrBlob;
     // tree tables
@@ -673,6 +675,10 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
     m.Dim = trees.ApproxDimension;
     m.Scale = trees.Scale;
     m.HostBias = trees.Bias;
+    {
+        const TFastExpConstants constants = FastExpConstants();
+        m.ExpMantissa.Upload(std::vector<unsigned long long>(constants.Mantissa, constants.Mantissa + 2048));
+    }
 
     // ---- binarize tables: one entry per bucket, float buckets first, then one-hot buckets, in
     // the order of BinarizeFeatures (cpu/quantization.h:366-409, 54-79). Borders are sorted inside
@@ -1480,6 +1486,36 @@ void THipEvaluator::ExportQuantizedDevice(const uint8_t* bins, size_t docCount, 
     HIP_CHECK(hipGetLastError());
 }
 
+void THipEvaluator::ApplyPredictionTypeDevice(int predictionType, size_t firstDoc, size_t totalDocs, size_t docCount,
+                                              const double* raw, double* result, void* stream) {
+    TImpl& m = *Impl;
+    const uint32_t dim = static_cast<uint32_t>(m.Dim);
+    CBAMD_ENSURE(predictionType >= dev::kPredRaw && predictionType <= dev::kPredMultiProbability, "unknown prediction type");
+    // one dimension: the types TEvalResultProcessor accepts (eval_processing.h:182-204)
+    CBAMD_ENSURE(dim > 1 || predictionType == dev::kPredRaw || predictionType == dev::kPredExponent ||
+                     predictionType == dev::kPredProbability || predictionType == dev::kPredClass,
+                 "unsupported prediction type");
+    CBAMD_ENSURE(firstDoc <= totalDocs && docCount <= totalDocs - firstDoc, "document range exceeds the batch");
+    CBAMD_ENSURE(firstDoc % 128 == 0, "a chunk must start at a multiple of 128 documents");
+    if (docCount == 0) {
+        return;
+    }
+    CBAMD_ENSURE(raw != nullptr && result != nullptr, "prediction buffers are null");
+    CBAMD_ENSURE(!(predictionType == dev::kPredClass && dim > 1 && raw == result),
+                 "Class of a multi-dimensional model cannot be computed in place");
+    HIP_CHECK(hipSetDevice(m.DeviceId));
+    hipStream_t s = m.Pick(stream);
+    const TFastExpConstants constants = FastExpConstants();
+    dev::TFastExpDev c;
+    c.Mantissa = m.ExpMantissa.Get();
+    c.Scale = constants.Scale;
+    c.InvScale = constants.InvScale;
+    CBAMD_ENSURE((docCount + 255) / 256 <= 0x7fffffffu, "too many documents in one batch");
+    hipLaunchKernelGGL(dev::ApplyPredictionTypeKernel, dim3(static_cast<uint32_t>((docCount + 255) / 256)), dim3(256), 0, s,
+                       predictionType, dim, firstDoc, totalDocs, docCount, c, raw, result);
+    HIP_CHECK(hipGetLastError());
+}
+
 void THipEvaluator::CalcDevice(const TFeatureBatch& batch, size_t docCount, size_t treeStart, size_t treeEnd,
                                double* results, void* stream) {
     std::lock_guard<std::mutex> guard(Lock);
@@ -1558,9 +1594,11 @@ size_t PipelineDocs(size_t rowFloats, size_t rowCats) {
 // staging memory; while the GPU copies in, binarizes, evaluates and copies out slot k, the host
 // gathers the rows of slot k + 1.
 void THipEvaluator::CalcHostRows(const float* const* rows, size_t rowLen, bool flat, const int32_t* const* catRows,
-                                 size_t catRowLen, size_t docCount, size_t treeStart, size_t treeEnd, double* results) {
+                                 size_t catRowLen, size_t docCount, size_t treeStart, size_t treeEnd, double* results,
+                                 int predictionType) {
     std::lock_guard<std::mutex> guard(Lock);
     TImpl& m = *Impl;
+    const size_t outDim = predictionType == dev::kPredClass ? 1 : static_cast<size_t>(m.Dim);
     HIP_CHECK(hipSetDevice(m.DeviceId));
     hipStream_t s = m.Stream;
     // only the columns the model can address are staged
@@ -1589,14 +1627,15 @@ void THipEvaluator::CalcHostRows(const float* const* rows, size_t rowLen, bool f
             stageCats[slot]->Reserve(stageDocs * needCats);
         }
         pinnedResults[slot]->Reserve(std::max<size_t>(1, stageDocs * m.Dim));
-        stageResults[slot]->Reserve(std::max<size_t>(1, stageDocs * m.Dim));
+        // raw values, and behind them room for a prediction type that cannot be computed in place
+        stageResults[slot]->Reserve(std::max<size_t>(1, stageDocs * (m.Dim + 1)));
     }
     m.ScratchBins.Reserve(QuantizedBytes(stageDocs));
     LastTimes = TKernelTimes();
     // takes the results of the chunk that went through `slot` and adds its kernel times
     const auto collect = [&](int slot, size_t begin, size_t n) {
         HIP_CHECK(hipEventSynchronize(m.SlotEv[slot][3]));
-        std::memcpy(results + begin * m.Dim, pinnedResults[slot]->Get(), n * m.Dim * sizeof(double));
+        std::memcpy(results + begin * outDim, pinnedResults[slot]->Get(), n * outDim * sizeof(double));
         float a = 0.f, b = 0.f;
         HIP_CHECK(hipEventElapsedTime(&a, m.SlotEv[slot][0], m.SlotEv[slot][1]));
         HIP_CHECK(hipEventElapsedTime(&b, m.SlotEv[slot][1], m.SlotEv[slot][2]));
@@ -1633,8 +1672,13 @@ void THipEvaluator::CalcHostRows(const float* const* rows, size_t rowLen, bool f
         HIP_CHECK(hipEventRecord(m.SlotEv[slot][1], s));
         EvalQuantizedDevice(m.ScratchBins.Get(), n, treeStart, treeEnd, stageResults[slot]->Get(), s);
         HIP_CHECK(hipEventRecord(m.SlotEv[slot][2], s));
-        HIP_CHECK(hipMemcpyAsync(pinnedResults[slot]->Get(), stageResults[slot]->Get(), n * m.Dim * sizeof(double),
-                                 hipMemcpyDeviceToHost, s));
+        const double* final = stageResults[slot]->Get();
+        if (predictionType != dev::kPredRaw) {
+            double* processed = stageResults[slot]->Get() + (outDim == static_cast<size_t>(m.Dim) ? 0 : stageDocs * m.Dim);
+            ApplyPredictionTypeDevice(predictionType, begin, docCount, n, stageResults[slot]->Get(), processed, s);
+            final = processed;
+        }
+        HIP_CHECK(hipMemcpyAsync(pinnedResults[slot]->Get(), final, n * outDim * sizeof(double), hipMemcpyDeviceToHost, s));
         HIP_CHECK(hipEventRecord(m.SlotEv[slot][3], s));
         pendingBegin[slot] = begin;
         pendingDocs[slot] = n;
@@ -1650,9 +1694,10 @@ void THipEvaluator::CalcHostRows(const float* const* rows, size_t rowLen, bool f
 }
 
 void THipEvaluator::CalcHostColumns(const float* const* columns, size_t columnCount, size_t docCount, size_t treeStart,
-                                    size_t treeEnd, double* results) {
+                                    size_t treeEnd, double* results, int predictionType) {
     std::lock_guard<std::mutex> guard(Lock);
     TImpl& m = *Impl;
+    const size_t outDim = predictionType == dev::kPredClass ? 1 : static_cast<size_t>(m.Dim);
     HIP_CHECK(hipSetDevice(m.DeviceId));
     hipStream_t s = m.Stream;
     const size_t need = m.FlatVectorSize;
@@ -1663,7 +1708,7 @@ void THipEvaluator::CalcHostColumns(const float* const* columns, size_t columnCo
     m.PinnedFloats.Reserve(std::max<size_t>(1, stageDocs * need));
     m.StageFloats.Reserve(std::max<size_t>(1, stageDocs * need));
     m.PinnedResults.Reserve(std::max<size_t>(1, stageDocs * m.Dim));
-    m.StageResults.Reserve(std::max<size_t>(1, stageDocs * m.Dim));
+    m.StageResults.Reserve(std::max<size_t>(1, stageDocs * (m.Dim + 1)));
     m.ScratchBins.Reserve(QuantizedBytes(stageDocs));
     LastTimes = TKernelTimes();
     for (size_t begin = 0; begin < docCount; begin += chunk) {
@@ -1688,10 +1733,15 @@ void THipEvaluator::CalcHostColumns(const float* const* columns, size_t columnCo
         HIP_CHECK(hipEventRecord(m.Ev[1], s));
         EvalQuantizedDevice(m.ScratchBins.Get(), n, treeStart, treeEnd, m.StageResults.Get(), s);
         HIP_CHECK(hipEventRecord(m.Ev[2], s));
-        HIP_CHECK(hipMemcpyAsync(m.PinnedResults.Get(), m.StageResults.Get(), n * m.Dim * sizeof(double),
-                                 hipMemcpyDeviceToHost, s));
+        const double* final = m.StageResults.Get();
+        if (predictionType != dev::kPredRaw) {
+            double* processed = m.StageResults.Get() + (outDim == static_cast<size_t>(m.Dim) ? 0 : stageDocs * m.Dim);
+            ApplyPredictionTypeDevice(predictionType, begin, docCount, n, m.StageResults.Get(), processed, s);
+            final = processed;
+        }
+        HIP_CHECK(hipMemcpyAsync(m.PinnedResults.Get(), final, n * outDim * sizeof(double), hipMemcpyDeviceToHost, s));
         HIP_CHECK(hipStreamSynchronize(s));
-        std::memcpy(results + begin * m.Dim, m.PinnedResults.Get(), n * m.Dim * sizeof(double));
+        std::memcpy(results + begin * outDim, m.PinnedResults.Get(), n * outDim * sizeof(double));
         float a = 0.f, b = 0.f;
         HIP_CHECK(hipEventElapsedTime(&a, m.Ev[0], m.Ev[1]));
         HIP_CHECK(hipEventElapsedTime(&b, m.Ev[1], m.Ev[2]));

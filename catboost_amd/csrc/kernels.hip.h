@@ -1364,6 +1364,139 @@ __global__ __launch_bounds__(256) void ExportBinsKernel(const uint8_t* __restric
     }
 }
 
+// ---- prediction types on the device --------------------------------------------------------
+// TEvalResultProcessor::PostprocessBlock (catboost/libs/model/eval_processing.h:174-240) over blocks of
+// min(128, total documents) documents, with the reference's exponent (fmath::expd_v / fmath::expd,
+// contrib/libs/fmath/fmath.hpp:474-512, 565-648). The library is compiled without contraction, so each
+// operation rounds on its own like the CPU's.
+
+struct TFastExpDev {
+    const unsigned long long* Mantissa;  // 2048 mantissas of 2^(i / 2048)
+    double Scale, InvScale;              // 2048 / ln 2 and its reciprocal
+};
+
+// the arithmetic both forms share; `indexBits`: table index in bits 0..10, binary exponent above
+__device__ __forceinline__ double FastExpCore(const TFastExpDev& c, double x, double rounded, unsigned long long indexBits) {
+    constexpr int kTableBits = 11;
+    const double kMagic = static_cast<double>(3ull << 51);
+    constexpr unsigned long long kAdjust = (1ull << (kTableBits + 10)) - (1ull << kTableBits);
+    const unsigned long long mantissa = c.Mantissa[indexBits & ((1u << kTableBits) - 1)];
+    const unsigned long long power = (((indexBits + kAdjust) >> kTableBits) << 52) | mantissa;
+    double t = rounded - kMagic;
+    t = t * c.InvScale;
+    t = t - x;
+    double y = 3.0000000027955394 - t;
+    y = y * (t * t);
+    y = y * 0.16666666685227835064;
+    y = y - t;
+    y = y + 1.0;
+    return y * __longlong_as_double(static_cast<long long>(power));
+}
+
+// element `index` of a run of `count` values handed to the exponent at once: the first count & ~3 take
+// the vector form (clamped argument, NaN -> upper clamp), the rest the scalar form (0 / +inf outside)
+__device__ __forceinline__ double FastExpAt(const TFastExpDev& c, double v, size_t index, size_t count) {
+    const double kMagic = static_cast<double>(3ull << 51);
+    if (index < (count & ~size_t(3))) {
+        v = v < 709.78272569338397 ? v : 709.78272569338397;
+        v = v > -708.39641853226408 ? v : -708.39641853226408;
+        double d = v * c.Scale;
+        d = d + kMagic;
+        return FastExpCore(c, v, d, static_cast<unsigned long long>(__double_as_longlong(d)));
+    }
+    if (v <= -708.39641853226408) {
+        return 0.0;
+    }
+    if (v >= 709.78271289338397) {
+        return __longlong_as_double(0x7ff0000000000000ll);
+    }
+    double d = v * c.Scale;
+    d = d + kMagic;
+    const long long low = static_cast<long long>(static_cast<int>(static_cast<unsigned int>(__double_as_longlong(d))));
+    return FastExpCore(c, v, d, static_cast<unsigned long long>(low));
+}
+
+constexpr int kPredRaw = 0, kPredExponent = 1, kPredRmseWithUncertainty = 2, kPredProbability = 3, kPredClass = 4,
+              kPredMultiProbability = 5;  // EApiPredictionType, catboost/libs/model_interface/c_api.h:50-57
+
+// One thread per document of a chunk that starts at document `firstDoc` of `totalDocs`.
+// raw[doc * dim + k] -> out (doc values for Class, doc * dim values otherwise). raw == out is allowed
+// except for Class with dim > 1.
+__global__ __launch_bounds__(256) void ApplyPredictionTypeKernel(int type, uint32_t dim, size_t firstDoc,
+                                                                 size_t totalDocs, size_t docCount, TFastExpDev c,
+                                                                 const double* raw, double* out) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= docCount) {
+        return;
+    }
+    const size_t doc = firstDoc + i;
+    const size_t blockSize = totalDocs < 128 ? totalDocs : 128;
+    const size_t inBlock = doc % blockSize;
+    const size_t blockDocs = min(blockSize, totalDocs - (doc - inBlock));  // documents of this document's block
+    const double* r = raw + i * dim;
+    if (type == kPredClass) {
+        if (dim == 1) {
+            out[i] = r[0] > 0.0 ? 1.0 : 0.0;
+        } else {
+            uint32_t best = 0;
+            double top = r[0];
+            for (uint32_t k = 1; k < dim; ++k) {
+                const double v = r[k];
+                if (top < v) {  // std::max_element: the first largest
+                    top = v;
+                    best = k;
+                }
+            }
+            out[i] = static_cast<double>(best);
+        }
+        return;
+    }
+    double* o = out + i * dim;
+    if (dim == 1) {
+        const double v = r[0];
+        if (type == kPredProbability) {
+            o[0] = 1. / (1. + FastExpAt(c, -v, inBlock, blockDocs));
+        } else if (type == kPredExponent) {
+            o[0] = FastExpAt(c, v, inBlock, blockDocs);
+        } else {
+            o[0] = v;
+        }
+        return;
+    }
+    if (type == kPredRmseWithUncertainty) {
+        for (uint32_t k = 0; k < dim; ++k) {
+            double v = r[k];
+            if (k == 1) {
+                v = FastExpAt(c, v * 2.0, 0, 1);
+            }
+            o[k] = v;
+        }
+    } else if (type == kPredProbability) {  // CalcSoftmax, eval_processing.h:15-27
+        double top = r[0];
+        for (uint32_t k = 1; k < dim; ++k) {
+            const double v = r[k];
+            top = top < v ? v : top;
+        }
+        double sum = 0;
+        for (uint32_t k = 0; k < dim; ++k) {
+            const double e = FastExpAt(c, r[k] - top, k, dim);
+            o[k] = e;
+            sum += e;
+        }
+        for (uint32_t k = 0; k < dim; ++k) {
+            o[k] = o[k] / sum;
+        }
+    } else if (type == kPredMultiProbability) {
+        for (uint32_t k = 0; k < dim; ++k) {
+            o[k] = 1. / (1. + FastExpAt(c, -r[k], inBlock * dim + k, blockDocs * dim));
+        }
+    } else {
+        for (uint32_t k = 0; k < dim; ++k) {
+            o[k] = r[k];
+        }
+    }
+}
+
 __global__ void FillBiasKernel(double* __restrict__ out, size_t count, const double* __restrict__ bias, int dim) {
     const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i < count) {

@@ -118,6 +118,15 @@ bool CbHipLeafIndexesQuantized(CbHipEvaluatorHandle* evaluator, const void* devi
 bool CbHipExportQuantized(CbHipEvaluatorHandle* evaluator, const void* deviceBins, size_t docCount,
                           uint8_t* deviceReferenceLayout, void* hipStream);
 
+/* Raw formula values deviceRaw[doc * dim + k] (what CbHipEvalQuantized / CbHipEvalData write) -> the
+ * prediction type `predictionType` (EApiPredictionType of c_api.h), on the device: what
+ * TEvalResultProcessor::PostprocessBlock (catboost/libs/model/eval_processing.h:174-240) does after the CPU
+ * evaluator and ProcessResultsImpl (cuda/evaluator.cu:262-296, Probability and Class of one dimension
+ * only) after the CUDA one. deviceResult holds docCount values for APT_CLASS, docCount * dim otherwise;
+ * it may be deviceRaw itself unless the type is APT_CLASS and the model has several dimensions. */
+bool CbHipApplyPredictionTypeDevice(CbHipEvaluatorHandle* evaluator, int predictionType, size_t docCount,
+                                    const double* deviceRaw, double* deviceResult, void* hipStream);
+
 bool CbHipSynchronize(CbHipEvaluatorHandle* evaluator, void* hipStream);
 
 /* hipEvent-measured duration of the binarize and evaluate kernels of the last CbHipEvalData or
@@ -185,7 +194,8 @@ bool CbHipQuantizeWithHashedCatFeatures(void* modelHandle, size_t docCount, cons
                                         uint8_t* bins, size_t binsSize);
 uint32_t CbHipModelBucketCount(void* modelHandle);
 
-/* ---- prediction types (host side; no GPU involved) ------------------------------------- */
+/* ---- prediction types on host arrays (no GPU involved; CbHipApplyPredictionTypeDevice is the
+ * device version) ----------------------------------------------------------------------- */
 
 /* values[i] = exp(values[i]) as NCB::FastExpWithInfInplace computes it on an AVX2 host
  * (catboost/libs/helpers/math_utils.cpp:14-27, contrib/libs/fmath/fmath.hpp:565-648). */

@@ -146,6 +146,57 @@ def test_rust_fixture_with_one_hot_string_cats(golden_dir):
     np.testing.assert_array_equal(g.quantize_hashed(rm.RUST_FLOATS, hashed), o.binarize(rm.RUST_FLOATS, hashed, layout="split"))
 
 
+def _same_bits(got, expected, what):
+    """Bit for bit, except that a NaN only has to be a NaN (x86 and the GPU give the NaN they make a
+    different sign)."""
+    nan = np.isnan(expected)
+    np.testing.assert_array_equal(np.isnan(got), nan, err_msg=what)
+    np.testing.assert_array_equal(got[~nan].view(np.uint64), expected[~nan].view(np.uint64), err_msg=what)
+
+
+@pytest.mark.parametrize("dim", [1, 2, 3, 10])
+def test_prediction_types_on_the_device(golden_dir, dim):
+    """CbHipApplyPredictionTypeDevice against the oracle's TEvalResultProcessor, bit for bit: the inputs of
+    the reference exponent's vectors (clamps, infinities, NaN, table boundaries) as raw values, and
+    document counts around the 128-document block and the 4-value vector width."""
+    import torch
+
+    from oracle.oracle import apply_prediction_type
+
+    rng = np.random.default_rng(dim)
+    ev = _gpu_model(_random_oblivious(rng, trees=2, dim=dim)[0]).evaluator()
+    pool = np.load(os.path.join(golden_dir, "fmath_exp_vectors.npz"))["x"]
+    names = {"RawFormulaVal": cb.APT_RAW_FORMULA_VAL, "Exponent": cb.APT_EXPONENT, "Probability": cb.APT_PROBABILITY,
+             "Class": cb.APT_CLASS}
+    if dim > 1:
+        names["MultiProbability"] = cb.APT_MULTI_PROBABILITY
+    if dim == 2:
+        names["RMSEWithUncertainty"] = cb.APT_RMSE_WITH_UNCERTAINTY
+    for docs in (1, 2, 3, 4, 5, 127, 128, 129, 131, 1000, len(pool) // dim):
+        raw = pool[rng.permutation(len(pool))[:docs * dim]].copy()
+        if dim > 1 and docs > 4:
+            raw[:dim] = raw[0]  # a tie for the first largest
+        for name, kind in names.items():
+            if name == "Exponent" and dim > 1:
+                continue  # several dimensions: the reference leaves the raw values (covered by the raw case)
+            expected = apply_prediction_type(raw, dim, name)
+            x = torch.from_numpy(raw).to("cuda:0")
+            out = torch.full((len(expected),), 777.0, dtype=torch.float64, device="cuda:0")
+            torch.cuda.synchronize()
+            ev.apply_prediction_type(kind, docs, x.data_ptr(), out.data_ptr())
+            ev.synchronize()
+            _same_bits(out.cpu().numpy(), expected, "%s dim %d docs %d" % (name, dim, docs))
+            if not (name == "Class" and dim > 1):  # in place
+                ev.apply_prediction_type(kind, docs, x.data_ptr(), x.data_ptr())
+                ev.synchronize()
+                _same_bits(x.cpu().numpy()[:len(expected)], expected, "in place")
+    with pytest.raises(cb.CatBoostError):
+        ev.apply_prediction_type(99, 1, 0, 0)
+    if dim == 1:
+        with pytest.raises(cb.CatBoostError, match="unsupported prediction type"):
+            ev.apply_prediction_type(cb.APT_MULTI_PROBABILITY, 1, 0, 0)
+
+
 # -------------------------------------------------------- CTR (target statistics) features ----
 
 def _hashed(rows):
