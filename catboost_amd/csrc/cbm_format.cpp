@@ -110,6 +110,11 @@ void ReadTrees(const fb::TTable& t, TModelTrees* trees) {
     *trees = TModelTrees();
     trees->ApproxDimension = t.Scalar<int32_t>(TS_ApproxDimension, 0);
     CBAMD_ENSURE(trees->ApproxDimension >= 1, "model approx dimension must be positive");
+    // a dimension that neither the leaf values nor the bias can back is a damaged file; refusing it here
+    // keeps a corrupted field from turning into gigabytes of bias
+    CBAMD_ENSURE(static_cast<size_t>(trees->ApproxDimension) <=
+                     std::max<size_t>({t.VectorLen(TS_LeafValues), t.VectorLen(TS_MultiBias), size_t(1)}),
+                 "model approx dimension exceeds the leaf values and the bias the file holds");
     trees->TreeSplits = t.Vector<int>(TS_TreeSplits);
     trees->TreeSizes = t.Vector<int>(TS_TreeSizes);
     trees->TreeStartOffsets = t.Vector<int>(TS_TreeStartOffsets);

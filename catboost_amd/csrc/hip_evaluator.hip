@@ -427,6 +427,9 @@ void BuildCtrTables(const TModelTrees& trees, const std::vector<TCtrValueTable>&
             }
             CBAMD_ENSURE(cat != nullptr && cat->FlatIndex >= 0 && cat->Index >= 0,
                          "CTR projection refers to an unknown or unused categorical feature");
+            CBAMD_ENSURE(static_cast<size_t>(cat->FlatIndex) < trees.GetFlatFeatureVectorExpectedSize() &&
+                             static_cast<size_t>(cat->Index) < trees.MinimalSufficientCatFeaturesVectorSize,
+                         "categorical feature position exceeds the model's feature vector size");
             items.push_back({dev::kCtrItemCat, static_cast<uint32_t>(cat->FlatIndex), static_cast<uint32_t>(cat->Index), 0});
         }
         for (const auto& split : ctr.Base.Projection.BinFeatures) {
@@ -691,6 +694,10 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
             continue;
         }
         CBAMD_ENSURE(f.FlatIndex >= 0 && f.Index >= 0, "float feature without a position");
+        // the vector sizes come from the last feature of each list (as in the reference); a feature
+        // that points past them would make the kernels read behind a caller's row
+        CBAMD_ENSURE(static_cast<size_t>(f.FlatIndex) < m.FlatVectorSize && static_cast<size_t>(f.Index) < m.MinFloatSize,
+                     "float feature position exceeds the model's feature vector size");
         for (size_t begin = 0; begin < f.Borders.size(); begin += kMaxValuesPerBin) {
             const size_t end = std::min(begin + kMaxValuesPerBin, f.Borders.size());
             std::vector<float> b;
@@ -721,6 +728,8 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         }
         CBAMD_ENSURE(cat != nullptr, "one-hot feature refers to an unknown or unused categorical feature");
         CBAMD_ENSURE(cat->FlatIndex >= 0 && cat->Index >= 0, "categorical feature without a position");
+        CBAMD_ENSURE(static_cast<size_t>(cat->FlatIndex) < m.FlatVectorSize && static_cast<size_t>(cat->Index) < m.MinCatSize,
+                     "categorical feature position exceeds the model's feature vector size");
         for (size_t begin = 0; begin < oh.Values.size(); begin += kMaxValuesPerBin) {
             const size_t end = std::min(begin + kMaxValuesPerBin, oh.Values.size());
             for (size_t i = begin; i < end; ++i) {

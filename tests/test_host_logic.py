@@ -3,6 +3,7 @@ writer, model builders, hashes, error reporting."""
 import ctypes
 import os
 import re
+import time
 
 import numpy as np
 import pytest
@@ -123,6 +124,14 @@ def test_loader_rejects_bad_input(golden_dir):
             cb.ModelCalcer(buffer=bytes(corrupted))
         except cb.CatBoostError:
             pass
+    # a damaged dimension field must not turn into gigabytes of bias before the loader gives up
+    start = time.time()
+    for pos, value in ((2243, 0x10), (2242, 0x7f)):
+        corrupted = bytearray(data)
+        corrupted[pos] = value
+        with pytest.raises(cb.CatBoostError, match="dimension"):
+            cb.ModelCalcer(buffer=bytes(corrupted))
+    assert time.time() - start < 5
     # text features stay out of reach: the model part that carries their dictionaries is refused
     with pytest.raises(cb.CatBoostError, match="not supported"):
         cb.ModelCalcer(os.path.join(golden_dir, "jvm_model_with_text_features.cbm"))
