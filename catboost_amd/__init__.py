@@ -153,6 +153,8 @@ def load_library():
         "CbHipLoadModelFromArrays": (ctypes.c_bool, [vp, ctypes.POINTER(ModelArrays)]),
         "CbHipBuildObliviousModel": (ctypes.c_bool, [vp, ctypes.POINTER(ModelArrays), ctypes.c_int32, vp, vp, vp]),
         "CbHipBuildNonSymmetricModel": (ctypes.c_bool, [vp, ctypes.POINTER(ModelArrays), ctypes.c_int32, vp, vp, vp, vp, vp, vp, vp]),
+        "CbHipLoadFullModelFromJsonFile": (ctypes.c_bool, [vp, ctypes.c_char_p]),
+        "CbHipLoadFullModelFromJsonBuffer": (ctypes.c_bool, [vp, ctypes.c_char_p, sz]),
         "CbHipSaveModelToFile": (ctypes.c_bool, [vp, ctypes.c_char_p]),
         "CbHipSaveModelToBuffer": (ctypes.c_bool, [vp, ctypes.POINTER(vp), ctypes.POINTER(sz)]),
         "CbHipConvertObliviousToAsymmetric": (ctypes.c_bool, [vp]),
@@ -388,15 +390,17 @@ class DeviceEvaluator:
 class ModelCalcer:
     """Model handle of the model_calcer C API (ModelCalcerWrapper, wrapped_calcer.h:17-110)."""
 
-    def __init__(self, filename=None, buffer=None):
+    def __init__(self, filename=None, buffer=None, model_format="cbm"):
         self._lib = load_library()
         self._h = self._lib.ModelCalcerCreate()
         if not self._h:
             raise CatBoostError(last_error())
+        if model_format not in ("cbm", "json"):
+            raise CatBoostError("unknown model format %r" % (model_format,))
         if filename is not None:
-            self.init_from_file(filename)
+            self.init_from_json_file(filename) if model_format == "json" else self.init_from_file(filename)
         elif buffer is not None:
-            self.init_from_memory(buffer)
+            self.init_from_json(buffer) if model_format == "json" else self.init_from_memory(buffer)
 
     def __del__(self):
         if getattr(self, "_h", None):
@@ -414,6 +418,13 @@ class ModelCalcer:
     def init_from_memory(self, data):
         data = bytes(data)
         _check(self._lib.LoadFullModelFromBuffer(self._h, data, len(data)))
+
+    def init_from_json_file(self, filename):
+        _check(self._lib.CbHipLoadFullModelFromJsonFile(self._h, os.fsencode(filename)))
+
+    def init_from_json(self, text):
+        data = text.encode("utf-8") if isinstance(text, str) else bytes(text)
+        _check(self._lib.CbHipLoadFullModelFromJsonBuffer(self._h, data, len(data)))
 
     def load_from_arrays(self, arrays):
         _check(self._lib.CbHipLoadModelFromArrays(self._h, ctypes.byref(arrays)))

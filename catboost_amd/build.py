@@ -14,7 +14,7 @@ LIB_DIR = os.path.join(HERE, "lib")
 OBJ_DIR = os.path.join(LIB_DIR, "obj")
 LIB_PATH = os.path.join(LIB_DIR, "libcatboostmodel.so")
 
-HOST_SOURCES = ["model.cpp", "cbm_format.cpp", "model_builder.cpp", "cat_hash.cpp", "fast_exp.cpp", "c_api.cpp"]
+HOST_SOURCES = ["model.cpp", "cbm_format.cpp", "json_model.cpp", "model_builder.cpp", "cat_hash.cpp", "fast_exp.cpp", "c_api.cpp"]
 HIP_SOURCES = ["hip_evaluator.hip"]
 
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-Wno-unused-parameter", "-ffp-contract=off"]

@@ -394,6 +394,28 @@ bool LoadFullModelFromBuffer(ModelCalcerHandle* modelHandle, const void* binaryB
     });
 }
 
+bool CbHipLoadFullModelFromJsonFile(void* modelHandle, const char* filename) {
+    return Guard([&] {
+        CBAMD_ENSURE(filename != nullptr, "file name is null");
+        TFullModel model;
+        model.LoadFromJsonFile(filename);
+        TModelHandle* h = H(modelHandle);
+        h->ResetEvaluator();
+        h->Model = std::move(model);
+    });
+}
+
+bool CbHipLoadFullModelFromJsonBuffer(void* modelHandle, const void* jsonText, size_t jsonTextSize) {
+    return Guard([&] {
+        CBAMD_ENSURE(jsonText != nullptr, "model buffer is null");
+        TFullModel model;
+        model.LoadFromJson(jsonText, jsonTextSize);
+        TModelHandle* h = H(modelHandle);
+        h->ResetEvaluator();
+        h->Model = std::move(model);
+    });
+}
+
 bool LoadFullModelZeroCopy(ModelCalcerHandle* modelHandle, const void* binaryBuffer, size_t binaryBufferSize) {
     return LoadFullModelFromBuffer(modelHandle, binaryBuffer, binaryBufferSize);
 }

@@ -168,6 +168,13 @@ bool CbHipBuildNonSymmetricModel(void* modelHandle, const CbHipModelArrays* feat
                                  const CbHipModelSplit* nodeSplits, const int32_t* nodeLeft, const int32_t* nodeRight,
                                  const int64_t* nodeValueOffset, const double* nodeValues);
 
+/* The "json" model format: what ReadModel(path, EModelType::Json) does for the reference's bindings
+ * (catboost/libs/model/model_export/json_model_helpers.cpp:583-608 ConvertJsonToCatboostModel; the JVM
+ * binding's loadModel(stream, "json")). Float and one-hot categorical features, oblivious and
+ * non-symmetric trees, scale and bias; a JSON model with CTR features is refused (load its .cbm form). */
+bool CbHipLoadFullModelFromJsonFile(void* modelHandle, const char* filename);
+bool CbHipLoadFullModelFromJsonBuffer(void* modelHandle, const void* jsonText, size_t jsonTextSize);
+
 /* TFullModel::Save (catboost/libs/model/model.cpp:1113-1163). The buffer is malloc'd. */
 bool CbHipSaveModelToFile(void* modelHandle, const char* filename);
 bool CbHipSaveModelToBuffer(void* modelHandle, void** buffer, size_t* size);

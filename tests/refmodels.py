@@ -257,3 +257,58 @@ def flat_rows(model, floats, cats):
     for c in cfs:
         flat[:, c["flat_index"]] = np.ascontiguousarray(cats[:, c["index"]]).view(np.float32)
     return flat
+
+
+def model_to_json(model):
+    """A model dict in CatBoost's "json" model format, as ConvertModelToJson writes it
+    (catboost/libs/model/model_export/json_model_helpers.cpp:293-364, 469-498): the keys the importer
+    reads, float and one-hot categorical features only."""
+    import json
+
+    dim = int(model["approx_dimension"])
+    leaves = np.asarray(model["leaf_values"], np.float64)
+    doc = {"model_info": dict(model.get("info", {})), "features_info": {}}
+    if model["float_features"]:
+        doc["features_info"]["float_features"] = [
+            {"has_nans": bool(f["has_nans"]), "feature_index": int(f["index"]), "flat_feature_index": int(f["flat_index"]),
+             "borders": [float(b) for b in np.asarray(f["borders"], np.float32)], "feature_id": f.get("feature_id", ""),
+             "nan_value_treatment": ["AsIs", "AsFalse", "AsTrue"][int(f["nan_treatment"])]}
+            for f in model["float_features"]]
+    if model["cat_features"]:
+        one_hot = {int(o["cat_index"]): o for o in model["one_hot_features"]}
+        cats = []
+        for c in model["cat_features"]:
+            item = {"feature_index": int(c["index"]), "flat_feature_index": int(c["flat_index"]),
+                    "feature_id": c.get("feature_id", "")}
+            if int(c["index"]) in one_hot:
+                item["values"] = [int(v) for v in one_hot[int(c["index"])]["values"]]
+            cats.append(item)
+        doc["features_info"]["categorical_features"] = cats
+    steps = np.asarray(model["step_nodes"]).reshape(-1, 2)
+    if len(steps) == 0:
+        trees, first = [], 0
+        for t, depth in enumerate(model["tree_sizes"]):
+            begin = int(model["tree_start_offsets"][t])
+            count = (1 << int(depth)) * dim
+            trees.append({"leaf_values": [float(v) for v in leaves[first:first + count]],
+                          "splits": [{"split_index": int(s)} for s in model["tree_splits"][begin:begin + int(depth)]]})
+            first += count
+        doc["oblivious_trees"] = trees
+    else:
+        leaf_of = np.asarray(model["node_id_to_leaf_id"])
+
+        def leaf(node):
+            values = leaves[int(leaf_of[node]):int(leaf_of[node]) + dim]
+            return {"value": float(values[0]) if dim == 1 else [float(v) for v in values]}
+
+        def node_json(node):
+            left, right = int(steps[node][0]), int(steps[node][1])
+            if left == 0 and right == 0:
+                return leaf(node)
+            return {"split": {"split_index": int(model["tree_splits"][node])},
+                    "left": node_json(node + left) if left else leaf(node),
+                    "right": node_json(node + right) if right else leaf(node)}
+
+        doc["trees"] = [node_json(int(start)) for start in model["tree_start_offsets"]]
+    doc["scale_and_bias"] = [float(model["scale"]), [float(b) for b in np.asarray(model["bias"], np.float64)]]
+    return json.dumps(doc)

@@ -132,6 +132,18 @@ def test_numeric_only_fixture(golden_dir):
     _close(g.calc_single(rm.NUMERIC_ONLY_ROWS[0], []), rm.NUMERIC_ONLY_EXPECTED[:1])
 
 
+def test_json_model_format(golden_dir):
+    # the json twin of the numeric-only model (CatBoostModelTest.java:181-200) predicts the binary's goldens
+    g = cb.ModelCalcer(os.path.join(golden_dir, "numeric_only_model.json"), model_format="json")
+    _close(g.calc_flat(rm.NUMERIC_ONLY_ROWS), rm.NUMERIC_ONLY_EXPECTED)
+    rng = np.random.default_rng(8)
+    model, cat_values = _random_oblivious(rng, dim=3, trees=40, max_depth=6)
+    model = mb.convert_oblivious_to_asymmetric(model)
+    x = _random_flat_data(rng, model, cat_values, 700)
+    g = cb.ModelCalcer(buffer=rm.model_to_json(model), model_format="json")
+    _close(g.calc_flat(x), OracleModel(model).calc(x))
+
+
 def test_rust_fixture_with_one_hot_string_cats(golden_dir):
     g = cb.ModelCalcer(os.path.join(golden_dir, "rust_tmp_model.cbm"))
     _close(g.calc(rm.RUST_FLOATS, rm.RUST_CATS), rm.RUST_EXPECTED)

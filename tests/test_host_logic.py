@@ -11,6 +11,7 @@ import pytest
 import catboost_amd as cb
 from oracle import model_builder as mb
 from oracle.cbm_reader import read_cbm, read_cbm_file
+from oracle.oracle import OracleModel
 from tests import refmodels as rm
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -285,3 +286,65 @@ def test_library_prediction_types_match_the_oracle():
             for name in types:
                 got = cb.apply_prediction_type(raw, dim, PREDICTION_TYPES[name])
                 np.testing.assert_array_equal(got.view(np.uint64), apply_prediction_type(raw, dim, name).view(np.uint64))
+
+
+# ------------------------------------------------------------------- json model format ----
+
+def test_json_twin_of_the_numeric_only_fixture(golden_dir):
+    """CatBoostModelTest.java:181-200 loads numeric_only_model.json; it must give the tables of its
+    binary twin."""
+    path = os.path.join(golden_dir, "numeric_only_model.json")
+    from_json = read_cbm(cb.ModelCalcer(path, model_format="json").save_to_buffer())
+    with open(path) as f:
+        same = read_cbm(cb.ModelCalcer(buffer=f.read(), model_format="json").save_to_buffer())
+    binary = read_cbm_file(os.path.join(golden_dir, "numeric_only_model.cbm"))
+    for model in (from_json, same):
+        for key in ("approx_dimension", "tree_splits", "tree_sizes", "tree_start_offsets", "leaf_values", "scale", "bias"):
+            np.testing.assert_array_equal(np.asarray(model[key]), np.asarray(binary[key]), err_msg=key)
+        for a, b in zip(model["float_features"], binary["float_features"]):
+            np.testing.assert_array_equal(a["borders"], b["borders"])
+            assert (a["index"], a["flat_index"], a["has_nans"], a["nan_treatment"]) == \
+                (b["index"], b["flat_index"], b["has_nans"], b["nan_treatment"])
+        assert "iterations" in model["info"]["params"]
+
+
+@pytest.mark.parametrize("dim", [1, 3])
+@pytest.mark.parametrize("asym", [False, True])
+def test_json_import_of_random_models(dim, asym):
+    """Random models (one-hot features, NaN modes, several dimensions, non-symmetric trees with nodes that
+    are terminal on one side) written as json by the test's restatement of the reference's exporter:
+    the imported model must predict what the original does (checked on the CPU oracle)."""
+    from tests.test_oracle import _random_flat_data, _random_oblivious
+
+    rng = np.random.default_rng(40 + dim + 10 * asym)
+    model, cat_values = _random_oblivious(rng, dim=dim, trees=15, max_depth=5, scale=0.5, bias=list(rng.normal(size=dim)))
+    if asym:
+        model = mb.convert_oblivious_to_asymmetric(model)
+    x = _random_flat_data(rng, model, cat_values, 500)
+    imported = read_cbm(cb.ModelCalcer(buffer=rm.model_to_json(model), model_format="json").save_to_buffer())
+    np.testing.assert_array_equal(OracleModel(imported).calc(x), OracleModel(model).calc(x))
+
+
+def test_json_import_error_paths(golden_dir):
+    text = open(os.path.join(golden_dir, "numeric_only_model.json")).read()
+    for bad in ("", "[]", "{", text[:len(text) // 2], text.replace("oblivious_trees", "x"), text + "}",
+                text.replace('"AsIs"', '"Maybe"', 1), text.replace("[", "[[[", 1)):
+        with pytest.raises(cb.CatBoostError):
+            cb.ModelCalcer(buffer=bad, model_format="json")
+    rng = np.random.default_rng(3)
+    raw = bytearray(text.encode())
+    for _ in range(300):  # damaged text fails cleanly or loads; it never crashes
+        corrupted = bytearray(raw)
+        for pos in rng.integers(0, len(raw), size=3):
+            corrupted[pos] = int(rng.integers(32, 127))
+        try:
+            cb.ModelCalcer(buffer=bytes(corrupted), model_format="json")
+        except cb.CatBoostError:
+            pass
+    import json
+    doc = json.loads(text)
+    doc["features_info"]["ctrs"] = [{"borders": [0.5]}]
+    with pytest.raises(cb.CatBoostError, match="CTR"):
+        cb.ModelCalcer(buffer=json.dumps(doc), model_format="json")
+    with pytest.raises(cb.CatBoostError, match="can't open"):
+        cb.ModelCalcer(os.path.join(golden_dir, "no_such_model.json"), model_format="json")
