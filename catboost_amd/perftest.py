@@ -1,0 +1,114 @@
+"""Throughput of a model on this machine's GPU, in the spirit of the reference's model_perftest tool
+(catboost/tools/model_perftest/lib/main.cpp:165-330: --model-path, --block-size, --repetitions; it times
+the evaluator's entry points block by block over a pool).
+
+    python -m catboost_amd.perftest -m model.cbm [--pool-path pool.tsv] [--docs N] [--block-size B]
+                                    [--repetitions R] [--model-format cbm|json] [--device-id D]
+
+Without a pool the documents are random: floats around the model's borders, categorical hashes at random.
+A pool is a tab-separated file of flat feature rows (categorical columns as strings). Reports documents
+per second of the flat host entry point (rows by pointer, PCIe both ways) and of the device entry points
+on features that already sit in HBM.
+"""
+import argparse
+import json
+import sys
+import time
+
+import numpy as np
+
+import catboost_amd as cb
+
+
+def _feature_positions(model):
+    """Flat indexes of the model's float and categorical features."""
+    return model.get_float_feature_indices(), model.get_cat_feature_indices()
+
+
+def _random_rows(model, docs, seed):
+    floats, cats = _feature_positions(model)
+    width = max(floats + cats, default=-1) + 1
+    rng = np.random.default_rng(seed)
+    rows = rng.normal(size=(docs, width)).astype(np.float32)
+    for c in cats:
+        rows[:, c] = rng.integers(-2 ** 31, 2 ** 31, size=docs, dtype=np.int64).astype(np.int32).view(np.float32)
+    return rows
+
+
+def _pool_rows(model, path):
+    floats, cats = _feature_positions(model)
+    width = max(floats + cats, default=-1) + 1
+    rows = []
+    with open(path) as f:
+        for line in f:
+            parts = line.rstrip("\n").split("\t")
+            if len(parts) < width:
+                raise cb.CatBoostError("pool row has %d columns, the model needs %d" % (len(parts), width))
+            row = np.zeros(width, np.float32)
+            for i in floats:
+                row[i] = np.float32(parts[i]) if parts[i] != "" else np.float32("nan")
+            for i in cats:
+                row[i:i + 1] = np.array([cb.string_cat_feature_hash(parts[i])], np.int32).view(np.float32)
+            rows.append(row)
+    return np.array(rows, np.float32).reshape(len(rows), width)
+
+
+def run(args):
+    import torch
+
+    model = cb.ModelCalcer(args.model_path, model_format=args.model_format)
+    model.enable_gpu_evaluation(args.device_id)
+    rows = _pool_rows(model, args.pool_path) if args.pool_path else _random_rows(model, args.docs, args.seed)
+    docs = rows.shape[0]
+    block = min(args.block_size or docs, docs)
+    if block <= 0:
+        raise cb.CatBoostError("Empty pool")
+    blocks = [rows[b:b + block] for b in range(0, docs - block + 1, block)]
+    report = {"model": args.model_path, "trees": model.tree_count, "dimensions": model.dimensions_count, "docs": docs,
+              "block_size": block, "repetitions": args.repetitions}
+
+    model.calc_flat(blocks[0])  # binds the model to the device, uploads its tables
+    start = time.perf_counter()
+    for _ in range(args.repetitions):
+        for b in blocks:
+            model.calc_flat(b)
+    seconds = time.perf_counter() - start
+    report["host_flat_docs_per_sec"] = args.repetitions * len(blocks) * block / seconds
+
+    ev = model.evaluator()
+    device = "cuda:%d" % args.device_id
+    resident = [torch.from_numpy(np.ascontiguousarray(b)).to(device) for b in blocks]
+    out = torch.zeros(block * ev.dim, dtype=torch.float64, device=device)
+    torch.cuda.synchronize()
+    feats = [ev.features(cb.LAYOUT_FLAT_ROWS, x.data_ptr(), x.shape[1]) for x in resident]
+    ev.eval_data(feats[0], block, out.data_ptr())
+    ev.synchronize()
+    start = time.perf_counter()
+    for _ in range(args.repetitions):
+        for f in feats:
+            ev.eval_data(f, block, out.data_ptr())
+    ev.synchronize()
+    seconds = time.perf_counter() - start
+    report["device_docs_per_sec"] = args.repetitions * len(blocks) * block / seconds
+    binarize_ms, evaluate_ms = ev.last_kernel_times()
+    report["last_block_kernel_ms"] = {"binarize": binarize_ms, "evaluate": evaluate_ms}
+    return report
+
+
+def main(argv=None):
+    parser = argparse.ArgumentParser(prog="python -m catboost_amd.perftest", description=__doc__.split("\n\n")[0])
+    parser.add_argument("-m", "--model-path", required=True)
+    parser.add_argument("--model-format", default="cbm", choices=["cbm", "json"])
+    parser.add_argument("-f", "--pool-path")
+    parser.add_argument("--docs", type=int, default=1_000_000, help="random documents when no pool is given")
+    parser.add_argument("--block-size", type=int, default=0, help="documents per call (default: all)")
+    parser.add_argument("--repetitions", type=int, default=10)
+    parser.add_argument("--device-id", type=int, default=0)
+    parser.add_argument("--seed", type=int, default=0)
+    args = parser.parse_args(argv)
+    print(json.dumps(run(args)))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

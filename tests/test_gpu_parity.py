@@ -536,6 +536,76 @@ def test_workload_configs_device_path(name, docs):
     assert binarize_ms > 0 and eval_ms > 0
 
 
+def test_concurrent_callers():
+    """Callers on threads of their own: the device entry points with caller-owned buffers and streams run
+    side by side without sharing state; the host entry points of one handle take turns. Every result must
+    equal the single-threaded one."""
+    import threading
+
+    import torch
+
+    model, info = syn.build_model("C1")
+    ev = model.evaluator()
+    docs = 40_000
+    x = syn.device_features(info, docs)
+    expected = torch.zeros(docs, dtype=torch.float64, device="cuda:0")
+    torch.cuda.synchronize()
+    feats = ev.features(cb.LAYOUT_FLAT_ROWS, x.data_ptr(), x.shape[1])
+    ev.eval_data(feats, docs, expected.data_ptr())
+    ev.synchronize()
+    host = x.cpu().numpy()
+    expected_host = expected.cpu().numpy()
+    errors = []
+
+    def device_worker(k):
+        try:
+            stream = torch.cuda.Stream()
+            bins = torch.zeros(ev.quantized_bytes(docs), dtype=torch.uint8, device="cuda:0")
+            out = torch.zeros(docs, dtype=torch.float64, device="cuda:0")
+            torch.cuda.synchronize()
+            for _ in range(20):
+                ev.quantize(feats, docs, bins.data_ptr(), stream=stream.cuda_stream)
+                ev.eval_quantized(bins.data_ptr(), docs, out.data_ptr(), stream=stream.cuda_stream)
+            ev.synchronize(stream=stream.cuda_stream)
+            if not torch.equal(out, expected):
+                errors.append("device worker %d differs" % k)
+        except Exception as e:  # noqa: BLE001 - reported through the list
+            errors.append("device worker %d: %r" % (k, e))
+
+    def host_worker(k):
+        try:
+            for _ in range(5):
+                if not np.array_equal(model.calc_flat(host[k * 1000:(k + 3) * 1000]), expected_host[k * 1000:(k + 3) * 1000]):
+                    errors.append("host worker %d differs" % k)
+        except Exception as e:  # noqa: BLE001
+            errors.append("host worker %d: %r" % (k, e))
+
+    threads = [threading.Thread(target=device_worker, args=(k,)) for k in range(4)]
+    threads += [threading.Thread(target=host_worker, args=(k,)) for k in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert errors == []
+
+
+def test_perftest_tool(golden_dir, tmp_path, capsys):
+    import json
+
+    from catboost_amd import perftest
+
+    path = os.path.join(golden_dir, "features_num_cat__dataset_adult.cbm")
+    assert perftest.main(["-m", path, "--docs", "20000", "--block-size", "4096", "--repetitions", "2"]) == 0
+    report = json.loads(capsys.readouterr().out)
+    assert report["docs"] == 20000 and report["block_size"] == 4096 and report["trees"] == 100
+    assert report["host_flat_docs_per_sec"] > 0 and report["device_docs_per_sec"] > report["host_flat_docs_per_sec"]
+    # a pool of flat rows: the rust fixture's three documents (one string categorical column)
+    pool = tmp_path / "pool.tsv"
+    pool.write_text("".join("%g\t%g\t%s\t%g\n" % (f[0], f[1], c[0], f[2]) for f, c in zip(rm.RUST_FLOATS, rm.RUST_CATS)))
+    assert perftest.main(["-m", os.path.join(golden_dir, "rust_tmp_model.cbm"), "-f", str(pool), "--repetitions", "1"]) == 0
+    assert json.loads(capsys.readouterr().out)["docs"] == 3
+
+
 def test_plain_c_client_of_the_c_abi(golden_dir):
     """A C program linked against libcatboostmodel.so the way users of the reference library are."""
     import subprocess
