@@ -328,11 +328,13 @@ void BuildLevelOrderTrees(const TModelTrees& trees, int dim, const std::vector<u
 void BuildCtrTables(const TModelTrees& trees, const std::vector<TCtrValueTable>& tables, std::vector<uint32_t>* srcFlat,
                     std::vector<uint32_t>* srcSplit, std::vector<uint32_t>* offsets, std::vector<uint32_t>* flags,
                     std::vector<uint32_t>* values, TDeviceVec<uint32_t>* featuresOut, TDeviceVec<uint32_t>* itemsOut,
-                    TDeviceVec<uint32_t>* indexOut, TDeviceVec<uint32_t>* blobOut) {
+                    TDeviceVec<uint32_t>* indexOut, TDeviceVec<uint32_t>* blobOut, TDeviceVec<uint32_t>* catColumnsFlatOut,
+                    TDeviceVec<uint32_t>* catColumnsSplitOut, uint32_t* catColumnCountOut) {
     static_assert(sizeof(dev::TCtrFeatureDev) == 64 && sizeof(dev::TCtrItemDev) == 16, "device CTR records changed size");
     std::vector<dev::TCtrFeatureDev> features;
     std::vector<dev::TCtrItemDev> items;
     std::vector<uint32_t> index, blob;
+    std::vector<uint32_t> catColumnsFlat, catColumnsSplit;  // distinct categorical columns of all projections
     std::vector<uint32_t> tableIndexBegin(tables.size(), 0), tableBlobBegin(tables.size(), 0), tableRows(tables.size(), 0);
     std::vector<bool> tableUploaded(tables.size(), false);
 
@@ -430,7 +432,15 @@ void BuildCtrTables(const TModelTrees& trees, const std::vector<TCtrValueTable>&
             CBAMD_ENSURE(static_cast<size_t>(cat->FlatIndex) < trees.GetFlatFeatureVectorExpectedSize() &&
                              static_cast<size_t>(cat->Index) < trees.MinimalSufficientCatFeaturesVectorSize,
                          "categorical feature position exceeds the model's feature vector size");
-            items.push_back({dev::kCtrItemCat, static_cast<uint32_t>(cat->FlatIndex), static_cast<uint32_t>(cat->Index), 0});
+            uint32_t tileRow = 0;
+            while (tileRow < catColumnsSplit.size() && catColumnsSplit[tileRow] != static_cast<uint32_t>(cat->Index)) {
+                ++tileRow;
+            }
+            if (tileRow == catColumnsSplit.size()) {
+                catColumnsFlat.push_back(static_cast<uint32_t>(cat->FlatIndex));
+                catColumnsSplit.push_back(static_cast<uint32_t>(cat->Index));
+            }
+            items.push_back({dev::kCtrItemCat, static_cast<uint32_t>(cat->FlatIndex), static_cast<uint32_t>(cat->Index), tileRow});
         }
         for (const auto& split : ctr.Base.Projection.BinFeatures) {
             bool found = false;
@@ -501,6 +511,8 @@ void BuildCtrTables(const TModelTrees& trees, const std::vector<TCtrValueTable>&
             flags->push_back(dev::kBucketFlagCtr);
         }
         f.BucketCount = static_cast<uint32_t>(srcFlat->size()) - f.FirstBucket;
+        f.SameProjectionAsPrevious =
+            !features.empty() && trees.CtrFeatures[features.size() - 1].Ctr.Base.Projection == ctr.Base.Projection ? 1u : 0u;
         features.push_back(f);
     }
     std::vector<uint32_t> raw(features.size() * (sizeof(dev::TCtrFeatureDev) / 4));
@@ -514,6 +526,9 @@ void BuildCtrTables(const TModelTrees& trees, const std::vector<TCtrValueTable>&
         blob.push_back(0);
     }
     blobOut->Upload(blob);
+    *catColumnCountOut = static_cast<uint32_t>(catColumnsFlat.size());
+    catColumnsFlatOut->Upload(catColumnsFlat);
+    catColumnsSplitOut->Upload(catColumnsSplit);
 }
 
 }  // namespace
@@ -550,7 +565,9 @@ struct THipEvaluator::TImpl {
     TDeviceVec<uint32_t> BucketLut;   // kLutCells bytes per bucket
     TDeviceVec<unsigned long long> ExpMantissa;  // the table of the prediction types' exponent
     // CTR tables: feature descriptors, projection items, the index buckets and the rows of all tables
-    TDeviceVec<uint32_t> CtrFeatures, CtrItems, CtrIndexBuckets, CtrBlob;
+    TDeviceVec<uint32_t> CtrFeatures, CtrItems, CtrIndexBuckets, CtrBlob, CtrCatColumnsFlat, CtrCatColumnsSplit;
+    uint32_t CtrCatColumnCount = 0;
+    bool CtrTileUsable = false;  // the projections' categorical columns fit the LDS tile of CtrBinarizeTileKernel
     // tree tables
     TDeviceVec<uint32_t> Splits, TreeStart, TreeSize, FirstLeaf, StepNodes, NodeToLeaf;
     TDeviceVec<double> Leaves, Bias;
@@ -628,6 +645,10 @@ struct THipEvaluator::TImpl {
         t.Items = reinterpret_cast<const dev::TCtrItemDev*>(CtrItems.Get());
         t.IndexBuckets = CtrIndexBuckets.Get();
         t.Blob = CtrBlob.Get();
+        t.CatColumnsFlat = CtrCatColumnsFlat.Get();
+        t.CatColumnsSplit = CtrCatColumnsSplit.Get();
+        t.CatColumnCount = CtrCatColumnCount;
+        t.FeatureCount = CtrCount;
         return t;
     }
     dev::TTreeTables TreeTables() const {
@@ -746,8 +767,10 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
     if (!trees.CtrFeatures.empty()) {
         CBAMD_ENSURE(ctrTables != nullptr, "Model has CTR features but no tables of learned statistics");
         BuildCtrTables(trees, *ctrTables, &srcFlat, &srcSplit, &offsets, &flags, &values, &m.CtrFeatures, &m.CtrItems,
-                       &m.CtrIndexBuckets, &m.CtrBlob);
+                       &m.CtrIndexBuckets, &m.CtrBlob, &m.CtrCatColumnsFlat, &m.CtrCatColumnsSplit, &m.CtrCatColumnCount);
         m.CtrCount = static_cast<uint32_t>(trees.CtrFeatures.size());
+        const char* tileSwitch = std::getenv("CATBOOST_AMD_CTR_TILE");
+        m.CtrTileUsable = m.CtrCatColumnCount <= dev::kCtrMaxTileColumns && !(tileSwitch && tileSwitch[0] == '0');
     }
     CBAMD_ENSURE(srcFlat.size() == BucketCount, "internal error: bucket count mismatch");
     for (size_t b = 0; b + 1 < offsets.size(); ++b) {
@@ -1211,9 +1234,17 @@ void THipEvaluator::QuantizeDevice(const TFeatureBatch& batch, size_t docCount, 
             cats.ColumnStride = batch.Stride;
         }
         CBAMD_ENSURE(m.CtrCount <= 65535, "too many CTR features for one launch");
-        const dim3 grid(static_cast<uint32_t>(blocks), m.CtrCount);
-        hipLaunchKernelGGL(dev::CtrBinarizeKernel, grid, dim3(64), 0, s, cats, static_cast<uint32_t>(docCount), m.CtrTables(),
-                           m.BinarizeTables(batch.Layout != TFeatureBatch::SplitRows), reinterpret_cast<uint32_t*>(bins));
+        const dev::TBinarizeTables tab = m.BinarizeTables(batch.Layout != TFeatureBatch::SplitRows);
+        if (m.CtrTileUsable) {
+            const dim3 grid(static_cast<uint32_t>(blocks), (m.CtrCount + dev::kCtrGroup - 1) / dev::kCtrGroup);
+            const size_t lds = static_cast<size_t>(std::max<uint32_t>(m.CtrCatColumnCount, 1)) * dev::kCtrTilePitch * 4;
+            hipLaunchKernelGGL(dev::CtrBinarizeTileKernel, grid, dim3(256), lds, s, cats, static_cast<uint32_t>(docCount),
+                               m.CtrTables(), tab, reinterpret_cast<uint32_t*>(bins));
+        } else {
+            const dim3 grid(static_cast<uint32_t>(blocks), m.CtrCount);
+            hipLaunchKernelGGL(dev::CtrBinarizeKernel, grid, dim3(64), 0, s, cats, static_cast<uint32_t>(docCount),
+                               m.CtrTables(), tab, reinterpret_cast<uint32_t*>(bins));
+        }
         HIP_CHECK(hipGetLastError());
     }
 }

@@ -315,7 +315,7 @@ struct TCtrFeatureDev {
     int32_t CounterDenominator;
     float PriorNum, PriorDenom, Shift, Scale;
     uint32_t FirstBucket, BucketCount;  // where the binarized CTR goes
-    uint32_t Pad;
+    uint32_t SameProjectionAsPrevious;  // the feature before this one hashes the same items
 };
 
 constexpr uint32_t kCtrItemCat = 0;       // hashed categorical value of column SrcFlat / SrcSplit
@@ -323,7 +323,7 @@ constexpr uint32_t kCtrItemBinGe = 1;     // float split: bin of bucket SrcFlat 
 constexpr uint32_t kCtrItemBinEq = 2;     // one-hot split: bin of bucket SrcFlat == Value
 
 struct TCtrItemDev {
-    uint32_t Kind, SrcFlat, SrcSplit, Value;
+    uint32_t Kind, SrcFlat, SrcSplit, Value;  // a categorical item keeps its row of the staged tile in Value
 };
 
 struct TCtrTablesDev {
@@ -331,6 +331,11 @@ struct TCtrTablesDev {
     const TCtrItemDev* Items;
     const uint32_t* IndexBuckets;  // {hash low, hash high, row} per bucket (helpers/dense_hash_view.h:12-26)
     const uint32_t* Blob;
+    // the categorical columns the projections read, as flat and as categorical feature indexes
+    const uint32_t* CatColumnsFlat;
+    const uint32_t* CatColumnsSplit;
+    uint32_t CatColumnCount;
+    uint32_t FeatureCount;
 };
 
 // hashed categorical values of a batch: Base[doc * DocStride + column * ColumnStride]
@@ -470,6 +475,83 @@ __global__ __launch_bounds__(64) void CtrBinarizeKernel(TCatSource cats, uint32_
         }
         bins[(static_cast<size_t>(block) * tab.BucketPitch + bucket) * kWave + lane] =
             count[0] | (count[1] << 8) | (count[2] << 16) | (count[3] << 24);
+    }
+}
+
+// The same for models whose CTR projections read at most kCtrMaxTileColumns categorical columns:
+// grid = (document blocks, groups of kCtrGroup CTR features), 4 waves per workgroup. The block's hashed
+// categorical values are staged once per workgroup into LDS ([column][document], read without bank
+// conflicts), each wave then works through kCtrGroup / 4 consecutive CTR features and keeps the hash
+// when the next feature has the same projection (features are sorted by projection).
+constexpr uint32_t kCtrGroup = 16;
+constexpr uint32_t kCtrMaxTileColumns = 60;
+constexpr uint32_t kCtrTilePitch = kDocsPerBlock + 1;
+
+__global__ __launch_bounds__(256) void CtrBinarizeTileKernel(TCatSource cats, uint32_t docCount, TCtrTablesDev ctr,
+                                                             TBinarizeTables tab, uint32_t* __restrict__ bins) {
+    extern __shared__ uint32_t sCats[];  // [CatColumnCount][kCtrTilePitch]
+    const uint32_t block = blockIdx.x, tid = threadIdx.x;
+    const uint32_t lane = tid & (kWave - 1), wave = tid / kWave;
+    const uint32_t columns = ctr.CatColumnCount;
+    const uint32_t* columnList = cats.SplitColumns ? ctr.CatColumnsSplit : ctr.CatColumnsFlat;
+    const size_t firstDoc = static_cast<size_t>(block) * kDocsPerBlock;
+    for (uint32_t i = tid; i < columns * kDocsPerBlock; i += 256) {
+        // neighbouring threads read neighbouring addresses: columns of one row, or documents of one column
+        const uint32_t c = cats.ColumnStride == 1 ? i % columns : i / kDocsPerBlock;
+        const uint32_t d = cats.ColumnStride == 1 ? i / columns : i % kDocsPerBlock;
+        const size_t doc = min(firstDoc + d, static_cast<size_t>(docCount) - 1);
+        sCats[c * kCtrTilePitch + d] = cats.Base[doc * cats.DocStride + static_cast<size_t>(columnList[c]) * cats.ColumnStride];
+    }
+    __syncthreads();
+    constexpr uint32_t kPerWave = kCtrGroup / 4;
+    const uint32_t first = blockIdx.y * kCtrGroup + wave * kPerWave;
+    uint64_t hash[4] = {0, 0, 0, 0};
+    for (uint32_t k = 0; k < kPerWave && first + k < ctr.FeatureCount; ++k) {
+        const TCtrFeatureDev f = ctr.Features[first + k];
+        if (k == 0 || !f.SameProjectionAsPrevious) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                hash[j] = 0;
+            }
+            for (uint32_t i = f.ItemBegin; i < f.ItemEnd; ++i) {
+                const TCtrItemDev item = ctr.Items[i];
+                if (item.Kind == kCtrItemCat) {
+                    const uint32_t* column = sCats + item.Value * kCtrTilePitch + lane;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const int32_t v = static_cast<int32_t>(column[j * kWave]);
+                        hash[j] = CtrCalcHash(hash[j], static_cast<uint64_t>(static_cast<int64_t>(v)));
+                    }
+                } else {
+                    const uint32_t word = bins[(static_cast<size_t>(block) * tab.BucketPitch + item.SrcFlat) * kWave + lane];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const uint32_t bin = (word >> (8 * j)) & 0xffu;
+                        const bool holds = item.Kind == kCtrItemBinGe ? bin >= item.Value : bin == item.Value;
+                        hash[j] = CtrCalcHash(hash[j], holds ? 1u : 0u);
+                    }
+                }
+            }
+        }
+        float value[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            value[j] = CtrValue(ctr, f, CtrTableRow(ctr, f, hash[j]));
+        }
+        for (uint32_t b = 0; b < f.BucketCount; ++b) {
+            const uint32_t bucket = f.FirstBucket + b;
+            const uint32_t begin = tab.BucketOffset[bucket], end = tab.BucketOffset[bucket + 1];
+            uint32_t count[4] = {0, 0, 0, 0};
+            for (uint32_t x = begin; x < end; ++x) {
+                const float border = __uint_as_float(tab.Values[x]);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    count[j] += value[j] > border ? 1u : 0u;
+                }
+            }
+            bins[(static_cast<size_t>(block) * tab.BucketPitch + bucket) * kWave + lane] =
+                count[0] | (count[1] << 8) | (count[2] << 16) | (count[3] << 24);
+        }
     }
 }
 

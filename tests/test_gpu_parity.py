@@ -270,6 +270,21 @@ def test_ctr_models_against_the_oracle(golden_dir, name, docs):
            o.calc(flat, tree_start=half, tree_end=o.tree_count))
 
 
+def test_ctr_kernel_without_the_staged_tile(golden_dir, monkeypatch):
+    """Models whose projections read more categorical columns than the LDS tile holds take the plain CTR
+    kernel; the switch forces it for models that would not."""
+    monkeypatch.setenv("CATBOOST_AMD_CTR_TILE", "0")
+    for name in ("mushroom_model.cbm", "features_num_cat__dataset_adult.cbm", "cloudness_small.cbm"):
+        path = os.path.join(golden_dir, name)
+        m = read_cbm_file(path)
+        o = OracleModel(m)
+        g = cb.ModelCalcer(path)
+        floats, cats = rm.random_ctr_inputs(m, 3000, 77, rm.known_cat_hashes(m))
+        np.testing.assert_array_equal(g.quantize_hashed(floats, cats), o.binarize(floats, cats, layout="split"))
+        flat = rm.flat_rows(m, floats, cats)
+        _close(g.calc_flat_transposed(np.ascontiguousarray(flat.T)), o.calc(flat))
+
+
 def test_ctr_model_on_the_device_path(golden_dir):
     """The device entry points (features already in HBM) on the adult model, 200 000 documents."""
     import torch
