@@ -1,7 +1,8 @@
-// .cbm reader / writer: "CBM1" + core size + flatbuffer TModelCore (+ refused trailing parts).
+// .cbm reader / writer: "CBM1" + core size + flatbuffer TModelCore + trailing model parts (the reader
+// takes the tables of the static CTR provider and refuses text / embedding parts; the writer emits none).
 // Follows TFullModel::Save / Load (catboost/libs/model/model.cpp:1113-1228), the schemas
-// catboost/libs/model/flatbuffers/model.fbs:22-54 and features.fbs:5-59 (vtable slot = field
-// declaration order) and the size prefix of util/ysaveload.h:277-296.
+// catboost/libs/model/flatbuffers/model.fbs:22-54, features.fbs:5-75 and ctr_data.fbs:5-43 (vtable slot =
+// field declaration order) and the size prefix of util/ysaveload.h:277-296.
 #include "flatbuf.h"
 #include "model.h"
 
