@@ -240,6 +240,99 @@ size_t WriteOneHotFeature(fb::TWriter& w, const TOneHotFeature& f) {
     return pos.Table;
 }
 
+// TModelCtrBase with its TFeatureCombination (ctr_data.fbs:15-19, features.fbs:71-75)
+size_t WriteCtrBase(fb::TWriter& w, const TModelCtrBase& base) {
+    fb::TWriter::TTableBuilder b;
+    b.Ref(0);
+    if (base.CtrType != ECtrType::Borders) {
+        b.Scalar<int8_t>(1, static_cast<int8_t>(base.CtrType));
+    }
+    if (base.TargetBorderClassifierIdx != 0) {
+        b.Scalar<int32_t>(2, base.TargetBorderClassifierIdx);
+    }
+    auto pos = w.WriteTable(b);
+    fb::TWriter::TTableBuilder pb;
+    pb.Ref(0);
+    pb.Ref(1);
+    pb.Ref(2);
+    auto proj = w.WriteTable(pb);
+    w.PatchRef(pos.RefPos(0), proj.Table);
+    w.PatchRef(proj.RefPos(0), w.WriteVector(base.Projection.CatFeatures));
+    w.PatchRef(proj.RefPos(1), w.WriteVector(base.Projection.BinFeatures.data(), base.Projection.BinFeatures.size(), 8, 4));
+    w.PatchRef(proj.RefPos(2),
+               w.WriteVector(base.Projection.OneHotFeatures.data(), base.Projection.OneHotFeatures.size(), 8, 4));
+    return pos.Table;
+}
+
+// TCtrFeature with its TModelCtr (ctr_data.fbs:21-33)
+size_t WriteCtrFeature(fb::TWriter& w, const TCtrFeature& f) {
+    fb::TWriter::TTableBuilder b;
+    b.Ref(0);
+    b.Ref(1);
+    auto pos = w.WriteTable(b);
+    fb::TWriter::TTableBuilder cb;
+    cb.Ref(0);
+    if (f.Ctr.TargetBorderIdx != 0) {
+        cb.Scalar<int32_t>(1, f.Ctr.TargetBorderIdx);
+    }
+    if (f.Ctr.PriorNum != 0.f) {
+        cb.Scalar<float>(2, f.Ctr.PriorNum);
+    }
+    if (f.Ctr.PriorDenom != 1.f) {
+        cb.Scalar<float>(3, f.Ctr.PriorDenom);
+    }
+    if (f.Ctr.Shift != 0.f) {
+        cb.Scalar<float>(4, f.Ctr.Shift);
+    }
+    if (f.Ctr.Scale != 1.f) {
+        cb.Scalar<float>(5, f.Ctr.Scale);
+    }
+    auto ctr = w.WriteTable(cb);
+    w.PatchRef(pos.RefPos(0), ctr.Table);
+    w.PatchRef(ctr.RefPos(0), WriteCtrBase(w, f.Ctr.Base));
+    w.PatchRef(pos.RefPos(1), w.WriteVector(f.Borders));
+    return pos.Table;
+}
+
+// SaveSize of util/ysaveload.h:277-296
+void AppendSize(std::string* out, uint64_t size) {
+    if (size < 0xffffffffu) {
+        const uint32_t s = static_cast<uint32_t>(size);
+        out->append(reinterpret_cast<const char*>(&s), 4);
+    } else {
+        const uint32_t marker = 0xffffffffu;
+        out->append(reinterpret_cast<const char*>(&marker), 4);
+        out->append(reinterpret_cast<const char*>(&size), 8);
+    }
+}
+
+// TCtrData::Save (ctr_data.cpp:9-22): the number of tables, then each as a size and a flatbuffer
+// whose root is TCtrValueTable (TCtrValueTable::Save, ctr_value_table.cpp:16-48)
+void AppendStaticCtrProvider(std::string* out, const std::vector<TCtrValueTable>& tables) {
+    AppendSize(out, tables.size());
+    for (const auto& table : tables) {
+        fb::TWriter w;
+        fb::TWriter::TTableBuilder b;
+        b.Ref(0);
+        b.Ref(1);
+        b.Ref(2);
+        if (table.CounterDenominator != 0) {
+            b.Scalar<int32_t>(3, table.CounterDenominator);
+        }
+        if (table.TargetClassesCount != 0) {
+            b.Scalar<int32_t>(4, table.TargetClassesCount);
+        }
+        auto pos = w.WriteTable(b);
+        w.SetRoot(pos.Table);
+        w.PatchRef(pos.RefPos(0), WriteCtrBase(w, table.ModelCtrBase));
+        w.PatchRef(pos.RefPos(1), w.WriteVector(table.IndexHashRaw));
+        w.PatchRef(pos.RefPos(2), w.WriteVector(table.CTRBlob));
+        const auto& buf = w.Buffer();
+        AppendSize(out, buf.size());
+        out->append(reinterpret_cast<const char*>(buf.data()), buf.size());
+    }
+}
+
 template <typename T, typename F>
 void WriteTableVector(fb::TWriter& w, size_t refPos, const std::vector<T>& items, F writeOne) {
     auto vec = w.WriteRefVector(items.size());
@@ -304,8 +397,7 @@ void TFullModel::LoadFromFile(const std::string& path) {
 }
 
 std::string TFullModel::Save() const {
-    CBAMD_ENSURE(Trees.CtrFeatures.empty() && CtrTables.empty(),
-                 "Saving a model with CTR features is not supported by the HIP evaluator library");
+    const bool withCtrPart = !CtrTables.empty();
     fb::TWriter w;
     // TModelCore
     fb::TWriter::TTableBuilder coreB;
@@ -313,6 +405,9 @@ std::string TFullModel::Save() const {
     coreB.Ref(1);
     if (!ModelInfo.empty()) {
         coreB.Ref(2);
+    }
+    if (withCtrPart) {
+        coreB.Ref(3);
     }
     auto core = w.WriteTable(coreB);
     w.SetRoot(core.Table);
@@ -338,7 +433,8 @@ std::string TFullModel::Save() const {
     WriteTableVector(w, tp.RefPos(TS_CatFeatures), Trees.CatFeatures, WriteCatFeature);
     WriteTableVector(w, tp.RefPos(TS_FloatFeatures), Trees.FloatFeatures, WriteFloatFeature);
     WriteTableVector(w, tp.RefPos(TS_OneHotFeatures), Trees.OneHotFeatures, WriteOneHotFeature);
-    for (int slot : {TS_CtrFeatures, TS_TextFeatures, TS_EstimatedFeatures, TS_EmbeddingFeatures}) {
+    WriteTableVector(w, tp.RefPos(TS_CtrFeatures), Trees.CtrFeatures, WriteCtrFeature);
+    for (int slot : {TS_TextFeatures, TS_EstimatedFeatures, TS_EmbeddingFeatures}) {
         w.PatchRef(tp.RefPos(slot), w.WriteRefVector(0).first);
     }
     w.PatchRef(tp.RefPos(TS_LeafValues), w.WriteVector(Trees.LeafValues));
@@ -367,19 +463,19 @@ std::string TFullModel::Save() const {
             ++i;
         }
     }
+    if (withCtrPart) {  // ModelPartIds, model.fbs:53 and model.cpp:1140-1161
+        auto vec = w.WriteRefVector(1);
+        w.PatchRef(core.RefPos(3), vec.first);
+        w.PatchRef(vec.second, w.WriteString("static_provider_v1"));
+    }
     const auto& buf = w.Buffer();
     std::string out;
     out.append("CBM1", 4);
-    if (buf.size() < 0xffffffffu) {
-        const uint32_t s = static_cast<uint32_t>(buf.size());
-        out.append(reinterpret_cast<const char*>(&s), 4);
-    } else {
-        const uint32_t marker = 0xffffffffu;
-        const uint64_t s = buf.size();
-        out.append(reinterpret_cast<const char*>(&marker), 4);
-        out.append(reinterpret_cast<const char*>(&s), 8);
-    }
+    AppendSize(&out, buf.size());
     out.append(reinterpret_cast<const char*>(buf.data()), buf.size());
+    if (withCtrPart) {
+        AppendStaticCtrProvider(&out, CtrTables);
+    }
     return out;
 }
 

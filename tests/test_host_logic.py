@@ -151,8 +151,21 @@ def test_loader_reads_ctr_models(golden_dir):
             sum((len(o["values"]) + 253) // 254 for o in expected["one_hot_features"]) + \
             sum((len(c["borders"]) + 253) // 254 for c in expected["ctr_features"])
         assert m.bucket_count == buckets and m.tree_count == len(expected["tree_sizes"]) and borders >= 0
-        with pytest.raises(cb.CatBoostError, match="CTR"):
-            m.save_to_buffer()
+        # saved again (CTR features in the core, the static CTR provider as a trailing part), the model
+        # reads back with the same tables through the oracle's reader and through the library
+        saved = m.save_to_buffer()
+        again = read_cbm(saved)
+        assert again["model_part_ids"] == ["static_provider_v1"]
+        assert len(again["ctr_tables"]) == len({bytes(str(t["base"]), "utf8") for t in expected["ctr_tables"]})
+        for a, b in zip(again["ctr_features"], expected["ctr_features"]):
+            np.testing.assert_array_equal(a["borders"], b["borders"])
+            assert str(a["base"]) == str(b["base"])
+            assert [a[k] for k in ("target_border_idx", "prior_num", "prior_denom", "shift", "scale")] == \
+                [b[k] for k in ("target_border_idx", "prior_num", "prior_denom", "shift", "scale")]
+        floats, cats = rm.random_ctr_inputs(expected, 800, 9, rm.known_cat_hashes(expected))
+        np.testing.assert_array_equal(OracleModel(again).calc(floats, cats, layout="split"),
+                                      OracleModel(expected).calc(floats, cats, layout="split"))
+        assert cb.ModelCalcer(buffer=saved).save_to_buffer() == saved
     # a damaged CTR part fails cleanly (or loads), and never crashes
     data = open(os.path.join(golden_dir, "jvm_model_with_ctr.cbm"), "rb").read()
     core = int.from_bytes(data[4:8], "little")
