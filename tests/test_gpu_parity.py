@@ -704,3 +704,49 @@ def test_c2_full_size_properties():
         parts += part
     torch.cuda.synchronize()
     assert torch.allclose(parts, out, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("name,base_docs,copies", [("C2", 1_000_000, 23), ("C4", 1_000_000, 15), ("C3", 500_000, 110)])
+def test_batches_beyond_four_gibibytes(name, base_docs, copies):
+    """Batches whose features, bins or results pass 4 GiB (C2: 18 GB of features, 4.6 GB of bins; C3: 4.4 GB
+    of results): a base batch repeated `copies` times plus a ragged tail must give the base batch's
+    predictions at every repetition, bit for bit - any 32-bit overflow in a kernel's addressing would
+    break that."""
+    import torch
+
+    model, info = syn.build_model(name)
+    ev = model.evaluator()
+    dim = info["dim"]
+    base = syn.device_features(info, base_docs)
+    tail = 777
+    docs = base_docs * copies + tail
+    x = torch.empty((docs, base.shape[1]), dtype=torch.float32, device="cuda:0")
+    for c in range(copies):
+        x[c * base_docs:(c + 1) * base_docs] = base
+    x[copies * base_docs:] = base[:tail]
+    expected = torch.zeros(base_docs * dim, dtype=torch.float64, device="cuda:0")
+    out = torch.zeros(docs * dim, dtype=torch.float64, device="cuda:0")
+    torch.cuda.synchronize()
+    ev.eval_data(ev.features(cb.LAYOUT_FLAT_ROWS, base.data_ptr(), base.shape[1]), base_docs, expected.data_ptr())
+    ev.eval_data(ev.features(cb.LAYOUT_FLAT_ROWS, x.data_ptr(), x.shape[1]), docs, out.data_ptr())
+    ev.synchronize()
+    assert ev.quantized_bytes(docs) > (1 << 32) or name == "C3"
+    # the huge batch may take another kernel than the base batch (C3: its output passes what the register
+    # kernels address), so the first repetition is held to the tolerance and the others to the first
+    first = out[:base_docs * dim]
+    _close(first.cpu().numpy(), expected.cpu().numpy())
+    for c in range(1, copies):
+        assert torch.equal(out[c * base_docs * dim:(c + 1) * base_docs * dim], first), "repetition %d" % c
+    assert torch.equal(out[copies * base_docs * dim:], first[:tail * dim])
+    # a tree sub-range takes the kernels that do not hold the model in registers
+    half = model.tree_count // 2
+    part = torch.zeros_like(out)
+    part_base = torch.zeros_like(expected)
+    torch.cuda.synchronize()
+    ev.eval_data(ev.features(cb.LAYOUT_FLAT_ROWS, base.data_ptr(), base.shape[1]), base_docs, part_base.data_ptr(),
+                 tree_start=half, tree_end=model.tree_count)
+    ev.eval_data(ev.features(cb.LAYOUT_FLAT_ROWS, x.data_ptr(), x.shape[1]), docs, part.data_ptr(),
+                 tree_start=half, tree_end=model.tree_count)
+    ev.synchronize()
+    assert torch.equal(part[(copies - 1) * base_docs * dim:copies * base_docs * dim], part_base)
+    assert torch.equal(part[:base_docs * dim], part_base)
