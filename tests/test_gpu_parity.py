@@ -120,6 +120,32 @@ def test_single_document_and_ragged_sizes():
     assert g.calc_flat(np.zeros((0, 3), np.float32)).size == 0
 
 
+def test_empty_batches(golden_dir):
+    """No documents: every entry point returns without touching the GPU buffers, whatever the model holds
+    (CTR features, several dimensions, a prediction type)."""
+    import torch
+
+    for name in ("numeric_only_model.cbm", "features_num_cat__dataset_adult.cbm", "iris_model.cbm"):
+        g = cb.ModelCalcer(os.path.join(golden_dir, name))
+        width = max(g.get_float_feature_indices() + g.get_cat_feature_indices()) + 1
+        for kind in ("RawFormulaVal", "Probability", "Class"):
+            g.set_prediction_type(kind)
+            assert g.calc_flat(np.zeros((0, width), np.float32)).size == 0
+            assert g.calc_flat_transposed(np.zeros((width, 0), np.float32)).size == 0
+        assert g.quantize_flat(np.zeros((0, width), np.float32)).size == 0
+        assert g.calc_leaf_indexes_flat(np.zeros((0, width), np.float32)).size == 0
+        ev = g.evaluator()
+        guard = torch.full((16,), 7.0, dtype=torch.float64, device="cuda:0")
+        torch.cuda.synchronize()
+        feats = ev.features(cb.LAYOUT_FLAT_ROWS, guard.data_ptr(), width)
+        ev.eval_data(feats, 0, guard.data_ptr())
+        ev.quantize(feats, 0, guard.data_ptr())
+        ev.eval_quantized(guard.data_ptr(), 0, guard.data_ptr())
+        ev.apply_prediction_type(cb.APT_PROBABILITY, 0, guard.data_ptr(), guard.data_ptr())
+        ev.synchronize()
+        assert bool((guard == 7.0).all())
+
+
 # ------------------------------------------------------------------- fixtures + goldens ----
 
 def test_numeric_only_fixture(golden_dir):
