@@ -126,9 +126,18 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed):
             e("  s_load_dwordx16 s[%d:%d], s[6:7], 0x%x" % (regs + 16 * part, regs + 16 * part + 15,
                                                             tree * tree_row_bytes + 64 * part))
 
+    # With eight levels the first level's sum needs no masking: each later level shifts the index
+    # right by one and replaces bit 7 of every byte, so the seven low bits of the first sum leave
+    # their byte one by one through bit 0, land on bit 7 of the byte below and are overwritten there.
+    # Six-level kernels keep the mask: two of those bits would stay below the index.
+    first_level_masked = depth < 8
+
     def levels_seven_bit(rows):
         for d in range(depth):
             e("  s_set_gpr_idx_idx s%d" % (rows + 2 * d))
+            if d == 0 and not first_level_masked:
+                e("  v_add_u32_e64 v3, v%d, s%d" % (b0, rows + 2 * d + 1))
+                continue
             e("  v_add_u32_e64 v4, v%d, s%d" % (b0, rows + 2 * d + 1))
             if d == 0:
                 e("  v_and_b32_e32 v3, s22, v4")
@@ -143,6 +152,9 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed):
             e("  v_xor_b32_e64 v4, v%d, s%d" % (b0, level + 1))       # x = bin ^ xorMask
             e("  v_or_b32_e32 v5, s22, v4")
             e("  v_subrev_u32_e32 v5, s%d, v5" % (level + 2))         # (x | 0x80) - (splitIdx & 0x7f), per byte
+            if d == 0 and not first_level_masked:
+                e("  v_bitop3_b32 v3, s%d, v4, v5 bitop3:0xe8" % (level + 3))  # majority
+                continue
             e("  v_bitop3_b32 v4, s%d, v4, v5 bitop3:0xe8" % (level + 3))  # majority
             if d == 0:
                 e("  v_and_b32_e32 v3, s22, v4")
