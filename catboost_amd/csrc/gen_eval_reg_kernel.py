@@ -109,16 +109,18 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed):
         lane l of wave w writes 16 bytes at lds_offset + w * 1024 + l * 16 (M0 holds the wave's
         base). M0 doubles as the VGPR index register, so its index-mode value is put back after."""
         e("  s_add_u32 m0, s100, %d" % lds_offset)
-        e("  s_nop 0")
+        # the thread's offset moves on to the next piece of the table; the instruction also fills the
+        # wait state that the M0 write needs before the copy
+        e("  v_add_u32_e32 v2, 0x%x, v2" % row_bytes)
         e("  global_load_lds_dwordx4 v2, s[26:27]")
-        e("  s_add_u32 s26, s26, %d" % row_bytes)
-        e("  s_addc_u32 s27, s27, 0")
 
     def add_leaf_values():
+        # sum + leaf as 1.0 * leaf + sum: the same single rounding, and with a constant in src0 the
+        # instruction does not depend on the register index that the levels leave in M0
         for j in range(4):
             for k in range(pitch):
-                e("  v_add_f64 v[%d:%d], v[%d:%d], v[%d:%d]" % (ac(j, k), ac(j, k) + 1, ac(j, k), ac(j, k) + 1,
-                                                                 lv(j, k), lv(j, k) + 1))
+                e("  v_fma_f64 v[%d:%d], 1.0, v[%d:%d], v[%d:%d]" % (ac(j, k), ac(j, k) + 1, lv(j, k), lv(j, k) + 1,
+                                                                      ac(j, k), ac(j, k) + 1))
 
     def load_rows(regs, tree):
         """Level table of tree `tree` (counted from the table position in s[6:7]) -> registers."""
@@ -175,7 +177,8 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed):
     e("  v_lshrrev_b32_e32 v5, 6, v0")
     e("  v_and_b32_e32 v1, 63, v0")
     e("  v_lshlrev_b32_e32 v1, 2, v1")           # lane * 4: offset inside a bucket's 256 bytes
-    e("  v_lshlrev_b32_e32 v2, 4, v0")           # thread * 16: offset of the thread's piece of a copy
+    e("  v_lshlrev_b32_e32 v2, 4, v0")           # thread * 16: offset of the thread's piece of a copy,
+    e("  v_subrev_u32_e32 v2, 0x%x, v2" % row_bytes)  # one piece back: every copy steps forward first
     # gfx940 family: a lane read needs one wait state behind the VALU write of its source register;
     # the three instructions above and the s_nop keep it well clear
     e("  s_nop 1")
@@ -232,7 +235,6 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed):
                 e("%s_j:" % label)
             else:
                 levels_seven_bit(rows)
-            e("  s_set_gpr_idx_idx 0")
             # previous tree's leaf values have arrived (and so has the next tree's row)
             e("  s_waitcnt lgkmcnt(0)")
             add_leaf_values()

@@ -997,7 +997,11 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         m.Oblivious && m.MaxDepth <= 8 && TreeCount > 0
             ? PickRegVariant(m.LayoutBuckets, static_cast<uint32_t>(m.Dim), m.MaxDepth, !m.PackedSevenBit)
             : nullptr;
-    if (regEnabled && variant) {
+    // a thread's 32-bit offset walks through the leaf table of a launch while it is copied to LDS
+    const bool regTableAddressable =
+        variant && (TreeCount / RegTreeBlock(*variant) + 3) * RegTreeBlock(*variant) * variant->Leaves * variant->Pitch * 8 <
+                       (uint64_t(1) << 32) - (1u << 20);
+    if (regEnabled && variant && regTableAddressable) {
         HIP_CHECK(hipModuleLoadData(&m.RegModule, kEvalRegCodeObject));
         HIP_CHECK(hipModuleGetFunction(&m.RegFunction, m.RegModule, variant->Name));
         const uint32_t block = RegTreeBlock(*variant);
