@@ -659,6 +659,44 @@ def test_plain_c_client_of_the_c_abi(golden_dir):
     assert abs(float(out.decode().split()[0]) - rm.NUMERIC_ONLY_EXPECTED[0]) < 1e-15
 
 
+def test_client_of_the_reference_wrapper_header(golden_dir):
+    """A C++ program written against the reference's own wrapped_calcer.h and c_api.h
+    (catboost/libs/model_interface), compiled unchanged and linked against this library: every
+    way that wrapper calls the model gives the goldens of the reference's own tests
+    (catboost/rust-package/src/model.rs:475-520, catboost/libs/model_interface/ut)."""
+    import subprocess
+
+    exe = os.path.join(os.path.dirname(__file__), "bin", "wrapped_calcer_client")
+    if not os.path.exists(exe):
+        pytest.skip("tests/bin/wrapped_calcer_client is not built (run __graft_entry__.build() where the reference is)")
+
+    def run(model, floats, cats):
+        text = "".join(" ".join("%r" % float(v) for v in f) + " | " + " ".join(c) + "\n" for f, c in zip(floats, cats))
+        out = subprocess.check_output([exe, os.path.join(golden_dir, model)], input=text.encode(), timeout=120)
+        lines = {}
+        for line in out.decode().splitlines():
+            name, _, rest = line.partition(" ")
+            lines[name] = rest
+        return lines
+
+    got = run("rust_tmp_model.cbm", rm.RUST_FLOATS, rm.RUST_CATS)
+    assert got["counts"].split()[1:] == ["3", "1", "0", "0"]
+    assert int(got["evaluators"]) >= 1
+    assert got["short_document"] == "refused" and got["missing_key"] == "[]"
+    for name in ("single", "batch", "hashed", "from_memory", "after_error"):
+        _close(np.array([float(v) for v in got[name].split()]), rm.RUST_EXPECTED)
+
+    got = run("numeric_only_model.cbm", rm.NUMERIC_ONLY_ROWS, [[] for _ in rm.NUMERIC_ONLY_ROWS])
+    assert got["counts"].split()[2] == "0"
+    for name in ("single", "batch", "hashed", "flat_single", "flat", "flat_transposed", "from_memory", "after_error"):
+        _close(np.array([float(v) for v in got[name].split()]), rm.NUMERIC_ONLY_EXPECTED)
+
+    # a model with CTR features through the same wrapper
+    got = run("features_num_cat__dataset_adult.cbm", rm.RUST_ADULT_FLOATS, rm.RUST_ADULT_CATS)
+    for name in ("single", "batch", "hashed", "from_memory"):
+        _close(np.array([float(v) for v in got[name].split()]), rm.RUST_ADULT_EXPECTED)
+
+
 # ----------------------------------------------------------------------------- error paths ----
 
 def test_error_paths(golden_dir):
