@@ -27,3 +27,6 @@ echo "built $OUT/standalone_eval"
 # the exponent of the prediction types (fmath::expd_v, AVX2 path as on the hosts this runs on)
 g++ -std=c++17 -O2 -mavx2 -w -I "$R" "$HERE/ref_fmath_main.cpp" -o "$OUT/fmath_exp"
 echo "built $OUT/fmath_exp"
+# the CTR calculator of exported models (model_export/resources/ctr_structs.cpp + ctr_calcer.cpp)
+g++ -std=c++17 -O2 -w -I "$R" "$HERE/ref_ctr_main.cpp" -o "$OUT/ctr_calc"
+echo "built $OUT/ctr_calc"

@@ -26,13 +26,20 @@
  * raw-split brute force below. CTR features: the golden predictions of the JVM, Rust and node
  * binding tests for models with CTRs of kinds Borders and Counter (reproduced to the last bit) and
  * the .NET mushroom test (8124 labels; projections of up to four categorical features, some with
- * a one-hot split).
+ * a one-hot split); and, for all six CTR kinds, tables with up to five target classes and
+ * projections with float splits (also past a feature's first 254 borders) and one-hot splits, the
+ * CTR calculator that the reference ships for exported models (model_export/resources/ctr_structs.cpp
+ * + ctr_calcer.cpp, built where they lie by oracle/build_ref.sh into oracle/_ref/ctr_calc): its values
+ * on the seeded models of tests/ctr_models.py are stored in tests/golden/ctr_ref_vectors.npz and
+ * reproduced bit for bit. That calculator answers an unknown hash with Calc(0, 0) for every kind,
+ * the evaluator's TStaticCtrProvider with Calc(0, denominator) for Counter and FeatureFreq
+ * (static_ctr_provider.cpp:63-75); this one case rests on the adult goldens (Counter CTRs, unknown
+ * categories) alone.
  * Parity unpinned (followed by reading only, cross-checked by the brute force): the NaN gating
- * "HasNans && treatment != AsIs", >254-border buckets combined with one-hot XorMask, and the
- * leaf numbering of non-symmetric multi-dimensional models; for CTRs the kinds Buckets,
- * BinarizedTargetMeanValue, FloatTargetMeanValue and FeatureFreq, float splits inside a projection
- * and the Borders branch for more than two target classes (the cloudness fixture has such CTRs
- * but no reference output): no fixture with reference outputs covers them.
+ * "HasNans && treatment != AsIs", >254-border buckets combined with one-hot XorMask, the
+ * leaf numbering of non-symmetric multi-dimensional models, and for CTR projections the table
+ * TStaticCtrProvider::SetupBinFeatureIndexes builds from a split to its (bin, value)
+ * (static_ctr_provider.cpp:139-170; the fixture generator restates it a second time in Python).
  */
 #include "cb_oracle.h"
 

@@ -13,6 +13,7 @@ from catboost_amd import synthetic as syn
 from oracle import model_builder as mb
 from oracle.cbm_reader import read_cbm, read_cbm_file
 from oracle.oracle import OracleModel, cat_feature_hash_signed
+from tests import ctr_models
 from tests import refmodels as rm
 from tests.test_oracle import _random_flat_data, _random_oblivious
 
@@ -294,6 +295,59 @@ def test_ctr_models_against_the_oracle(golden_dir, name, docs):
     half = o.tree_count // 2
     _close(g.calc_flat(flat, tree_start=half, tree_end=o.tree_count),
            o.calc(flat, tree_start=half, tree_end=o.tree_count))
+
+
+@pytest.mark.parametrize("seed", [seed for seed, _ in ctr_models.CASES])
+@pytest.mark.parametrize("tile", ["1", "0"])
+def test_synthetic_ctr_models_of_every_kind(golden_dir, monkeypatch, seed, tile):
+    """Synthetic models with all six CTR types, tables with up to five target classes and projections
+    over categorical features, float splits and one-hot splits (tests/ctr_models.py), through both CTR
+    kernels. The CTR buckets of the quantized documents must equal, bit for bit, the bins of the CTR
+    values that the reference's own calculator printed for the stored documents; on more documents the
+    oracle (which reproduces those values) is the checker."""
+    monkeypatch.setenv("CATBOOST_AMD_CTR_TILE", tile)
+    path = os.path.join(golden_dir, "synthetic_ctr_%d.cbm" % seed)
+    m = read_cbm_file(path)
+    o = OracleModel(m)
+    g = cb.ModelCalcer(path)
+    ref = np.load(os.path.join(golden_dir, "ctr_ref_vectors.npz"))
+    floats, cats = ref["floats_%d" % seed], ref["cats_%d" % seed]
+    bins = g.quantize_hashed(floats, cats)
+    np.testing.assert_array_equal(bins, o.binarize(floats, cats, layout="split"))
+    # straight against the reference's values: a CTR bucket holds the count of borders below the value
+    # (one bucket per CTR here, none has more than 254 borders)
+    doc_major = np.zeros((floats.shape[0], o.bucket_count), np.uint8)
+    for start in range(0, floats.shape[0], 128):
+        dc = min(128, floats.shape[0] - start)
+        doc_major[start:start + dc] = bins[start * o.bucket_count:(start + dc) * o.bucket_count].reshape(-1, dc).T
+    first = o.bucket_count - len(m["ctr_features"])
+    values, comparable = ref["ctrs_%d" % seed], ref["comparable_%d" % seed]
+    for i, c in enumerate(m["ctr_features"]):
+        expected = (values[i][:, None] > np.asarray(c["borders"], np.float32)[None, :]).sum(axis=1)
+        np.testing.assert_array_equal(doc_major[comparable[i], first + i], expected[comparable[i]])
+    _close(g.calc_hashed(floats, cats), o.calc(floats, cats, layout="split"))
+    # more documents, ragged tail, every host layout
+    model, known = ctr_models.random_ctr_model(seed, **dict(ctr_models.CASES)[seed])
+    for docs in (1, 3000):
+        floats, cats = ctr_models.random_documents(model, known, docs, 50 + docs)
+        expected = o.calc(floats, cats, layout="split")
+        np.testing.assert_array_equal(g.quantize_hashed(floats, cats), o.binarize(floats, cats, layout="split"))
+        _close(g.calc_hashed(floats, cats), expected)
+        flat = rm.flat_rows(m, floats, cats)
+        _close(g.calc_flat(flat), expected)
+        _close(g.calc_flat_transposed(np.ascontiguousarray(flat.T)), expected)
+        np.testing.assert_array_equal(g.calc_leaf_indexes_flat(flat), o.leaf_indexes(flat))
+
+
+def test_synthetic_ctr_model_survives_save_and_load(golden_dir, tmp_path):
+    """The library's own writer keeps CTR features of every kind: load, save, load again, same bins."""
+    path = os.path.join(golden_dir, "synthetic_ctr_5.cbm")
+    ref = np.load(os.path.join(golden_dir, "ctr_ref_vectors.npz"))
+    floats, cats = ref["floats_5"], ref["cats_5"]
+    g = cb.ModelCalcer(path)
+    again = cb.ModelCalcer(buffer=g.save_to_buffer())
+    np.testing.assert_array_equal(g.quantize_hashed(floats, cats), again.quantize_hashed(floats, cats))
+    np.testing.assert_array_equal(g.calc_hashed(floats, cats), again.calc_hashed(floats, cats))
 
 
 def test_ctr_kernel_without_the_staged_tile(golden_dir, monkeypatch):

@@ -8,9 +8,10 @@ import numpy as np
 import pytest
 
 from oracle import model_builder as mb
-from oracle.cbm_reader import read_cbm, read_cbm_file
+from oracle.cbm_reader import ctr_base_key, read_cbm, read_cbm_file
 from oracle.oracle import (OracleModel, cat_feature_hash_signed, city_hash64,
                            integer_cat_feature_hash)
+from tests import cbm_writer, ctr_models
 from tests import refmodels as rm
 
 
@@ -275,6 +276,86 @@ def test_ctr_models_against_the_raw_definition(golden_dir, name):
     # known and unknown categories both occur
     ctrs = o.ctrs(floats, cats, layout="split")
     assert all(len(np.unique(row)) > 1 for row in ctrs)
+
+
+@pytest.mark.parametrize("seed", [seed for seed, _ in ctr_models.CASES])
+def test_ctr_values_match_the_reference_ctr_calculator(golden_dir, seed):
+    """CTR values on synthetic models with all six CTR types, tables with up to five target classes and
+    projections over categorical features, float splits (also beyond the first 254 borders of a feature)
+    and one-hot splits, against what the reference's own calculator for exported models printed
+    (model_export/resources/ctr_calcer.cpp, run by tests/golden/make_ctr_vectors.py): bit for bit. Pairs
+    where that calculator and the evaluator differ by design (a hash that a Counter or FeatureFreq
+    table does not hold) are excluded by the stored mask and checked against Calc(0, denominator)."""
+    g = np.load(os.path.join(golden_dir, "ctr_ref_vectors.npz"))
+    m = read_cbm_file(os.path.join(golden_dir, "synthetic_ctr_%d.cbm" % seed))
+    o = OracleModel(m)
+    floats, cats = g["floats_%d" % seed], g["cats_%d" % seed]
+    got = o.ctrs(floats, cats, layout="split")
+    expected, comparable = g["ctrs_%d" % seed], g["comparable_%d" % seed]
+    assert comparable.mean() > 0.7
+    np.testing.assert_array_equal(got.view(np.uint32)[comparable], expected.view(np.uint32)[comparable])
+    tables = {ctr_base_key(t["base"]): t for t in m["ctr_tables"]}
+    for i, c in enumerate(m["ctr_features"]):
+        rest = ~comparable[i]
+        if rest.any():
+            assert c["base"]["ctr_type"] in (4, 5)
+            denominator = np.float32(tables[ctr_base_key(c["base"])]["counter_denominator"])
+            value = (np.float32(c["prior_num"]) / (denominator + np.float32(c["prior_denom"])) +
+                     np.float32(c["shift"])) * np.float32(c["scale"])
+            np.testing.assert_array_equal(got[i][rest], np.full(int(rest.sum()), value, np.float32))
+    # every CTR type and both kinds of split occur in the cases taken together
+    assert {c["base"]["ctr_type"] for c in m["ctr_features"]} <= set(range(6))
+    # the block path over these models equals the per-document definition
+    pred = o.calc(floats, cats, layout="split")
+    bf, bf_idx = o.bruteforce(floats, cats, layout="split")
+    np.testing.assert_array_equal(pred, bf)
+    np.testing.assert_array_equal(o.leaf_indexes(floats, cats, layout="split"), bf_idx)
+
+
+def test_synthetic_ctr_cases_cover_every_kind(golden_dir):
+    types, classes, float_splits, one_hot_splits, wide = set(), set(), 0, 0, 0
+    for seed, kwargs in ctr_models.CASES:
+        path = os.path.join(golden_dir, "synthetic_ctr_%d.cbm" % seed)
+        m = read_cbm_file(path)
+        # the committed files are what the seeded generator and the writer produce
+        with open(path, "rb") as f:
+            assert f.read() == cbm_writer.write_cbm(ctr_models.random_ctr_model(seed, **kwargs)[0])
+        borders = {f["index"]: f["borders"] for f in m["float_features"]}
+        for c in m["ctr_features"]:
+            types.add(c["base"]["ctr_type"])
+            float_splits += len(c["base"]["float_splits"])
+            one_hot_splits += len(c["base"]["one_hot_splits"])
+            wide += sum(int(np.searchsorted(borders[f], b)) >= 254 for f, b in c["base"]["float_splits"])
+        for t in m["ctr_tables"]:
+            if t["base"]["ctr_type"] in (0, 1):
+                classes.add((t["base"]["ctr_type"], t["target_classes_count"]))
+    assert types == set(range(6)) and float_splits > 10 and one_hot_splits > 5 and wide > 0
+    assert {(0, 2), (0, 3), (0, 5)} <= classes and len([c for c in classes if c[0] == 1]) >= 2
+
+
+def test_python_cbm_writer_round_trips_the_fixtures(golden_dir):
+    """tests/cbm_writer.py writes what oracle/cbm_reader.py reads, on every fixture of the reference."""
+    def same(a, b):
+        if isinstance(a, dict):
+            assert a.keys() == b.keys()
+            for k in a:
+                same(a[k], b[k])
+        elif isinstance(a, (list, tuple)):
+            assert len(a) == len(b)
+            for x, y in zip(a, b):
+                same(x, y)
+        elif isinstance(a, np.ndarray):
+            assert a.dtype == b.dtype and a.shape == b.shape and a.tobytes() == b.tobytes()
+        else:
+            assert a == b
+
+    names = ["numeric_only_model.cbm", "rust_tmp_model.cbm", "iris_model.cbm", "boston_housing_model.cbm"]
+    for name in names + rm.CTR_FIXTURES:
+        m = read_cbm_file(os.path.join(golden_dir, name))
+        again = read_cbm(cbm_writer.write_cbm(m))
+        m.pop("repacked_bins_in_file")
+        again.pop("repacked_bins_in_file")
+        same(m, again)
 
 
 def test_not_a_model_is_rejected(golden_dir):
