@@ -150,6 +150,7 @@ def load_library():
         "CbHipSynchronize": (ctypes.c_bool, [vp, vp]),
         "CbHipLastKernelTimes": (ctypes.c_bool, [vp, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float)]),
         "CbHipGetEvaluator": (vp, [vp]),
+        "CbHipSetFeatureLayout": (ctypes.c_bool, [vp, vp, sz, vp, sz, vp, sz]),
         "CbHipLoadModelFromArrays": (ctypes.c_bool, [vp, ctypes.POINTER(ModelArrays)]),
         "CbHipBuildObliviousModel": (ctypes.c_bool, [vp, ctypes.POINTER(ModelArrays), ctypes.c_int32, vp, vp, vp]),
         "CbHipBuildNonSymmetricModel": (ctypes.c_bool, [vp, ctypes.POINTER(ModelArrays), ctypes.c_int32, vp, vp, vp, vp, vp, vp, vp]),
@@ -523,6 +524,17 @@ class ModelCalcer:
 
     def set_model_info(self, key, value):
         _check(self._lib.CbHipSetModelInfo(self._h, key.encode(), value.encode()))
+
+    def set_feature_layout(self, float_feature_indexes=None, cat_feature_indexes=None, flat_indexes=None):
+        """TFeatureLayout (evaluation_interface.h:17-69): a feature at model position p is read at
+        list[p] of the caller's data; None leaves a kind of position as the model has it."""
+        lists = [None if v is None else np.ascontiguousarray(v, np.uint32)
+                 for v in (float_feature_indexes, cat_feature_indexes, flat_indexes)]
+        args = []
+        for a in lists:
+            # a defined but empty list still needs a non-null pointer
+            args += [None, 0] if a is None else [a.ctypes.data if a.size else ctypes.addressof(ctypes.c_uint32()), a.size]
+        _check(self._lib.CbHipSetFeatureLayout(self._h, *args))
 
     # ---- evaluator selection
     def enable_gpu_evaluation(self, device_id=0):

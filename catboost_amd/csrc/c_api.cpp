@@ -34,6 +34,7 @@ struct TModelHandle {
     std::mutex EvaluatorLock;
     int DeviceId = 0;
     EApiPredictionType PredictionType = APT_RAW_FORMULA_VAL;
+    TFeatureLayout Layout;  // IModelEvaluator::SetFeatureLayout, evaluation_interface.h:82
 
     void ResetEvaluator() {
         std::lock_guard<std::mutex> g(EvaluatorLock);
@@ -44,7 +45,7 @@ struct TModelHandle {
         std::lock_guard<std::mutex> g(EvaluatorLock);
         if (!Evaluator) {
             Model.EnsureSupported();
-            Evaluator.reset(new THipEvaluator(Model.Trees, DeviceId, &Model.CtrTables));
+            Evaluator.reset(new THipEvaluator(Model.Trees, DeviceId, &Model.CtrTables, &Layout));
         }
         return *Evaluator;
     }
@@ -879,6 +880,40 @@ CbHipEvaluatorHandle* CbHipGetEvaluator(void* modelHandle) {
         LastError = e.what();
     }
     return nullptr;
+}
+
+bool CbHipSetFeatureLayout(void* modelHandle, const uint32_t* floatFeatureIndexes, size_t floatFeatureIndexesSize,
+                           const uint32_t* catFeatureIndexes, size_t catFeatureIndexesSize, const uint32_t* flatIndexes,
+                           size_t flatIndexesSize) {
+    return Guard([&] {
+        TModelHandle* h = H(modelHandle);
+        TFeatureLayout layout;
+        if (floatFeatureIndexes != nullptr) {
+            layout.HasFloatFeatureIndexes = true;
+            layout.FloatFeatureIndexes.assign(floatFeatureIndexes, floatFeatureIndexes + floatFeatureIndexesSize);
+        }
+        if (catFeatureIndexes != nullptr) {
+            layout.HasCatFeatureIndexes = true;
+            layout.CatFeatureIndexes.assign(catFeatureIndexes, catFeatureIndexes + catFeatureIndexesSize);
+        }
+        if (flatIndexes != nullptr) {
+            layout.HasFlatIndexes = true;
+            layout.FlatIndexes.assign(flatIndexes, flatIndexes + flatIndexesSize);
+        }
+        // every position the evaluator would read must have an entry; checked now, not at the next call
+        for (const auto& f : h->Model.Trees.FloatFeatures) {
+            if (f.UsedInModel()) {
+                layout.Remap(f);
+            }
+        }
+        for (const auto& c : h->Model.Trees.CatFeatures) {
+            if (c.UsedInModel) {
+                layout.Remap(c);
+            }
+        }
+        h->ResetEvaluator();
+        h->Layout = std::move(layout);
+    });
 }
 
 bool CbHipLoadModelFromArrays(void* modelHandle, const CbHipModelArrays* model) {

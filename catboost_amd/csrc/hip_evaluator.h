@@ -35,7 +35,10 @@ class THipEvaluator {
 public:
     // Uploads the model tables (model upload of cuda/evaluator.cpp:30-84, re-laid out as SoA).
     // `ctrTables`: the tables of the model's static CTR provider; needed when the model has CTR features.
-    THipEvaluator(const TModelTrees& trees, int deviceId, const std::vector<TCtrValueTable>* ctrTables = nullptr);
+    // `layout`: where the model's features sit in the callers' data (TFeatureLayout,
+    // evaluation_interface.h:17-69); it is resolved into the device tables here, so it costs nothing per call
+    THipEvaluator(const TModelTrees& trees, int deviceId, const std::vector<TCtrValueTable>* ctrTables = nullptr,
+                  const TFeatureLayout* layout = nullptr);
     ~THipEvaluator();
     THipEvaluator(const THipEvaluator&) = delete;
     THipEvaluator& operator=(const THipEvaluator&) = delete;

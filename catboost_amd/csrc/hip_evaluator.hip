@@ -320,12 +320,56 @@ void BuildLevelOrderTrees(const TModelTrees& trees, int dim, const std::vector<u
     }
 }
 
+// Where the kernels read the model's features in a caller's data: the positions stored in the model, or
+// those positions sent through a feature layout. The vector sizes a caller must provide follow the
+// reference without a layout (the last feature of each list decides, model.h:494-541) and are the
+// largest position read plus one with a layout.
+struct TFeaturePositions {
+    const TFeatureLayout* Layout = nullptr;
+    size_t FlatVectorSize = 0;
+    size_t MinFloatSize = 0;
+    size_t MinCatSize = 0;
+
+    TFeaturePosition Of(const TFloatFeature& f) const {
+        return Layout ? Layout->Remap(f) : TFeaturePosition{f.Index, f.FlatIndex};
+    }
+    TFeaturePosition Of(const TCatFeature& c) const {
+        return Layout ? Layout->Remap(c) : TFeaturePosition{c.Index, c.FlatIndex};
+    }
+
+    TFeaturePositions(const TModelTrees& trees, const TFeatureLayout* layout)
+        : Layout(layout && layout->Defined() ? layout : nullptr)
+    {
+        if (!Layout) {
+            FlatVectorSize = trees.GetFlatFeatureVectorExpectedSize();
+            MinFloatSize = trees.MinimalSufficientFloatFeaturesVectorSize;
+            MinCatSize = trees.MinimalSufficientCatFeaturesVectorSize;
+            return;
+        }
+        for (const auto& f : trees.FloatFeatures) {
+            if (f.UsedInModel() && f.Index >= 0 && f.FlatIndex >= 0) {
+                const TFeaturePosition p = Of(f);
+                FlatVectorSize = std::max(FlatVectorSize, static_cast<size_t>(p.FlatIndex) + 1);
+                MinFloatSize = std::max(MinFloatSize, static_cast<size_t>(p.Index) + 1);
+            }
+        }
+        for (const auto& c : trees.CatFeatures) {
+            if (c.UsedInModel && c.Index >= 0 && c.FlatIndex >= 0) {
+                const TFeaturePosition p = Of(c);
+                FlatVectorSize = std::max(FlatVectorSize, static_cast<size_t>(p.FlatIndex) + 1);
+                MinCatSize = std::max(MinCatSize, static_cast<size_t>(p.Index) + 1);
+            }
+        }
+    }
+};
+
 // Device tables of the model's CTR features (TStaticCtrProvider, catboost/libs/model/static_ctr_provider.cpp):
 // per feature a descriptor and its projection (SetupBinFeatureIndexes, :142-178, resolved to bucket
 // numbers and input columns), all index buckets and all rows. Every row index and class index the kernel
 // can reach is checked here, so a damaged model fails at load instead of reading out of bounds.
 // Appends one bucket entry per 254 borders of a CTR feature to the binarize bucket tables.
-void BuildCtrTables(const TModelTrees& trees, const std::vector<TCtrValueTable>& tables, std::vector<uint32_t>* srcFlat,
+void BuildCtrTables(const TModelTrees& trees, const TFeaturePositions& positions,
+                    const std::vector<TCtrValueTable>& tables, std::vector<uint32_t>* srcFlat,
                     std::vector<uint32_t>* srcSplit, std::vector<uint32_t>* offsets, std::vector<uint32_t>* flags,
                     std::vector<uint32_t>* values, TDeviceVec<uint32_t>* featuresOut, TDeviceVec<uint32_t>* itemsOut,
                     TDeviceVec<uint32_t>* indexOut, TDeviceVec<uint32_t>* blobOut, TDeviceVec<uint32_t>* catColumnsFlatOut,
@@ -429,18 +473,19 @@ void BuildCtrTables(const TModelTrees& trees, const std::vector<TCtrValueTable>&
             }
             CBAMD_ENSURE(cat != nullptr && cat->FlatIndex >= 0 && cat->Index >= 0,
                          "CTR projection refers to an unknown or unused categorical feature");
-            CBAMD_ENSURE(static_cast<size_t>(cat->FlatIndex) < trees.GetFlatFeatureVectorExpectedSize() &&
-                             static_cast<size_t>(cat->Index) < trees.MinimalSufficientCatFeaturesVectorSize,
+            const TFeaturePosition at = positions.Of(*cat);
+            CBAMD_ENSURE(static_cast<size_t>(at.FlatIndex) < positions.FlatVectorSize &&
+                             static_cast<size_t>(at.Index) < positions.MinCatSize,
                          "categorical feature position exceeds the model's feature vector size");
             uint32_t tileRow = 0;
-            while (tileRow < catColumnsSplit.size() && catColumnsSplit[tileRow] != static_cast<uint32_t>(cat->Index)) {
+            while (tileRow < catColumnsSplit.size() && catColumnsSplit[tileRow] != static_cast<uint32_t>(at.Index)) {
                 ++tileRow;
             }
             if (tileRow == catColumnsSplit.size()) {
-                catColumnsFlat.push_back(static_cast<uint32_t>(cat->FlatIndex));
-                catColumnsSplit.push_back(static_cast<uint32_t>(cat->Index));
+                catColumnsFlat.push_back(static_cast<uint32_t>(at.FlatIndex));
+                catColumnsSplit.push_back(static_cast<uint32_t>(at.Index));
             }
-            items.push_back({dev::kCtrItemCat, static_cast<uint32_t>(cat->FlatIndex), static_cast<uint32_t>(cat->Index), tileRow});
+            items.push_back({dev::kCtrItemCat, static_cast<uint32_t>(at.FlatIndex), static_cast<uint32_t>(at.Index), tileRow});
         }
         for (const auto& split : ctr.Base.Projection.BinFeatures) {
             bool found = false;
@@ -668,9 +713,11 @@ struct THipEvaluator::TImpl {
     hipStream_t Pick(void* stream) const { return stream ? static_cast<hipStream_t>(stream) : Stream; }
 };
 
-THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::vector<TCtrValueTable>* ctrTables)
+THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::vector<TCtrValueTable>* ctrTables,
+                             const TFeatureLayout* layout)
     : Impl(new TImpl)
 {
+    const TFeaturePositions positions(trees, layout);
     const int deviceCount = GetHipDeviceCount();
     CBAMD_ENSURE(deviceCount > 0, "no HIP device found: the HIP evaluator needs an AMD GPU");
     CBAMD_ENSURE(deviceId >= 0 && deviceId < deviceCount, "HIP device id out of range");
@@ -692,9 +739,9 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
     m.Oblivious = trees.IsOblivious();
     m.RealBucketCount = BucketCount;
     m.LayoutBuckets = std::max<uint32_t>(1, BucketCount);
-    m.FlatVectorSize = trees.GetFlatFeatureVectorExpectedSize();
-    m.MinFloatSize = trees.MinimalSufficientFloatFeaturesVectorSize;
-    m.MinCatSize = trees.MinimalSufficientCatFeaturesVectorSize;
+    m.FlatVectorSize = positions.FlatVectorSize;
+    m.MinFloatSize = positions.MinFloatSize;
+    m.MinCatSize = positions.MinCatSize;
     m.HasCats = trees.UsedCatFeaturesCount > 0;
     m.Dim = trees.ApproxDimension;
     m.Scale = trees.Scale;
@@ -717,7 +764,8 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         CBAMD_ENSURE(f.FlatIndex >= 0 && f.Index >= 0, "float feature without a position");
         // the vector sizes come from the last feature of each list (as in the reference); a feature
         // that points past them would make the kernels read behind a caller's row
-        CBAMD_ENSURE(static_cast<size_t>(f.FlatIndex) < m.FlatVectorSize && static_cast<size_t>(f.Index) < m.MinFloatSize,
+        const TFeaturePosition at = positions.Of(f);
+        CBAMD_ENSURE(static_cast<size_t>(at.FlatIndex) < m.FlatVectorSize && static_cast<size_t>(at.Index) < m.MinFloatSize,
                      "float feature position exceeds the model's feature vector size");
         for (size_t begin = 0; begin < f.Borders.size(); begin += kMaxValuesPerBin) {
             const size_t end = std::min(begin + kMaxValuesPerBin, f.Borders.size());
@@ -734,8 +782,8 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
                 values.push_back(bits);
             }
             offsets.push_back(static_cast<uint32_t>(values.size()));
-            srcFlat.push_back(static_cast<uint32_t>(f.FlatIndex));
-            srcSplit.push_back(static_cast<uint32_t>(f.Index));
+            srcFlat.push_back(static_cast<uint32_t>(at.FlatIndex));
+            srcSplit.push_back(static_cast<uint32_t>(at.Index));
             const bool nanToInf = f.HasNans && f.NanValueTreatment == ENanValueTreatment::AsTrue;
             flags.push_back(nanToInf ? dev::kBucketFlagNanToInf : 0);
         }
@@ -749,7 +797,8 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         }
         CBAMD_ENSURE(cat != nullptr, "one-hot feature refers to an unknown or unused categorical feature");
         CBAMD_ENSURE(cat->FlatIndex >= 0 && cat->Index >= 0, "categorical feature without a position");
-        CBAMD_ENSURE(static_cast<size_t>(cat->FlatIndex) < m.FlatVectorSize && static_cast<size_t>(cat->Index) < m.MinCatSize,
+        const TFeaturePosition at = positions.Of(*cat);
+        CBAMD_ENSURE(static_cast<size_t>(at.FlatIndex) < m.FlatVectorSize && static_cast<size_t>(at.Index) < m.MinCatSize,
                      "categorical feature position exceeds the model's feature vector size");
         for (size_t begin = 0; begin < oh.Values.size(); begin += kMaxValuesPerBin) {
             const size_t end = std::min(begin + kMaxValuesPerBin, oh.Values.size());
@@ -757,8 +806,8 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
                 values.push_back(static_cast<uint32_t>(oh.Values[i]));
             }
             offsets.push_back(static_cast<uint32_t>(values.size()));
-            srcFlat.push_back(static_cast<uint32_t>(cat->FlatIndex));
-            srcSplit.push_back(static_cast<uint32_t>(cat->Index));
+            srcFlat.push_back(static_cast<uint32_t>(at.FlatIndex));
+            srcSplit.push_back(static_cast<uint32_t>(at.Index));
             flags.push_back(dev::kBucketFlagOneHot);
         }
     }
@@ -766,7 +815,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
     CBAMD_ENSURE(m.BinarizeBuckets == trees.CtrFirstBucket, "internal error: bucket count mismatch");
     if (!trees.CtrFeatures.empty()) {
         CBAMD_ENSURE(ctrTables != nullptr, "Model has CTR features but no tables of learned statistics");
-        BuildCtrTables(trees, *ctrTables, &srcFlat, &srcSplit, &offsets, &flags, &values, &m.CtrFeatures, &m.CtrItems,
+        BuildCtrTables(trees, positions, *ctrTables, &srcFlat, &srcSplit, &offsets, &flags, &values, &m.CtrFeatures, &m.CtrItems,
                        &m.CtrIndexBuckets, &m.CtrBlob, &m.CtrCatColumnsFlat, &m.CtrCatColumnsSplit, &m.CtrCatColumnCount);
         m.CtrCount = static_cast<uint32_t>(trees.CtrFeatures.size());
         const char* tileSwitch = std::getenv("CATBOOST_AMD_CTR_TILE");

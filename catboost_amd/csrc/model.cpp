@@ -271,6 +271,34 @@ void TFullModel::EnsureSupported() const {
     CBAMD_ENSURE(Trees.EmbeddingFeatureCount == 0, "Model contains embedding features, HIP evaluation impossible");
 }
 
+namespace {
+
+int RemapOne(bool defined, const std::vector<uint32_t>& list, int position, const char* what) {
+    if (!defined) {
+        return position;
+    }
+    CBAMD_ENSURE(position >= 0 && static_cast<size_t>(position) < list.size(),
+                 "feature layout: " + what + " has no entry for position " + std::to_string(position));
+    CBAMD_ENSURE(list[position] <= 0x7fffffffu, "feature layout: position is too large");
+    return static_cast<int>(list[position]);
+}
+
+}  // namespace
+
+TFeaturePosition TFeatureLayout::Remap(const TFloatFeature& feature) const {
+    TFeaturePosition p;
+    p.Index = RemapOne(HasFloatFeatureIndexes, FloatFeatureIndexes, feature.Index, "FloatFeatureIndexes");
+    p.FlatIndex = RemapOne(HasFlatIndexes, FlatIndexes, feature.FlatIndex, "FlatIndexes");
+    return p;
+}
+
+TFeaturePosition TFeatureLayout::Remap(const TCatFeature& feature) const {
+    TFeaturePosition p;
+    p.Index = RemapOne(HasCatFeatureIndexes, CatFeatureIndexes, feature.Index, "CatFeatureIndexes");
+    p.FlatIndex = RemapOne(HasFlatIndexes, FlatIndexes, feature.FlatIndex, "FlatIndexes");
+    return p;
+}
+
 const TCtrValueTable* TFullModel::FindCtrTable(const TModelCtrBase& base) const {
     for (const auto& table : CtrTables) {
         if (table.ModelCtrBase == base) {

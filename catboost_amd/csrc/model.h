@@ -227,6 +227,29 @@ struct TModelTrees {
     void AddBinTree(const std::vector<int>& binSplits);
 };
 
+struct TFeaturePosition {  // features.h:16-48
+    int Index = -1;
+    int FlatIndex = -1;
+};
+
+// Where the model's features sit in a caller's data when that differs from the positions stored in
+// the model (NCB::NModelEvaluation::TFeatureLayout, evaluation_interface.h:17-69): a feature at model
+// position p is read at FloatFeatureIndexes[p] / CatFeatureIndexes[p] (separate float and categorical
+// arrays) or FlatIndexes[p] (flat vectors). A list that is not defined leaves its positions as they are.
+struct TFeatureLayout {
+    bool HasFloatFeatureIndexes = false;
+    bool HasCatFeatureIndexes = false;
+    bool HasFlatIndexes = false;
+    std::vector<uint32_t> FloatFeatureIndexes;
+    std::vector<uint32_t> CatFeatureIndexes;
+    std::vector<uint32_t> FlatIndexes;
+
+    bool Defined() const { return HasFloatFeatureIndexes || HasCatFeatureIndexes || HasFlatIndexes; }
+    // GetRemappedPosition; a position outside a defined list is an error (TVector::at there)
+    TFeaturePosition Remap(const TFloatFeature& feature) const;
+    TFeaturePosition Remap(const TCatFeature& feature) const;
+};
+
 struct TFullModel {
     TModelTrees Trees;
     std::map<std::string, std::string> ModelInfo;

@@ -139,6 +139,19 @@ bool CbHipLastKernelTimes(CbHipEvaluatorHandle* evaluator, float* binarizeMs, fl
  * the handle; invalidated by the next Load* / CbHipLoad* / CbHipBuild* call on it. */
 CbHipEvaluatorHandle* CbHipGetEvaluator(void* modelHandle);
 
+/* IModelEvaluator::SetFeatureLayout (catboost/libs/model/evaluation_interface.h:17-82; the reference's
+ * CUDA evaluator refuses layouts, cuda/evaluator.cpp:129,176): tells where the model's features sit in
+ * the caller's data. A feature whose position in the model is p is then read at floatFeatureIndexes[p]
+ * or catFeatureIndexes[p] of the separate float / categorical arrays, and at flatIndexes[p] of flat
+ * vectors (TFeatureLayout::GetRemappedPosition). A null list leaves those positions as the model has
+ * them; three nulls remove the layout. Every used feature needs an entry in a list that is given. The
+ * vector sizes every Calc* then asks for are the largest position read plus one. Applies to all later
+ * calls on the handle, host and device entry points alike (the handle's evaluator is rebuilt: pointers
+ * from CbHipGetEvaluator are invalidated); a Load* call keeps it. */
+bool CbHipSetFeatureLayout(void* modelHandle, const uint32_t* floatFeatureIndexes, size_t floatFeatureIndexesSize,
+                           const uint32_t* catFeatureIndexes, size_t catFeatureIndexesSize, const uint32_t* flatIndexes,
+                           size_t flatIndexesSize);
+
 /* Install a model given as raw tables (the AddBinTree / AddLeafValue route of TModelTrees,
  * catboost/libs/model/model.cpp:238-254). */
 bool CbHipLoadModelFromArrays(void* modelHandle, const CbHipModelArrays* model);

@@ -350,6 +350,61 @@ def test_synthetic_ctr_model_survives_save_and_load(golden_dir, tmp_path):
     np.testing.assert_array_equal(g.calc_hashed(floats, cats), again.calc_hashed(floats, cats))
 
 
+def test_feature_layout_remaps_positions(golden_dir):
+    """TFeatureLayout (evaluation_interface.h:17-69): with a layout installed, a feature at model
+    position p is read at list[p] of the caller's data. Documents whose columns are scattered that way
+    must give what the unscattered documents give without a layout, bit for bit (same kernels, same
+    bins), through flat rows, flat columns, separate float / hashed categorical arrays and strings."""
+    rng = np.random.default_rng(42)
+    for name in ("synthetic_ctr_2.cbm", "rust_tmp_model.cbm", "features_num__dataset_querywise.cbm"):
+        path = os.path.join(golden_dir, name)
+        m = read_cbm_file(path)
+        o = OracleModel(m)
+        g = cb.ModelCalcer(path)
+        floats, cats = rm.random_ctr_inputs(m, 700, 3, rm.known_cat_hashes(m))
+        flat = rm.flat_rows(m, floats, cats)
+        expected = g.calc_flat(flat)
+        _close(expected, o.calc(flat))
+        expected_bins = g.quantize_flat(flat)
+        # flat vectors: scatter into wider rows
+        width = flat.shape[1] + 5
+        where = rng.permutation(width)[:flat.shape[1]].astype(np.uint32)
+        scattered = rng.normal(size=(flat.shape[0], width)).astype(np.float32)
+        scattered[:, where] = flat
+        g.set_feature_layout(flat_indexes=where)
+        used = [f["flat_index"] for f in m["float_features"] if len(f["borders"])] + \
+               [c["flat_index"] for c in m["cat_features"] if c.get("used", True)]
+        need = int(where[used].max()) + 1
+        np.testing.assert_array_equal(g.calc_flat(scattered), expected)
+        np.testing.assert_array_equal(g.calc_flat(scattered[:, :need]), expected)
+        np.testing.assert_array_equal(g.quantize_flat(scattered), expected_bins)
+        np.testing.assert_array_equal(g.calc_flat_transposed(np.ascontiguousarray(scattered.T)), expected)
+        with pytest.raises(cb.CatBoostError, match="insufficient"):
+            g.calc_flat(scattered[:, :need - 1])
+        # separate arrays: scatter the float and the categorical columns on their own
+        fw, cw = floats.shape[1] + 3, cats.shape[1] + 2
+        fwhere = rng.permutation(fw)[:floats.shape[1]].astype(np.uint32)
+        cwhere = rng.permutation(cw)[:cats.shape[1]].astype(np.uint32)
+        sf = rng.normal(size=(floats.shape[0], fw)).astype(np.float32)
+        sc = rng.integers(-5, 5, size=(cats.shape[0], cw)).astype(np.int32)
+        sf[:, fwhere] = floats
+        sc[:, cwhere] = cats
+        g.set_feature_layout(float_feature_indexes=fwhere, cat_feature_indexes=cwhere)
+        np.testing.assert_array_equal(g.calc_hashed(sf, sc), expected)
+        np.testing.assert_array_equal(g.calc_flat(flat), expected)  # flat positions untouched by these lists
+        # a list without an entry for a used feature is refused and changes nothing
+        if floats.shape[1] > 1:
+            with pytest.raises(cb.CatBoostError, match="feature layout"):
+                g.set_feature_layout(float_feature_indexes=fwhere[:0])
+            np.testing.assert_array_equal(g.calc_hashed(sf, sc), expected)
+        g.set_feature_layout()
+        np.testing.assert_array_equal(g.calc_hashed(floats, cats), expected)
+    # strings: the rust fixture's one categorical feature moved to the third of three strings
+    g = cb.ModelCalcer(os.path.join(golden_dir, "rust_tmp_model.cbm"))
+    g.set_feature_layout(cat_feature_indexes=np.array([2], np.uint32))
+    _close(g.calc(rm.RUST_FLOATS, [["x", "y", c[0]] for c in rm.RUST_CATS]), rm.RUST_EXPECTED)
+
+
 def test_ctr_kernel_without_the_staged_tile(golden_dir, monkeypatch):
     """Models whose projections read more categorical columns than the LDS tile holds take the plain CTR
     kernel; the switch forces it for models that would not."""

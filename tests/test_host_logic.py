@@ -361,3 +361,17 @@ def test_json_import_error_paths(golden_dir):
         cb.ModelCalcer(buffer=json.dumps(doc), model_format="json")
     with pytest.raises(cb.CatBoostError, match="can't open"):
         cb.ModelCalcer(os.path.join(golden_dir, "no_such_model.json"), model_format="json")
+
+
+def test_feature_layout_is_checked_when_it_is_set(golden_dir):
+    """CbHipSetFeatureLayout needs an entry for every used feature in a list that is given
+    (TFeatureLayout::GetRemappedPosition indexes the lists with at(), evaluation_interface.h:27-47)."""
+    g = cb.ModelCalcer(os.path.join(golden_dir, "rust_tmp_model.cbm"))  # 3 float features, 1 categorical
+    g.set_feature_layout(float_feature_indexes=[4, 0, 2], cat_feature_indexes=[1], flat_indexes=[3, 2, 1, 0])
+    with pytest.raises(cb.CatBoostError, match="FloatFeatureIndexes has no entry"):
+        g.set_feature_layout(float_feature_indexes=[4, 0])
+    with pytest.raises(cb.CatBoostError, match="CatFeatureIndexes has no entry"):
+        g.set_feature_layout(cat_feature_indexes=[])
+    with pytest.raises(cb.CatBoostError, match="FlatIndexes has no entry"):
+        g.set_feature_layout(flat_indexes=[0, 1, 2])
+    g.set_feature_layout()
