@@ -1226,7 +1226,12 @@ void THipEvaluator::QuantizeDevice(const TFeatureBatch& batch, size_t docCount, 
     const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
     CBAMD_ENSURE(blocks <= 0x7fffffffu, "too many documents in one batch");
     if (m.RealBucketCount == 0) {
-        HIP_CHECK(hipMemsetAsync(bins, 0, QuantizedBytes(docCount), s));
+        // a model without splits: one all-zero bucket per block keeps the layout non-empty
+        CBAMD_ENSURE(bins != nullptr, "quantized buffer is null");
+        const size_t dwords = QuantizedBytes(docCount) / 4;
+        hipLaunchKernelGGL(dev::FillZeroKernel, dim3(static_cast<uint32_t>(std::min<size_t>((dwords + 255) / 256, 4096))),
+                           dim3(256), 0, s, reinterpret_cast<uint32_t*>(bins), dwords);
+        HIP_CHECK(hipGetLastError());
         return;
     }
     CBAMD_ENSURE(bins != nullptr, "quantized buffer is null");

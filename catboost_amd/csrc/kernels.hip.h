@@ -1586,4 +1586,13 @@ __global__ void FillBiasKernel(double* __restrict__ out, size_t count, const dou
     }
 }
 
+// Clears `dwords` 32-bit words. A kernel rather than hipMemsetAsync, so that callers may capture the
+// launch into a HIP graph.
+__global__ void FillZeroKernel(uint32_t* __restrict__ out, size_t dwords) {
+    const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < dwords; i += stride) {
+        out[i] = 0;
+    }
+}
+
 }  // namespace cbamd::dev

@@ -3,12 +3,13 @@
 the evaluator's entry points block by block over a pool).
 
     python -m catboost_amd.perftest -m model.cbm [--pool-path pool.tsv] [--docs N] [--block-size B]
-                                    [--repetitions R] [--model-format cbm|json] [--device-id D]
+                                    [--repetitions R] [--model-format cbm|json] [--device-id D] [--graph]
 
 Without a pool the documents are random: floats around the model's borders, categorical hashes at random.
 A pool is a tab-separated file of flat feature rows (categorical columns as strings). Reports documents
 per second of the flat host entry point (rows by pointer, PCIe both ways) and of the device entry points
-on features that already sit in HBM.
+on features that already sit in HBM; with --graph also of a block's quantize + evaluate launches captured
+once into a HIP graph and replayed per block (what a serving loop with small blocks does).
 """
 import argparse
 import json
@@ -92,6 +93,36 @@ def run(args):
     report["device_docs_per_sec"] = args.repetitions * len(blocks) * block / seconds
     binarize_ms, evaluate_ms = ev.last_kernel_times()
     report["last_block_kernel_ms"] = {"binarize": binarize_ms, "evaluate": evaluate_ms}
+
+    if args.graph:
+        # quantize + evaluate of one block captured once into a HIP graph (the quantized-data entry points
+        # only launch kernels); a call is then a copy into the captured input buffer and a replay
+        captured_in = resident[0].clone()
+        bins = torch.zeros(ev.quantized_bytes(block), dtype=torch.uint8, device=device)
+        captured = ev.features(cb.LAYOUT_FLAT_ROWS, captured_in.data_ptr(), captured_in.shape[1])
+
+        def launch(stream):
+            ev.quantize(captured, block, bins.data_ptr(), stream=stream)
+            ev.eval_quantized(bins.data_ptr(), block, out.data_ptr(), stream=stream)
+
+        side = torch.cuda.Stream(device=device)
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            launch(side.cuda_stream)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            launch(torch.cuda.current_stream().cuda_stream)
+        stream = torch.cuda.current_stream()
+        start = time.perf_counter()
+        for _ in range(args.repetitions):
+            for x in resident:
+                captured_in.copy_(x, non_blocking=True)
+                graph.replay()
+                stream.synchronize()  # like eval_data, a call ends when its results are there
+        seconds = time.perf_counter() - start
+        report["graph_replay_docs_per_sec"] = args.repetitions * len(blocks) * block / seconds
     return report
 
 
@@ -103,6 +134,7 @@ def main(argv=None):
     parser.add_argument("--docs", type=int, default=1_000_000, help="random documents when no pool is given")
     parser.add_argument("--block-size", type=int, default=0, help="documents per call (default: all)")
     parser.add_argument("--repetitions", type=int, default=10)
+    parser.add_argument("--graph", action="store_true", help="also time the block as a replayed HIP graph")
     parser.add_argument("--device-id", type=int, default=0)
     parser.add_argument("--seed", type=int, default=0)
     args = parser.parse_args(argv)

@@ -93,7 +93,9 @@ size_t CbHipQuantizedBytes(CbHipEvaluatorHandle* evaluator, size_t docCount);
 
 /* Binarize device-resident features into `deviceBins` (TGPUCatboostEvaluationContext::QuantizeData,
  * cuda/evaluator.cu:379-416; IModelEvaluator::Quantize). `hipStream` is a hipStream_t or NULL for
- * the evaluator's own stream; the call is asynchronous on that stream. */
+ * the evaluator's own stream; the call is asynchronous on that stream. Like CbHipEvalQuantized,
+ * CbHipLeafIndexesQuantized, CbHipExportQuantized and CbHipApplyPredictionTypeDevice it only launches
+ * kernels (no allocation, synchronisation or memset), so a caller may capture it into a HIP graph. */
 bool CbHipQuantize(CbHipEvaluatorHandle* evaluator, const CbHipFeatures* deviceFeatures, size_t docCount,
                    void* deviceBins, void* hipStream);
 

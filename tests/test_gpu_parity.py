@@ -451,6 +451,89 @@ def test_ctr_model_on_the_device_path(golden_dir):
     np.testing.assert_array_equal(exported.cpu().numpy(), o.binarize(flat))
 
 
+def test_device_entry_points_in_a_hip_graph(golden_dir):
+    """CbHipQuantize, CbHipEvalQuantized, CbHipLeafIndexesQuantized and CbHipApplyPredictionTypeDevice only
+    launch kernels on the caller's stream (no allocation, no synchronisation, no memset), so a caller may
+    capture them into a HIP graph. Every replay, with new documents in the captured input buffer and eager
+    work in between, must equal the eager one-call path bit for bit."""
+    import torch
+
+    cases = []
+    for cfg, docs in (("C1", 10_000), ("C3", 3000), ("C4", 3000), ("C5", 2000)):
+        model, info = syn.build_model(cfg, trees=100)
+        cases.append((cfg, model, syn.device_features(info, docs), None, info["dim"]))
+    path = os.path.join(golden_dir, "features_num_cat__dataset_adult.cbm")
+    m = read_cbm_file(path)
+    floats, cats = rm.random_ctr_inputs(m, 5000, 9, rm.known_cat_hashes(m))
+    cases.append(("adult", cb.ModelCalcer(path), torch.from_numpy(floats).to("cuda:0"),
+                  torch.from_numpy(cats).to("cuda:0"), 1))
+    no_splits = cb.ModelCalcer()
+    no_splits.build_oblivious([dict(index=0, flat_index=0)], [], 1, [([], [0.25]), ([], [0.5])], bias=[1.0])
+    cases.append(("no splits", no_splits, torch.zeros(1000, 1, device="cuda:0"), None, 1))
+    for name, model, x, c, dim in cases:
+        model.enable_gpu_evaluation(0)
+        ev = model.evaluator()
+        docs = x.shape[0]
+        static_x = x.clone()
+        static_c = c.clone() if c is not None else None
+        bins = torch.zeros(ev.quantized_bytes(docs), dtype=torch.uint8, device="cuda:0")
+        out = torch.zeros(docs * dim, dtype=torch.float64, device="cuda:0")
+        proba = torch.zeros_like(out)
+        leaves = torch.zeros(docs * ev.tree_count, dtype=torch.int32, device="cuda:0")
+
+        def features(a, b):
+            if b is None:
+                return ev.features(cb.LAYOUT_FLAT_ROWS, a.data_ptr(), a.shape[1])
+            return ev.features(cb.LAYOUT_SPLIT_ROWS, a.data_ptr(), a.shape[1], b.data_ptr(), b.shape[1])
+
+        prediction = cb.APT_PROBABILITY if dim == 1 else cb.APT_MULTI_PROBABILITY
+
+        def run(stream):
+            ev.quantize(features(static_x, static_c), docs, bins.data_ptr(), stream=stream)
+            ev.eval_quantized(bins.data_ptr(), docs, out.data_ptr(), stream=stream)
+            ev.leaf_indexes_quantized(bins.data_ptr(), docs, leaves.data_ptr(), stream=stream)
+            ev.apply_prediction_type(prediction, docs, out.data_ptr(), proba.data_ptr(), stream=stream)
+
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            run(side.cuda_stream)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            run(torch.cuda.current_stream().cuda_stream)
+        eager = torch.zeros_like(out)
+        eager_proba = torch.zeros_like(out)
+        eager_bins = torch.zeros_like(bins)
+        eager_leaves = torch.zeros_like(leaves)
+        for replay in range(3):
+            order = torch.randperm(docs, device="cuda:0")
+            static_x.copy_(x[order])
+            if c is not None:
+                static_c.copy_(c[order])
+            out.zero_()
+            proba.zero_()
+            leaves.zero_()
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            # eager, through the one-call entry point and separate buffers
+            xe = x[order].contiguous()
+            ce = c[order].contiguous() if c is not None else None
+            ev.eval_data(features(xe, ce), docs, eager.data_ptr())
+            ev.quantize(features(xe, ce), docs, eager_bins.data_ptr())
+            ev.leaf_indexes_quantized(eager_bins.data_ptr(), docs, eager_leaves.data_ptr())
+            ev.apply_prediction_type(prediction, docs, eager.data_ptr(), eager_proba.data_ptr())
+            ev.synchronize()
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager), (name, replay)
+            assert torch.equal(leaves, eager_leaves), (name, replay)
+            assert torch.equal(proba, eager_proba), (name, replay)
+        if name == "no splits":
+            assert torch.equal(out, torch.full_like(out, 1.75))
+
+
 def test_querywise_fixture(golden_dir):
     g = cb.ModelCalcer(os.path.join(golden_dir, "features_num__dataset_querywise.cbm"))
     np.testing.assert_allclose(g.calc_flat(rm.querywise_rows()), rm.QUERYWISE_EXPECTED, rtol=1e-12, atol=1e-15)
@@ -749,6 +832,8 @@ def test_perftest_tool(golden_dir, tmp_path, capsys):
     report = json.loads(capsys.readouterr().out)
     assert report["docs"] == 20000 and report["block_size"] == 4096 and report["trees"] == 100
     assert report["host_flat_docs_per_sec"] > 0 and report["device_docs_per_sec"] > report["host_flat_docs_per_sec"]
+    assert perftest.main(["-m", str(path), "--docs", "4096", "--block-size", "256", "--repetitions", "2", "--graph"]) == 0
+    assert json.loads(capsys.readouterr().out)["graph_replay_docs_per_sec"] > 0
     # a pool of flat rows: the rust fixture's three documents (one string categorical column)
     pool = tmp_path / "pool.tsv"
     pool.write_text("".join("%g\t%g\t%s\t%g\n" % (f[0], f[1], c[0], f[2]) for f, c in zip(rm.RUST_FLOATS, rm.RUST_CATS)))
