@@ -65,6 +65,38 @@ def cpu_baseline(model_bytes, info, target_seconds=12.0):
     }
 
 
+def reference_standalone(model_bytes, rows, gpu_values):
+    """Times the reference's own standalone evaluator (catboost/libs/standalone_evaluator, built from the
+    reference's sources into oracle/_ref/standalone_eval by oracle/build_ref.sh; one scalar thread, float-only
+    oblivious one-dimensional models) on `rows` and compares what it prints with the GPU's values.
+    Returns None where the binary is not there."""
+    import subprocess
+    import tempfile
+
+    import numpy as np
+
+    exe = os.path.join(ROOT, "oracle", "_ref", "standalone_eval")
+    if not os.path.exists(exe):
+        return None
+    with tempfile.TemporaryDirectory() as tmp:
+        model_path = os.path.join(tmp, "model.cbm")
+        with open(model_path, "wb") as f:
+            f.write(model_bytes)
+        seconds, printed = [], None
+        # two sizes: their difference takes the process start and the model load out of the rate
+        for count in (rows.shape[0] // 10, rows.shape[0]):
+            docs_path = os.path.join(tmp, "docs_%d.f32" % count)
+            np.ascontiguousarray(rows[:count], np.float32).tofile(docs_path)
+            t0 = time.perf_counter()
+            printed = subprocess.run([exe, "apply", model_path, docs_path, str(count)], check=True,
+                                     stdout=subprocess.PIPE).stdout
+            seconds.append(time.perf_counter() - t0)
+    values = np.array(printed.split(), dtype=np.float64)
+    rate = (rows.shape[0] - rows.shape[0] // 10) / max(seconds[1] - seconds[0], 1e-9)
+    return {"docs_per_sec": rate, "cores": 1, "sample": "%d docs of the same workload, %.1f s" % (rows.shape[0], seconds[1]),
+            "max_abs_diff_gpu_vs_reference": float(np.abs(values - gpu_values).max())}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -182,6 +214,11 @@ def main():
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(model_bytes, info)
+        if info["kind"] == "oblivious" and dim == 1 and not info["cat_hashes"]:
+            # the sampled documents of the parity check, through the reference's own scalar evaluator
+            ref = reference_standalone(model_bytes, sample, got)
+            if ref is not None:
+                result["cpu_baseline"]["reference_standalone_evaluator"] = ref
     print(json.dumps(result))
     if not ok:
         sys.exit(1)
