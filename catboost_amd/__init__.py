@@ -531,9 +531,9 @@ class ModelCalcer:
         lists = [None if v is None else np.ascontiguousarray(v, np.uint32)
                  for v in (float_feature_indexes, cat_feature_indexes, flat_indexes)]
         args = []
+        placeholder = ctypes.c_uint32()  # a defined but empty list still needs a non-null pointer
         for a in lists:
-            # a defined but empty list still needs a non-null pointer
-            args += [None, 0] if a is None else [a.ctypes.data if a.size else ctypes.addressof(ctypes.c_uint32()), a.size]
+            args += [None, 0] if a is None else [a.ctypes.data if a.size else ctypes.addressof(placeholder), a.size]
         _check(self._lib.CbHipSetFeatureLayout(self._h, *args))
 
     # ---- evaluator selection

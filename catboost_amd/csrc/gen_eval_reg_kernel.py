@@ -220,6 +220,15 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed):
     e("  s_waitcnt vmcnt(0) lgkmcnt(0)")
     e("  s_barrier")
     e("  s_set_gpr_idx_on s22, 0x1")             # src0 of VALU instructions becomes index relative
+    # every wave warms its own share of a tree block's level tables, every WARM_WAYS-th 64-byte line
+    # from line (wave mod WARM_WAYS) on: s[30:31] = table + that line
+    warm_lines = block * tree_row_bytes // 64
+    warm_ways = min(waves, warm_lines)
+    assert warm_ways & (warm_ways - 1) == 0 and warm_lines % warm_ways == 0
+    e("  s_and_b32 s28, s20, %d" % (warm_ways - 1))
+    e("  s_lshl_b32 s28, s28, 6")
+    e("  s_add_u32 s30, s6, s28")
+    e("  s_addc_u32 s31, s7, 0")
     e("%s_loop:" % name)
     for buf in range(2):
         for i in range(block):
@@ -258,9 +267,12 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed):
                 e("  s_mov_b32 m0, 0x1000")      # index mode value again: src0 relative, index 0
             if i == 0:
                 # the rows of the next tree block are pulled into the scalar cache now, so that the
-                # per-tree row loads of that block do not each wait for a miss
-                for k in range(block * tree_row_bytes // 64):
-                    e("  s_load_dword s3, s[6:7], 0x%x" % ((buf * block + block + 2) * tree_row_bytes + 64 * k))
+                # per-tree row loads of that block do not each wait for a miss. The waves of a workgroup
+                # share the cache and reach this point together, so each touches a share of the lines
+                # (a scalar load is dear here: sixteen per wave and block cost 5 % of the launch)
+                for k in range(warm_lines // warm_ways):
+                    e("  s_load_dword s3, s[30:31], 0x%x" % ((buf * block + block + 2) * tree_row_bytes
+                                                            + 64 * warm_ways * k))
         # every wave is done reading this buffer and writing the other one
         e("  s_waitcnt vmcnt(0) lgkmcnt(0)")
         e("  s_barrier")
@@ -269,6 +281,8 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed):
         e("  s_cbranch_scc1 %s_done" % name)
     e("  s_add_u32 s6, s6, %d" % (2 * block * tree_row_bytes))
     e("  s_addc_u32 s7, s7, 0")
+    e("  s_add_u32 s30, s30, %d" % (2 * block * tree_row_bytes))
+    e("  s_addc_u32 s31, s31, 0")
     e("  s_branch %s_loop" % name)
     e("%s_done:" % name)
     add_leaf_values()
