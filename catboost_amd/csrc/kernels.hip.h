@@ -218,6 +218,8 @@ __global__ __launch_bounds__(256) void BinarizeRowsKernel(const float* __restric
         if (block + 1 < blockEnd) {
             CBAMD_LOAD_BLOCK(block + 1);  // in flight while this block is binarized
         }
+        // this lane's dword of the block's first bucket of the tile; bucket bb sits bb * 256 bytes further
+        uint32_t* blockBins = bins + (static_cast<size_t>(block) * tab.BucketPitch + b0) * kWave + lane;
 #pragma unroll
         for (int k = 0; k < kBucketsPerWave; ++k) {
             const uint32_t bb = wave + k * (256 / kWave);
@@ -234,18 +236,37 @@ __global__ __launch_bounds__(256) void BinarizeRowsKernel(const float* __restric
                     packed |= OneHotBin(values, count, column[j * kWave]) << (8 * j);
                 }
             } else {
+                // the lane's four documents go through the search side by side: one pass of the loop
+                // control and one LDS round trip per step for all four (CountBelowInCell, four at once)
                 const uint8_t* lut = reinterpret_cast<const uint8_t*>(sLut + bb * (kLutCells / 4));
-                const bool nanToInf = (myFlags[k] & kBucketFlagNanToInf) != 0;
+                float v[4];
+                uint32_t below[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    float v = __uint_as_float(column[j * kWave]);
-                    if (nanToInf) {
-                        v = isnan(v) ? __uint_as_float(0x7f800000u) : v;
-                    }
-                    packed |= CountBelowInCell(values, lut, myLo[k], myScale[k], myTopStep[k], v) << (8 * j);
+                    v[j] = __uint_as_float(column[j * kWave]);
                 }
+                if (myFlags[k] & kBucketFlagNanToInf) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        v[j] = isnan(v[j]) ? __uint_as_float(0x7f800000u) : v[j];
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    below[j] = static_cast<uint32_t>(lut[GridCell(v[j], myLo[k], myScale[k])]) * 4;  // byte offsets
+                }
+                const uint8_t* valueBytes = reinterpret_cast<const uint8_t*>(values);
+                for (uint32_t step4 = __builtin_amdgcn_readfirstlane(myTopStep[k]) * 4; step4 >= 4; step4 >>= 1) {
+                    const uint8_t* probe = valueBytes + step4 - 4;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float b = *reinterpret_cast<const float*>(probe + below[j]);
+                        below[j] += (b < v[j]) ? step4 : 0u;
+                    }
+                }
+                packed = (below[0] >> 2) | (below[1] << 6) | (below[2] << 14) | (below[3] << 22);
             }
-            bins[(static_cast<size_t>(block) * tab.BucketPitch + b0 + bb) * kWave + lane] = packed;
+            blockBins[bb * kWave] = packed;
         }
     }
 #undef CBAMD_LOAD_BLOCK
