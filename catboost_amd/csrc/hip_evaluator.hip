@@ -984,15 +984,21 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
                 for (int d = 0; d < 8; ++d) {
                     if (d < trees.TreeSizes[t]) {
                         const auto& rb = trees.RepackedBins[trees.TreeStartOffsets[t] + d];
-                        row[d] = sevenBit ? (static_cast<uint32_t>(rb.FeatureIndex) << 8) | (128u - rb.SplitIdx)
-                                          : (static_cast<uint32_t>(rb.FeatureIndex) << 16) |
-                                                (static_cast<uint32_t>(rb.XorMask) << 8) | rb.SplitIdx;
+                        if (sevenBit) {
+                            // ready for use: byte offset of the bucket's row in the half tile, compare constant
+                            row[d] = static_cast<uint32_t>(rb.FeatureIndex) * 128u;
+                            row[8 + d] = (128u - rb.SplitIdx) * 0x0101u;
+                        } else {
+                            row[d] = (static_cast<uint32_t>(rb.FeatureIndex) << 16) |
+                                     (static_cast<uint32_t>(rb.XorMask) << 8) | rb.SplitIdx;
+                        }
                     } else {
-                        row[d] = sevenBit ? 0u : 0xffu;
+                        row[d] = sevenBit ? 0u : 0xffu;  // a split that no bin passes
                     }
                 }
-                row[dev::kPackedFirstLeafSlot] = firstLeaf[t];
-                row[dev::kPackedFormSlot] = sevenBit ? 0u : 1u;
+                if (!sevenBit) {
+                    row[dev::kPackedFormSlot] |= 0x80000000u;
+                }
             }
             m.PackedMixed.Upload(mixed);
             if (TileLdsBytes(m.LayoutBuckets, 1) > kMaxTileLdsBytes) {

@@ -895,24 +895,35 @@ __global__ __launch_bounds__(64 * kTileWaves) __attribute__((amdgpu_waves_per_eu
 // (buckets x 128 bytes, two documents per lane: documents (2 * half + j) * 64 + lane of the block)
 // and its waves split the trees; everything else is EvalObliviousTileKernel with DCHUNK == 1 and
 // leaf values through LDS. `leaves` holds (1 << MAXD) values per tree at a fixed pitch.
-// The packed rows come in the form chosen per tree (slot kPackedFormSlot): the 7-bit form when
-// the tree has no one-hot split and all float bins of the model fit 7 bits, else the 8-bit form;
+// The packed rows come in the form chosen per tree (bit 31 of slot kPackedFormSlot): the 7-bit form
+// when the tree has no one-hot split and all float bins of the model fit 7 bits, else the 8-bit form;
 // a model with a few one-hot splits pays the longer compare only in the trees that have them.
+// A 7-bit row holds what a level needs ready for use, so that a level costs two lane reads and no scalar
+// arithmetic: slot d the byte offset of the level's bucket in the half tile (bucket * 128), slot 8 + d
+// (128 - splitIdx) * 0x0101. An 8-bit row holds bucket << 16 | xorMask << 8 | splitIdx in slot d.
 // grid = 2 * doc blocks, block = 64 * kTileWaves threads, dynamic LDS = buckets * 128 (rounded up
 // to 8) + 128 * 8 + kTileWaves * (1 << MAXD) * 8 bytes.
-constexpr int kPackedFormSlot = 11;  // mixed table: 0 = 7-bit form, 1 = 8-bit form
+constexpr int kPackedFormSlot = 8;  // mixed table, bit 31: clear = 7-bit form, set = 8-bit form
 
 template <bool SEVEN_BIT, int MAXD>
 __device__ __forceinline__ uint32_t TreeIndexesPair(const uint8_t* laneTile, uint32_t packedRow) {
     uint32_t idx2 = 0;
 #pragma unroll
     for (int d = 0; d < MAXD; ++d) {
-        const uint32_t level = __builtin_amdgcn_readlane(packedRow, d);
-        const uint32_t a = *reinterpret_cast<const uint16_t*>(laneTile + (LevelTileOffset<SEVEN_BIT>(level) >> 1));
-        const uint32_t r = CompareBytes<SEVEN_BIT>(a, level);
-        idx2 = (r & 0x8080u) | ((idx2 >> 1) & 0x7f7fu);
+        uint32_t r;
+        if (SEVEN_BIT) {
+            const uint32_t a = *reinterpret_cast<const uint16_t*>(laneTile + __builtin_amdgcn_readlane(packedRow, d));
+            r = a + __builtin_amdgcn_readlane(packedRow, 8 + d);
+        } else {
+            const uint32_t level = __builtin_amdgcn_readlane(packedRow, d);
+            const uint32_t a = *reinterpret_cast<const uint16_t*>(laneTile + (LevelTileOffset<false>(level) >> 1));
+            r = CompareBytes<false>(a, level);
+        }
+        // bits 7 and 15 from r, the rest from the shifted index: one v_bfi. What a sum carries past bit 15
+        // moves down one bit per level and is replaced when it reaches bit 15.
+        idx2 = (r & 0x8080u) | ((idx2 >> 1) & ~0x8080u);
     }
-    return idx2 >> (8 - MAXD);
+    return (idx2 & 0xffffu) >> (8 - MAXD);
 }
 
 template <int MAXD>
@@ -989,7 +1000,7 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousHalfTileKernel(
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                 __builtin_amdgcn_wave_barrier();
                 uint32_t idx2;
-                if (__builtin_amdgcn_readlane(row, kPackedFormSlot) != 0) {
+                if (__builtin_amdgcn_readlane(row, kPackedFormSlot) >> 31) {
                     idx2 = TreeIndexesPair<false, MAXD>(laneTile, row);
                 } else {
                     idx2 = TreeIndexesPair<true, MAXD>(laneTile, row);
