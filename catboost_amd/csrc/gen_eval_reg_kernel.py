@@ -84,8 +84,20 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed):
     buf_bytes = block * tree_bytes
     lds_bytes = 2 * buf_bytes
     assert buf_bytes % row_bytes == 0 and lds_bytes <= 65536
-    chunks = buf_bytes // row_bytes       # pieces of a tree block per thread
-    per_tree = (chunks + block - 1) // block
+    # A wave copies its own contiguous share of a tree block, 1 KB (16 bytes per lane) per instruction;
+    # up to four instructions of a group differ only in the immediate offset, which moves the source
+    # and the LDS destination alike.
+    wave_bytes = buf_bytes // waves
+    pieces = wave_bytes // 1024
+    assert wave_bytes % 1024 == 0 and pieces >= 1
+    groups = [(first, min(4, pieces - first)) for first in range(0, pieces, 4)]
+    assert len(groups) <= block
+
+    def group_step(g):
+        """Distance of group g's first piece from the previous group's, the previous block's last one for g = 0."""
+        if g == 0:
+            return buf_bytes - groups[-1][0] * 1024
+        return (groups[g][0] - groups[g - 1][0]) * 1024
     # vector registers: v0 thread, v1 lane * 4, v2 thread * 16, v3 leaf indexes, v4/v5 scratch
     lv0 = 6                               # leaf values in flight: 4 documents x pitch doubles
     ac0 = lv0 + 8 * pitch                 # the sums
@@ -104,15 +116,18 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed):
     o = []
     e = o.append
 
-    def stage(lds_offset):
-        """One piece of the leaf table, global memory -> LDS without passing through registers:
-        lane l of wave w writes 16 bytes at lds_offset + w * 1024 + l * 16 (M0 holds the wave's
-        base). M0 doubles as the VGPR index register, so its index-mode value is put back after."""
-        e("  s_add_u32 m0, s100, %d" % lds_offset)
-        # the thread's offset moves on to the next piece of the table; the instruction also fills the
-        # wait state that the M0 write needs before the copy
-        e("  v_add_u32_e32 v2, 0x%x, v2" % row_bytes)
-        e("  global_load_lds_dwordx4 v2, s[26:27]")
+    def stage(buffer_offset, g):
+        """Group g of the wave's pieces of a tree block, global memory -> LDS without passing through
+        registers: lane l writes 16 bytes at buffer_offset + wave * wave_bytes + piece * 1024 + l * 16 (M0
+        holds the wave's base). M0 doubles as the VGPR index register, so its index-mode value is put
+        back after."""
+        first, count = groups[g]
+        e("  s_add_u32 m0, s100, %d" % (buffer_offset + first * 1024))
+        # the thread's offset moves on to the group's first piece; the instruction also fills the wait
+        # state that the M0 write needs before the copy
+        e("  v_add_u32_e32 v2, 0x%x, v2" % group_step(g))
+        for piece in range(count):
+            e("  global_load_lds_dwordx4 v2, s[26:27]%s" % (" offset:%d" % (piece * 1024) if piece else ""))
 
     def add_leaf_values():
         # sum + leaf as 1.0 * leaf + sum: the same single rounding, and with a constant in src0 the
@@ -177,8 +192,8 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed):
     e("  v_lshrrev_b32_e32 v5, 6, v0")
     e("  v_and_b32_e32 v1, 63, v0")
     e("  v_lshlrev_b32_e32 v1, 2, v1")           # lane * 4: offset inside a bucket's 256 bytes
-    e("  v_lshlrev_b32_e32 v2, 4, v0")           # thread * 16: offset of the thread's piece of a copy,
-    e("  v_subrev_u32_e32 v2, 0x%x, v2" % row_bytes)  # one piece back: every copy steps forward first
+    e("  v_lshlrev_b32_e32 v2, 2, v1")           # lane * 16: offset of the lane's part of a copied piece;
+    #                                              the wave's share and the first step are added below
     # gfx940 family: a lane read needs one wait state behind the VALU write of its source register;
     # the three instructions above and the s_nop keep it well clear
     e("  s_nop 1")
@@ -187,13 +202,16 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed):
     # byte j of the leaf indexes times s23 = offset of the document's leaf row in a tree's table
     # (a six-level index sits in bits 2..7 of its byte)
     e("  s_mov_b32 s23, %d" % (pitch * 8 >> (8 - depth)))
-    e("  s_lshl_b32 s100, s20, 10")              # LDS offset of the wave's part of a copied piece
+    e("  s_mul_i32 s100, s20, %d" % wave_bytes)  # offset of the wave's share of a tree block
+    # one step back: every group of copies steps forward first
+    e("  s_sub_u32 s28, s100, %d" % group_step(0))
+    e("  v_add_u32_e32 v2, s28, v2")
     e("  s_waitcnt lgkmcnt(0)")
     # first tree block -> buffer 0
     e("  s_mov_b32 s26, s8")
     e("  s_mov_b32 s27, s9")
-    for c in range(chunks):
-        stage(c * row_bytes)
+    for g in range(len(groups)):
+        stage(0, g)
     # document block of this wave; waves past the last block redo the last one and store nothing
     e("  s_mul_i32 s21, s2, %d" % waves)
     e("  s_add_u32 s21, s21, s20")
@@ -260,9 +278,10 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed):
             load_rows(rows, buf * block + i + 2)
             # copy of the next tree block into the other buffer, spread over this block's trees
             staged = False
-            for c in range(i * per_tree, min(chunks, (i + 1) * per_tree)):
-                stage((1 - buf) * buf_bytes + c * row_bytes)
-                staged = True
+            for g in range(len(groups)):
+                if g * block // len(groups) == i:
+                    stage((1 - buf) * buf_bytes, g)
+                    staged = True
             if staged:
                 e("  s_mov_b32 m0, 0x1000")      # index mode value again: src0 relative, index 0
             if i == 0:
