@@ -2,7 +2,8 @@
 
 The kernels evaluate oblivious trees of depth <= 8. The plain variants take models whose bins and
 split indexes all fit 7 bits (no xor masks), the case of float-feature models with at most 127
-used borders per feature; the "_m" (mixed) variants take any bins and xor masks (one-hot splits)
+used borders per feature; the "_s" variants take such models when no feature uses more than 63
+borders, which lets two levels share their merge; the "_m" (mixed) variants take any bins and xor masks (one-hot splits)
 and choose the compare per tree. One launch produces PITCH consecutive dimensions of the result
 (1 for a one-dimensional model).
 
@@ -19,6 +20,8 @@ Layout of the work:
     (global_load_lds);
   * a tree's levels come from a table of 16 dwords per tree, (bucket, (128 - splitIdx) * 0x01010101)
     per level, read with one scalar load two trees ahead; kernels for LEAVES = 64 use the first six.
+    Six-bit variants: the even levels' constant is (64 - splitIdx) * 0x01010101, which puts the level's
+    bit in bit 6 of every byte (all bins are below 64), next to the following level's in bit 7.
     Mixed variants: 32 dwords per tree. Bit 31 of the first dword clear: the 7-bit form above (the
     tree has no xor mask and all bins of its buckets fit 7 bits). Set: 4 dwords per level, bucket,
     xorMask, splitIdx & 0x7f (both times 0x01010101) and 0x80808080 if splitIdx < 128 else 0; the
@@ -48,18 +51,18 @@ import sys
 
 LDS_BUFFER_LIMIT = 32 * 1024
 
-# (bins registers, waves per workgroup, PITCH, LEAVES), each in a plain and a mixed form;
+# (bins registers, waves per workgroup, PITCH, LEAVES), each in a plain, a six-bit and a mixed form;
 # hip_evaluator.hip lists the same variants
 SHAPES = [
     (208, 4, 1, 256), (200, 4, 1, 256), (96, 8, 1, 256),
     (192, 4, 2, 64), (160, 4, 4, 64), (128, 4, 6, 64),
     (192, 4, 2, 256), (160, 4, 4, 256), (128, 4, 6, 256),
 ]
-VARIANTS = [shape + (mixed,) for mixed in (False, True) for shape in SHAPES]
+VARIANTS = [shape + (mixed, six) for mixed, six in ((False, False), (False, True), (True, False)) for shape in SHAPES]
 
 
-def kernel_name(buckets, waves, pitch, leaves, mixed):
-    return "cbamd_eval_reg_b%d_w%d_p%d_l%d%s" % (buckets, waves, pitch, leaves, "_m" if mixed else "")
+def kernel_name(buckets, waves, pitch, leaves, mixed, six=False):
+    return "cbamd_eval_reg_b%d_w%d_p%d_l%d%s" % (buckets, waves, pitch, leaves, "_m" if mixed else "_s" if six else "")
 
 
 def tree_block(pitch, leaves):
@@ -70,8 +73,9 @@ def tree_block(pitch, leaves):
     return block
 
 
-def gen_kernel(buckets, waves, pitch, leaves, mixed):
-    name = kernel_name(buckets, waves, pitch, leaves, mixed)
+def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False):
+    assert not (mixed and six)
+    name = kernel_name(buckets, waves, pitch, leaves, mixed, six)
     row_dwords = 32 if mixed else 16      # level table of a tree
     tree_row_bytes = row_dwords * 4
     rows_a, rows_b = 32, 32 + row_dwords  # the two sets of scalar registers holding level tables
@@ -162,6 +166,27 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed):
                 e("  v_lshrrev_b32_e32 v3, 1, v3")
                 e("  v_bfi_b32 v3, s22, v4, v3")
 
+    def levels_six_bit(rows):
+        """Bins below 64 everywhere: the host gives the even levels the constant (64 - splitIdx), whose sum
+        has the level's bit in bit 6 (and bit 7 clear), the odd levels (128 - splitIdx) as in the 7-bit
+        form. A pair of levels is then merged into the index with one shift: five instructions for two
+        levels instead of six. What the first pair leaves below its two bits goes the way the 7-bit
+        form's first sum goes; six-level kernels mask it."""
+        for pair in range(depth // 2):
+            even, odd = rows + 4 * pair, rows + 4 * pair + 2
+            e("  s_set_gpr_idx_idx s%d" % even)
+            e("  v_add_u32_e64 v4, v%d, s%d" % (b0, even + 1))
+            e("  s_set_gpr_idx_idx s%d" % odd)
+            e("  v_add_u32_e64 v%d, v%d, s%d" % (3 if pair == 0 else 5, b0, odd + 1))
+            if pair == 0:
+                e("  v_bfi_b32 v3, s22, v3, v4")           # bit 7 of the odd level's sum over the even level's
+                if first_level_masked:
+                    e("  v_and_b32_e32 v3, s29, v3")
+            else:
+                e("  v_bfi_b32 v4, s22, v5, v4")
+                e("  v_lshrrev_b32_e32 v3, 2, v3")
+                e("  v_bfi_b32 v3, s29, v4, v3")
+
     def levels_eight_bit(rows):
         for d in range(depth):
             level = rows + 4 * d
@@ -199,6 +224,8 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed):
     e("  s_nop 1")
     e("  v_readfirstlane_b32 s20, v5")           # wave of the workgroup
     e("  s_mov_b32 s22, 0x80808080")
+    if six:
+        e("  s_mov_b32 s29, 0xc0c0c0c0")
     # byte j of the leaf indexes times s23 = offset of the document's leaf row in a tree's table
     # (a six-level index sits in bits 2..7 of its byte)
     e("  s_mov_b32 s23, %d" % (pitch * 8 >> (8 - depth)))
@@ -260,6 +287,8 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed):
                 e("%s_x:" % label)
                 levels_eight_bit(rows)
                 e("%s_j:" % label)
+            elif six:
+                levels_six_bit(rows)
             else:
                 levels_seven_bit(rows)
             # previous tree's leaf values have arrived (and so has the next tree's row)
@@ -401,8 +430,8 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed):
 def generate():
     parts = ['.amdgcn_target "amdgcn-amd-amdhsa--gfx950"', ".amdhsa_code_object_version 6", ""]
     metas = []
-    for buckets, waves, pitch, leaves, mixed in VARIANTS:
-        text, meta = gen_kernel(buckets, waves, pitch, leaves, mixed)
+    for buckets, waves, pitch, leaves, mixed, six in VARIANTS:
+        text, meta = gen_kernel(buckets, waves, pitch, leaves, mixed, six)
         parts.append(text)
         metas.append(meta)
     parts.append(".amdgpu_metadata")

@@ -116,27 +116,37 @@ struct TEvalRegVariant {
     uint32_t Pitch;   // dimensions per launch = doubles per leaf row
     uint32_t Leaves;  // leaf rows per tree (64: trees of depth <= 6)
     bool Mixed;       // 32-dword level tables, compare form chosen per tree
+    bool Six;         // every bin below 64: even levels compare into bit 6, two levels share a merge
     const char* Name;
 };
 constexpr TEvalRegVariant kEvalRegVariants[] = {
-    {96, 8, 1, 256, false, "cbamd_eval_reg_b96_w8_p1_l256"},
-    {200, 4, 1, 256, false, "cbamd_eval_reg_b200_w4_p1_l256"},
-    {208, 4, 1, 256, false, "cbamd_eval_reg_b208_w4_p1_l256"},
-    {192, 4, 2, 64, false, "cbamd_eval_reg_b192_w4_p2_l64"},
-    {160, 4, 4, 64, false, "cbamd_eval_reg_b160_w4_p4_l64"},
-    {128, 4, 6, 64, false, "cbamd_eval_reg_b128_w4_p6_l64"},
-    {192, 4, 2, 256, false, "cbamd_eval_reg_b192_w4_p2_l256"},
-    {160, 4, 4, 256, false, "cbamd_eval_reg_b160_w4_p4_l256"},
-    {128, 4, 6, 256, false, "cbamd_eval_reg_b128_w4_p6_l256"},
-    {96, 8, 1, 256, true, "cbamd_eval_reg_b96_w8_p1_l256_m"},
-    {200, 4, 1, 256, true, "cbamd_eval_reg_b200_w4_p1_l256_m"},
-    {208, 4, 1, 256, true, "cbamd_eval_reg_b208_w4_p1_l256_m"},
-    {192, 4, 2, 64, true, "cbamd_eval_reg_b192_w4_p2_l64_m"},
-    {160, 4, 4, 64, true, "cbamd_eval_reg_b160_w4_p4_l64_m"},
-    {128, 4, 6, 64, true, "cbamd_eval_reg_b128_w4_p6_l64_m"},
-    {192, 4, 2, 256, true, "cbamd_eval_reg_b192_w4_p2_l256_m"},
-    {160, 4, 4, 256, true, "cbamd_eval_reg_b160_w4_p4_l256_m"},
-    {128, 4, 6, 256, true, "cbamd_eval_reg_b128_w4_p6_l256_m"},
+    {96, 8, 1, 256, false, false, "cbamd_eval_reg_b96_w8_p1_l256"},
+    {200, 4, 1, 256, false, false, "cbamd_eval_reg_b200_w4_p1_l256"},
+    {208, 4, 1, 256, false, false, "cbamd_eval_reg_b208_w4_p1_l256"},
+    {192, 4, 2, 64, false, false, "cbamd_eval_reg_b192_w4_p2_l64"},
+    {160, 4, 4, 64, false, false, "cbamd_eval_reg_b160_w4_p4_l64"},
+    {128, 4, 6, 64, false, false, "cbamd_eval_reg_b128_w4_p6_l64"},
+    {192, 4, 2, 256, false, false, "cbamd_eval_reg_b192_w4_p2_l256"},
+    {160, 4, 4, 256, false, false, "cbamd_eval_reg_b160_w4_p4_l256"},
+    {128, 4, 6, 256, false, false, "cbamd_eval_reg_b128_w4_p6_l256"},
+    {96, 8, 1, 256, true, false, "cbamd_eval_reg_b96_w8_p1_l256_m"},
+    {200, 4, 1, 256, true, false, "cbamd_eval_reg_b200_w4_p1_l256_m"},
+    {208, 4, 1, 256, true, false, "cbamd_eval_reg_b208_w4_p1_l256_m"},
+    {192, 4, 2, 64, true, false, "cbamd_eval_reg_b192_w4_p2_l64_m"},
+    {160, 4, 4, 64, true, false, "cbamd_eval_reg_b160_w4_p4_l64_m"},
+    {128, 4, 6, 64, true, false, "cbamd_eval_reg_b128_w4_p6_l64_m"},
+    {192, 4, 2, 256, true, false, "cbamd_eval_reg_b192_w4_p2_l256_m"},
+    {160, 4, 4, 256, true, false, "cbamd_eval_reg_b160_w4_p4_l256_m"},
+    {128, 4, 6, 256, true, false, "cbamd_eval_reg_b128_w4_p6_l256_m"},
+    {96, 8, 1, 256, false, true, "cbamd_eval_reg_b96_w8_p1_l256_s"},
+    {200, 4, 1, 256, false, true, "cbamd_eval_reg_b200_w4_p1_l256_s"},
+    {208, 4, 1, 256, false, true, "cbamd_eval_reg_b208_w4_p1_l256_s"},
+    {192, 4, 2, 64, false, true, "cbamd_eval_reg_b192_w4_p2_l64_s"},
+    {160, 4, 4, 64, false, true, "cbamd_eval_reg_b160_w4_p4_l64_s"},
+    {128, 4, 6, 64, false, true, "cbamd_eval_reg_b128_w4_p6_l64_s"},
+    {192, 4, 2, 256, false, true, "cbamd_eval_reg_b192_w4_p2_l256_s"},
+    {160, 4, 4, 256, false, true, "cbamd_eval_reg_b160_w4_p4_l256_s"},
+    {128, 4, 6, 256, false, true, "cbamd_eval_reg_b128_w4_p6_l256_s"},
 };
 
 // trees per LDS buffer of a variant: a power of two, at most 16, buffer at most 32 KB
@@ -151,12 +161,12 @@ uint32_t RegTreeBlock(const TEvalRegVariant& v) {
 // The variant for a model: one-dimensional models take the smallest register file that holds
 // their buckets; others the pitch that needs the fewest launches (then the smallest such pitch).
 // mixed: the model has one-hot splits or bins above 127.
-const TEvalRegVariant* PickRegVariant(uint32_t buckets, uint32_t dim, uint32_t maxDepth, bool mixed) {
+const TEvalRegVariant* PickRegVariant(uint32_t buckets, uint32_t dim, uint32_t maxDepth, bool mixed, bool six) {
     const TEvalRegVariant* best = nullptr;
     uint32_t bestLaunches = 0;
     for (const auto& v : kEvalRegVariants) {
         if (buckets > v.Buckets || (dim == 1) != (v.Pitch == 1) || v.Leaves != (dim > 1 && maxDepth <= 6 ? 64u : 256u) ||
-            v.Mixed != mixed) {
+            v.Mixed != mixed || v.Six != six) {
             continue;
         }
         const uint32_t launches = (dim + v.Pitch - 1) / v.Pitch;
@@ -1048,9 +1058,12 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
 
     const char* regSwitch = std::getenv("CATBOOST_AMD_REG_KERNEL");
     const bool regEnabled = !(regSwitch && regSwitch[0] == '0');
+    // six-bit form: no one-hot split and no bucket with more than 63 values, so that every bin is below 64
+    const char* sixSwitch = std::getenv("CATBOOST_AMD_REG_SIX");
+    const bool six = m.PackedSevenBit && m.MaxBucketValues <= 63 && !(sixSwitch && sixSwitch[0] == '0');
     const TEvalRegVariant* variant =
         m.Oblivious && m.MaxDepth <= 8 && TreeCount > 0
-            ? PickRegVariant(m.LayoutBuckets, static_cast<uint32_t>(m.Dim), m.MaxDepth, !m.PackedSevenBit)
+            ? PickRegVariant(m.LayoutBuckets, static_cast<uint32_t>(m.Dim), m.MaxDepth, !m.PackedSevenBit, six)
             : nullptr;
     // a thread's 32-bit offset walks through the leaf table of a launch while it is copied to LDS
     const bool regTableAddressable =
@@ -1089,7 +1102,8 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
                 for (int d = 0; d < depth; ++d) {
                     const auto& rb = trees.RepackedBins[trees.TreeStartOffsets[t] + d];
                     row[2 * d] = rb.FeatureIndex;
-                    row[2 * d + 1] = (128u - rb.SplitIdx) * 0x01010101u;
+                    // the level's bit is the carry into bit 7; six-bit kernels want the even levels' in bit 6
+                    row[2 * d + 1] = ((variant->Six && d % 2 == 0 ? 64u : 128u) - rb.SplitIdx) * 0x01010101u;
                 }
                 for (int d = depth; d < 8 && depth > 0; ++d) {
                     row[2 * d] = row[0];

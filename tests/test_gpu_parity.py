@@ -617,10 +617,10 @@ def test_random_oblivious_models(seed, dim):
     _close(g.calc_hashed(floats, cats), o.calc(floats, cats, layout="split"))
 
 
-def _float_only_model(rng, n_float, trees, max_depth, scale=1.0, bias=None, dim=1):
-    """Oblivious model over float features only (at most 40 borders each), every feature used."""
+def _float_only_model(rng, n_float, trees, max_depth, scale=1.0, bias=None, dim=1, max_borders=40):
+    """Oblivious model over float features only (fewer than `max_borders` borders each), every feature used."""
     ffs = [mb.float_feature(i, i) for i in range(n_float)]
-    cands = [np.unique(rng.normal(size=int(rng.integers(1, 40))).astype(np.float32)) for _ in range(n_float)]
+    cands = [np.unique(rng.normal(size=int(rng.integers(1, max_borders))).astype(np.float32)) for _ in range(n_float)]
     tree_list = []
     order = rng.permutation(n_float)
     next_feature = 0
@@ -643,12 +643,16 @@ def _float_only_model(rng, n_float, trees, max_depth, scale=1.0, bias=None, dim=
 # Models of this kind (one-dimensional, float features with < 128 borders, depth <= 8, at most
 # 208 buckets) run on the register-resident kernels, which add leaf values in tree order like the
 # CPU evaluator: their predictions are compared bit for bit. 209 buckets fall back to the LDS tile
-# kernel (sums per wave, then across waves), which only meets the tolerance.
+# kernel (sums per wave, then across waves), which only meets the tolerance. Models whose features all
+# have fewer than 64 borders take the six-bit form of these kernels (two levels share a merge); the
+# switch sends them through the 7-bit form as well.
+@pytest.mark.parametrize("six", ["1", "0"])
 @pytest.mark.parametrize("n_float,trees,max_depth,docs", [
     (1, 1, 1, 1), (1, 1, 8, 255), (3, 15, 8, 256), (5, 16, 8, 257), (7, 17, 6, 2049), (20, 33, 8, 1000),
     (96, 40, 8, 3000), (97, 40, 8, 3000), (208, 70, 8, 5000), (209, 70, 8, 1500), (50, 200, 4, 70001),
 ])
-def test_register_kernel_shapes(n_float, trees, max_depth, docs):
+def test_register_kernel_shapes(monkeypatch, n_float, trees, max_depth, docs, six):
+    monkeypatch.setenv("CATBOOST_AMD_REG_SIX", six)
     rng = np.random.default_rng(1000 * n_float + trees)
     model = _float_only_model(rng, n_float, trees, max_depth, scale=0.75, bias=[0.125])
     x = rng.normal(size=(docs, n_float)).astype(np.float32)
@@ -668,13 +672,15 @@ def test_register_kernel_shapes(n_float, trees, max_depth, docs):
                o.calc(x, tree_start=1, tree_end=len(model["tree_sizes"]) - 1))
 
 
+@pytest.mark.parametrize("six", ["1", "0"])
 @pytest.mark.parametrize("dim,max_depth,n_float,trees,docs", [
     (2, 6, 10, 20, 1000), (3, 6, 30, 33, 3000), (5, 8, 12, 9, 700), (6, 6, 128, 50, 2500), (7, 8, 100, 21, 1300),
     (10, 6, 100, 100, 5000), (13, 8, 60, 18, 900), (20, 6, 40, 30, 2049), (4, 6, 160, 60, 600), (2, 8, 192, 70, 600),
 ])
-def test_register_kernel_multi_dimensional(dim, max_depth, n_float, trees, docs):
+def test_register_kernel_multi_dimensional(monkeypatch, dim, max_depth, n_float, trees, docs, six):
     """Multi-dimensional float-only models: several launches of a register-resident kernel, each
     adding its dimensions in tree order like the CPU evaluator, hence bit for bit."""
+    monkeypatch.setenv("CATBOOST_AMD_REG_SIX", six)
     rng = np.random.default_rng(77 * dim + trees)
     model = _float_only_model(rng, n_float, trees, max_depth, scale=1.25, bias=list(rng.normal(size=dim)), dim=dim)
     x = rng.normal(size=(docs, n_float)).astype(np.float32)
@@ -683,6 +689,26 @@ def test_register_kernel_multi_dimensional(dim, max_depth, n_float, trees, docs)
     np.testing.assert_array_equal(g.calc_flat(x), o.calc(x))
     _close(g.calc_flat(x, tree_start=1, tree_end=len(model["tree_sizes"])),
            o.calc(x, tree_start=1, tree_end=len(model["tree_sizes"])))
+
+
+@pytest.mark.parametrize("max_borders", [64, 65, 128])
+def test_register_kernel_border_counts(max_borders):
+    """Features with exactly 63 borders still take the six-bit form, one feature with 64 or more sends
+    the model to the 7-bit form (127 is its limit): bit for bit either way."""
+    rng = np.random.default_rng(max_borders)
+    model = _float_only_model(rng, 24, 60, 8, scale=1.5, bias=[-0.25], max_borders=max_borders)
+    # one feature with every border the form allows, all of them used by some tree
+    full = np.unique(rng.normal(size=4 * max_borders).astype(np.float32))[:max_borders - 1]
+    ffs = [mb.float_feature(i, i) for i in range(25)]
+    trees = [([("float", 24, float(b)), ("float", int(rng.integers(0, 24)), 0.0)], rng.normal(size=4)) for b in full]
+    extra = mb.build_oblivious(ffs, [], 1, trees)
+    assert max(len(f["borders"]) for f in extra["float_features"]) == max_borders - 1
+    x = rng.normal(size=(3000, 25)).astype(np.float32)
+    x[:1000, 24] = rng.choice(full, size=1000)  # on the borders
+    for m in (model, extra):
+        xx = x[:, :len(m["float_features"])]
+        np.testing.assert_array_equal(_gpu_model(m).calc_flat(xx), OracleModel(m).calc(xx))
+        np.testing.assert_array_equal(_gpu_model(m).quantize_flat(xx), OracleModel(m).binarize(xx))
 
 
 def test_register_kernel_against_tile_kernel():
