@@ -19,7 +19,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
 # HBM bytes of one step (both launches, fetched + written), from rocprofv3 FETCH_SIZE / WRITE_SIZE
 # runs scaled by a copy kernel of known size; only known for workloads that were profiled
-MEASURED_TRAFFIC_BYTES = {("C2", 4000000, 1000): 6.14e9}
+MEASURED_TRAFFIC_BYTES = {("C2", 4000000, 1000): 6.12e9}
 
 
 def cpu_baseline(model_bytes, info, target_seconds=12.0):
