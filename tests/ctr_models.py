@@ -92,7 +92,7 @@ def random_ctr_model(seed, n_float=4, n_cat=4, n_bases=8, n_trees=40, max_depth=
         projections.append(proj)
         ctr_type = int(b % 6) if b < 6 else int(rng.integers(0, 6))
         base = dict(proj, ctr_type=ctr_type, target_border_classifier_idx=int(rng.integers(0, 2)))
-        if any(_same_base(base, t["base"]) for t in tables):
+        while any(_same_base(base, t["base"]) for t in tables):
             base["target_border_classifier_idx"] += 2
         keys = set()
         for _ in range(int(rng.integers(20, 200))):
