@@ -2,7 +2,8 @@
 // Follows ConvertJsonToCatboostModel (catboost/libs/model/model_export/json_model_helpers.cpp:583-608)
 // with its helpers GetObliviousModelTrees (:366-391), GetNonSymmetricModelTrees (:393-431),
 // GetFeaturesInfo (:267-291), FloatFeatureFromJson (:180-189) and CatFeatureFromJson (:199-205).
-// Models whose JSON carries CTR features are refused: their tables are only read from .cbm files.
+// CTR features and their tables: CtrFeatureFromJson (:119-136), FeatureCombinationFromJson (:54-78) and
+// CtrDataFromJson (:531-580); the json format does not carry TModelCtrBase::TargetBorderClassifierIdx (0 then).
 #include "model.h"
 
 #include <cerrno>
@@ -458,6 +459,56 @@ void ReadNonSymmetricTrees(const TJson& treesJson, TModelTrees* trees) {
 }
 
 // json_model_helpers.cpp:267-291
+ECtrType CtrTypeFromString(const std::string& s) {  // ECtrType, catboost/private/libs/ctr_description/ctr_type.h
+    static const char* const names[] = {"Borders", "Buckets", "BinarizedTargetMeanValue", "FloatTargetMeanValue",
+                                        "Counter", "FeatureFreq"};
+    for (int i = 0; i < 6; ++i) {
+        if (s == names[i]) {
+            return static_cast<ECtrType>(i);
+        }
+    }
+    CBAMD_ENSURE(false, "JSON model: unknown CTR type \"" + s + "\"");
+    return ECtrType::Borders;
+}
+
+// FeatureCombinationFromJson, json_model_helpers.cpp:54-78
+TFeatureCombination ReadProjection(const TJson& elements) {
+    TFeatureCombination projection;
+    for (const TJson& v : elements.Array_("the elements of a CTR")) {
+        const std::string& kind = v.At("combination_element").Str("combination_element");
+        if (kind == "cat_feature_value") {
+            projection.CatFeatures.push_back(v.At("cat_feature_index").Int32("cat_feature_index"));
+        } else if (kind == "float_feature") {
+            TFloatSplit split;
+            split.FloatFeature = v.At("float_feature_index").Int32("float_feature_index");
+            split.Split = static_cast<float>(v.At("border").Double("border"));
+            projection.BinFeatures.push_back(split);
+        } else {
+            TOneHotSplit split;
+            split.CatFeatureIdx = v.At("cat_feature_index").Int32("cat_feature_index");
+            split.Value = v.At("value").Int32("value");
+            projection.OneHotFeatures.push_back(split);
+        }
+    }
+    return projection;
+}
+
+// CtrFeatureFromJson / ModelCtrFromJson, json_model_helpers.cpp:119-136
+TCtrFeature ReadCtrFeature(const TJson& v) {
+    TCtrFeature feature;
+    feature.Ctr.Base.Projection = ReadProjection(v.At("elements"));
+    feature.Ctr.Base.CtrType = CtrTypeFromString(v.At("ctr_type").Str("ctr_type"));
+    feature.Ctr.TargetBorderIdx = v.At("target_border_idx").Int32("target_border_idx");
+    feature.Ctr.PriorNum = static_cast<float>(v.At("prior_numerator").Double("prior_numerator"));
+    feature.Ctr.PriorDenom = static_cast<float>(v.At("prior_denomerator").Double("prior_denomerator"));
+    feature.Ctr.Shift = static_cast<float>(v.At("shift").Double("shift"));
+    feature.Ctr.Scale = static_cast<float>(v.At("scale").Double("scale"));
+    for (const TJson& b : v.At("borders").Array_("the borders of a CTR")) {
+        feature.Borders.push_back(static_cast<float>(b.Double("a border")));
+    }
+    return feature;
+}
+
 void ReadFeaturesInfo(const TJson& info, TModelTrees* trees) {
     if (const TJson* floats = info.Find("float_features")) {
         for (const TJson& v : floats->Array_("float_features")) {
@@ -506,8 +557,97 @@ void ReadFeaturesInfo(const TJson& info, TModelTrees* trees) {
         }
     }
     if (const TJson* ctrs = info.Find("ctrs")) {
-        CBAMD_ENSURE(ctrs->Type != TJson::Array || ctrs->Items.empty(),
-                     "JSON models with CTR features are not supported: load the .cbm form of the model");
+        if (ctrs->Type == TJson::Array) {
+            for (const TJson& v : ctrs->Items) {
+                trees->CtrFeatures.push_back(ReadCtrFeature(v));
+            }
+        }
+    }
+}
+
+// CtrDataFromJson, json_model_helpers.cpp:531-580: a map from the text of a {"type", "identifier"} object
+// to {"hash_map": [hash as a decimal string, the row's values, ...], "hash_stride", "counter_denominator"}.
+// Rows are numbered in the order of their hashes (TDenseIndexHashBuilder::AddIndex,
+// catboost/libs/helpers/dense_hash_view.h:74-121: 2^k buckets at a load factor of at most one half,
+// linear probing, a hash seen again keeps its row).
+void ReadCtrData(const TJson& data, std::vector<TCtrValueTable>* tables) {
+    if (data.Type != TJson::Object) {
+        return;
+    }
+    for (const auto& entry : data.Fields) {
+        TJsonParser keyParser(entry.first.data(), entry.first.size());
+        const TJson key = keyParser.ParseDocument();
+        TCtrValueTable table;
+        table.ModelCtrBase.CtrType = CtrTypeFromString(key.At("type").Str("type"));
+        table.ModelCtrBase.Projection = ReadProjection(key.At("identifier"));
+        const ECtrType type = table.ModelCtrBase.CtrType;
+        const bool mean = type == ECtrType::BinarizedTargetMeanValue || type == ECtrType::FloatTargetMeanValue;
+        const bool counter = type == ECtrType::Counter || type == ECtrType::FeatureFreq;
+        const long long stride = entry.second.At("hash_stride").Integer("hash_stride");
+        const auto& items = entry.second.At("hash_map").Array_("hash_map");
+        CBAMD_ENSURE(stride >= 2 && stride <= 65536 && items.size() % static_cast<size_t>(stride) == 0,
+                     "JSON model: hash_map does not hold whole rows of hash_stride values");
+        CBAMD_ENSURE(!mean || stride == 3, "JSON model: a mean CTR table has rows of a sum and a count");
+        CBAMD_ENSURE(!counter || stride == 2, "JSON model: a counter CTR table has rows of one value");
+        const size_t rows = items.size() / static_cast<size_t>(stride);
+        const size_t values = static_cast<size_t>(stride) - 1;
+        size_t buckets = 2;
+        while (buckets < 2 * rows) {
+            buckets *= 2;
+        }
+        CBAMD_ENSURE(buckets < (size_t(1) << 31), "JSON model: CTR table is too large");
+        std::vector<uint64_t> hashes(buckets, ~uint64_t(0));
+        std::vector<uint32_t> rowOf(buckets, 0);
+        std::vector<uint32_t> blob(rows * (mean ? 2 : values), 0);
+        if (counter) {
+            table.CounterDenominator = entry.second.At("counter_denominator").Int32("counter_denominator");
+        } else if (!mean) {
+            table.TargetClassesCount = static_cast<int>(values);
+        }
+        uint32_t rowCount = 0;
+        for (size_t r = 0; r < rows; ++r) {
+            const TJson* item = &items[r * static_cast<size_t>(stride)];
+            const std::string& text = item[0].Str("a hash of hash_map");
+            errno = 0;
+            char* end = nullptr;
+            const unsigned long long hash = std::strtoull(text.c_str(), &end, 10);
+            CBAMD_ENSURE(!text.empty() && text[0] != '-' && errno == 0 && end != nullptr && *end == '\0',
+                         "JSON model: a hash of hash_map is not a 64-bit number");
+            CBAMD_ENSURE(hash != ~0ull, "JSON model: a hash of hash_map has the value of an empty bucket");
+            size_t z = hash & (buckets - 1);
+            while (hashes[z] != ~uint64_t(0) && hashes[z] != hash) {
+                z = (z + 1) & (buckets - 1);
+            }
+            if (hashes[z] == ~uint64_t(0)) {
+                hashes[z] = hash;
+                rowOf[z] = rowCount++;
+            }
+            const uint32_t row = rowOf[z];
+            if (mean) {
+                // the reference reads the sum with GetInteger (json_model_helpers.cpp:562): a sum that is
+                // not a whole number becomes 0 there, and so it does here
+                const double sum = item[1].Double("a sum of hash_map");
+                const float kept = (std::isfinite(sum) && sum == std::floor(sum) && std::fabs(sum) < 9.0e18)
+                                       ? static_cast<float>(static_cast<long long>(sum)) : 0.f;
+                std::memcpy(&blob[2 * row], &kept, 4);
+                blob[2 * row + 1] = static_cast<uint32_t>(item[2].Int32("a count of hash_map"));
+            } else {
+                for (size_t k = 0; k < values; ++k) {
+                    blob[row * values + k] = static_cast<uint32_t>(item[1 + k].Int32("a value of hash_map"));
+                }
+            }
+        }
+        table.IndexHashRaw.resize(buckets * 12);
+        for (size_t z = 0; z < buckets; ++z) {
+            std::memcpy(&table.IndexHashRaw[12 * z], &hashes[z], 8);
+            std::memcpy(&table.IndexHashRaw[12 * z + 8], &rowOf[z], 4);
+        }
+        blob.resize(static_cast<size_t>(rowCount) * (mean ? 2 : values));
+        table.CTRBlob.resize(blob.size() * 4);
+        if (!blob.empty()) {
+            std::memcpy(table.CTRBlob.data(), blob.data(), table.CTRBlob.size());
+        }
+        tables->push_back(std::move(table));
     }
 }
 
@@ -537,9 +677,12 @@ void TFullModel::LoadFromJson(const void* data, size_t size) {
         ReadNonSymmetricTrees(root.At("trees"), &Trees);
     }
     ReadFeaturesInfo(root.At("features_info"), &Trees);
-    CBAMD_ENSURE(!root.Has("ctr_data") || root.At("ctr_data").Type == TJson::Null ||
-                     (root.At("ctr_data").Type == TJson::Object && root.At("ctr_data").Fields.empty()),
-                 "JSON models with CTR features are not supported: load the .cbm form of the model");
+    if (const TJson* ctrData = root.Find("ctr_data")) {
+        ReadCtrData(*ctrData, &CtrTables);
+        if (!CtrTables.empty()) {
+            ModelPartIds.push_back("static_provider_v1");
+        }
+    }
     if (const TJson* sb = root.Find("scale_and_bias")) {
         const auto& items = sb->Array_("scale_and_bias");
         CBAMD_ENSURE(items.size() == 2, "JSON model: scale_and_bias must hold a scale and a bias");

@@ -261,7 +261,7 @@ struct TFullModel {
     // .cbm (de)serialisation, model.cpp:1113-1228
     void Load(const void* data, size_t size);
     void LoadFromFile(const std::string& path);
-    // the "json" model format (model_export/json_model_helpers.cpp:583-608); no CTR features
+    // the "json" model format (model_export/json_model_helpers.cpp:583-608)
     void LoadFromJson(const void* data, size_t size);
     void LoadFromJsonFile(const std::string& path);
     std::string Save() const;

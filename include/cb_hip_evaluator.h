@@ -185,8 +185,9 @@ bool CbHipBuildNonSymmetricModel(void* modelHandle, const CbHipModelArrays* feat
 
 /* The "json" model format: what ReadModel(path, EModelType::Json) does for the reference's bindings
  * (catboost/libs/model/model_export/json_model_helpers.cpp:583-608 ConvertJsonToCatboostModel; the JVM
- * binding's loadModel(stream, "json")). Float and one-hot categorical features, oblivious and
- * non-symmetric trees, scale and bias; a JSON model with CTR features is refused (load its .cbm form). */
+ * binding's loadModel(stream, "json")). Float, one-hot categorical and CTR features with their tables
+ * (CtrDataFromJson, :531-580), oblivious and non-symmetric trees, scale and bias. As in the reference
+ * the format loses TModelCtrBase::TargetBorderClassifierIdx and the fraction of a mean CTR's sum. */
 bool CbHipLoadFullModelFromJsonFile(void* modelHandle, const char* filename);
 bool CbHipLoadFullModelFromJsonBuffer(void* modelHandle, const void* jsonText, size_t jsonTextSize);
 

@@ -262,7 +262,7 @@ def flat_rows(model, floats, cats):
 def model_to_json(model):
     """A model dict in CatBoost's "json" model format, as ConvertModelToJson writes it
     (catboost/libs/model/model_export/json_model_helpers.cpp:293-364, 469-498): the keys the importer
-    reads, float and one-hot categorical features only."""
+    reads."""
     import json
 
     dim = int(model["approx_dimension"])
@@ -311,4 +311,49 @@ def model_to_json(model):
 
         doc["trees"] = [node_json(int(start)) for start in model["tree_start_offsets"]]
     doc["scale_and_bias"] = [float(model["scale"]), [float(b) for b in np.asarray(model["bias"], np.float64)]]
+    if model.get("ctr_features"):
+        # ToJson(TCtrFeature) and ConvertCtrsToJson, json_model_helpers.cpp:105-117, 433-485
+        type_names = ["Borders", "Buckets", "BinarizedTargetMeanValue", "FloatTargetMeanValue", "Counter", "FeatureFreq"]
+
+        def elements(base):
+            items = [{"cat_feature_index": int(c), "combination_element": "cat_feature_value"} for c in base["cat_features"]]
+            items += [{"float_feature_index": int(f), "border": float(np.float32(b)), "combination_element": "float_feature"}
+                      for f, b in base["float_splits"]]
+            items += [{"cat_feature_index": int(f), "value": int(v), "combination_element": "cat_feature_exact_value"}
+                      for f, v in base["one_hot_splits"]]
+            return items
+
+        def identifier(base):
+            return json.dumps({"type": type_names[int(base["ctr_type"])], "identifier": elements(base)})
+
+        doc["features_info"]["ctrs"] = [
+            {"identifier": identifier(c["base"]), "elements": elements(c["base"]),
+             "ctr_type": type_names[int(c["base"]["ctr_type"])], "prior_numerator": float(c["prior_num"]),
+             "prior_denomerator": float(c["prior_denom"]), "shift": float(c["shift"]), "scale": float(c["scale"]),
+             "target_border_idx": int(c["target_border_idx"]), "borders": [float(b) for b in np.asarray(c["borders"], np.float32)]}
+            for c in model["ctr_features"]]
+        data = {}
+        for t in model.get("ctr_tables", []):
+            kind = int(t["base"]["ctr_type"])
+            raw = np.asarray(t["index_hash_raw"], np.uint8).reshape(-1, 12)
+            keys = raw[:, :8].copy().view(np.uint64).ravel()
+            rows = raw[:, 8:].copy().view(np.uint32).ravel()
+            blob = np.asarray(t["ctr_blob"], np.uint8)
+            flat = []
+            for k, r in zip(keys, rows):
+                if int(k) == 0xFFFFFFFFFFFFFFFF:
+                    continue
+                flat.append(str(int(k)))
+                if kind in (2, 3):
+                    flat.append(float(blob[8 * r:8 * r + 4].view(np.float32)[0]))
+                    flat.append(int(blob[8 * r + 4:8 * r + 8].view(np.int32)[0]))
+                elif kind in (4, 5):
+                    flat.append(int(blob[4 * r:4 * r + 4].view(np.int32)[0]))
+                else:
+                    n = int(t["target_classes_count"])
+                    flat += [int(v) for v in blob[4 * n * r:4 * n * (r + 1)].view(np.int32)]
+            stride = 3 if kind in (2, 3) else 2 if kind in (4, 5) else int(t["target_classes_count"]) + 1
+            data[identifier(t["base"])] = {"hash_map": flat, "hash_stride": stride,
+                                           "counter_denominator": int(t["counter_denominator"])}
+        doc["ctr_data"] = data
     return json.dumps(doc)

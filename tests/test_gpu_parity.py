@@ -171,6 +171,31 @@ def test_json_model_format(golden_dir):
     _close(g.calc_flat(x), OracleModel(model).calc(x))
 
 
+def test_json_model_format_with_ctr_features(golden_dir):
+    """Models with CTR features through the json format: bins and predictions equal the oracle's on what
+    the format keeps of the model (tests/test_host_logic.py::json_view_of_ctr_model)."""
+    from tests.test_host_logic import json_view_of_ctr_model
+
+    cases = [(read_cbm_file(os.path.join(golden_dir, n)), None) for n in ("mushroom_model.cbm", "jvm_model_with_ctr.cbm",
+                                                                          "features_num_cat__dataset_adult.cbm")]
+    cases += [ctr_models.random_ctr_model(seed, **kwargs) for seed, kwargs in ctr_models.CASES]
+    checked = 0
+    for model, known in cases:
+        kept = json_view_of_ctr_model(model)
+        if kept is None:
+            continue
+        checked += 1
+        g = cb.ModelCalcer(buffer=rm.model_to_json(model), model_format="json")
+        o = OracleModel(kept)
+        if known is None:
+            floats, cats = rm.random_ctr_inputs(model, 1500, 21, rm.known_cat_hashes(model))
+        else:
+            floats, cats = ctr_models.random_documents(model, known, 1500, 21)
+        np.testing.assert_array_equal(g.quantize_hashed(floats, cats), o.binarize(floats, cats, layout="split"))
+        _close(g.calc_hashed(floats, cats), o.calc(floats, cats, layout="split"))
+    assert checked >= 5
+
+
 def test_rust_fixture_with_one_hot_string_cats(golden_dir):
     g = cb.ModelCalcer(os.path.join(golden_dir, "rust_tmp_model.cbm"))
     _close(g.calc(rm.RUST_FLOATS, rm.RUST_CATS), rm.RUST_EXPECTED)

@@ -10,7 +10,7 @@ import pytest
 
 import catboost_amd as cb
 from oracle import model_builder as mb
-from oracle.cbm_reader import read_cbm, read_cbm_file
+from oracle.cbm_reader import ctr_base_key, read_cbm, read_cbm_file
 from oracle.oracle import OracleModel
 from tests import refmodels as rm
 
@@ -356,8 +356,8 @@ def test_json_import_error_paths(golden_dir):
             pass
     import json
     doc = json.loads(text)
-    doc["features_info"]["ctrs"] = [{"borders": [0.5]}]
-    with pytest.raises(cb.CatBoostError, match="CTR"):
+    doc["features_info"]["ctrs"] = [{"borders": [0.5]}]  # a CTR feature without its description
+    with pytest.raises(cb.CatBoostError, match="elements"):
         cb.ModelCalcer(buffer=json.dumps(doc), model_format="json")
     with pytest.raises(cb.CatBoostError, match="can't open"):
         cb.ModelCalcer(os.path.join(golden_dir, "no_such_model.json"), model_format="json")
@@ -375,3 +375,98 @@ def test_feature_layout_is_checked_when_it_is_set(golden_dir):
     with pytest.raises(cb.CatBoostError, match="FlatIndexes has no entry"):
         g.set_feature_layout(flat_indexes=[0, 1, 2])
     g.set_feature_layout()
+
+
+def json_view_of_ctr_model(model):
+    """What the json format keeps of a model dict with CTR features: no TargetBorderClassifierIdx, and a
+    mean CTR's sum only when it is a whole number (the reference reads it with GetInteger,
+    json_model_helpers.cpp:562). None if two tables would share a key of ctr_data."""
+    import copy
+
+    kept = copy.deepcopy(model)
+    keys = set()
+    for t in kept["ctr_tables"]:
+        t["base"]["target_border_classifier_idx"] = 0
+        key = ctr_base_key(t["base"])
+        if key in keys:
+            return None
+        keys.add(key)
+        if t["base"]["ctr_type"] in (2, 3):
+            rows = t["ctr_blob"].view(np.dtype([("sum", "<f4"), ("count", "<i4")]))
+            whole = rows["sum"] == np.floor(rows["sum"])
+            rows["sum"] = np.where(whole, rows["sum"], np.float32(0))
+    for c in kept["ctr_features"]:
+        c["base"]["target_border_classifier_idx"] = 0
+    return kept
+
+
+def test_json_import_of_ctr_models(golden_dir):
+    """CTR features and their tables through the json format (CtrFeatureFromJson, CtrDataFromJson,
+    json_model_helpers.cpp:119-136, 531-580): what the library saves afterwards holds the same features and,
+    row for row, the same statistics as the model the json was written from."""
+    from tests import ctr_models
+
+    cases = [read_cbm_file(os.path.join(golden_dir, n)) for n in rm.CTR_FIXTURES]
+    cases += [ctr_models.random_ctr_model(seed, **kwargs)[0] for seed, kwargs in ctr_models.CASES]
+    checked = 0
+    for model in cases:
+        kept = json_view_of_ctr_model(model)
+        if kept is None:
+            continue
+        checked += 1
+        g = cb.ModelCalcer(buffer=rm.model_to_json(model), model_format="json")
+        back = read_cbm(g.save_to_buffer())
+        assert [ctr_base_key(c["base"]) for c in back["ctr_features"]] == [ctr_base_key(c["base"]) for c in kept["ctr_features"]]
+        for a, b in zip(back["ctr_features"], kept["ctr_features"]):
+            for k in ("target_border_idx", "prior_num", "prior_denom", "shift", "scale"):
+                assert a[k] == b[k]
+            np.testing.assert_array_equal(a["borders"], b["borders"])
+        tables = {ctr_base_key(t["base"]): t for t in back["ctr_tables"]}
+        assert len(tables) == len(kept["ctr_tables"])
+        for t in kept["ctr_tables"]:
+            got = tables[ctr_base_key(t["base"])]
+            assert got["counter_denominator"] == t["counter_denominator"]
+            if t["base"]["ctr_type"] in (0, 1):
+                assert got["target_classes_count"] == t["target_classes_count"]
+
+            def rows_by_hash(table):
+                raw = np.asarray(table["index_hash_raw"], np.uint8).reshape(-1, 12)
+                keys = raw[:, :8].copy().view(np.uint64).ravel()
+                rows = raw[:, 8:].copy().view(np.uint32).ravel()
+                width = {2: 8, 3: 8, 4: 4, 5: 4}.get(table["base"]["ctr_type"], 4 * max(table["target_classes_count"], 1))
+                blob = np.asarray(table["ctr_blob"], np.uint8)
+                return {int(k): blob[width * r:width * (r + 1)].tobytes() for k, r in zip(keys, rows)
+                        if int(k) != 0xFFFFFFFFFFFFFFFF}
+
+            assert rows_by_hash(got) == rows_by_hash(t)
+    assert checked >= 8
+
+
+def test_json_import_of_damaged_ctr_models(golden_dir):
+    """Damaged text of a model with CTR features fails cleanly or loads; it never crashes."""
+    import json
+
+    model = read_cbm_file(os.path.join(golden_dir, "jvm_model_with_ctr.cbm"))
+    text = rm.model_to_json(model)
+    rng = np.random.default_rng(17)
+    raw = bytearray(text.encode())
+    for _ in range(400):
+        corrupted = bytearray(raw)
+        for pos in rng.integers(0, len(raw), size=3):
+            corrupted[pos] = int(rng.integers(32, 127))
+        try:
+            cb.ModelCalcer(buffer=bytes(corrupted), model_format="json")
+        except cb.CatBoostError:
+            pass
+    doc = json.loads(text)
+    key = next(iter(doc["ctr_data"]))
+    for change in ({"hash_stride": 0}, {"hash_stride": 7}, {"hash_map": ["12", 1]}, {"hash_map": [12, 1, 2]},
+                   {"hash_map": ["-5", 1, 2]}, {"hash_map": ["18446744073709551615", 1, 2]}):
+        bad = json.loads(text)
+        bad["ctr_data"][key].update(change)
+        with pytest.raises(cb.CatBoostError):
+            cb.ModelCalcer(buffer=json.dumps(bad), model_format="json")
+    bad = json.loads(text)
+    del bad["ctr_data"][key]  # a CTR feature without its table
+    with pytest.raises(cb.CatBoostError, match="CTR"):
+        cb.ModelCalcer(buffer=json.dumps(bad), model_format="json")
