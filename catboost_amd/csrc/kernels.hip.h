@@ -1354,7 +1354,9 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalNonSymmetricLdsKernel(
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const uint32_t e = entry[g][j];
-                    pair[g][j] = *reinterpret_cast<const uint2*>(sEntries + start[g] + (e >> 21));
+                    // bits 18-20 of an entry are clear: e >> 19 is the byte offset of the pair of children
+                    pair[g][j] = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint8_t*>(sEntries + start[g]) +
+                                                                 (e >> 19));
                     bin[g][j] = tileBytes[((e & 0x3ff00u) | laneOff) + j];
                 }
             }
