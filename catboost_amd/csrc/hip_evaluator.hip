@@ -1337,8 +1337,8 @@ size_t HalfTileLdsBytes(uint32_t buckets, int maxd) {
 }
 
 // LDS of the per-wave leaf regions of the tile kernel
-size_t TileLeafLdsBytes(int maxd, int dchunk) {
-    return static_cast<size_t>(dev::kTileWaves) * (size_t(1) << maxd) * dchunk * sizeof(double);
+size_t TileLeafLdsBytes(int maxd, int dchunk, int waves = dev::kTileWaves) {
+    return static_cast<size_t>(waves) * (size_t(1) << maxd) * dchunk * sizeof(double);
 }
 
 struct TTileArgs {
@@ -1356,18 +1356,30 @@ struct TTileArgs {
     bool LeavesPairAligned;
 };
 
-template <bool SEVEN_BIT, int MAXD, int DCHUNK, bool LEAF_LDS>
-void LaunchEvalTileL(const TTileArgs& a) {
+template <bool SEVEN_BIT, int MAXD, int DCHUNK, bool LEAF_LDS, int WAVES>
+void LaunchEvalTileW(const TTileArgs& a) {
     const size_t blocks = (a.DocCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
-    const size_t lds = TileLdsBytes(a.Buckets, DCHUNK) + (LEAF_LDS ? TileLeafLdsBytes(MAXD, DCHUNK) : 0);
-    auto kernel = dev::EvalObliviousTileKernel<SEVEN_BIT, MAXD, DCHUNK, LEAF_LDS>;
+    const size_t lds = TileLdsBytes(a.Buckets, DCHUNK) + (LEAF_LDS ? TileLeafLdsBytes(MAXD, DCHUNK, WAVES) : 0);
+    auto kernel = dev::EvalObliviousTileKernel<SEVEN_BIT, MAXD, DCHUNK, LEAF_LDS, WAVES>;
     if (lds > 64 * 1024) {
         HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       static_cast<int>(lds)));
     }
-    hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(blocks)), dim3(64 * dev::kTileWaves), lds, a.Stream,
+    hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(blocks)), dim3(64 * WAVES), lds, a.Stream,
                        reinterpret_cast<const uint32_t*>(a.Bins), a.DocCount, a.Buckets, a.PackedTrees, a.Leaves, a.Bias,
                        a.Scale, a.Dim, a.TreeBegin, a.TreeEnd, a.Out);
+}
+
+template <bool SEVEN_BIT, int MAXD, int DCHUNK, bool LEAF_LDS>
+void LaunchEvalTileL(const TTileArgs& a) {
+    // a tile of which only one workgroup fits a CU gets sixteen waves instead of eight, LDS permitting
+    const size_t narrow = TileLdsBytes(a.Buckets, DCHUNK) + (LEAF_LDS ? TileLeafLdsBytes(MAXD, DCHUNK) : 0);
+    const size_t wide = TileLdsBytes(a.Buckets, DCHUNK) + (LEAF_LDS ? TileLeafLdsBytes(MAXD, DCHUNK, dev::kWideTileWaves) : 0);
+    if (2 * narrow > kMaxTileLdsBytes && wide <= kMaxTileLdsBytes) {
+        LaunchEvalTileW<SEVEN_BIT, MAXD, DCHUNK, LEAF_LDS, dev::kWideTileWaves>(a);
+    } else {
+        LaunchEvalTileW<SEVEN_BIT, MAXD, DCHUNK, LEAF_LDS, dev::kTileWaves>(a);
+    }
 }
 
 template <bool SEVEN_BIT, int MAXD, int DCHUNK>

@@ -719,14 +719,18 @@ __device__ __forceinline__ uint32_t TreeIndexes(const uint8_t* laneTile, uint32_
 // when that takes at most 8 loads per lane, and gathers from there; otherwise the values are
 // gathered straight from global memory. `leaves` must be readable for (1 << MAXD) * DCHUNK values
 // past the first value of the last tree.
-// grid = doc blocks, block = 64 * kTileWaves threads, dynamic LDS = buckets * 256 (rounded up to
-// 8) + 256 * DCHUNK * 8 [+ kTileWaves * (1 << MAXD) * DCHUNK * 8 with LEAF_LDS] bytes.
+// WAVES waves share a block (tree t goes to wave t % WAVES): kTileWaves, or kWideTileWaves when the
+// tile is so large that only one workgroup fits a CU: the waves of a workgroup wait on LDS round trips
+// most of the time, and sixteen of them hide what eight cannot (400 buckets: 1.75 instead of 2.79 ms).
+// grid = doc blocks, block = 64 * WAVES threads, dynamic LDS = buckets * 256 (rounded up to
+// 8) + 256 * DCHUNK * 8 [+ WAVES * (1 << MAXD) * DCHUNK * 8 with LEAF_LDS] bytes.
 constexpr int kTileWaves = 8;
+constexpr int kWideTileWaves = 16;
 constexpr int kPackedPaddedLeafSlot = 9;
 constexpr int kPackedLeafCountSlot = 10;
 
-template <bool SEVEN_BIT, int MAXD, int DCHUNK, bool LEAF_LDS>
-__global__ __launch_bounds__(64 * kTileWaves) __attribute__((amdgpu_waves_per_eu(2, 4))) void EvalObliviousTileKernel(
+template <bool SEVEN_BIT, int MAXD, int DCHUNK, bool LEAF_LDS, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(2, 4))) void EvalObliviousTileKernel(
     const uint32_t* __restrict__ bins, size_t docCount, uint32_t bucketCount, const uint32_t* __restrict__ packedTrees,
     const double* __restrict__ leaves, const double* __restrict__ bias, double scale, int dim, uint32_t treeBegin,
     uint32_t treeEnd, double* __restrict__ out) {
@@ -744,7 +748,7 @@ __global__ __launch_bounds__(64 * kTileWaves) __attribute__((amdgpu_waves_per_eu
     const size_t block = blockIdx.x;
     const uint32_t tileDwords = bucketCount * kWave;
     const uint32_t* src = bins + block * tileDwords;
-    for (uint32_t i = tid; i < tileDwords; i += 64 * kTileWaves) {
+    for (uint32_t i = tid; i < tileDwords; i += 64 * WAVES) {
         sTile[i] = src[i];
     }
     const bool addBias = treeBegin == 0;
@@ -787,13 +791,13 @@ __global__ __launch_bounds__(64 * kTileWaves) __attribute__((amdgpu_waves_per_eu
     ((tree) < treeEnd ? packedTrees[static_cast<size_t>(tree) * kPackedTreeDwords + slot] : 0u)
         uint32_t t = treeBegin + wave;
         uint32_t row = CBAMD_FETCH_ROW(t);
-        uint32_t rowNext = CBAMD_FETCH_ROW(t + kTileWaves);
+        uint32_t rowNext = CBAMD_FETCH_ROW(t + WAVES);
         if (LEAF_LDS && kPrefetch && t < treeEnd) {
             CBAMD_FETCH_LEAVES(row);
         }
         while (t < treeEnd) {
-            const uint32_t tNext = t + kTileWaves;
-            const uint32_t rowNext2 = CBAMD_FETCH_ROW(tNext + kTileWaves);
+            const uint32_t tNext = t + WAVES;
+            const uint32_t rowNext2 = CBAMD_FETCH_ROW(tNext + WAVES);
             const double* leaf = CBAMD_TREE_VALUES(row);
             if (LEAF_LDS) {
                 // publish this tree's leaf values in the wave's region; the previous tree's gathers
@@ -861,7 +865,7 @@ __global__ __launch_bounds__(64 * kTileWaves) __attribute__((amdgpu_waves_per_eu
 #undef CBAMD_TREE_VALUES
         // waves add their partial sums in wave order into the LDS accumulator; the last wave
         // finishes the values and writes them out
-        for (uint32_t w = 0; w + 1 < kTileWaves; ++w) {
+        for (uint32_t w = 0; w + 1 < WAVES; ++w) {
             if (wave == w) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
@@ -874,7 +878,7 @@ __global__ __launch_bounds__(64 * kTileWaves) __attribute__((amdgpu_waves_per_eu
             }
             __syncthreads();
         }
-        if (wave == kTileWaves - 1) {
+        if (wave == WAVES - 1) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const size_t doc = block * kDocsPerBlock + j * kWave + lane;

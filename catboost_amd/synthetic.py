@@ -17,6 +17,9 @@
   C2B C2 over 20 features instead of 200, so that about 200 borders of every feature are used: bins
       above 127 (the 8-bit compare of the mixed kernels). Not one of the baseline workloads.
 
+  C2W C2 over 400 features and 2M docs: more buckets than the register-resident kernels hold, the LDS tile
+      kernel's case. Not one of the baseline workloads.
+
 Every split is (feature, border) drawn uniformly; models go through the builder, so only the
 borders that some split uses survive. Leaf values are N(0, sigma).
 """
@@ -32,6 +35,8 @@ CONFIGS = {
                docs=4_000_000, dist="normal_lognormal", nan_rate=0.05),
     "C2B": dict(kind="oblivious", trees=1000, depth=8, floats=20, borders=254, dim=1, leaf_sigma=0.005,
                 docs=4_000_000, dist="normal_lognormal", nan_rate=0.05),
+    "C2W": dict(kind="oblivious", trees=1000, depth=8, floats=400, borders=254, dim=1, leaf_sigma=0.005,
+                docs=2_000_000, dist="normal_lognormal", nan_rate=0.05),
     "C3": dict(kind="oblivious", trees=2000, depth=6, floats=100, borders=64, dim=10, leaf_sigma=0.01,
                docs=2_000_000, dist="uniform3", nan_rate=0.0),
     "C4": dict(kind="nonsymmetric", trees=500, depth=10, floats=300, borders=254, dim=1, leaf_sigma=0.01,
