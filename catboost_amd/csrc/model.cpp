@@ -191,10 +191,12 @@ void TModelTrees::UpdateRuntimeData() {
                          NonSymmetricStepNodes.size() == TreeSplits.size(),
                      "non-symmetric node tables differ in length");
         for (size_t t = 0; t < TreeSizes.size(); ++t) {
+            CBAMD_ENSURE(TreeStartOffsets[t] >= 0 && TreeSizes[t] > 0 &&
+                             static_cast<size_t>(TreeStartOffsets[t]) + static_cast<size_t>(TreeSizes[t]) <=
+                                 NonSymmetricStepNodes.size(),
+                         "tree nodes out of range");
             const int begin = TreeStartOffsets[t];
             const int end = begin + TreeSizes[t];
-            CBAMD_ENSURE(begin >= 0 && TreeSizes[t] > 0 && static_cast<size_t>(end) <= NonSymmetricStepNodes.size(),
-                         "tree nodes out of range");
             uint32_t minLeaf = std::numeric_limits<uint32_t>::max();
             for (int n = begin; n < end; ++n) {
                 const auto& node = NonSymmetricStepNodes[n];

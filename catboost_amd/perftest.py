@@ -1,15 +1,18 @@
 """Throughput of a model on this machine's GPU, in the spirit of the reference's model_perftest tool
-(catboost/tools/model_perftest/lib/main.cpp:165-330: --model-path, --block-size, --repetitions; it times
-the evaluator's entry points block by block over a pool).
+(catboost/tools/model_perftest/lib/main.cpp:165-330: --model-path, --block-size, --threads, --repetitions;
+it times the evaluator's entry points block by block over a pool).
 
     python -m catboost_amd.perftest -m model.cbm [--pool-path pool.tsv] [--docs N] [--block-size B]
-                                    [--repetitions R] [--model-format cbm|json] [--device-id D] [--graph]
+                                    [--repetitions R] [--threads T] [--model-format cbm|json] [--device-id D]
+                                    [--graph]
 
 Without a pool the documents are random: floats around the model's borders, categorical hashes at random.
 A pool is a tab-separated file of flat feature rows (categorical columns as strings). Reports documents
 per second of the flat host entry point (rows by pointer, PCIe both ways) and of the device entry points
 on features that already sit in HBM; with --graph also of a block's quantize + evaluate launches captured
-once into a HIP graph and replayed per block (what a serving loop with small blocks does).
+once into a HIP graph and replayed per block (what a serving loop with small blocks does). With
+--threads T above 1 the flat host entry point is also timed from T caller threads at once, each with the
+blocks of its share (one model handle: calls from several threads are allowed and run on streams of their own).
 """
 import argparse
 import json
@@ -76,6 +79,32 @@ def run(args):
     seconds = time.perf_counter() - start
     report["host_flat_docs_per_sec"] = args.repetitions * len(blocks) * block / seconds
 
+    if args.threads > 1:
+        import threading
+
+        shares = [blocks[t::args.threads] for t in range(args.threads)]
+        failures = []
+
+        def caller(share):
+            try:
+                for _ in range(args.repetitions):
+                    for b in share:
+                        model.calc_flat(b)
+            except Exception as e:  # reported by the main thread
+                failures.append(e)
+
+        callers = [threading.Thread(target=caller, args=(share,)) for share in shares if share]
+        start = time.perf_counter()
+        for t in callers:
+            t.start()
+        for t in callers:
+            t.join()
+        seconds = time.perf_counter() - start
+        if failures:
+            raise failures[0]
+        report["threads"] = len(callers)
+        report["host_flat_threads_docs_per_sec"] = args.repetitions * len(blocks) * block / seconds
+
     ev = model.evaluator()
     device = "cuda:%d" % args.device_id
     resident = [torch.from_numpy(np.ascontiguousarray(b)).to(device) for b in blocks]
@@ -134,6 +163,7 @@ def main(argv=None):
     parser.add_argument("--docs", type=int, default=1_000_000, help="random documents when no pool is given")
     parser.add_argument("--block-size", type=int, default=0, help="documents per call (default: all)")
     parser.add_argument("--repetitions", type=int, default=10)
+    parser.add_argument("-T", "--threads", type=int, default=1, help="caller threads for the host entry point")
     parser.add_argument("--graph", action="store_true", help="also time the block as a replayed HIP graph")
     parser.add_argument("--device-id", type=int, default=0)
     parser.add_argument("--seed", type=int, default=0)

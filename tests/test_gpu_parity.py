@@ -885,6 +885,9 @@ def test_perftest_tool(golden_dir, tmp_path, capsys):
     assert report["host_flat_docs_per_sec"] > 0 and report["device_docs_per_sec"] > report["host_flat_docs_per_sec"]
     assert perftest.main(["-m", str(path), "--docs", "4096", "--block-size", "256", "--repetitions", "2", "--graph"]) == 0
     assert json.loads(capsys.readouterr().out)["graph_replay_docs_per_sec"] > 0
+    assert perftest.main(["-m", str(path), "--docs", "16384", "--block-size", "1024", "--repetitions", "2", "-T", "4"]) == 0
+    report = json.loads(capsys.readouterr().out)
+    assert report["threads"] == 4 and report["host_flat_threads_docs_per_sec"] > 0
     # a pool of flat rows: the rust fixture's three documents (one string categorical column)
     pool = tmp_path / "pool.tsv"
     pool.write_text("".join("%g\t%g\t%s\t%g\n" % (f[0], f[1], c[0], f[2]) for f, c in zip(rm.RUST_FLOATS, rm.RUST_CATS)))
