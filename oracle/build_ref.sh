@@ -30,3 +30,10 @@ echo "built $OUT/fmath_exp"
 # the CTR calculator of exported models (model_export/resources/ctr_structs.cpp + ctr_calcer.cpp)
 g++ -std=c++17 -O2 -w -I "$R" "$HERE/ref_ctr_main.cpp" -o "$OUT/ctr_calc"
 echo "built $OUT/ctr_calc"
+# models that the reference holds as exported C++ code (canonical outputs of its export tests)
+CANON="$R/catboost/python-package/ut/medium/canondata"
+g++ -std=c++20 -O1 -w -DWITH_CATS=1 "-DMODEL_SOURCE=\"$CANON/test.test_cpp_export_with_cat_features_CPU_/model.cpp\"" \
+  "$HERE/ref_export_main.cpp" -o "$OUT/export_cat"
+g++ -std=c++20 -O1 -w -DWITH_CATS=0 "-DMODEL_SOURCE=\"$CANON/test.test_cpp_export_no_cat_features_CPU_/model.cpp\"" \
+  "$HERE/ref_export_main.cpp" -o "$OUT/export_nocat"
+echo "built $OUT/export_cat $OUT/export_nocat"

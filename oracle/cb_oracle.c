@@ -34,7 +34,11 @@
  * reproduced bit for bit. That calculator answers an unknown hash with Calc(0, 0) for every kind,
  * the evaluator's TStaticCtrProvider with Calc(0, denominator) for Counter and FeatureFreq
  * (static_ctr_provider.cpp:63-75); this one case rests on the adult goldens (Counter CTRs, unknown
- * categories) alone.
+ * categories) alone. Whole models: the two trained models that the reference keeps as exported C++
+ * code, tables and applier in one file (python-package/ut/medium/canondata/test.test_cpp_export_*;
+ * built where they lie into oracle/_ref/export_{cat,nocat}): that applier's predictions on 3000
+ * seeded documents each (tests/golden/cpp_export_vectors.npz) are reproduced bit for bit, and the
+ * (bucket, split index, xor mask) derived here per tree split equal the arrays in that code.
  * Parity unpinned (followed by reading only, cross-checked by the brute force): the NaN gating
  * "HasNans && treatment != AsIs", >254-border buckets combined with one-hot XorMask, the
  * leaf numbering of non-symmetric multi-dimensional models, and for CTR projections the table

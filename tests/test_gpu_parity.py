@@ -364,6 +364,34 @@ def test_synthetic_ctr_models_of_every_kind(golden_dir, monkeypatch, seed, tile)
         np.testing.assert_array_equal(g.calc_leaf_indexes_flat(flat), o.leaf_indexes(flat))
 
 
+@pytest.mark.parametrize("name", ["cat", "nocat"])
+def test_models_that_the_reference_holds_as_exported_cpp(golden_dir, name):
+    """The two models that the reference keeps as exported C++ code (tests/golden/make_export_vectors.py):
+    the library's predictions against that code's own applier on the stored documents, bins and leaf
+    indexes against the oracle, the split tables the library derives against the exporter's arrays."""
+    v = np.load(os.path.join(golden_dir, "cpp_export_vectors.npz"))
+    path = os.path.join(golden_dir, "cpp_export_%s.cbm" % name)
+    m = read_cbm_file(path)
+    o = OracleModel(m)
+    g = cb.ModelCalcer(path)
+    floats, cats = v["floats_" + name], v["cats_" + name]
+    expected, comparable = v["predictions_" + name], v["comparable_" + name]
+    got = g.calc_hashed(floats, cats)
+    _close(got[comparable], expected[comparable])
+    _close(got, o.calc(floats, cats, layout="split"))
+    np.testing.assert_array_equal(g.quantize_hashed(floats, cats), o.binarize(floats, cats, layout="split"))
+    flat = rm.flat_rows(m, floats, cats)
+    _close(g.calc_flat(flat), got)
+    np.testing.assert_array_equal(g.calc_leaf_indexes_flat(flat), o.leaf_indexes(flat))
+    if name == "cat":
+        # the strings of the code's own table through the string entry point
+        strings = {int(h): str(s) for s, h in zip(v["hash_strings_cat"], v["hash_values_cat"])}
+        rows = [i for i in range(200) if all(int(h) in strings for h in cats[i])]
+        assert len(rows) > 50
+        as_text = [[strings[int(h)] for h in cats[i]] for i in rows]
+        _close(g.calc(floats[rows], as_text), got[rows])
+
+
 def test_synthetic_ctr_model_survives_save_and_load(golden_dir, tmp_path):
     """The library's own writer keeps CTR features of every kind: load, save, load again, same bins."""
     path = os.path.join(golden_dir, "synthetic_ctr_5.cbm")

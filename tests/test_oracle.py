@@ -278,6 +278,35 @@ def test_ctr_models_against_the_raw_definition(golden_dir, name):
     assert all(len(np.unique(row)) > 1 for row in ctrs)
 
 
+@pytest.mark.parametrize("name", ["cat", "nocat"])
+def test_models_that_the_reference_holds_as_exported_cpp(golden_dir, name):
+    """Two trained models that the reference keeps as exported C++ code, tables and applier in one file
+    (canonical outputs of its export tests; run by tests/golden/make_export_vectors.py, which also put
+    the tables together into tests/golden/cpp_export_<name>.cbm): predictions of the oracle against that
+    applier's on 3000 documents, floats on and around the borders, known and unknown categories. The
+    sums run in the same order, so the values are equal bit for bit. For the model with categorical
+    features (20 trees, 13 Borders and Counter CTRs) also the (bucket, split index, xor mask) of every
+    tree split against the arrays the reference's exporter wrote, and the string hash on the 58 category
+    names of the code's own table."""
+    v = np.load(os.path.join(golden_dir, "cpp_export_vectors.npz"))
+    m = read_cbm_file(os.path.join(golden_dir, "cpp_export_%s.cbm" % name))
+    o = OracleModel(m)
+    floats, cats = v["floats_" + name], v["cats_" + name]
+    expected, comparable = v["predictions_" + name], v["comparable_" + name]
+    assert comparable.mean() > 0.8 and len(np.unique(expected)) > 500
+    got = o.calc(floats, cats, layout="split")
+    np.testing.assert_array_equal(got[comparable], expected[comparable])
+    np.testing.assert_array_equal(got, o.bruteforce(floats, cats, layout="split")[0])
+    if name == "cat":
+        bucket, xor_mask, split_idx = o.repacked_bins()
+        np.testing.assert_array_equal(bucket, v["split_bucket_cat"])
+        np.testing.assert_array_equal(split_idx, v["split_idx_cat"])
+        np.testing.assert_array_equal(xor_mask, v["split_xor_mask_cat"])
+        assert len(v["hash_strings_cat"]) == 58
+        for text, value in zip(v["hash_strings_cat"], v["hash_values_cat"]):
+            assert cat_feature_hash_signed(str(text)) == int(value)
+
+
 @pytest.mark.parametrize("seed", [seed for seed, _ in ctr_models.CASES])
 def test_ctr_values_match_the_reference_ctr_calculator(golden_dir, seed):
     """CTR values on synthetic models with all six CTR types, tables with up to five target classes and
