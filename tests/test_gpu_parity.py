@@ -614,6 +614,34 @@ def test_iris_fixture(golden_dir):
     np.testing.assert_allclose(g.calc_flat(feats).reshape(-1, 3).sum(axis=1), 1.0, atol=1e-12)
 
 
+@pytest.mark.parametrize("name", ["all", "missed"])
+def test_multiclass_probabilities_of_the_reference_canondata(golden_dir, name):
+    """The multi-class model and the 17-digit probability table of the reference's own
+    test_multiclass_classes_count: the library's Probability predictions, host and device post-processing."""
+    from tests.test_oracle import multiclass_classes_count_case
+    path, features, expected = multiclass_classes_count_case(golden_dir, name)
+    g = cb.ModelCalcer(path)
+    g.set_prediction_type("Probability")
+    got = g.calc_flat(features).reshape(100, -1)
+    np.testing.assert_allclose(got, expected, rtol=1e-9, atol=1e-12)
+    np.testing.assert_allclose(g.calc_flat_transposed(np.ascontiguousarray(features.T)).reshape(100, -1), expected,
+                               rtol=1e-9, atol=1e-12)
+    g.set_prediction_type("Class")
+    # classes from the raw values (documents with equal stored probabilities may differ in the raw ones)
+    raw = OracleModel(read_cbm_file(path)).calc(features).reshape(100, -1)
+    np.testing.assert_array_equal(g.calc_flat(features), np.argmax(raw, axis=1).astype(np.float64))
+    # on the device: raw values, then the prediction type applied in place by the library's kernel
+    import torch
+    ev = g.evaluator()
+    dim = expected.shape[1]
+    x = torch.from_numpy(features).cuda()
+    out = torch.zeros(100 * dim, dtype=torch.float64, device="cuda")
+    ev.eval_data(ev.features(cb.LAYOUT_FLAT_ROWS, x.data_ptr(), x.shape[1]), 100, out.data_ptr())
+    ev.apply_prediction_type(cb.APT_PROBABILITY, 100, out.data_ptr(), out.data_ptr())
+    ev.synchronize()
+    np.testing.assert_allclose(out.cpu().numpy().reshape(100, dim), expected, rtol=1e-9, atol=1e-12)
+
+
 def test_prediction_types_of_the_reference_unit_test():
     """TestFlatCalcMultiValMultiProba (formula_evaluator_ut.cpp:148-165) through the C API, and the
     one-dimensional types on the two-tree model with scale and bias."""

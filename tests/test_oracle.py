@@ -9,7 +9,7 @@ import pytest
 
 from oracle import model_builder as mb
 from oracle.cbm_reader import ctr_base_key, read_cbm, read_cbm_file
-from oracle.oracle import (OracleModel, cat_feature_hash_signed, city_hash64,
+from oracle.oracle import (OracleModel, apply_prediction_type, cat_feature_hash_signed, city_hash64,
                            integer_cat_feature_hash)
 from tests import cbm_writer, ctr_models
 from tests import refmodels as rm
@@ -276,6 +276,35 @@ def test_ctr_models_against_the_raw_definition(golden_dir, name):
     # known and unknown categories both occur
     ctrs = o.ctrs(floats, cats, layout="split")
     assert all(len(np.unique(row)) > 1 for row in ctrs)
+
+
+def multiclass_classes_count_case(golden_dir, name):
+    """(model path, features, expected probabilities of the model's own dimensions) of a canonical case of
+    the reference's test_multiclass_classes_count (catboost/python-package/ut/medium/test.py:1979-2031):
+    model.bin and predictions.txt are its canondata, the 100 x 10 features are the numpy RandomState(0)
+    draw that the test makes. With labels 1 and 3 only ("missed") the model has two dimensions and the
+    stored table four columns: the Python package spreads the two over the declared classes
+    (class_to_label [1, 3] in the model's class_params) and leaves ~1e-308 in the others."""
+    path = os.path.join(golden_dir, "multiclass_classes_count_%s.cbm" % name)
+    features = np.random.RandomState(seed=0).random_sample(size=(100, 10)).astype(np.float32)
+    expected = np.loadtxt(os.path.join(golden_dir, "multiclass_classes_count_%s.predictions.txt" % name))
+    assert expected.shape == (100, 4)
+    if name == "missed":
+        assert np.abs(expected[:, [0, 2]]).max() < 1e-300
+        expected = expected[:, [1, 3]]
+    return path, features, expected
+
+
+@pytest.mark.parametrize("name", ["all", "missed"])
+def test_multiclass_probabilities_of_the_reference_canondata(golden_dir, name):
+    """Softmax probabilities of a trained multi-class model against the 17-digit table that the
+    reference's own test stores: equal to the last bit (multi-dimensional leaves, the sum over trees,
+    CalcSoftmax with the reference's exponent)."""
+    path, features, expected = multiclass_classes_count_case(golden_dir, name)
+    o = OracleModel(read_cbm_file(path))
+    assert o.dim == expected.shape[1]
+    got = apply_prediction_type(o.calc(features), o.dim, "Probability").reshape(100, -1)
+    np.testing.assert_array_equal(got, expected)
 
 
 @pytest.mark.parametrize("name", ["cat", "nocat"])
