@@ -642,6 +642,16 @@ def test_multiclass_probabilities_of_the_reference_canondata(golden_dir, name):
     np.testing.assert_allclose(out.cpu().numpy().reshape(100, dim), expected, rtol=1e-9, atol=1e-12)
 
 
+def test_model_of_the_backward_compatibility_test(golden_dir):
+    """The old-version three-class model of the reference's test_multiclass_model_backward_compatibility and
+    the canonical outputs of `catboost calc` for it (10 digits), through the library."""
+    v = np.load(os.path.join(golden_dir, "cloudness_backward_compatibility.npz"))
+    g = cb.ModelCalcer(os.path.join(golden_dir, "cloudness_backward_compatibility.cbm"))
+    for kind in ("RawFormulaVal", "Probability", "Class"):
+        g.set_prediction_type(kind)
+        np.testing.assert_allclose(g.calc_flat(v["features"]), v[kind].ravel(), rtol=6e-10, atol=0)
+
+
 def test_prediction_types_of_the_reference_unit_test():
     """TestFlatCalcMultiValMultiProba (formula_evaluator_ut.cpp:148-165) through the C API, and the
     one-dimensional types on the two-tree model with scale and bias."""

@@ -307,6 +307,23 @@ def test_multiclass_probabilities_of_the_reference_canondata(golden_dir, name):
     np.testing.assert_array_equal(got, expected)
 
 
+def test_model_of_the_backward_compatibility_test(golden_dir):
+    """test_multiclass_model_backward_compatibility (catboost/pytest/test.py:7543-7571): a three-class model
+    written by an old version (catboost/pytest/data/multiclass_model.bin, copied) applied to
+    cloudness_small/train_small; the canonical outputs of `catboost calc` for the three prediction types
+    are printed with 10 digits. The .npz holds the pool's numeric columns (categorical ones, which the
+    model's tree does not look at, as zeros) and those tables."""
+    v = np.load(os.path.join(golden_dir, "cloudness_backward_compatibility.npz"))
+    m = read_cbm_file(os.path.join(golden_dir, "cloudness_backward_compatibility.cbm"))
+    assert "class_params" not in m["info"]
+    o = OracleModel(m)
+    raw = o.calc(v["features"])
+    np.testing.assert_allclose(raw.reshape(-1, 3), v["RawFormulaVal"], rtol=6e-10, atol=0)
+    np.testing.assert_allclose(apply_prediction_type(raw, 3, "Probability").reshape(-1, 3), v["Probability"],
+                               rtol=6e-10, atol=0)
+    np.testing.assert_array_equal(apply_prediction_type(raw, 3, "Class"), v["Class"].ravel())
+
+
 @pytest.mark.parametrize("name", ["cat", "nocat"])
 def test_models_that_the_reference_holds_as_exported_cpp(golden_dir, name):
     """Two trained models that the reference keeps as exported C++ code, tables and applier in one file
