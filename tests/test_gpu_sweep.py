@@ -84,8 +84,12 @@ def _ctr_model_case(seed, rng, monkeypatch):
                                err_msg=tag)
 
 
-def test_random_model_shapes(monkeypatch):
-    for seed in _seeds():
+def test_random_model_shapes(monkeypatch, capsys):
+    seeds = _seeds()
+    for seed in seeds:
+        if (seed - seeds[0]) % 2000 == 1999:
+            with capsys.disabled():  # a long run shows that it is alive
+                print("sweep: %d of %d seeds" % (seed - seeds[0] + 1, len(seeds)), flush=True)
         rng = np.random.default_rng(seed)
         kind = seed % 3
         monkeypatch.setenv("CATBOOST_AMD_REG_SIX", str(int(rng.integers(0, 2))))
