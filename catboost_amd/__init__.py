@@ -144,6 +144,7 @@ def load_library():
         "CbHipQuantize": (ctypes.c_bool, [vp, ctypes.POINTER(DeviceFeatures), sz, vp, vp]),
         "CbHipEvalQuantized": (ctypes.c_bool, [vp, vp, sz, sz, sz, vp, vp]),
         "CbHipEvalData": (ctypes.c_bool, [vp, ctypes.POINTER(DeviceFeatures), sz, sz, sz, vp, vp]),
+        "CbHipEvalDataNoAlloc": (ctypes.c_bool, [vp, ctypes.POINTER(DeviceFeatures), sz, sz, sz, vp, vp]),
         "CbHipLeafIndexesQuantized": (ctypes.c_bool, [vp, vp, sz, sz, sz, vp, vp]),
         "CbHipExportQuantized": (ctypes.c_bool, [vp, vp, sz, vp, vp]),
         "CbHipApplyPredictionTypeDevice": (ctypes.c_bool, [vp, ctypes.c_int, sz, vp, vp, vp]),
@@ -366,6 +367,11 @@ class DeviceEvaluator:
     def eval_data(self, features, doc_count, results_ptr, tree_start=0, tree_end=None, stream=None):
         tree_end = self.tree_count if tree_end is None else tree_end
         _check(self._lib.CbHipEvalData(self._h, ctypes.byref(features), doc_count, tree_start, tree_end, results_ptr, stream))
+
+    def eval_data_no_alloc(self, features, doc_count, results_ptr, tree_start=0, tree_end=None, stream=None):
+        """eval_data with the bins in the library's fixed device array: allocates nothing, asynchronous."""
+        tree_end = self.tree_count if tree_end is None else tree_end
+        _check(self._lib.CbHipEvalDataNoAlloc(self._h, ctypes.byref(features), doc_count, tree_start, tree_end, results_ptr, stream))
 
     def leaf_indexes_quantized(self, bins_ptr, doc_count, indexes_ptr, tree_start=0, tree_end=None, stream=None):
         tree_end = self.tree_count if tree_end is None else tree_end

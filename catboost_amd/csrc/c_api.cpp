@@ -834,6 +834,13 @@ bool CbHipEvalData(CbHipEvaluatorHandle* evaluator, const CbHipFeatures* deviceF
     });
 }
 
+bool CbHipEvalDataNoAlloc(CbHipEvaluatorHandle* evaluator, const CbHipFeatures* deviceFeatures, size_t docCount,
+                          size_t treeStart, size_t treeEnd, double* deviceResults, void* hipStream) {
+    return Guard([&] {
+        E(evaluator)->CalcDeviceNoAlloc(ToBatch(deviceFeatures), docCount, treeStart, treeEnd, deviceResults, hipStream);
+    });
+}
+
 bool CbHipLeafIndexesQuantized(CbHipEvaluatorHandle* evaluator, const void* deviceBins, size_t docCount,
                                size_t treeStart, size_t treeEnd, uint32_t* deviceIndexes, void* hipStream) {
     return Guard([&] {

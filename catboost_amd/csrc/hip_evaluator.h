@@ -67,6 +67,12 @@ public:
     // binarize + evaluate with a scratch bin buffer owned by the evaluator; records kernel times
     void CalcDevice(const TFeatureBatch& batch, size_t docCount, size_t treeStart, size_t treeEnd,
                     double* results, void* stream);
+    // the same two launches with the bins in a fixed array that every GPU holds from library load on:
+    // no allocation, no synchronisation, nothing recorded. At most kNoAllocScratchBytes of bins per call
+    // (QuantizedBytes tells); calls that overlap on one GPU share the array and race
+    static constexpr size_t kNoAllocScratchBytes = size_t(32) << 20;
+    void CalcDeviceNoAlloc(const TFeatureBatch& batch, size_t docCount, size_t treeStart, size_t treeEnd,
+                           double* results, void* stream);
     void Synchronize(void* stream);
     TKernelTimes LastKernelTimes() const { return LastTimes; }
 

@@ -12,6 +12,11 @@
 #include <thread>
 #include <vector>
 
+// Bin buffer of the entry point that allocates nothing (THipEvaluator::CalcDeviceNoAlloc): every GPU the
+// library runs on holds one copy of this array, at its own address, until the process ends. In host code
+// the name is only a handle for hipGetSymbolAddress; kernels get the address that call returns.
+static __device__ __align__(256) unsigned char scratch[cbamd::THipEvaluator::kNoAllocScratchBytes];
+
 namespace cbamd {
 
 namespace {
@@ -84,6 +89,23 @@ private:
     T* Ptr = nullptr;
     size_t Cap = 0;
 };
+
+// Address of `scratch` on a device, asked for once per device, with that device current.
+uint8_t* NoAllocScratchOfCurrentDevice(int deviceId) {
+    static std::mutex lock;
+    static std::vector<uint8_t*> perDevice;
+    std::lock_guard<std::mutex> guard(lock);
+    if (perDevice.size() <= static_cast<size_t>(deviceId)) {
+        perDevice.resize(static_cast<size_t>(deviceId) + 1, nullptr);
+    }
+    if (perDevice[deviceId] == nullptr) {
+        void* ptr = nullptr;
+        HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        CBAMD_ENSURE(ptr != nullptr, "the device holds no copy of the no-allocation bin buffer");
+        perDevice[deviceId] = static_cast<uint8_t*>(ptr);
+    }
+    return perDevice[deviceId];
+}
 
 // Code object of the register-resident evaluate kernels (assembled from the output of
 // gen_eval_reg_kernel.py at build time).
@@ -601,6 +623,7 @@ struct THipEvaluator::TImpl {
     int DeviceId = 0;
     hipStream_t Stream = nullptr;
     hipEvent_t Ev[3] = {nullptr, nullptr, nullptr};
+    uint8_t* NoAllocScratch = nullptr;  // this device's copy of the file-scope array `scratch`
     bool Oblivious = true;
     uint32_t RealBucketCount = 0;  // buckets of the model; the device layout uses max(1, this)
     uint32_t LayoutBuckets = 1;
@@ -734,6 +757,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
     HIP_CHECK(hipSetDevice(deviceId));
     TImpl& m = *Impl;
     m.DeviceId = deviceId;
+    m.NoAllocScratch = NoAllocScratchOfCurrentDevice(deviceId);
     HIP_CHECK(hipStreamCreateWithFlags(&m.Stream, hipStreamNonBlocking));
     for (auto& e : m.Ev) {
         HIP_CHECK(hipEventCreate(&e));
@@ -1661,6 +1685,18 @@ void THipEvaluator::CalcDevice(const TFeatureBatch& batch, size_t docCount, size
     HIP_CHECK(hipStreamSynchronize(s));
     HIP_CHECK(hipEventElapsedTime(&LastTimes.BinarizeMs, m.Ev[0], m.Ev[1]));
     HIP_CHECK(hipEventElapsedTime(&LastTimes.EvalMs, m.Ev[1], m.Ev[2]));
+}
+
+void THipEvaluator::CalcDeviceNoAlloc(const TFeatureBatch& batch, size_t docCount, size_t treeStart, size_t treeEnd,
+                                      double* results, void* stream) {
+    TImpl& m = *Impl;
+    const size_t maxDocs = kNoAllocScratchBytes / (static_cast<size_t>(m.LayoutBuckets) * dev::kDocsPerBlock) * dev::kDocsPerBlock;
+    CBAMD_ENSURE(docCount <= maxDocs, "batch of " + std::to_string(docCount) + " documents exceeds the fixed bin buffer: at most " +
+                                          std::to_string(maxDocs) + " documents per call for this model");
+    // every (block, bucket) cell that the evaluate kernels read is written by the binarize kernels of
+    // the same call, so nothing of the previous call's contents has to be cleared
+    QuantizeDevice(batch, docCount, m.NoAllocScratch, stream);
+    EvalQuantizedDevice(m.NoAllocScratch, docCount, treeStart, treeEnd, results, stream);
 }
 
 // ---------------------------------------------------------------------------- host staging ----

@@ -110,6 +110,18 @@ bool CbHipEvalQuantized(CbHipEvaluatorHandle* evaluator, const void* deviceBins,
 bool CbHipEvalData(CbHipEvaluatorHandle* evaluator, const CbHipFeatures* deviceFeatures, size_t docCount,
                    size_t treeStart, size_t treeEnd, double* deviceResults, void* hipStream);
 
+/* CbHipEvalData for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc). No counterpart in the reference. The bins of the
+ * call sit in a fixed 32 MiB array that every GPU the library runs on holds until the process ends,
+ * instead of the evaluator's grow-only scratch buffer; the call allocates nothing, waits for nothing
+ * and records no kernel times: it only launches the binarize and evaluate kernels on `hipStream`
+ * (NULL = the evaluator's own stream). Fails when CbHipQuantizedBytes(evaluator, docCount) exceeds
+ * 32 MiB (the error names the largest document count for the model). All calls on one GPU share the
+ * array, so calls that overlap there (two streams, two threads, two evaluators) race; calls in stream
+ * order on one stream are safe. */
+bool CbHipEvalDataNoAlloc(CbHipEvaluatorHandle* evaluator, const CbHipFeatures* deviceFeatures, size_t docCount,
+                          size_t treeStart, size_t treeEnd, double* deviceResults, void* hipStream);
+
 /* Leaf indexes deviceIndexes[doc * (treeEnd - treeStart) + t] (IModelEvaluator::CalcLeafIndexes on
  * quantized data, evaluation_interface.h:289-294; unimplemented in cuda/evaluator.cpp:337-348). */
 bool CbHipLeafIndexesQuantized(CbHipEvaluatorHandle* evaluator, const void* deviceBins, size_t docCount,

@@ -1,0 +1,74 @@
+"""CbHipEvalDataNoAlloc, the entry point that allocates nothing, against CbHipEvalData. Needs an MI355X.
+
+Both run the same binarize and evaluate kernels; one keeps the bins in the evaluator's scratch buffer,
+the other in the library's fixed device array. Bar: bit for bit, and against the oracle within
+1e-9 relative / 1e-12 absolute. Two calls in a row, the second with fewer documents, so that what the
+first call left in the array sits behind (and under) the second call's bins.
+"""
+import numpy as np
+import pytest
+
+import catboost_amd as cb
+from catboost_amd import synthetic as syn
+from oracle.cbm_reader import read_cbm
+from oracle.oracle import OracleModel
+
+pytestmark = pytest.mark.gpu
+
+NO_ALLOC_BYTES = 32 << 20
+
+
+def _run_both(ev, feats, docs, dim, tree_range=(0, None)):
+    import torch
+
+    a = torch.full((docs * dim,), -7.0, dtype=torch.float64, device="cuda:0")
+    b = torch.full((docs * dim,), -9.0, dtype=torch.float64, device="cuda:0")
+    torch.cuda.synchronize()
+    ev.eval_data_no_alloc(feats, docs, a.data_ptr(), tree_start=tree_range[0], tree_end=tree_range[1])
+    ev.synchronize()
+    ev.eval_data(feats, docs, b.data_ptr(), tree_start=tree_range[0], tree_end=tree_range[1])
+    torch.cuda.synchronize()
+    return a, b
+
+
+@pytest.mark.parametrize("cfg,trees", [("C2", 60), ("C3", 40), ("C4", 30), ("C5", 20)])
+def test_no_alloc_entry_point_equals_eval_data(cfg, trees):
+    import torch
+
+    model, info = syn.build_model(cfg, trees=trees)
+    model.enable_gpu_evaluation(0)
+    ev = model.evaluator()
+    oracle = OracleModel(read_cbm(model.save_to_buffer()))
+    dim = info["dim"]
+    first_docs = 7001
+    assert ev.quantized_bytes(first_docs) <= NO_ALLOC_BYTES
+    x = syn.device_features(info, first_docs)
+    for docs in (first_docs, 1300):  # the second call is smaller: the first call's bins stay behind it
+        part = x[:docs].contiguous()
+        feats = ev.features(cb.LAYOUT_FLAT_ROWS, part.data_ptr(), part.shape[1])
+        got, expected = _run_both(ev, feats, docs, dim)
+        assert torch.equal(got, expected), (cfg, docs)
+        np.testing.assert_allclose(got.cpu().numpy(), oracle.calc(part.cpu().numpy(), threads=8), rtol=1e-9, atol=1e-12)
+    # a tree sub-range goes the same way
+    feats = ev.features(cb.LAYOUT_FLAT_ROWS, x.data_ptr(), x.shape[1])
+    got, expected = _run_both(ev, feats, 900, dim, tree_range=(3, trees - 2))
+    assert torch.equal(got, expected)
+
+
+def test_no_alloc_entry_point_refuses_batches_beyond_its_buffer():
+    import torch
+
+    model, info = syn.build_model("C2", trees=5)
+    model.enable_gpu_evaluation(0)
+    ev = model.evaluator()
+    per_block = ev.quantized_bytes(256)
+    max_docs = NO_ALLOC_BYTES // per_block * 256
+    assert ev.quantized_bytes(max_docs) <= NO_ALLOC_BYTES < ev.quantized_bytes(max_docs + 1)
+    x = syn.device_features(info, max_docs)
+    out = torch.zeros(max_docs + 1, dtype=torch.float64, device="cuda:0")
+    feats = ev.features(cb.LAYOUT_FLAT_ROWS, x.data_ptr(), x.shape[1])
+    with pytest.raises(cb.CatBoostError, match="at most %d documents" % max_docs):
+        ev.eval_data_no_alloc(feats, max_docs + 1, out.data_ptr())
+    # the largest batch that fits runs and equals the allocating entry point
+    got, expected = _run_both(ev, feats, max_docs, 1)
+    assert torch.equal(got, expected)
