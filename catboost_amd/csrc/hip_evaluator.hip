@@ -183,11 +183,12 @@ uint32_t RegTreeBlock(const TEvalRegVariant& v) {
 // The variant for a model: one-dimensional models take the smallest register file that holds
 // their buckets; others the pitch that needs the fewest launches (then the smallest such pitch).
 // mixed: the model has one-hot splits or bins above 127.
-const TEvalRegVariant* PickRegVariant(uint32_t buckets, uint32_t dim, uint32_t maxDepth, bool mixed, bool six) {
+const TEvalRegVariant* PickRegVariant(uint32_t buckets, uint32_t dim, uint32_t maxDepth, bool mixed, bool six,
+                                      uint32_t minVariantBuckets = 0) {
     const TEvalRegVariant* best = nullptr;
     uint32_t bestLaunches = 0;
     for (const auto& v : kEvalRegVariants) {
-        if (buckets > v.Buckets || (dim == 1) != (v.Pitch == 1) || v.Leaves != (dim > 1 && maxDepth <= 6 ? 64u : 256u) ||
+        if (buckets > v.Buckets || v.Buckets < minVariantBuckets || (dim == 1) != (v.Pitch == 1) || v.Leaves != (dim > 1 && maxDepth <= 6 ? 64u : 256u) ||
             v.Mixed != mixed || v.Six != six) {
             continue;
         }
@@ -199,6 +200,30 @@ const TEvalRegVariant* PickRegVariant(uint32_t buckets, uint32_t dim, uint32_t m
     }
     return best;
 }
+
+// Diagnostic switches, read from the environment when an evaluator is built (cb_hip_evaluator.h lists them).
+// They choose between kernels that give the same results; tests use them to reach every kernel with one model.
+struct TKernelSwitches {
+    bool RegKernel = true;        // CATBOOST_AMD_REG_KERNEL=0: no register-resident assembly kernels
+    bool RegSix = true;           // CATBOOST_AMD_REG_SIX=0: no six-bit form of those kernels
+    bool CtrTile = true;          // CATBOOST_AMD_CTR_TILE=0: the plain CTR kernel instead of the tile kernel
+    uint32_t RegMinBuckets = 0;   // CATBOOST_AMD_REG_MIN_BUCKETS=n: only register kernels that hold n buckets or more
+
+    static TKernelSwitches FromEnvironment() {
+        const auto off = [](const char* name) {
+            const char* v = std::getenv(name);
+            return v != nullptr && v[0] == '0';
+        };
+        TKernelSwitches k;
+        k.RegKernel = !off("CATBOOST_AMD_REG_KERNEL");
+        k.RegSix = !off("CATBOOST_AMD_REG_SIX");
+        k.CtrTile = !off("CATBOOST_AMD_CTR_TILE");
+        if (const char* v = std::getenv("CATBOOST_AMD_REG_MIN_BUCKETS")) {
+            k.RegMinBuckets = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
+        }
+        return k;
+    }
+};
 
 // log2 of the LDS slots per bucket of the row binarize kernel: the smallest count that still
 // exceeds the largest bucket of the model
@@ -265,7 +290,10 @@ void BuildLevelOrderTrees(const TModelTrees& trees, int dim, const std::vector<u
         uint32_t height = 0;
         // first pass: breadth-first order; second pass below fills the entries
         std::vector<std::pair<uint32_t, uint32_t>> children;  // entry index of (left, right); terminals: unused
-        for (size_t i = 0; i < order.size(); ++i) {
+        // A tree whose nodes share children (the loader only checks that every step stays inside the tree)
+        // unfolds into more entries than it has nodes, up to 2^depth: the walk stops as soon as the entries
+        // no longer fit the 16-bit offsets, and the model goes to the kernel that follows the step nodes.
+        for (size_t i = 0; i < order.size() && order.size() * 8 <= 0xffffu; ++i) {
             const TItem item = order[i];
             const auto& st = trees.NonSymmetricStepNodes[item.Node];
             const bool terminal = item.Terminal || (st.LeftSubtreeDiff == 0 && st.RightSubtreeDiff == 0);
@@ -744,6 +772,33 @@ struct THipEvaluator::TImpl {
         return t;
     }
     hipStream_t Pick(void* stream) const { return stream ? static_cast<hipStream_t>(stream) : Stream; }
+
+    // Also runs when the evaluator's constructor throws half way (a refused model), so that the
+    // stream, the events and the code object of a partly built evaluator are released.
+    ~TImpl() {
+        (void)hipSetDevice(DeviceId);
+        if (Stream) {
+            (void)hipStreamSynchronize(Stream);
+        }
+        for (auto& e : Ev) {
+            if (e) {
+                (void)hipEventDestroy(e);
+            }
+        }
+        for (auto& slot : SlotEv) {
+            for (auto& e : slot) {
+                if (e) {
+                    (void)hipEventDestroy(e);
+                }
+            }
+        }
+        if (Stream) {
+            (void)hipStreamDestroy(Stream);
+        }
+        if (RegModule) {
+            (void)hipModuleUnload(RegModule);
+        }
+    }
 };
 
 THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::vector<TCtrValueTable>* ctrTables,
@@ -751,6 +806,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
     : Impl(new TImpl)
 {
     const TFeaturePositions positions(trees, layout);
+    const TKernelSwitches switches = TKernelSwitches::FromEnvironment();
     const int deviceCount = GetHipDeviceCount();
     CBAMD_ENSURE(deviceCount > 0, "no HIP device found: the HIP evaluator needs an AMD GPU");
     CBAMD_ENSURE(deviceId >= 0 && deviceId < deviceCount, "HIP device id out of range");
@@ -852,8 +908,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         BuildCtrTables(trees, positions, *ctrTables, &srcFlat, &srcSplit, &offsets, &flags, &values, &m.CtrFeatures, &m.CtrItems,
                        &m.CtrIndexBuckets, &m.CtrBlob, &m.CtrCatColumnsFlat, &m.CtrCatColumnsSplit, &m.CtrCatColumnCount);
         m.CtrCount = static_cast<uint32_t>(trees.CtrFeatures.size());
-        const char* tileSwitch = std::getenv("CATBOOST_AMD_CTR_TILE");
-        m.CtrTileUsable = m.CtrCatColumnCount <= dev::kCtrMaxTileColumns && !(tileSwitch && tileSwitch[0] == '0');
+        m.CtrTileUsable = m.CtrCatColumnCount <= dev::kCtrMaxTileColumns && switches.CtrTile;
     }
     CBAMD_ENSURE(srcFlat.size() == BucketCount, "internal error: bucket count mismatch");
     for (size_t b = 0; b + 1 < offsets.size(); ++b) {
@@ -1080,14 +1135,13 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         }
     }
 
-    const char* regSwitch = std::getenv("CATBOOST_AMD_REG_KERNEL");
-    const bool regEnabled = !(regSwitch && regSwitch[0] == '0');
+    const bool regEnabled = switches.RegKernel;
     // six-bit form: no one-hot split and no bucket with more than 63 values, so that every bin is below 64
-    const char* sixSwitch = std::getenv("CATBOOST_AMD_REG_SIX");
-    const bool six = m.PackedSevenBit && m.MaxBucketValues <= 63 && !(sixSwitch && sixSwitch[0] == '0');
+    const bool six = m.PackedSevenBit && m.MaxBucketValues <= 63 && switches.RegSix;
     const TEvalRegVariant* variant =
         m.Oblivious && m.MaxDepth <= 8 && TreeCount > 0
-            ? PickRegVariant(m.LayoutBuckets, static_cast<uint32_t>(m.Dim), m.MaxDepth, !m.PackedSevenBit, six)
+            ? PickRegVariant(m.LayoutBuckets, static_cast<uint32_t>(m.Dim), m.MaxDepth, !m.PackedSevenBit, six,
+                             switches.RegMinBuckets)
             : nullptr;
     // a thread's 32-bit offset walks through the leaf table of a launch while it is copied to LDS
     const bool regTableAddressable =
@@ -1168,32 +1222,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
     }
 }
 
-THipEvaluator::~THipEvaluator() {
-    if (Impl) {
-        (void)hipSetDevice(Impl->DeviceId);
-        if (Impl->Stream) {
-            (void)hipStreamSynchronize(Impl->Stream);
-        }
-        for (auto& e : Impl->Ev) {
-            if (e) {
-                (void)hipEventDestroy(e);
-            }
-        }
-        for (auto& slot : Impl->SlotEv) {
-            for (auto& e : slot) {
-                if (e) {
-                    (void)hipEventDestroy(e);
-                }
-            }
-        }
-        if (Impl->Stream) {
-            (void)hipStreamDestroy(Impl->Stream);
-        }
-        if (Impl->RegModule) {
-            (void)hipModuleUnload(Impl->RegModule);
-        }
-    }
-}
+THipEvaluator::~THipEvaluator() = default;
 
 size_t THipEvaluator::QuantizedBytes(size_t docCount) const {
     const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
@@ -1756,6 +1785,18 @@ size_t PipelineDocs(size_t rowFloats, size_t rowCats) {
 
 }  // namespace
 
+namespace {
+
+// A model without trees answers with its bias whatever the prediction type: the reference fills the result
+// array with the bias values in turn and returns before any post-processing (cpu/formula_evaluator.cpp:29-41).
+void FillBiasOnly(const std::vector<double>& bias, size_t count, double* results) {
+    for (size_t i = 0; i < count; ++i) {
+        results[i] = bias.empty() ? 0.0 : bias[i % bias.size()];
+    }
+}
+
+}  // namespace
+
 // Rows by pointer (the reference API's float** / hashed int**): two slots of pinned and device
 // staging memory; while the GPU copies in, binarizes, evaluates and copies out slot k, the host
 // gathers the rows of slot k + 1.
@@ -1776,6 +1817,10 @@ void THipEvaluator::CalcHostRows(const float* const* rows, size_t rowLen, bool f
     CBAMD_ENSURE(needCats == 0 || catRows != nullptr, "Model has categorical features but no categorical features provided");
     CBAMD_ENSURE(catRowLen >= needCats, "insufficient cat features vector size: " + std::to_string(catRowLen) +
                                             " expected: " + std::to_string(needCats));
+    if (TreeCount == 0) {
+        FillBiasOnly(m.HostBias, docCount * outDim, results);
+        return;
+    }
     const size_t chunk = PipelineDocs(needFloats, needCats);
     const size_t stageDocs = std::min(chunk, docCount);
     const bool twoSlots = docCount > chunk;
@@ -1869,6 +1914,10 @@ void THipEvaluator::CalcHostColumns(const float* const* columns, size_t columnCo
     const size_t need = m.FlatVectorSize;
     CBAMD_ENSURE(columnCount >= need, "Not enough features provided");
     CBAMD_ENSURE(need == 0 || columns != nullptr, "Not enough features provided");
+    if (TreeCount == 0) {
+        FillBiasOnly(m.HostBias, docCount * outDim, results);
+        return;
+    }
     const size_t chunk = ChunkDocs(need, 0);
     const size_t stageDocs = std::min(chunk, docCount);
     m.PinnedFloats.Reserve(std::max<size_t>(1, stageDocs * need));

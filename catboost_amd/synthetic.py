@@ -20,6 +20,10 @@
   C2W C2 over 400 features and 2M docs: more buckets than the register-resident kernels hold, the LDS tile
       kernel's case. Not one of the baseline workloads.
 
+  C2N C2 over 90 features: few enough buckets for the 96-register kernel shape (four waves per SIMD), which the
+      CATBOOST_AMD_REG_MIN_BUCKETS switch can trade for the 200-register shape (two waves per SIMD) on the
+      same model. Not one of the baseline workloads.
+
 Every split is (feature, border) drawn uniformly; models go through the builder, so only the
 borders that some split uses survive. Leaf values are N(0, sigma).
 """
@@ -37,6 +41,8 @@ CONFIGS = {
                 docs=4_000_000, dist="normal_lognormal", nan_rate=0.05),
     "C2W": dict(kind="oblivious", trees=1000, depth=8, floats=400, borders=254, dim=1, leaf_sigma=0.005,
                 docs=2_000_000, dist="normal_lognormal", nan_rate=0.05),
+    "C2N": dict(kind="oblivious", trees=1000, depth=8, floats=90, borders=254, dim=1, leaf_sigma=0.005,
+                docs=4_000_000, dist="normal_lognormal", nan_rate=0.05),
     "C3": dict(kind="oblivious", trees=2000, depth=6, floats=100, borders=64, dim=10, leaf_sigma=0.01,
                docs=2_000_000, dist="uniform3", nan_rate=0.0),
     "C4": dict(kind="nonsymmetric", trees=500, depth=10, floats=300, borders=254, dim=1, leaf_sigma=0.01,

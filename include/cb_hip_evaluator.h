@@ -78,6 +78,14 @@ typedef struct CbHipFeatures {
     size_t CatStride;
 } CbHipFeatures;
 
+/* Diagnostic switches, read from the environment whenever an evaluator is built (CbHipEvaluatorCreate, the
+ * first prediction of a model handle, CbHipSetFeatureLayout). They select between kernels that return the
+ * same results and exist for tests and measurements; production callers leave them unset.
+ *   CATBOOST_AMD_REG_KERNEL=0        no register-resident assembly kernels (the LDS tile kernels instead)
+ *   CATBOOST_AMD_REG_SIX=0           no six-bit form of the register-resident kernels
+ *   CATBOOST_AMD_REG_MIN_BUCKETS=n   only register-resident kernel shapes that hold n buckets or more
+ *   CATBOOST_AMD_CTR_TILE=0          the plain CTR kernel instead of the LDS tile one */
+
 /* Model upload: validates the tables, derives buckets / repacked splits / leaf offsets and
  * copies SoA tables to device `deviceId` (takes the place of the TGpuEvaluator constructor,
  * cuda/evaluator.cpp:18-85). */

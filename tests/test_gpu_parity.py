@@ -103,9 +103,37 @@ def test_simple_asymmetric_model():
     np.testing.assert_array_equal(r.calc_flat(rm.DATA), rm.ASYMMETRIC_PREDICTIONS)
 
 
+def test_non_symmetric_tree_whose_nodes_share_children():
+    """A chain of 60 nodes in which both steps of every node lead to the next one passes the loader's
+    range checks; unfolded level by level it would have 2^60 entries. The level-order tables give up
+    on it and the model runs on the kernel that follows the step nodes, like the reference."""
+    depth = 60
+    head = mb.leaf_node(float(depth))
+    for level in reversed(range(depth)):
+        head = mb.split_node(("float", level % 3, 0.5), mb.leaf_node(float(level)), head)
+    model = mb.build_non_symmetric([mb.float_feature(i) for i in range(3)], [], 1, [head])
+    steps = np.array(model["step_nodes"])
+    chain = (steps == [0, 1]).all(axis=1)
+    assert chain.sum() == depth - 1
+    steps[chain] = [1, 1]
+    model["step_nodes"] = steps
+    _, o = _check_flat(model, rm.DATA)
+    assert set(o.calc(rm.DATA)) == {depth - 1.0, float(depth)}
+
+
 def test_zero_trees_gives_bias():
     g = _gpu_model(rm.simple_float_model(tree_count=0, bias=[0.75]))
     np.testing.assert_array_equal(g.calc_flat(rm.DATA), np.full(8, 0.75))
+
+
+def test_zero_trees_ignore_the_prediction_type():
+    """The reference fills the results with the bias and returns before TEvalResultProcessor runs
+    (cpu/formula_evaluator.cpp:29-41): Probability, Exponent and Class of a model without trees are the raw bias."""
+    g = _gpu_model(rm.simple_float_model(tree_count=0, bias=[0.75]))
+    for kind in ("Probability", "Exponent", "Class", "RawFormulaVal"):
+        g.set_prediction_type(kind)
+        np.testing.assert_array_equal(g.calc_flat(rm.DATA), np.full(8, 0.75))
+        np.testing.assert_array_equal(g.calc_flat_transposed(np.ascontiguousarray(rm.DATA.T)), np.full(8, 0.75))
 
 
 def test_single_document_and_ragged_sizes():
