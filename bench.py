@@ -206,7 +206,8 @@ def main():
             "kernel": "binarize + evaluate (the two launches of one step)",
         },
         "kernels": {
-            "binarize": {"avg_ms": avg_bin, "GBps": (4 * (used_floats + used_cats) + buckets) * docs / (avg_bin * 1e-3) / 1e9},
+            "binarize": {"avg_ms": avg_bin, "GBps": (4 * (used_floats + used_cats) + buckets) * docs / (avg_bin * 1e-3) / 1e9
+                         if avg_bin > 0 else None},
             "evaluate": {"avg_ms": avg_eval, "GBps": (buckets + 8 * dim) * docs / (avg_eval * 1e-3) / 1e9,
                          "tree_evals_per_sec": docs * model.tree_count / (avg_eval * 1e-3)},
         },

@@ -45,6 +45,26 @@ Kernel arguments (80 bytes):
 grid = ceil(blockCount / WAVES) workgroups of WAVES * 64 threads, LDS = 2 * TREE_BLOCK * LEAVES *
 PITCH * 8 bytes.
 
+Fused variants ("cbamd_fused_..."; one-dimensional float-only models, plain and six-bit forms) take the
+documents' fp32 rows instead of bins and binarize them into the bins registers themselves, so the bins
+never exist in memory. Their leaf table is preceded by FUSED_CHUNKS 32 KB images of border tables, which
+go through the same two LDS buffers as the tree blocks that follow them:
+  * a lane owns the documents block * 256 + lane + 64 * j as before and reads its own rows, 16 bytes (four
+    columns) per load, 64 bytes (a "unit" of sixteen columns = sixteen bins registers) per document and
+    turn; the two units that share a 128-byte stretch of the rows are taken one right after the other;
+  * a value's bin is found as the HIP binarize kernel finds it: the value's cell in the bucket's uniform
+    grid of 256 cells, min(255, u32((v - lo) * scale)), indexes a byte table of search starts, and a
+    branch-free binary search over the next 2^steps - 1 borders finishes the count of borders below the
+    value; four columns of a document go through it side by side. steps (at most FUSED_MAX_STEPS) is
+    common to the four columns of a load;
+  * per unit a record of 40 dwords: sixteen lo, sixteen scale, a flags dword (bit q: the unit's q-th four
+    columns need four steps, bit 4 + q: three or more, bit 8 + q: two or more, bit 16 + i: NaN counts
+    as +inf in column i), the unit's byte offset in a row.
+Additional kernel arguments (104 bytes in all):
+  80 floats const float*  88 units const uint32* [unitCount + 1][40]  96 row stride in bytes uint32
+ 100 unitCount uint32 (1 .. BUCKETS / 16)
+and argument 0 is unused, argument 16 points at the border table images.
+
 Usage: gen_eval_reg_kernel.py OUT.s
 """
 import sys
@@ -59,9 +79,28 @@ SHAPES = [
     (192, 4, 2, 256), (160, 4, 4, 256), (128, 4, 6, 256),
 ]
 VARIANTS = [shape + (mixed, six) for mixed, six in ((False, False), (False, True), (True, False)) for shape in SHAPES]
+# shapes of the fused kernels (one dimension, 256 leaf rows), each in a plain and a six-bit form
+FUSED_SHAPES = [(208, 4), (96, 8)]
+FUSED_MAX_STEPS = 4
+FUSED_UNIT_DWORDS = 40
 
 
-def kernel_name(buckets, waves, pitch, leaves, mixed, six=False):
+def fused_layout(six):
+    """(buckets per border table image, bytes of a bucket's borders): the borders of the image's buckets,
+    then from byte 16384 on their 256-byte tables of search starts."""
+    return (64, 256) if six else (32, 512)
+
+
+def fused_chunks(buckets, six):
+    """Border table images in front of the leaf table: enough for `buckets`, an even number."""
+    per_chunk = fused_layout(six)[0]
+    chunks = (buckets + per_chunk - 1) // per_chunk
+    return chunks + chunks % 2
+
+
+def kernel_name(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
+    if fused:
+        return "cbamd_fused_b%d_w%d%s" % (buckets, waves, "_s" if six else "")
     return "cbamd_eval_reg_b%d_w%d_p%d_l%d%s" % (buckets, waves, pitch, leaves, "_m" if mixed else "_s" if six else "")
 
 
@@ -73,9 +112,10 @@ def tree_block(pitch, leaves):
     return block
 
 
-def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False):
+def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
     assert not (mixed and six)
-    name = kernel_name(buckets, waves, pitch, leaves, mixed, six)
+    assert not fused or (pitch == 1 and leaves == 256 and not mixed and buckets % 16 == 0)
+    name = kernel_name(buckets, waves, pitch, leaves, mixed, six, fused)
     row_dwords = 32 if mixed else 16      # level table of a tree
     tree_row_bytes = row_dwords * 4
     rows_a, rows_b = 32, 32 + row_dwords  # the two sets of scalar registers holding level tables
@@ -109,6 +149,16 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False):
     te0 = ga0 + 4                         # two scratch registers of the epilogue
     b0 = te0 + 2                          # the bins
     vgprs = b0 + buckets
+    if fused:
+        # registers of the binarize phase: those below the bins except v0 and v2, and 20 above the bins
+        high = vgprs
+        vgprs += 20
+        row_off = [1, 3, 4, 5]            # byte offset of the lane's four rows from the block's first row
+        srch_p = [6, 7, 8, 9]             # four searches side by side: position, border / scratch
+        srch_b = [10, 11, 12, 13]
+        # two sets of four 16-byte loads (first registers of the quads)
+        values = [[16, 20, 24, high], [high + 4, high + 8, high + 12, high + 16]]
+        assert b0 == 28
     assert vgprs <= 256
 
     def lv(j, k):
@@ -204,6 +254,188 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False):
                 e("  v_lshrrev_b32_e32 v3, 1, v3")
                 e("  v_bfi_b32 v3, s22, v4, v3")
 
+    def fused_binarize():
+        """The binarize phase of a fused kernel: fills the bins registers from the documents' rows. On
+        entry the first border table image is on its way into buffer 0 and s24 holds the wave's document
+        block; on exit the first tree block sits in buffer 0 and every wave has passed the barrier behind it."""
+        per_chunk, border_bytes = fused_layout(six)
+        units_per_chunk = per_chunk // 16
+        max_units = buckets // 16
+        chunks = fused_chunks(buckets, six)
+        # scalar registers of the two unit records in flight: sixteen lo, sixteen scale, (flags, offset)
+        rec_lo, rec_scale, rec_fo = [32, 68], [48, 84], [64, 66]
+        e("  s_lshl_b32 s30, s24, 8")                 # first row of the block
+        e("  s_sub_u32 s31, s12, s30")
+        e("  s_add_u32 s31, s31, -1")
+        e("  s_min_u32 s31, s31, 0xff")               # last row of the batch, counted from the block's first, at most 255
+        e("  s_mul_hi_u32 s3, s30, s88")
+        e("  s_mul_i32 s25, s30, s88")
+        e("  s_add_u32 s4, s84, s25")                 # s[4:5]: the block's first row
+        e("  s_addc_u32 s5, s85, s3")
+        e("  v_and_b32_e32 v%d, 63, v0" % srch_p[0])
+        for j in range(4):
+            # rows past the last document are read as the last document
+            e("  v_add_u32_e32 v%d, %d, v%d" % (row_off[j], 64 * j, srch_p[0]))
+            e("  v_min_u32_e32 v%d, s31, v%d" % (row_off[j], row_off[j]))
+            e("  v_mul_lo_u32 v%d, v%d, s88" % (row_off[j], row_off[j]))
+        e("  s_mov_b32 s24, s86")                     # s[24:25]: unit records, s28: units of the model
+        e("  s_mov_b32 s25, s87")
+        e("  s_mov_b32 s28, s89")
+
+        def load_record(unit):
+            x = unit % 2
+            at = unit * FUSED_UNIT_DWORDS * 4
+            e("  s_load_dwordx16 s[%d:%d], s[24:25], 0x%x" % (rec_lo[x], rec_lo[x] + 15, at))
+            e("  s_load_dwordx16 s[%d:%d], s[24:25], 0x%x" % (rec_scale[x], rec_scale[x] + 15, at + 64))
+            e("  s_load_dwordx2 s[%d:%d], s[24:25], 0x%x" % (rec_fo[x], rec_fo[x] + 1, at + 128))
+
+        # every unit for each of the lane's four documents; the two units of a pair share 128-byte stretches
+        # of the rows and follow each other
+        seq = [(2 * k + h, j) for k in range((max_units + 1) // 2) for j in range(4) for h in range(2)
+               if 2 * k + h < max_units]
+        pending = []                      # vector memory operations in flight, oldest first
+
+        def issue_loads(n):
+            unit, j = seq[n]
+            e("  s_add_u32 s30, s4, s%d" % (rec_fo[unit % 2] + 1))
+            e("  s_addc_u32 s31, s5, 0")
+            for q in range(4):
+                first = values[n % 2][q]
+                e("  global_load_dwordx4 v[%d:%d], v%d, s[30:31]%s" % (first, first + 3, row_off[j],
+                                                                      " offset:%d" % (16 * q) if q else ""))
+                pending.append(("unit", n))
+
+        def wait_loads(n):
+            last = max((i for i, op in enumerate(pending) if op == ("unit", n)), default=None)
+            if last is not None:
+                e("  s_waitcnt vmcnt(%d)" % (len(pending) - 1 - last))
+                del pending[:last + 1]
+
+        def search_step(step, vals):
+            """Step `step` (counted from the last one, 1) of the four searches: looks at the border 2^(step-1)
+            places on and moves on behind it when it lies below the value."""
+            size = 4 << (step - 1)
+            for d in range(4):
+                e("  ds_read_b32 v%d, v%d offset:%d" % (srch_b[d], srch_p[d], search_step.border_at[d] + size - 4))
+            e("  s_waitcnt lgkmcnt(0)")
+            for d in range(4):
+                e("  v_cmp_lt_f32_e32 vcc, v%d, v%d" % (srch_b[d], vals + d))
+                e("  v_cndmask_b32_e64 v%d, 0, %d, vcc" % (srch_b[d], size))
+                e("  v_add_u32_e32 v%d, v%d, v%d" % (srch_p[d], srch_p[d], srch_b[d]))
+
+        def process(n, buf):
+            unit, j = seq[n]
+            lo, scale, flags = rec_lo[unit % 2], rec_scale[unit % 2], rec_fo[unit % 2]
+            label = "%s_u%d_%d" % (name, unit, j)
+            # NaN counts as +inf in the columns whose flag says so
+            e("  s_lshr_b32 s3, s%d, 16" % flags)
+            e("  s_cmp_eq_u32 s3, 0")
+            e("  s_cbranch_scc1 %s_n" % label)
+            e("  v_mov_b32_e32 v%d, 0x7f800000" % srch_b[0])
+            for i in range(16):
+                reg = values[n % 2][i // 4] + i % 4
+                e("  s_bitcmp1_b32 s%d, %d" % (flags, 16 + i))
+                e("  s_cbranch_scc0 %s_n%d" % (label, i))
+                e("  v_cmp_u_f32_e32 vcc, v%d, v%d" % (reg, reg))
+                e("  v_cndmask_b32_e32 v%d, v%d, v%d, vcc" % (reg, reg, srch_b[0]))
+                e("%s_n%d:" % (label, i))
+            e("%s_n:" % label)
+            for q in range(4):
+                vals = values[n % 2][q]
+                local = (unit % units_per_chunk) * 16 + 4 * q
+                search_step.border_at = [buf * buf_bytes + (local + d) * border_bytes for d in range(4)]
+                for d in range(4):
+                    i = 4 * q + d
+                    # the value's cell in the column's grid and the search start stored for it
+                    e("  v_subrev_f32_e32 v%d, s%d, v%d" % (srch_b[d], lo + i, vals + d))
+                    e("  v_mul_f32_e32 v%d, s%d, v%d" % (srch_b[d], scale + i, srch_b[d]))
+                    e("  v_cvt_u32_f32_e32 v%d, v%d" % (srch_b[d], srch_b[d]))
+                    e("  v_min_u32_e32 v%d, 0xff, v%d" % (srch_b[d], srch_b[d]))
+                    e("  ds_read_u8 v%d, v%d offset:%d" % (srch_p[d], srch_b[d],
+                                                           buf * buf_bytes + 16384 + (local + d) * 256))
+                e("  s_waitcnt lgkmcnt(0)")
+                if not six:
+                    for d in range(4):
+                        e("  v_lshlrev_b32_e32 v%d, 2, v%d" % (srch_p[d], srch_p[d]))
+                # the search: steps above two are rare and sit out of line
+                e("  s_bitcmp1_b32 s%d, %d" % (flags, 4 + q))
+                e("  s_cbranch_scc1 %s_q%d_hi" % (label, q))
+                e("%s_q%d_back:" % (label, q))
+                e("  s_bitcmp1_b32 s%d, %d" % (flags, 8 + q))
+                e("  s_cbranch_scc0 %s_q%d_one" % (label, q))
+                search_step(2, vals)
+                e("%s_q%d_one:" % (label, q))
+                search_step(1, vals)
+                for d in range(4):
+                    reg = b0 + unit * 16 + 4 * q + d
+                    if j == 0:
+                        e("  v_lshrrev_b32_e32 v%d, 2, v%d" % (reg, srch_p[d]))
+                    else:
+                        e("  v_lshl_add_u32 v%d, v%d, %d, v%d" % (reg, srch_p[d], 8 * j - 2, reg))
+                out_of_line.append((label, q, vals, list(search_step.border_at), flags))
+
+        def emit_out_of_line():
+            for label, q, vals, border_at, flags in out_of_line:
+                search_step.border_at = border_at
+                e("%s_q%d_hi:" % (label, q))
+                e("  s_bitcmp1_b32 s%d, %d" % (flags, q))
+                e("  s_cbranch_scc0 %s_q%d_three" % (label, q))
+                search_step(4, vals)
+                e("%s_q%d_three:" % (label, q))
+                search_step(3, vals)
+                e("  s_branch %s_q%d_back" % (label, q))
+            del out_of_line[:]
+
+        out_of_line = []
+        load_record(0)
+        if max_units > 1:
+            load_record(1)
+        e("  s_waitcnt lgkmcnt(0)")
+        issue_loads(0)
+        e("  s_waitcnt vmcnt(0)")                      # the first image (and the first loads)
+        e("  s_barrier")
+        del pending[:]
+        done = {0}                                    # unit loads known to have arrived
+        n = 0
+        for c in range(chunks):
+            buf = c % 2
+            for g in range(len(groups)):
+                stage((1 - buf) * buf_bytes, g)
+                pending.extend([("stage", c)] * groups[g][1])
+            while n < len(seq) and seq[n][0] // units_per_chunk == c:
+                unit, j = seq[n]
+                if unit % 2 == 0 and j == 0:
+                    # no such pair of units in this model: nothing left to do in this image
+                    e("  s_cmp_le_u32 s28, %d" % unit)
+                    e("  s_cbranch_scc1 %s_c%d_end" % (name, c))
+                if n + 1 < len(seq):
+                    nxt_unit, nxt_j = seq[n + 1]
+                    if nxt_j == 0:
+                        e("  s_waitcnt lgkmcnt(0)")    # the record of a unit that starts
+                    issue_loads(n + 1)
+                if n in done:
+                    done.discard(n)
+                else:
+                    wait_loads(n)
+                if unit % 2 == 1:
+                    e("  s_cmp_le_u32 s28, %d" % unit)
+                    e("  s_cbranch_scc1 %s_u%d_%d_skip" % (name, unit, j))
+                process(n, buf)
+                e("%s_u%d_%d_skip:" % (name, unit, j))
+                if j == 3 and unit + 2 < max_units:
+                    load_record(unit + 2)
+                n += 1
+            e("  s_branch %s_c%d_end" % (name, c))
+            emit_out_of_line()
+            e("%s_c%d_end:" % (name, c))
+            e("  s_waitcnt vmcnt(0) lgkmcnt(0)")
+            e("  s_barrier")
+            if any(op[0] == "unit" for op in pending):
+                done.update(op[1] for op in pending if op[0] == "unit")
+            del pending[:]
+        assert n == len(seq)
+        e("  s_load_dwordx4 s[96:99], s[0:1], 0x40")   # the record registers held these arguments
+
     e(".text")
     e(".globl %s" % name)
     e(".p2align 8")
@@ -213,6 +445,9 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False):
     e("  s_load_dwordx8 s[4:11], s[0:1], 0x0")
     e("  s_load_dwordx8 s[12:19], s[0:1], 0x20")
     e("  s_load_dwordx4 s[96:99], s[0:1], 0x40")
+    if fused:
+        e("  s_load_dwordx4 s[84:87], s[0:1], 0x50")   # floats, unit records
+        e("  s_load_dwordx2 s[88:89], s[0:1], 0x60")   # row stride in bytes, units
     e("  v_and_b32_e32 v0, 0x3ff, v0")           # work-item ids come packed; keep x
     e("  v_lshrrev_b32_e32 v5, 6, v0")
     e("  v_and_b32_e32 v1, 63, v0")
@@ -244,20 +479,23 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False):
     e("  s_add_u32 s21, s21, s20")
     e("  s_add_u32 s24, s13, -1")
     e("  s_min_u32 s24, s21, s24")
-    # (the level table registers are free until the first tables are loaded)
-    e("  s_lshl_b32 s25, s96, 8")                # bytes of bins per document block
-    e("  s_mul_hi_u32 s31, s24, s25")
-    e("  s_mul_i32 s30, s24, s25")
-    e("  s_add_u32 s32, s4, s30")
-    e("  s_addc_u32 s33, s5, s31")
-    e("  s_add_u32 s28, s96, -1")
-    for i in range(buckets):
-        # registers past the model's bucket count reload the last bucket and are never indexed
-        e("  s_min_u32 s24, %d, s28" % i)
-        e("  s_lshl_b32 s24, s24, 8")
-        e("  s_add_u32 s34, s32, s24")
-        e("  s_addc_u32 s35, s33, 0")
-        e("  global_load_dword v%d, v1, s[34:35]" % (b0 + i))
+    if fused:
+        fused_binarize()
+    else:
+        # (the level table registers are free until the first tables are loaded)
+        e("  s_lshl_b32 s25, s96, 8")                # bytes of bins per document block
+        e("  s_mul_hi_u32 s31, s24, s25")
+        e("  s_mul_i32 s30, s24, s25")
+        e("  s_add_u32 s32, s4, s30")
+        e("  s_addc_u32 s33, s5, s31")
+        e("  s_add_u32 s28, s96, -1")
+        for i in range(buckets):
+            # registers past the model's bucket count reload the last bucket and are never indexed
+            e("  s_min_u32 s24, %d, s28" % i)
+            e("  s_lshl_b32 s24, s24, 8")
+            e("  s_add_u32 s34, s32, s24")
+            e("  s_addc_u32 s35, s33, 0")
+            e("  global_load_dword v%d, v1, s[34:35]" % (b0 + i))
     load_rows(rows_a, 0)
     load_rows(rows_b, 1)
     for r in range(lv0, ga0):
@@ -374,7 +612,7 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False):
     e(".amdhsa_kernel %s" % name)
     e("  .amdhsa_group_segment_fixed_size %d" % lds_bytes)
     e("  .amdhsa_private_segment_fixed_size 0")
-    e("  .amdhsa_kernarg_size 80")
+    e("  .amdhsa_kernarg_size %d" % (104 if fused else 80))
     e("  .amdhsa_user_sgpr_count 2")
     e("  .amdhsa_user_sgpr_kernarg_segment_ptr 1")
     e("  .amdhsa_system_sgpr_workgroup_id_x 1")
@@ -409,9 +647,9 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False):
       - {.offset: 68, .size: 4, .value_kind: by_value}
       - {.offset: 72, .size: 4, .value_kind: by_value}
       - {.offset: 76, .size: 4, .value_kind: by_value}
-    .group_segment_fixed_size: %d
+%s    .group_segment_fixed_size: %d
     .kernarg_segment_align: 8
-    .kernarg_segment_size: 80
+    .kernarg_segment_size: %d
     .max_flat_workgroup_size: %d
     .name: %s
     .private_segment_fixed_size: 0
@@ -423,7 +661,11 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False):
     .vgpr_count: %d
     .vgpr_spill_count: 0
     .wavefront_size: 64
-""" % (lds_bytes, threads, name, name, vgprs)
+""" % ("""      - {.address_space: global, .offset: 80, .size: 8, .value_kind: global_buffer}
+      - {.address_space: global, .offset: 88, .size: 8, .value_kind: global_buffer}
+      - {.offset: 96, .size: 4, .value_kind: by_value}
+      - {.offset: 100, .size: 4, .value_kind: by_value}
+""" if fused else "", lds_bytes, 104 if fused else 80, threads, name, name, vgprs)
     return "\n".join(o), meta
 
 
@@ -434,6 +676,11 @@ def generate():
         text, meta = gen_kernel(buckets, waves, pitch, leaves, mixed, six)
         parts.append(text)
         metas.append(meta)
+    for buckets, waves in FUSED_SHAPES:
+        for six in (False, True):
+            text, meta = gen_kernel(buckets, waves, 1, 256, False, six, fused=True)
+            parts.append(text)
+            metas.append(meta)
     parts.append(".amdgpu_metadata")
     parts.append("---")
     parts.append("amdhsa.kernels:")

@@ -55,6 +55,10 @@ public:
     void QuantizeDevice(const TFeatureBatch& batch, size_t docCount, uint8_t* bins, void* stream);
     void EvalQuantizedDevice(const uint8_t* bins, size_t docCount, size_t treeStart, size_t treeEnd,
                              double* results, void* stream);
+    // binarize + evaluate in one launch of a fused kernel, the bins in registers only; false (and nothing
+    // launched) when the model, the batch layout or the tree range has no fused kernel
+    bool EvalRowsFusedDevice(const TFeatureBatch& batch, size_t docCount, size_t treeStart, size_t treeEnd,
+                             double* results, void* stream);
     void LeafIndexesQuantizedDevice(const uint8_t* bins, size_t docCount, size_t treeStart, size_t treeEnd,
                                     uint32_t* indexes, void* stream);
     // bins in the reference's layout: blocks of 128 docs, [block][bucket][doc in block]

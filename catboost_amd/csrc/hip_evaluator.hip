@@ -171,6 +171,35 @@ constexpr TEvalRegVariant kEvalRegVariants[] = {
     {128, 4, 6, 256, false, true, "cbamd_eval_reg_b128_w4_p6_l256_s"},
 };
 
+// Fused kernels (binarize + evaluate in one launch, bins only ever in registers): shapes of
+// gen_eval_reg_kernel.py's FUSED_SHAPES, each in a plain and a six-bit form.
+struct TFusedVariant {
+    uint32_t Buckets;  // bins registers = 16 per unit of sixteen columns
+    uint32_t Waves;
+    bool Six;
+    const char* Name;
+};
+constexpr TFusedVariant kFusedVariants[] = {
+    {96, 8, false, "cbamd_fused_b96_w8"},
+    {96, 8, true, "cbamd_fused_b96_w8_s"},
+    {208, 4, false, "cbamd_fused_b208_w4"},
+    {208, 4, true, "cbamd_fused_b208_w4_s"},
+};
+constexpr uint32_t kFusedUnitColumns = 16;
+constexpr uint32_t kFusedUnitDwords = 40;   // sixteen lo, sixteen scale, flags, byte offset in the row, padding
+constexpr uint32_t kFusedMaxSteps = 4;
+constexpr size_t kFusedImageBytes = 32 * 1024;
+constexpr size_t kFusedLutOffset = 16 * 1024;
+
+struct TEvalFusedArgs {
+    TEvalRegArgs Reg;       // Bins unused; Leaves: the border table images, then the leaf table
+    const void* Floats;
+    const void* Units;
+    uint32_t StrideBytes;
+    uint32_t UnitCount;
+};
+static_assert(sizeof(TEvalFusedArgs) == 104, "kernel argument block of the fused kernels");
+
 // trees per LDS buffer of a variant: a power of two, at most 16, buffer at most 32 KB
 uint32_t RegTreeBlock(const TEvalRegVariant& v) {
     uint32_t block = 16;
@@ -208,6 +237,7 @@ struct TKernelSwitches {
     bool RegSix = true;           // CATBOOST_AMD_REG_SIX=0: no six-bit form of those kernels
     bool CtrTile = true;          // CATBOOST_AMD_CTR_TILE=0: the plain CTR kernel instead of the tile kernel
     uint32_t RegMinBuckets = 0;   // CATBOOST_AMD_REG_MIN_BUCKETS=n: only register kernels that hold n buckets or more
+    bool Fused = true;            // CATBOOST_AMD_FUSED=0: binarize and evaluate always as two launches
 
     static TKernelSwitches FromEnvironment() {
         const auto off = [](const char* name) {
@@ -218,6 +248,7 @@ struct TKernelSwitches {
         k.RegKernel = !off("CATBOOST_AMD_REG_KERNEL");
         k.RegSix = !off("CATBOOST_AMD_REG_SIX");
         k.CtrTile = !off("CATBOOST_AMD_CTR_TILE");
+        k.Fused = !off("CATBOOST_AMD_FUSED");
         if (const char* v = std::getenv("CATBOOST_AMD_REG_MIN_BUCKETS")) {
             k.RegMinBuckets = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
         }
@@ -243,6 +274,47 @@ uint32_t GridCell(float v, float lo, float scale) {
         return dev::kLutCells - 1;
     }
     return std::min<uint32_t>(static_cast<uint32_t>(tt), dev::kLutCells - 1);
+}
+
+// The uniform grid over a float bucket's sorted borders that starts the border search: lowest border,
+// cells per unit, the search steps that cover the tallest cell, and per cell the number of borders in
+// lower cells (what a search in that cell may skip).
+struct TBucketGrid {
+    float Lo = 0.0f;
+    float Scale = 0.0f;
+    uint32_t Steps = 0;
+    uint32_t Start[dev::kLutCells] = {};
+};
+
+TBucketGrid MakeBucketGrid(const std::vector<float>& borders) {
+    TBucketGrid g;
+    if (borders.empty()) {
+        return g;
+    }
+    g.Lo = borders.front();
+    const float span = borders.back() - g.Lo;
+    if (std::isfinite(g.Lo) && std::isfinite(span) && span > 0.0f) {
+        g.Scale = static_cast<float>(dev::kLutCells) / span;
+        if (!std::isfinite(g.Scale)) {
+            g.Scale = 0.0f;
+        }
+    } else {
+        g.Lo = 0.0f;
+    }
+    uint32_t population[dev::kLutCells] = {};
+    for (float x : borders) {
+        ++population[GridCell(x, g.Lo, g.Scale)];
+    }
+    const uint32_t tallest = *std::max_element(population, population + dev::kLutCells);
+    while ((1u << g.Steps) - 1 < tallest) {
+        ++g.Steps;
+    }
+    uint32_t start = 0;
+    for (int c = 0; c < dev::kLutCells; ++c) {
+        g.Start[c] = start;
+        start += population[c];
+    }
+    return g;
 }
 
 constexpr size_t kMaxTileLdsBytes = 160 * 1024;
@@ -711,6 +783,18 @@ struct THipEvaluator::TImpl {
     TDeviceVec<double> RegLeaves;  // [launch][tree][leaf row][pitch]
     TDeviceVec<double> RegBias;    // the bias, readable for a whole pitch behind every dimension
 
+    // fused kernels, per row layout (0: flat rows, 1: split rows of a model without categorical features)
+    struct TFused {
+        bool Usable = false;
+        uint32_t UnitCount = 0;
+        TDeviceVec<uint32_t> Rows;    // level rows that name bins registers of the fused layout
+        TDeviceVec<uint32_t> Units;   // unit records
+        TDeviceVec<uint8_t> Table;    // border table images, then a copy of the leaf table
+    };
+    TFused Fused[2];
+    hipFunction_t FusedFunction = nullptr;
+    uint32_t FusedWaves = 0;
+
     // scratch (grow-only, guarded by THipEvaluator::Lock)
     TDeviceVec<uint8_t> ScratchBins;
     TDeviceVec<float> StageFloats;
@@ -938,33 +1022,14 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
             }
             std::vector<float> borders(n);
             std::memcpy(borders.data(), values.data() + offsets[b], n * sizeof(float));
-            float lo = borders.front(), scale = 0.0f;
-            const float span = borders.back() - lo;
-            if (std::isfinite(lo) && std::isfinite(span) && span > 0.0f) {
-                scale = static_cast<float>(dev::kLutCells) / span;
-                if (!std::isfinite(scale)) {
-                    scale = 0.0f;
-                }
-            } else {
-                lo = 0.0f;
-            }
-            // start[c] = borders in cells below c; the tallest cell decides the number of steps
-            std::vector<uint32_t> population(dev::kLutCells, 0);
-            for (float x : borders) {
-                ++population[GridCell(x, lo, scale)];
-            }
-            const uint32_t tallest = *std::max_element(population.begin(), population.end());
-            uint32_t steps = 0;
-            while ((1u << steps) - 1 < tallest) {
-                ++steps;
-            }
+            const TBucketGrid g = MakeBucketGrid(borders);
+            const float lo = g.Lo, scale = g.Scale;
+            const uint32_t steps = g.Steps;
             CBAMD_ENSURE((1u << steps) <= slots, "internal error: search window exceeds the bucket's slots");
             uint8_t* cells = reinterpret_cast<uint8_t*>(lut.data() + b * (dev::kLutCells / 4));
-            uint32_t start = 0;
             for (int c = 0; c < dev::kLutCells; ++c) {
                 // a lower start only adds borders known to be below the value; it keeps the window inside the slots
-                cells[c] = static_cast<uint8_t>(std::min(start, slots - (1u << steps)));
-                start += population[c];
+                cells[c] = static_cast<uint8_t>(std::min(g.Start[c], slots - (1u << steps)));
             }
             std::memcpy(&grid[b * 4 + 0], &lo, 4);
             std::memcpy(&grid[b * 4 + 1], &scale, 4);
@@ -1219,6 +1284,142 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         m.RegLeaves.Upload(leaves);
         m.RegBias.Upload(biasPadded);
         m.RegKernelUsable = true;
+
+        // ---- fused kernels: float-only one-dimensional models in the 7-bit or six-bit form whose rows are
+        // at least sixteen columns wide. The bins registers follow the columns of the rows (a unit = sixteen
+        // consecutive columns = sixteen registers), so the level rows are rewritten per row layout.
+        const bool fusedCandidate = switches.Fused && !variant->Mixed && variant->Pitch == 1 && m.Dim == 1 && !m.HasCats &&
+                                    m.CtrCount == 0 && m.BinarizeBuckets == BucketCount && BucketCount > 0;
+        for (int layoutIndex = 0; layoutIndex < 2 && fusedCandidate; ++layoutIndex) {
+            const std::vector<uint32_t>& columns = layoutIndex == 0 ? srcFlat : srcSplit;
+            const size_t rowWidth = layoutIndex == 0 ? m.FlatVectorSize : m.MinFloatSize;
+            if (rowWidth < kFusedUnitColumns) {
+                continue;
+            }
+            std::vector<std::pair<uint32_t, uint32_t>> byColumn;  // (column, bucket)
+            for (uint32_t b = 0; b < BucketCount; ++b) {
+                byColumn.emplace_back(columns[b], b);
+            }
+            std::sort(byColumn.begin(), byColumn.end());
+            bool distinct = true;
+            for (size_t i = 1; i < byColumn.size(); ++i) {
+                distinct = distinct && byColumn[i].first != byColumn[i - 1].first;
+            }
+            if (!distinct) {
+                continue;
+            }
+            // units: sixteen columns from a used column on, moved back where they would leave the row
+            std::vector<uint32_t> unitStart, slotOfBucket(BucketCount, 0);
+            for (size_t i = 0; i < byColumn.size();) {
+                const uint32_t start = static_cast<uint32_t>(std::min<size_t>(byColumn[i].first, rowWidth - kFusedUnitColumns));
+                const uint32_t unit = static_cast<uint32_t>(unitStart.size());
+                unitStart.push_back(start);
+                while (i < byColumn.size() && byColumn[i].first < start + kFusedUnitColumns) {
+                    slotOfBucket[byColumn[i].second] = unit * kFusedUnitColumns + (byColumn[i].first - start);
+                    ++i;
+                }
+            }
+            const TFusedVariant* fused = nullptr;
+            for (const auto& v : kFusedVariants) {
+                if (v.Six == variant->Six && unitStart.size() * kFusedUnitColumns <= v.Buckets && !fused) {
+                    fused = &v;
+                }
+            }
+            if (!fused || (m.FusedFunction && m.FusedWaves != fused->Waves)) {
+                continue;
+            }
+            const uint32_t slots = fused->Six ? 64 : 128;           // border slots of a bucket in an image
+            const uint32_t bucketsPerImage = fused->Six ? 64 : 32;
+            const uint32_t unitsPerImage = bucketsPerImage / kFusedUnitColumns;
+            const uint32_t maxUnits = fused->Buckets / kFusedUnitColumns;
+            uint32_t images = (fused->Buckets + bucketsPerImage - 1) / bucketsPerImage;
+            images += images % 2;
+            std::vector<uint32_t> bucketOfSlot(fused->Buckets, UINT32_MAX);
+            for (uint32_t b = 0; b < BucketCount; ++b) {
+                bucketOfSlot[slotOfBucket[b]] = b;
+            }
+            // grids first: the four columns of a load share their number of search steps
+            std::vector<TBucketGrid> grids(fused->Buckets);
+            std::vector<std::vector<float>> bordersOfSlot(fused->Buckets);
+            std::vector<uint32_t> groupSteps(fused->Buckets / 4, 1);
+            bool fits = true;
+            for (uint32_t slot = 0; slot < fused->Buckets; ++slot) {
+                const uint32_t b = bucketOfSlot[slot];
+                if (b == UINT32_MAX) {
+                    continue;
+                }
+                const uint32_t n = offsets[b + 1] - offsets[b];
+                bordersOfSlot[slot].resize(n);
+                std::memcpy(bordersOfSlot[slot].data(), values.data() + offsets[b], n * sizeof(float));
+                grids[slot] = MakeBucketGrid(bordersOfSlot[slot]);
+                groupSteps[slot / 4] = std::max(groupSteps[slot / 4], grids[slot].Steps);
+                fits = fits && n < slots;
+            }
+            for (uint32_t steps : groupSteps) {
+                fits = fits && steps <= kFusedMaxSteps && (1u << steps) <= slots;
+            }
+            if (!fits) {
+                continue;
+            }
+            std::vector<uint32_t> units((static_cast<size_t>(maxUnits) + 1) * kFusedUnitDwords, 0);
+            std::vector<uint8_t> table(images * kFusedImageBytes + leaves.size() * sizeof(double), 0);
+            for (uint32_t slot = 0; slot < fused->Buckets; ++slot) {
+                const uint32_t unit = slot / kFusedUnitColumns, column = slot % kFusedUnitColumns;
+                uint32_t* record = units.data() + static_cast<size_t>(unit) * kFusedUnitDwords;
+                const uint32_t steps = groupSteps[slot / 4], group = column / 4;
+                record[32] |= (steps >= 4 ? 1u << group : 0u) | (steps >= 3 ? 16u << group : 0u) | (steps >= 2 ? 256u << group : 0u);
+                if (unit < unitStart.size()) {
+                    record[33] = unitStart[unit] * 4;
+                }
+                const uint32_t b = bucketOfSlot[slot];
+                if (b == UINT32_MAX) {
+                    continue;  // a column no split reads: all-zero record and tables, its register is never indexed
+                }
+                std::memcpy(&record[column], &grids[slot].Lo, 4);
+                std::memcpy(&record[16 + column], &grids[slot].Scale, 4);
+                if (flags[b] & dev::kBucketFlagNanToInf) {
+                    record[32] |= 0x10000u << column;
+                }
+                uint8_t* image = table.data() + (unit / unitsPerImage) * kFusedImageBytes;
+                const uint32_t local = (unit % unitsPerImage) * kFusedUnitColumns + column;
+                uint32_t* borders = reinterpret_cast<uint32_t*>(image + static_cast<size_t>(local) * slots * 4);
+                for (uint32_t k = 0; k < slots; ++k) {
+                    uint32_t bits = 0x7f800000u;  // +inf behind the real borders
+                    if (k < bordersOfSlot[slot].size()) {
+                        std::memcpy(&bits, &bordersOfSlot[slot][k], 4);
+                    }
+                    borders[k] = bits;
+                }
+                uint8_t* lut = image + kFusedLutOffset + static_cast<size_t>(local) * dev::kLutCells;
+                for (int c = 0; c < dev::kLutCells; ++c) {
+                    const uint32_t start = std::min(grids[slot].Start[c], slots - (1u << steps));
+                    lut[c] = static_cast<uint8_t>(fused->Six ? start * 4 : start);  // the six-bit form stores byte offsets
+                }
+            }
+            std::memcpy(table.data() + images * kFusedImageBytes, leaves.data(), leaves.size() * sizeof(double));
+            // level rows of the same form as the register kernel's, naming bins registers of this layout
+            std::vector<uint32_t> fusedRows(rows);
+            for (size_t t = 0; t < TreeCount; ++t) {
+                const int depth = trees.TreeSizes[t];
+                uint32_t* row = fusedRows.data() + t * rowDwords;
+                for (int d = 0; d < depth; ++d) {
+                    row[2 * d] = slotOfBucket[trees.RepackedBins[trees.TreeStartOffsets[t] + d].FeatureIndex];
+                }
+                for (int d = depth; d < 8 && depth > 0; ++d) {
+                    row[2 * d] = row[0];
+                }
+            }
+            if (!m.FusedFunction) {
+                HIP_CHECK(hipModuleGetFunction(&m.FusedFunction, m.RegModule, fused->Name));
+                m.FusedWaves = fused->Waves;
+            }
+            TImpl::TFused& f = m.Fused[layoutIndex];
+            f.UnitCount = static_cast<uint32_t>(unitStart.size());
+            f.Rows.Upload(fusedRows);
+            f.Units.Upload(units);
+            f.Table.Upload(table);
+            f.Usable = true;
+        }
     }
 }
 
@@ -1642,6 +1843,45 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
     HIP_CHECK(hipGetLastError());
 }
 
+bool THipEvaluator::EvalRowsFusedDevice(const TFeatureBatch& batch, size_t docCount, size_t treeStart, size_t treeEnd,
+                                        double* results, void* stream) {
+    TImpl& m = *Impl;
+    const int layoutIndex = batch.Layout == TFeatureBatch::FlatRows ? 0 : batch.Layout == TFeatureBatch::SplitRows ? 1 : -1;
+    if (layoutIndex < 0 || !m.Fused[layoutIndex].Usable || docCount == 0 || treeStart != 0 || treeEnd != TreeCount ||
+        docCount >= (size_t(1) << 29) || batch.Stride >= (size_t(1) << 20)) {
+        return false;
+    }
+    const TImpl::TFused& f = m.Fused[layoutIndex];
+    CBAMD_ENSURE(results != nullptr, "results pointer is null");
+    CBAMD_ENSURE(batch.Floats != nullptr, "float features pointer is null");
+    const size_t need = layoutIndex == 0 ? m.FlatVectorSize : m.MinFloatSize;
+    CBAMD_ENSURE(batch.Stride >= need, (layoutIndex == 0 ? "insufficient flat features vector size: " : "insufficient float features vector size: ") +
+                                           std::to_string(batch.Stride) + " expected: " + std::to_string(need));
+    TEvalFusedArgs args = {};
+    args.Reg.Rows = f.Rows.Get();
+    args.Reg.Leaves = f.Table.Get();
+    args.Reg.Out = results;
+    args.Reg.DocCount = static_cast<uint32_t>(docCount);
+    args.Reg.BlockCount = static_cast<uint32_t>((docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock);
+    args.Reg.TreeBlocks = m.RegTreeBlocks;
+    args.Reg.Flags = 1;
+    args.Reg.Scale = m.Scale;
+    args.Reg.Bias = m.RegBias.Get();
+    args.Reg.BucketCount = m.LayoutBuckets;
+    args.Reg.Dim = 1;
+    args.Reg.FirstDim = 0;
+    args.Reg.StoreDims = 1;
+    args.Floats = batch.Floats;
+    args.Units = f.Units.Get();
+    args.StrideBytes = static_cast<uint32_t>(batch.Stride * sizeof(float));
+    args.UnitCount = f.UnitCount;
+    const uint32_t grid = (args.Reg.BlockCount + m.FusedWaves - 1) / m.FusedWaves;
+    size_t argSize = sizeof(args);
+    void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &argSize, HIP_LAUNCH_PARAM_END};
+    HIP_CHECK(hipModuleLaunchKernel(m.FusedFunction, grid, 1, 1, 64 * m.FusedWaves, 1, 1, 0, m.Pick(stream), nullptr, config));
+    return true;
+}
+
 void THipEvaluator::LeafIndexesQuantizedDevice(const uint8_t* bins, size_t docCount, size_t treeStart, size_t treeEnd,
                                                uint32_t* indexes, void* stream) {
     TImpl& m = *Impl;
@@ -1705,8 +1945,16 @@ void THipEvaluator::CalcDevice(const TFeatureBatch& batch, size_t docCount, size
     TImpl& m = *Impl;
     HIP_CHECK(hipSetDevice(m.DeviceId));
     hipStream_t s = m.Pick(stream);
-    m.ScratchBins.Reserve(QuantizedBytes(docCount));
     HIP_CHECK(hipEventRecord(m.Ev[0], s));
+    if (EvalRowsFusedDevice(batch, docCount, treeStart, treeEnd, results, s)) {
+        // one launch does both: its whole duration is reported as the evaluate time
+        HIP_CHECK(hipEventRecord(m.Ev[2], s));
+        HIP_CHECK(hipStreamSynchronize(s));
+        LastTimes.BinarizeMs = 0.0f;
+        HIP_CHECK(hipEventElapsedTime(&LastTimes.EvalMs, m.Ev[0], m.Ev[2]));
+        return;
+    }
+    m.ScratchBins.Reserve(QuantizedBytes(docCount));
     QuantizeDevice(batch, docCount, m.ScratchBins.Get(), s);
     HIP_CHECK(hipEventRecord(m.Ev[1], s));
     EvalQuantizedDevice(m.ScratchBins.Get(), docCount, treeStart, treeEnd, results, s);
@@ -1719,6 +1967,9 @@ void THipEvaluator::CalcDevice(const TFeatureBatch& batch, size_t docCount, size
 void THipEvaluator::CalcDeviceNoAlloc(const TFeatureBatch& batch, size_t docCount, size_t treeStart, size_t treeEnd,
                                       double* results, void* stream) {
     TImpl& m = *Impl;
+    if (EvalRowsFusedDevice(batch, docCount, treeStart, treeEnd, results, stream)) {
+        return;  // the fused kernel keeps the bins in registers: no buffer at all
+    }
     const size_t maxDocs = kNoAllocScratchBytes / (static_cast<size_t>(m.LayoutBuckets) * dev::kDocsPerBlock) * dev::kDocsPerBlock;
     CBAMD_ENSURE(docCount <= maxDocs, "batch of " + std::to_string(docCount) + " documents exceeds the fixed bin buffer: at most " +
                                           std::to_string(maxDocs) + " documents per call for this model");
@@ -1879,9 +2130,13 @@ void THipEvaluator::CalcHostRows(const float* const* rows, size_t rowLen, bool f
         batch.Cats = needCats ? stageCats[slot]->Get() : nullptr;
         batch.CatStride = needCats;
         HIP_CHECK(hipEventRecord(m.SlotEv[slot][0], s));
-        QuantizeDevice(batch, n, m.ScratchBins.Get(), s);
-        HIP_CHECK(hipEventRecord(m.SlotEv[slot][1], s));
-        EvalQuantizedDevice(m.ScratchBins.Get(), n, treeStart, treeEnd, stageResults[slot]->Get(), s);
+        if (EvalRowsFusedDevice(batch, n, treeStart, treeEnd, stageResults[slot]->Get(), s)) {
+            HIP_CHECK(hipEventRecord(m.SlotEv[slot][1], s));
+        } else {
+            QuantizeDevice(batch, n, m.ScratchBins.Get(), s);
+            HIP_CHECK(hipEventRecord(m.SlotEv[slot][1], s));
+            EvalQuantizedDevice(m.ScratchBins.Get(), n, treeStart, treeEnd, stageResults[slot]->Get(), s);
+        }
         HIP_CHECK(hipEventRecord(m.SlotEv[slot][2], s));
         const double* final = stageResults[slot]->Get();
         if (predictionType != dev::kPredRaw) {

@@ -1,0 +1,132 @@
+"""The fused kernels (binarize + evaluate in one launch, the bins in registers only) against the two-launch
+path and the oracle. Needs an MI355X.
+
+CbHipEvalData and the host entry points take the fused kernel for float-only one-dimensional oblivious
+models whose rows are at least sixteen columns wide; CATBOOST_AMD_FUSED=0 keeps an evaluator on the two
+launches. Both add the leaves in tree order in fp64: results must be equal bit for bit, and within
+1e-9 relative / 1e-12 absolute of the oracle.
+"""
+import numpy as np
+import pytest
+
+import catboost_amd as cb
+from catboost_amd import synthetic as syn
+from oracle import model_builder as mb
+from oracle.cbm_reader import read_cbm
+from oracle.oracle import OracleModel
+
+pytestmark = pytest.mark.gpu
+
+
+def _evaluators(model_bytes, monkeypatch):
+    """(fused, two-launch) evaluators of one model."""
+    out = []
+    for switch in ("1", "0"):
+        monkeypatch.setenv("CATBOOST_AMD_FUSED", switch)
+        m = cb.ModelCalcer(buffer=model_bytes)
+        m.enable_gpu_evaluation(0)
+        out.append((m, m.evaluator()))
+    monkeypatch.delenv("CATBOOST_AMD_FUSED")
+    return out
+
+
+def _compare(model_bytes, x, monkeypatch, stride=None):
+    import torch
+
+    oracle = OracleModel(read_cbm(model_bytes))
+    (fm, fev), (tm, tev) = _evaluators(model_bytes, monkeypatch)
+    docs, width = x.shape
+    stride = stride or width
+    padded = np.full((docs, stride), np.float32(7.5))
+    padded[:, :width] = x
+    dx = torch.from_numpy(np.ascontiguousarray(padded, np.float32)).to("cuda:0")
+    a = torch.full((docs,), -1.0, dtype=torch.float64, device="cuda:0")
+    b = torch.full((docs,), -2.0, dtype=torch.float64, device="cuda:0")
+    torch.cuda.synchronize()
+    fev.eval_data(fev.features(cb.LAYOUT_FLAT_ROWS, dx.data_ptr(), stride), docs, a.data_ptr())
+    tev.eval_data(tev.features(cb.LAYOUT_FLAT_ROWS, dx.data_ptr(), stride), docs, b.data_ptr())
+    torch.cuda.synchronize()
+    assert fev.last_kernel_times()[0] == 0.0, "the fused kernel did not run"
+    assert tev.last_kernel_times()[0] > 0.0
+    assert torch.equal(a, b)
+    np.testing.assert_allclose(a.cpu().numpy(), oracle.calc(x, threads=8), rtol=1e-9, atol=1e-12)
+    # the host entry point takes the same kernel
+    np.testing.assert_array_equal(fm.calc_flat(x[:3000]), a.cpu().numpy()[:3000])
+    return a
+
+
+@pytest.mark.parametrize("cfg,trees,docs", [("C2", 50, 1), ("C2", 50, 255), ("C2", 50, 257), ("C2", 64, 5000),
+                                             ("C2", 1000, 20000), ("C1", 200, 30011), ("C2N", 40, 4097)])
+def test_fused_equals_two_launches(cfg, trees, docs, monkeypatch):
+    model, info = syn.build_model(cfg, trees=trees)
+    x = syn.host_features(info, docs, seed=3)
+    _compare(model.save_to_buffer(), x, monkeypatch)
+    if docs == 5000:
+        _compare(model.save_to_buffer(), x, monkeypatch, stride=x.shape[1] + 5)
+
+
+def _random_model(rng, columns, used, trees, depth, borders_of, nan_true=()):
+    """An oblivious model over `columns` float columns of which `used` are split on; borders_of(f) draws
+    the candidate borders of column f."""
+    feats = []
+    for f in range(columns):
+        ff = mb.float_feature(f)
+        if f in nan_true:
+            ff["has_nans"], ff["nan_treatment"] = True, 2
+        feats.append(ff)
+    cands = {f: np.unique(np.asarray(borders_of(f), np.float32)) for f in used}
+    tree_list = []
+    for _ in range(trees):
+        splits = []
+        for _ in range(depth):
+            f = int(rng.choice(used))
+            splits.append(("float", f, float(rng.choice(cands[f]))))
+        tree_list.append((splits, rng.normal(0, 0.01, size=1 << depth)))
+    return mb.build_oblivious(feats, [], 1, tree_list, scale=0.75, bias=[0.125])
+
+
+def _bytes(model_dict):
+    m = cb.ModelCalcer()
+    m.load_from_dict(model_dict)
+    return m.save_to_buffer()
+
+
+def test_fused_sparse_columns_clustered_borders_and_nan_as_true(monkeypatch):
+    """Columns that no split reads between the used ones, a row whose last unit is moved back, borders so
+    close together that a grid cell holds up to fifteen of them (three and four search steps), NaN that
+    counts as +inf, values on the borders and infinities."""
+    rng = np.random.default_rng(11)
+    columns = 75
+    used = sorted(rng.choice(columns, size=31, replace=False).tolist() + [74])
+    used = sorted(set(used))
+
+    def borders_of(f):
+        if f % 3 == 0:  # clustered: a few tight groups far apart
+            centers = rng.normal(0, 3, size=4)
+            return np.concatenate([c + rng.normal(0, 1e-3, size=rng.integers(3, 12)) for c in centers])
+        return rng.normal(0, 1, size=rng.integers(1, 50))
+
+    model = _random_model(rng, columns, used, trees=70, depth=8, borders_of=borders_of, nan_true=set(used[::4]))
+    x = rng.normal(0, 2, size=(6000, columns)).astype(np.float32)
+    for f in used:
+        b = np.asarray(model["float_features"][f]["borders"], np.float32)
+        rows = rng.integers(0, x.shape[0], size=200)
+        x[rows, f] = rng.choice(b, size=200)
+    x[rng.random(x.shape) < 0.05] = np.nan
+    x[rng.random(x.shape) < 0.01] = np.inf
+    x[rng.random(x.shape) < 0.01] = -np.inf
+    _compare(_bytes(model), x, monkeypatch)
+
+
+def test_fused_shallow_trees_and_mixed_depths(monkeypatch):
+    rng = np.random.default_rng(5)
+    columns = 20
+    feats = [mb.float_feature(f) for f in range(columns)]
+    trees = []
+    for t in range(45):
+        depth = int(rng.integers(0, 9))
+        splits = [("float", int(rng.integers(0, columns)), float(np.float32(rng.normal()))) for _ in range(depth)]
+        trees.append((splits, rng.normal(0, 0.01, size=1 << depth)))
+    model = mb.build_oblivious(feats, [], 1, trees)
+    x = rng.normal(size=(3001, columns)).astype(np.float32)
+    _compare(_bytes(model), x, monkeypatch)

@@ -911,7 +911,7 @@ def test_workload_configs_device_path(name, docs):
     assert torch.equal(out, out2)
     np.testing.assert_array_equal(exported.cpu().numpy(), o.binarize(host))
     binarize_ms, eval_ms = ev.last_kernel_times()
-    assert binarize_ms > 0 and eval_ms > 0
+    assert binarize_ms >= 0 and eval_ms > 0  # a fused kernel reports its whole time as the evaluate time
 
 
 def test_concurrent_callers():
