@@ -59,15 +59,19 @@ go through the same two LDS buffers as the tree blocks that follow them:
     common to the four columns of a load;
   * per unit a record of 40 dwords: sixteen lo, sixteen scale, a flags dword (bit q: the unit's q-th four
     columns need four steps, bit 4 + q: three or more, bit 8 + q: two or more, bit 16 + i: NaN counts
-    as +inf in column i), the unit's byte offset in a row.
+    as +inf in column i); behind the BUCKETS / 16 + 1 records, the units' byte offsets in a row.
 Additional kernel arguments (104 bytes in all):
-  80 floats const float*  88 units const uint32* [unitCount + 1][40]  96 row stride in bytes uint32
+  80 floats const float*  88 units const uint32* [BUCKETS / 16 + 1][40] + [16]  96 row stride in bytes uint32
  100 unitCount uint32 (1 .. BUCKETS / 16)
 and argument 0 is unused, argument 16 points at the border table images.
 
 Usage: gen_eval_reg_kernel.py OUT.s
 """
+import os
 import sys
+
+# (the CBAMD_GEN_* variables are for timing experiments; a build that ships sets none of them)
+EXPERIMENT = os.environ.get("CBAMD_GEN_EXPERIMENT", "")  # timing experiments only; never set in a build that ships
 
 LDS_BUFFER_LIMIT = 32 * 1024
 
@@ -82,6 +86,7 @@ VARIANTS = [shape + (mixed, six) for mixed, six in ((False, False), (False, True
 # shapes of the fused kernels (one dimension, 256 leaf rows), each in a plain and a six-bit form
 FUSED_SHAPES = [(208, 4), (96, 8)]
 FUSED_MAX_STEPS = 4
+FUSED_EXTRA_SETS = int(os.environ.get("CBAMD_GEN_SETS", "1"))
 FUSED_UNIT_DWORDS = 40
 
 
@@ -272,6 +277,9 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
         e("  s_mul_i32 s25, s30, s88")
         e("  s_add_u32 s4, s84, s25")                 # s[4:5]: the block's first row
         e("  s_addc_u32 s5, s85, s3")
+        if EXPERIMENT == "l2loads":
+            e("  s_mov_b32 s4, s84")
+            e("  s_mov_b32 s5, s85")
         e("  v_and_b32_e32 v%d, 63, v0" % srch_p[0])
         for j in range(4):
             # rows past the last document are read as the last document
@@ -281,26 +289,36 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
         e("  s_mov_b32 s24, s86")                     # s[24:25]: unit records, s28: units of the model
         e("  s_mov_b32 s25, s87")
         e("  s_mov_b32 s28, s89")
+        # the units' byte offsets in a row (they follow the records) stay in s6 .. s19 for the whole phase;
+        # the arguments that sat there are loaded again behind it
+        assert max_units <= 14
+        offsets_at = (max_units + 1) * FUSED_UNIT_DWORDS * 4
+        e("  s_load_dwordx2 s[6:7], s[24:25], 0x%x" % offsets_at)
+        e("  s_load_dwordx8 s[8:15], s[24:25], 0x%x" % (offsets_at + 8))
+        e("  s_load_dwordx4 s[16:19], s[24:25], 0x%x" % (offsets_at + 40))
 
-        def load_record(unit):
-            x = unit % 2
+        def load_record(n):
+            unit, x = seq[n][0], n % 2
             at = unit * FUSED_UNIT_DWORDS * 4
             e("  s_load_dwordx16 s[%d:%d], s[24:25], 0x%x" % (rec_lo[x], rec_lo[x] + 15, at))
             e("  s_load_dwordx16 s[%d:%d], s[24:25], 0x%x" % (rec_scale[x], rec_scale[x] + 15, at + 64))
             e("  s_load_dwordx2 s[%d:%d], s[24:25], 0x%x" % (rec_fo[x], rec_fo[x] + 1, at + 128))
 
-        # every unit for each of the lane's four documents; the two units of a pair share 128-byte stretches
-        # of the rows and follow each other
-        seq = [(2 * k + h, j) for k in range((max_units + 1) // 2) for j in range(4) for h in range(2)
-               if 2 * k + h < max_units]
+        # every unit for each of the lane's four documents: image by image, inside an image document by
+        # document, so that neighbouring units of a row, which share 128-byte lines, follow each other
+        seq = [(unit, j) for c in range(chunks) for j in range(4)
+               for unit in range(c * units_per_chunk, min((c + 1) * units_per_chunk, max_units))]
         pending = []                      # vector memory operations in flight, oldest first
 
-        def issue_loads(n):
+        def issue_loads(n, pieces=range(4)):
             unit, j = seq[n]
-            e("  s_add_u32 s30, s4, s%d" % (rec_fo[unit % 2] + 1))
-            e("  s_addc_u32 s31, s5, 0")
-            for q in range(4):
-                first = values[n % 2][q]
+            if 0 in pieces:
+                e("  s_add_u32 s30, s4, s%d" % (6 + unit))
+                e("  s_addc_u32 s31, s5, 0")
+            for q in pieces:
+                first = value_set[n][q]
+                if EXPERIMENT == "noloads":
+                    continue
                 e("  global_load_dwordx4 v[%d:%d], v%d, s[30:31]%s" % (first, first + 3, row_off[j],
                                                                       " offset:%d" % (16 * q) if q else ""))
                 pending.append(("unit", n))
@@ -315,6 +333,8 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
             """Step `step` (counted from the last one, 1) of the four searches: looks at the border 2^(step-1)
             places on and moves on behind it when it lies below the value."""
             size = 4 << (step - 1)
+            if EXPERIMENT == "nosearch":
+                return
             for d in range(4):
                 e("  ds_read_b32 v%d, v%d offset:%d" % (srch_b[d], srch_p[d], search_step.border_at[d] + size - 4))
             e("  s_waitcnt lgkmcnt(0)")
@@ -325,15 +345,16 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
 
         def process(n, buf):
             unit, j = seq[n]
-            lo, scale, flags = rec_lo[unit % 2], rec_scale[unit % 2], rec_fo[unit % 2]
+            lo, scale, flags = rec_lo[n % 2], rec_scale[n % 2], rec_fo[n % 2]
             label = "%s_u%d_%d" % (name, unit, j)
+            e("  s_waitcnt lgkmcnt(0)")                # the unit's record
             # NaN counts as +inf in the columns whose flag says so
             e("  s_lshr_b32 s3, s%d, 16" % flags)
             e("  s_cmp_eq_u32 s3, 0")
             e("  s_cbranch_scc1 %s_n" % label)
             e("  v_mov_b32_e32 v%d, 0x7f800000" % srch_b[0])
             for i in range(16):
-                reg = values[n % 2][i // 4] + i % 4
+                reg = value_set[n][i // 4] + i % 4
                 e("  s_bitcmp1_b32 s%d, %d" % (flags, 16 + i))
                 e("  s_cbranch_scc0 %s_n%d" % (label, i))
                 e("  v_cmp_u_f32_e32 vcc, v%d, v%d" % (reg, reg))
@@ -341,7 +362,7 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
                 e("%s_n%d:" % (label, i))
             e("%s_n:" % label)
             for q in range(4):
-                vals = values[n % 2][q]
+                vals = value_set[n][q]
                 local = (unit % units_per_chunk) * 16 + 4 * q
                 search_step.border_at = [buf * buf_bytes + (local + d) * border_bytes for d in range(4)]
                 for d in range(4):
@@ -386,45 +407,76 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
                 e("  s_branch %s_q%d_back" % (label, q))
             del out_of_line[:]
 
+        # Two neighbouring units of a document (128 bytes of its row) are loaded together, eight loads one
+        # behind the other, so that a line of the row is asked for once (the cache merges requests that
+        # meet there; asked for piece by piece a line came from memory up to twice). Registers of the loads
+        # in flight: the 32 below and above the bins and, while the bins registers of the last units are
+        # not yet written, FUSED_EXTRA_SETS more sets of 32 among those. Inside an image the sets go round,
+        # so that a pair's loads are issued that many pairs ahead of its turn; images that have no such
+        # set left load, wait and search in turn (the other waves of the CU fill the wait).
+        chunk_positions = [[n for n in range(len(seq)) if seq[n][0] // units_per_chunk == c] for c in range(chunks)]
+        value_set = {}
+        plan = []                                      # per image: (pairs of positions, sets in use, pair loaded ahead across the boundary)
+        for c, positions in enumerate(chunk_positions):
+            pairs = []
+            for n in positions:
+                if pairs and len(pairs[-1]) < 2 and seq[pairs[-1][0]][1] == seq[n][1]:
+                    pairs[-1].append(n)
+                else:
+                    pairs.append([n])
+            later_units = [u for u in range(max_units - 1, -1, -1) if u // units_per_chunk > c]
+            sets = [values[0] + values[1]]
+            for k in range(min(FUSED_EXTRA_SETS, len(later_units) // 2)):
+                sets.append([b0 + 16 * u + 4 * q for u in later_units[2 * k:2 * k + 2] for q in range(4)])
+            for k, pair in enumerate(pairs):
+                for h, n in enumerate(pair):
+                    value_set[n] = sets[k % len(sets)][4 * h:4 * h + 4]
+            cross = bool(pairs) and len(sets) > 1 and (len(pairs) - 1) % len(sets) != 0
+            plan.append((pairs, len(sets), cross))
+
         out_of_line = []
         load_record(0)
-        if max_units > 1:
+        if len(seq) > 1:
             load_record(1)
         e("  s_waitcnt lgkmcnt(0)")
-        issue_loads(0)
+        issued = set()
+        for n in plan[0][0][0]:
+            issue_loads(n)
+            issued.add(n)
         e("  s_waitcnt vmcnt(0)")                      # the first image (and the first loads)
         e("  s_barrier")
         del pending[:]
-        done = {0}                                    # unit loads known to have arrived
-        n = 0
-        for c in range(chunks):
+        done = set(issued)                            # unit loads known to have arrived
+        for c, (pairs, set_count, cross) in enumerate(plan):
             buf = c % 2
             for g in range(len(groups)):
                 stage((1 - buf) * buf_bytes, g)
                 pending.extend([("stage", c)] * groups[g][1])
-            while n < len(seq) and seq[n][0] // units_per_chunk == c:
-                unit, j = seq[n]
-                if unit % 2 == 0 and j == 0:
-                    # no such pair of units in this model: nothing left to do in this image
-                    e("  s_cmp_le_u32 s28, %d" % unit)
-                    e("  s_cbranch_scc1 %s_c%d_end" % (name, c))
-                if n + 1 < len(seq):
-                    nxt_unit, nxt_j = seq[n + 1]
-                    if nxt_j == 0:
-                        e("  s_waitcnt lgkmcnt(0)")    # the record of a unit that starts
-                    issue_loads(n + 1)
-                if n in done:
-                    done.discard(n)
+            if pairs:
+                # the model has no unit in this image: nothing to do but to pass it on
+                e("  s_cmp_le_u32 s28, %d" % seq[pairs[0][0]][0])
+                e("  s_cbranch_scc1 %s_c%d_end" % (name, c))
+            for k, pair in enumerate(pairs):
+                ahead = [p for p in pairs[k:k + set_count] if p[0] not in issued]
+                if k == len(pairs) - 1 and cross and c + 1 < len(plan) and plan[c + 1][0]:
+                    ahead.append(plan[c + 1][0][0])
+                for p in ahead:
+                    for n in p:
+                        issue_loads(n)
+                        issued.add(n)
+                if pair[-1] in done:
+                    done.difference_update(pair)
                 else:
-                    wait_loads(n)
-                if unit % 2 == 1:
-                    e("  s_cmp_le_u32 s28, %d" % unit)
-                    e("  s_cbranch_scc1 %s_u%d_%d_skip" % (name, unit, j))
-                process(n, buf)
-                e("%s_u%d_%d_skip:" % (name, unit, j))
-                if j == 3 and unit + 2 < max_units:
-                    load_record(unit + 2)
-                n += 1
+                    wait_loads(pair[-1])
+                for n in pair:
+                    unit, j = seq[n]
+                    if unit > 0:
+                        e("  s_cmp_le_u32 s28, %d" % unit)
+                        e("  s_cbranch_scc1 %s_u%d_%d_skip" % (name, unit, j))
+                    process(n, buf)
+                    e("%s_u%d_%d_skip:" % (name, unit, j))
+                    if n + 2 < len(seq):
+                        load_record(n + 2)
             e("  s_branch %s_c%d_end" % (name, c))
             emit_out_of_line()
             e("%s_c%d_end:" % (name, c))
@@ -433,8 +485,13 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
             if any(op[0] == "unit" for op in pending):
                 done.update(op[1] for op in pending if op[0] == "unit")
             del pending[:]
+        n = len(issued)
         assert n == len(seq)
-        e("  s_load_dwordx4 s[96:99], s[0:1], 0x40")   # the record registers held these arguments
+        # the record and offset registers held these arguments
+        e("  s_load_dwordx4 s[96:99], s[0:1], 0x40")
+        e("  s_load_dwordx8 s[4:11], s[0:1], 0x0")
+        e("  s_load_dwordx8 s[12:19], s[0:1], 0x20")
+        e("  s_waitcnt lgkmcnt(0)")                    # the level tables are loaded through s[6:7] next
 
     e(".text")
     e(".globl %s" % name)

@@ -186,7 +186,7 @@ constexpr TFusedVariant kFusedVariants[] = {
     {208, 4, true, "cbamd_fused_b208_w4_s"},
 };
 constexpr uint32_t kFusedUnitColumns = 16;
-constexpr uint32_t kFusedUnitDwords = 40;   // sixteen lo, sixteen scale, flags, byte offset in the row, padding
+constexpr uint32_t kFusedUnitDwords = 40;   // sixteen lo, sixteen scale, flags, padding
 constexpr uint32_t kFusedMaxSteps = 4;
 constexpr size_t kFusedImageBytes = 32 * 1024;
 constexpr size_t kFusedLutOffset = 16 * 1024;
@@ -1361,16 +1361,17 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
             if (!fits) {
                 continue;
             }
-            std::vector<uint32_t> units((static_cast<size_t>(maxUnits) + 1) * kFusedUnitDwords, 0);
+            // the records of all units the kernel has code for, one more, and the units' byte offsets in a row
+            std::vector<uint32_t> units((static_cast<size_t>(maxUnits) + 1) * kFusedUnitDwords + 16, 0);
+            for (size_t u = 0; u < unitStart.size(); ++u) {
+                units[(static_cast<size_t>(maxUnits) + 1) * kFusedUnitDwords + u] = unitStart[u] * 4;
+            }
             std::vector<uint8_t> table(images * kFusedImageBytes + leaves.size() * sizeof(double), 0);
             for (uint32_t slot = 0; slot < fused->Buckets; ++slot) {
                 const uint32_t unit = slot / kFusedUnitColumns, column = slot % kFusedUnitColumns;
                 uint32_t* record = units.data() + static_cast<size_t>(unit) * kFusedUnitDwords;
                 const uint32_t steps = groupSteps[slot / 4], group = column / 4;
                 record[32] |= (steps >= 4 ? 1u << group : 0u) | (steps >= 3 ? 16u << group : 0u) | (steps >= 2 ? 256u << group : 0u);
-                if (unit < unitStart.size()) {
-                    record[33] = unitStart[unit] * 4;
-                }
                 const uint32_t b = bucketOfSlot[slot];
                 if (b == UINT32_MAX) {
                     continue;  // a column no split reads: all-zero record and tables, its register is never indexed

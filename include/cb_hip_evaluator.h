@@ -125,7 +125,8 @@ bool CbHipEvalData(CbHipEvaluatorHandle* evaluator, const CbHipFeatures* deviceF
  * instead of the evaluator's grow-only scratch buffer; the call allocates nothing, waits for nothing
  * and records no kernel times: it only launches the binarize and evaluate kernels on `hipStream`
  * (NULL = the evaluator's own stream). Fails when CbHipQuantizedBytes(evaluator, docCount) exceeds
- * 32 MiB (the error names the largest document count for the model). All calls on one GPU share the
+ * 32 MiB (the error names the largest document count for the model); a model that runs on a fused
+ * kernel keeps its bins in registers, uses no buffer and has no such limit. All calls on one GPU share the
  * array, so calls that overlap there (two streams, two threads, two evaluators) race; calls in stream
  * order on one stream are safe. */
 bool CbHipEvalDataNoAlloc(CbHipEvaluatorHandle* evaluator, const CbHipFeatures* deviceFeatures, size_t docCount,

@@ -31,10 +31,13 @@ def _run_both(ev, feats, docs, dim, tree_range=(0, None)):
     return a, b
 
 
-@pytest.mark.parametrize("cfg,trees", [("C2", 60), ("C3", 40), ("C4", 30), ("C5", 20)])
-def test_no_alloc_entry_point_equals_eval_data(cfg, trees):
+@pytest.mark.parametrize("cfg,trees,fused", [("C2", 60, "0"), ("C2", 60, "1"), ("C3", 40, "1"), ("C4", 30, "1"), ("C5", 20, "1")])
+def test_no_alloc_entry_point_equals_eval_data(cfg, trees, fused, monkeypatch):
     import torch
 
+    # C2 has a fused kernel (no bins in memory at all); CATBOOST_AMD_FUSED=0 keeps it on the two launches
+    # whose bins sit in the fixed array, as the other models' do
+    monkeypatch.setenv("CATBOOST_AMD_FUSED", fused)
     model, info = syn.build_model(cfg, trees=trees)
     model.enable_gpu_evaluation(0)
     ev = model.evaluator()
@@ -55,9 +58,10 @@ def test_no_alloc_entry_point_equals_eval_data(cfg, trees):
     assert torch.equal(got, expected)
 
 
-def test_no_alloc_entry_point_refuses_batches_beyond_its_buffer():
+def test_no_alloc_entry_point_refuses_batches_beyond_its_buffer(monkeypatch):
     import torch
 
+    monkeypatch.setenv("CATBOOST_AMD_FUSED", "0")
     model, info = syn.build_model("C2", trees=5)
     model.enable_gpu_evaluation(0)
     ev = model.evaluator()
