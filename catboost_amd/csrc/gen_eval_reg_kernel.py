@@ -67,11 +67,8 @@ and argument 0 is unused, argument 16 points at the border table images.
 
 Usage: gen_eval_reg_kernel.py OUT.s
 """
-import os
 import sys
 
-# (the CBAMD_GEN_* variables are for timing experiments; a build that ships sets none of them)
-EXPERIMENT = os.environ.get("CBAMD_GEN_EXPERIMENT", "")  # timing experiments only; never set in a build that ships
 
 LDS_BUFFER_LIMIT = 32 * 1024
 
@@ -86,7 +83,7 @@ VARIANTS = [shape + (mixed, six) for mixed, six in ((False, False), (False, True
 # shapes of the fused kernels (one dimension, 256 leaf rows), each in a plain and a six-bit form
 FUSED_SHAPES = [(208, 4), (96, 8)]
 FUSED_MAX_STEPS = 4
-FUSED_EXTRA_SETS = int(os.environ.get("CBAMD_GEN_SETS", "1"))
+FUSED_EXTRA_SETS = 1
 FUSED_UNIT_DWORDS = 40
 
 
@@ -277,9 +274,6 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
         e("  s_mul_i32 s25, s30, s88")
         e("  s_add_u32 s4, s84, s25")                 # s[4:5]: the block's first row
         e("  s_addc_u32 s5, s85, s3")
-        if EXPERIMENT == "l2loads":
-            e("  s_mov_b32 s4, s84")
-            e("  s_mov_b32 s5, s85")
         e("  v_and_b32_e32 v%d, 63, v0" % srch_p[0])
         for j in range(4):
             # rows past the last document are read as the last document
@@ -317,8 +311,6 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
                 e("  s_addc_u32 s31, s5, 0")
             for q in pieces:
                 first = value_set[n][q]
-                if EXPERIMENT == "noloads":
-                    continue
                 e("  global_load_dwordx4 v[%d:%d], v%d, s[30:31]%s" % (first, first + 3, row_off[j],
                                                                       " offset:%d" % (16 * q) if q else ""))
                 pending.append(("unit", n))
@@ -333,8 +325,6 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
             """Step `step` (counted from the last one, 1) of the four searches: looks at the border 2^(step-1)
             places on and moves on behind it when it lies below the value."""
             size = 4 << (step - 1)
-            if EXPERIMENT == "nosearch":
-                return
             for d in range(4):
                 e("  ds_read_b32 v%d, v%d offset:%d" % (srch_b[d], srch_p[d], search_step.border_at[d] + size - 4))
             e("  s_waitcnt lgkmcnt(0)")

@@ -238,6 +238,7 @@ struct TKernelSwitches {
     bool CtrTile = true;          // CATBOOST_AMD_CTR_TILE=0: the plain CTR kernel instead of the tile kernel
     uint32_t RegMinBuckets = 0;   // CATBOOST_AMD_REG_MIN_BUCKETS=n: only register kernels that hold n buckets or more
     bool Fused = true;            // CATBOOST_AMD_FUSED=0: binarize and evaluate always as two launches
+    bool LevelOrder = true;       // CATBOOST_AMD_LEVEL_ORDER=0: register kernels keep the model's order of a tree's levels
 
     static TKernelSwitches FromEnvironment() {
         const auto off = [](const char* name) {
@@ -249,6 +250,7 @@ struct TKernelSwitches {
         k.RegSix = !off("CATBOOST_AMD_REG_SIX");
         k.CtrTile = !off("CATBOOST_AMD_CTR_TILE");
         k.Fused = !off("CATBOOST_AMD_FUSED");
+        k.LevelOrder = !off("CATBOOST_AMD_LEVEL_ORDER");
         if (const char* v = std::getenv("CATBOOST_AMD_REG_MIN_BUCKETS")) {
             k.RegMinBuckets = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
         }
@@ -1227,12 +1229,39 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         m.RegLaunchLeaves = tableTrees * rowsPerTree * pitch;
         std::vector<uint32_t> rows(tableTrees * rowDwords, 0);  // 7-bit form (bucket 0, add 0): false for every bin
         std::vector<double> leaves(launches * m.RegLaunchLeaves, 0.0);
+        // Order of a tree's levels in these tables (levelOrder[t][position] = level of the model). The leaf
+        // gathers of a wave meet in the LDS banks that the low bits of the leaf indexes choose; lanes with the
+        // same index share one access, lanes that differ only in high bits wait for each other. So the levels
+        // that split the documents most evenly go to the low bits and the lopsided ones, on which most lanes
+        // agree, to the high bits: fewer lanes of a bank then differ. How evenly a level splits is estimated
+        // from the rank of its border among the feature's borders (borders are quantiles of the training data).
+        // The leaf tables are permuted to match; the sums and their order do not change.
+        std::vector<std::vector<int>> levelOrder(TreeCount);
         for (size_t t = 0; t < TreeCount; ++t) {
             const int depth = trees.TreeSizes[t];
+            std::vector<std::pair<double, int>> lopsided;
+            for (int d = 0; d < depth; ++d) {
+                const auto& rb = trees.RepackedBins[trees.TreeStartOffsets[t] + d];
+                const uint32_t n = offsets[rb.FeatureIndex + 1] - offsets[rb.FeatureIndex];
+                const bool oneHot = (flags[rb.FeatureIndex] & dev::kBucketFlagOneHot) != 0 || rb.XorMask != 0;
+                const double share = oneHot ? 0.05 : static_cast<double>(rb.SplitIdx) / (n + 1.0);
+                lopsided.emplace_back(switches.LevelOrder ? std::fabs(share - 0.5) : 0.0, d);
+            }
+            std::stable_sort(lopsided.begin(), lopsided.end(),
+                             [](const auto& a, const auto& b) { return a.first < b.first; });
+            for (const auto& item : lopsided) {
+                levelOrder[t].push_back(item.second);
+            }
+        }
+        for (size_t t = 0; t < TreeCount; ++t) {
+            const int depth = trees.TreeSizes[t];
+            const auto levelAt = [&](int position) -> const TRepackedBin& {
+                return trees.RepackedBins[trees.TreeStartOffsets[t] + levelOrder[t][position]];
+            };
             // 7-bit form: no xor mask in the tree and every bin of its buckets below 128
             bool sevenBit = true;
             for (int d = 0; d < depth; ++d) {
-                const auto& rb = trees.RepackedBins[trees.TreeStartOffsets[t] + d];
+                const auto& rb = levelAt(d);
                 sevenBit = sevenBit && rb.XorMask == 0 && offsets[rb.FeatureIndex + 1] - offsets[rb.FeatureIndex] <= 127;
             }
             CBAMD_ENSURE(sevenBit || variant->Mixed, "internal error: tree needs the 8-bit compare");
@@ -1243,7 +1272,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
             uint32_t* row = rows.data() + t * rowDwords;
             if (sevenBit) {
                 for (int d = 0; d < depth; ++d) {
-                    const auto& rb = trees.RepackedBins[trees.TreeStartOffsets[t] + d];
+                    const auto& rb = levelAt(d);
                     row[2 * d] = rb.FeatureIndex;
                     // the level's bit is the carry into bit 7; six-bit kernels want the even levels' in bit 6
                     row[2 * d + 1] = ((variant->Six && d % 2 == 0 ? 64u : 128u) - rb.SplitIdx) * 0x01010101u;
@@ -1256,7 +1285,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
                     // levels past the tree's depth: splitIdx 255, false for every bin (bins are at most 254)
                     uint32_t bucket = 0, xorMask = 0, splitIdx = 255;
                     if (d < depth) {
-                        const auto& rb = trees.RepackedBins[trees.TreeStartOffsets[t] + d];
+                        const auto& rb = levelAt(d);
                         bucket = rb.FeatureIndex;
                         xorMask = rb.XorMask;
                         splitIdx = rb.SplitIdx;
@@ -1272,8 +1301,13 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
             for (size_t launch = 0; launch < launches; ++launch) {
                 double* table = leaves.data() + launch * m.RegLaunchLeaves + t * rowsPerTree * pitch;
                 for (size_t leaf = 0; leaf < (size_t(1) << depth); ++leaf) {
+                    // the leaf of the model whose level bits are this table row's position bits
+                    size_t modelLeaf = 0;
+                    for (int d = 0; d < depth; ++d) {
+                        modelLeaf |= ((leaf >> d) & 1) << levelOrder[t][d];
+                    }
                     for (size_t k = 0; k < pitch && launch * pitch + k < static_cast<size_t>(m.Dim); ++k) {
-                        table[leaf * pitch + k] = values[leaf * m.Dim + launch * pitch + k];
+                        table[leaf * pitch + k] = values[modelLeaf * m.Dim + launch * pitch + k];
                     }
                 }
             }
@@ -1404,7 +1438,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
                 const int depth = trees.TreeSizes[t];
                 uint32_t* row = fusedRows.data() + t * rowDwords;
                 for (int d = 0; d < depth; ++d) {
-                    row[2 * d] = slotOfBucket[trees.RepackedBins[trees.TreeStartOffsets[t] + d].FeatureIndex];
+                    row[2 * d] = slotOfBucket[trees.RepackedBins[trees.TreeStartOffsets[t] + levelOrder[t][d]].FeatureIndex];
                 }
                 for (int d = depth; d < 8 && depth > 0; ++d) {
                     row[2 * d] = row[0];
