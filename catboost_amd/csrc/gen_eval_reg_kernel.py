@@ -547,6 +547,26 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
     load_rows(rows_b, 1)
     for r in range(lv0, ga0):
         e("  v_mov_b32_e32 v%d, 0" % r)          # leaf values in flight and the sums
+    # a launch that continues the sums of earlier trees takes them from `out`
+    e("  s_bitcmp1_b32 s15, 1")
+    e("  s_cbranch_scc0 %s_fresh" % name)
+    e("  v_and_b32_e32 v5, 63, v0")
+    e("  s_lshl_b32 s24, s21, 8")
+    e("  v_add_u32_e32 v5, s24, v5")
+    for j in range(4):
+        e("  v_add_u32_e32 v%d, %d, v5" % (te0, 64 * j))
+        e("  v_cmp_gt_u32_e32 vcc, s12, v%d" % te0)
+        e("  s_and_saveexec_b64 s[30:31], vcc")
+        e("  v_mul_lo_u32 v%d, v%d, s97" % (te0 + 1, te0))
+        e("  v_add_lshl_u32 v%d, v%d, s98, 3" % (te0 + 1, te0 + 1))
+        for k in range(pitch):
+            if k > 0:
+                e("  s_cmp_gt_u32 s99, %d" % k)
+                e("  s_cbranch_scc0 %s_taken_%d" % (name, j))
+            e("  global_load_dwordx2 v[%d:%d], v%d, s[10:11] offset:%d" % (ac(j, k), ac(j, k) + 1, te0 + 1, 8 * k))
+        e("%s_taken_%d:" % (name, j))
+        e("  s_mov_b64 exec, s[30:31]")
+    e("%s_fresh:" % name)
     e("  s_waitcnt vmcnt(0) lgkmcnt(0)")
     e("  s_barrier")
     e("  s_set_gpr_idx_on s22, 0x1")             # src0 of VALU instructions becomes index relative
@@ -620,6 +640,8 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
     e("%s_done:" % name)
     add_leaf_values()
     e("  s_set_gpr_idx_off")
+    e("  s_bitcmp1_b32 s15, 2")                  # raw sums for a launch that continues them
+    e("  s_cbranch_scc1 %s_store" % name)
     # scale, bias of the launch's dimensions (rows registers are free now)
     for k in range(pitch):
         e("  s_load_dwordx2 s[%d:%d], s[18:19], 0x%x" % (32 + 2 * k, 33 + 2 * k, 8 * k))

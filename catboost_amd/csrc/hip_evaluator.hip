@@ -780,6 +780,9 @@ struct THipEvaluator::TImpl {
     uint32_t RegWaves = 0;
     uint32_t RegPitch = 1;
     uint32_t RegTreeBlocks = 0;
+    uint32_t RegTreeBlockSize = 16;   // trees per LDS buffer of the chosen kernel
+    uint32_t RegRowDwords = 16;       // dwords of a tree's level table
+    size_t RegTreeLeafDoubles = 256;  // doubles of a tree's leaf table (leaf rows x pitch)
     size_t RegLaunchLeaves = 0;  // doubles of the leaf table of one launch
     TDeviceVec<uint32_t> RegRows;
     TDeviceVec<double> RegLeaves;  // [launch][tree][leaf row][pitch]
@@ -1222,6 +1225,9 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         const size_t rowDwords = variant->Mixed ? 32 : 16;
         m.RegWaves = variant->Waves;
         m.RegPitch = variant->Pitch;
+        m.RegTreeBlockSize = block;
+        m.RegRowDwords = static_cast<uint32_t>(rowDwords);
+        m.RegTreeLeafDoubles = rowsPerTree * pitch;
         m.RegTreeBlocks = static_cast<uint32_t>((TreeCount + block - 1) / block);
         // two blocks of null trees behind the last one: the kernels prefetch that far
         const size_t tableTrees = (static_cast<size_t>(m.RegTreeBlocks) + 2) * block;
@@ -1746,7 +1752,7 @@ void LaunchEval(bool oblivious, const uint8_t* bins, size_t docCount, uint32_t b
     if (oblivious) {
         const uint32_t grid = static_cast<uint32_t>((blocks + 3) / 4);
         hipLaunchKernelGGL(dev::EvalObliviousKernel<DCHUNK>, dim3(grid), dim3(256), 0, s,
-                           reinterpret_cast<const uint32_t*>(bins), docCount, buckets, tt, treeBegin, treeEnd, out);
+                           reinterpret_cast<const uint32_t*>(bins), docCount, buckets, tt, treeBegin, treeEnd, out, 0u, 2u);
     } else {
         hipLaunchKernelGGL(dev::EvalNonSymmetricKernel<DCHUNK>, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, s,
                            bins, docCount, buckets, tt, treeBegin, treeEnd, out);
@@ -1775,22 +1781,67 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
     CBAMD_ENSURE(bins != nullptr, "quantized buffer is null");
     const dev::TTreeTables tt = m.TreeTables();
     const uint32_t tb = static_cast<uint32_t>(treeStart), te = static_cast<uint32_t>(treeEnd);
-    if (m.RegKernelUsable && treeStart == 0 && treeEnd == TreeCount && docCount * m.Dim < (size_t(1) << 29)) {
-        // whole model over bins kept in registers, RegPitch dimensions per launch
+    if (m.RegKernelUsable) {
+        // Bins kept in registers, RegPitch dimensions per launch. A launch addresses its results with 32
+        // bits, so a very large batch goes in slices of whole document blocks.
+        const size_t sliceDocs = ((size_t(1) << 29) - 1) / m.Dim / dev::kDocsPerBlock * dev::kDocsPerBlock;
+        if (docCount > sliceDocs) {
+            for (size_t first = 0; first < docCount; first += sliceDocs) {
+                const size_t n = std::min(sliceDocs, docCount - first);
+                EvalQuantizedDevice(bins + first * m.LayoutBuckets, n, treeStart, treeEnd, results + first * m.Dim, stream);
+            }
+            return;
+        }
+        // The kernels walk whole blocks of RegTreeBlock trees. A range that starts or ends inside a block has
+        // those few trees evaluated by the kernel that follows the model's own tables, before and after the
+        // whole blocks: the launches hand on raw sums, each adds its trees in tree order, so the result is the
+        // same sequence of additions as one pass over the range.
+        const uint32_t block = m.RegTreeBlockSize;
+        const uint32_t wholeBegin = (tb + block - 1) / block * block;
+        const uint32_t wholeEnd = te == TreeCount ? te : te / block * block;  // null trees pad the model's last block
+        const bool biased = treeStart == 0;
+        const auto generic = [&](uint32_t begin, uint32_t end, uint32_t mode) {
+            const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
+            const dim3 grid(static_cast<uint32_t>((blocks + 3) / 4));
+            const auto launch = [&](auto kernel) {
+                hipLaunchKernelGGL(kernel, grid, dim3(256), 0, s, reinterpret_cast<const uint32_t*>(bins), docCount,
+                                   m.LayoutBuckets, tt, begin, end, results, mode, biased ? 1u : 0u);
+            };
+            if (m.Dim == 1) {
+                launch(dev::EvalObliviousKernel<1>);
+            } else if (m.Dim == 2) {
+                launch(dev::EvalObliviousKernel<2>);
+            } else if (m.Dim <= 4) {
+                launch(dev::EvalObliviousKernel<4>);
+            } else if (m.Dim <= 8) {
+                launch(dev::EvalObliviousKernel<8>);
+            } else {
+                launch(dev::EvalObliviousKernel<16>);
+            }
+            HIP_CHECK(hipGetLastError());
+        };
+        if (wholeBegin >= wholeEnd) {
+            generic(tb, te, 0);  // fewer trees than a block holds (or none: the bias alone)
+            return;
+        }
+        const bool head = tb < wholeBegin, tail = wholeEnd < te;
+        if (head) {
+            generic(tb, wholeBegin, dev::kEvalRaw);
+        }
         TEvalRegArgs args = {};
         args.Bins = bins;
-        args.Rows = m.RegRows.Get();
+        args.Rows = m.RegRows.Get() + static_cast<size_t>(wholeBegin) * m.RegRowDwords;
         args.Out = results;
         args.DocCount = static_cast<uint32_t>(docCount);
         args.BlockCount = static_cast<uint32_t>((docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock);
-        args.TreeBlocks = m.RegTreeBlocks;
-        args.Flags = 1;  // the range starts at tree 0: add the bias
+        args.TreeBlocks = (wholeEnd - wholeBegin + block - 1) / block;
+        args.Flags = (biased && !tail ? 1u : 0u) | (head ? 2u : 0u) | (tail ? 4u : 0u);
         args.Scale = m.Scale;
         args.BucketCount = m.LayoutBuckets;
         args.Dim = static_cast<uint32_t>(m.Dim);
         const uint32_t grid = (args.BlockCount + m.RegWaves - 1) / m.RegWaves;
         for (uint32_t first = 0, launch = 0; first < args.Dim; first += m.RegPitch, ++launch) {
-            args.Leaves = m.RegLeaves.Get() + launch * m.RegLaunchLeaves;
+            args.Leaves = m.RegLeaves.Get() + launch * m.RegLaunchLeaves + static_cast<size_t>(wholeBegin) * m.RegTreeLeafDoubles;
             args.Bias = m.RegBias.Get() + first;
             args.FirstDim = first;
             args.StoreDims = std::min(m.RegPitch, args.Dim - first);
@@ -1798,6 +1849,9 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
             void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &argSize,
                               HIP_LAUNCH_PARAM_END};
             HIP_CHECK(hipModuleLaunchKernel(m.RegFunction, grid, 1, 1, 64 * m.RegWaves, 1, 1, 0, s, nullptr, config));
+        }
+        if (tail) {
+            generic(wholeEnd, te, dev::kEvalContinue);
         }
         return;
     }

@@ -589,11 +589,18 @@ __device__ __forceinline__ double Finish(double sum, double scale, double bias, 
 // Oblivious trees, any model: one wave per 256-document block, four documents per lane, leaf
 // sums kept in registers in fp64 and accumulated in tree order (as the CPU evaluator does).
 // DCHUNK output dimensions are accumulated per pass over the trees.
+// mode: kEvalContinue - the sums start from the raw sums of earlier trees found in `out`; kEvalRaw - store raw
+// sums (neither scaled nor biased) for a launch that continues them; `addBias` tells the launch that finishes
+// whether the whole range started at tree 0 (0 no, 1 yes, 2: this launch is the whole range, treeBegin tells).
 // grid = ceil(doc blocks / 4), block = 256 threads.
+constexpr uint32_t kEvalContinue = 1;
+constexpr uint32_t kEvalRaw = 2;
+
 template <int DCHUNK>
 __global__ __launch_bounds__(256) void EvalObliviousKernel(const uint32_t* __restrict__ bins, size_t docCount,
                                                            uint32_t bucketCount, TTreeTables tt, uint32_t treeBegin,
-                                                           uint32_t treeEnd, double* __restrict__ out) {
+                                                           uint32_t treeEnd, double* out, uint32_t mode,
+                                                           uint32_t addBiasFlag) {
     const uint32_t lane = threadIdx.x & (kWave - 1);
     const size_t block = static_cast<size_t>(blockIdx.x) * (256 / kWave) + threadIdx.x / kWave;
     const size_t blockCount = (docCount + kDocsPerBlock - 1) / kDocsPerBlock;
@@ -602,14 +609,18 @@ __global__ __launch_bounds__(256) void EvalObliviousKernel(const uint32_t* __res
     }
     const uint32_t* myBins = bins + block * bucketCount * kWave + lane;
     const int dim = tt.Dim;
-    const bool addBias = treeBegin == 0;
+    const bool addBias = addBiasFlag == 2 ? treeBegin == 0 : addBiasFlag != 0;
     for (int d0 = 0; d0 < dim; d0 += DCHUNK) {
         double acc[4][DCHUNK];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
+            const size_t doc = block * kDocsPerBlock + j * kWave + lane;
 #pragma unroll
             for (int k = 0; k < DCHUNK; ++k) {
                 acc[j][k] = 0.0;
+                if ((mode & kEvalContinue) && doc < docCount && (DCHUNK == 1 || d0 + k < dim)) {
+                    acc[j][k] = out[doc * dim + d0 + k];
+                }
             }
         }
         for (uint32_t t = treeBegin; t < treeEnd; ++t) {
@@ -646,7 +657,8 @@ __global__ __launch_bounds__(256) void EvalObliviousKernel(const uint32_t* __res
 #pragma unroll
                 for (int k = 0; k < DCHUNK; ++k) {
                     if (DCHUNK == 1 || d0 + k < dim) {
-                        out[doc * dim + d0 + k] = Finish(acc[j][k], tt.Scale, tt.Bias[d0 + k], addBias);
+                        out[doc * dim + d0 + k] =
+                            (mode & kEvalRaw) ? acc[j][k] : Finish(acc[j][k], tt.Scale, tt.Bias[d0 + k], addBias);
                     }
                 }
             }

@@ -1112,6 +1112,39 @@ def test_c2_full_size_properties():
     assert torch.allclose(parts, out, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("cfg,trees", [("C2", 210), ("C3", 75), ("C1", 200)])
+def test_tree_ranges_stay_on_the_register_kernels_and_equal_the_oracle(cfg, trees):
+    """CalcTreesBlockedImpl (cpu/evaluator_impl.cpp:257-414) runs any [treeStart, treeEnd) through its one loop
+    and ApplyScaleAndBias adds the bias only when the range starts at tree 0 (scale_and_bias.cpp:13-24). Here
+    the whole tree blocks of a range go through the register-resident kernel and the few trees before and after
+    them through the kernel that follows the model's tables, all adding in tree order: equal to the oracle bit
+    for bit, for the device and the host entry points."""
+    import torch
+
+    model, info = syn.build_model(cfg, trees=trees)
+    model.set_scale_and_bias(0.5, [0.25 * (k + 1) for k in range(info["dim"])])
+    ev = model.evaluator()
+    oracle = OracleModel(read_cbm(model.save_to_buffer()))
+    docs, dim = 3001, info["dim"]
+    x = syn.device_features(info, docs)
+    host = x.cpu().numpy()
+    bins = torch.zeros(ev.quantized_bytes(docs), dtype=torch.uint8, device="cuda:0")
+    out = torch.zeros(docs * dim, dtype=torch.float64, device="cuda:0")
+    torch.cuda.synchronize()
+    ev.quantize(ev.features(cb.LAYOUT_FLAT_ROWS, x.data_ptr(), x.shape[1]), docs, bins.data_ptr())
+    ranges = [(0, trees), (0, 16), (0, 17), (3, 17), (5, 9), (16, 48), (1, trees), (15, trees - 1), (33, 64),
+              (31, 33), (7, 7), (0, 0), (trees, trees), (trees - 3, trees), (64, trees)]
+    for begin, end in ranges:
+        out.fill_(-3.0)
+        torch.cuda.synchronize()
+        ev.eval_quantized(bins.data_ptr(), docs, out.data_ptr(), tree_start=begin, tree_end=end)
+        ev.synchronize()
+        expected = oracle.calc(host, tree_start=begin, tree_end=end, threads=8)
+        np.testing.assert_array_equal(out.cpu().numpy(), expected, err_msg="trees [%d, %d)" % (begin, end))
+    np.testing.assert_array_equal(model.calc_flat(host[:700], tree_start=19, tree_end=trees - 20),
+                                  oracle.calc(host[:700], tree_start=19, tree_end=trees - 20))
+
+
 @pytest.mark.parametrize("name,base_docs,copies", [("C2", 1_000_000, 23), ("C4", 1_000_000, 15), ("C3", 500_000, 110)])
 def test_batches_beyond_four_gibibytes(name, base_docs, copies):
     """Batches whose features, bins or results pass 4 GiB (C2: 18 GB of features, 4.6 GB of bins; C3: 4.4 GB
@@ -1137,14 +1170,14 @@ def test_batches_beyond_four_gibibytes(name, base_docs, copies):
     ev.eval_data(ev.features(cb.LAYOUT_FLAT_ROWS, x.data_ptr(), x.shape[1]), docs, out.data_ptr())
     ev.synchronize()
     assert ev.quantized_bytes(docs) > (1 << 32) or name == "C3"
-    # the huge batch may take another kernel than the base batch (C3: its output passes what the register
-    # kernels address), so the first repetition is held to the tolerance and the others to the first
+    # a batch whose results pass what a launch of the register kernels addresses (C3) goes in slices through
+    # the same kernels: every repetition equals the base batch bit for bit
     first = out[:base_docs * dim]
-    _close(first.cpu().numpy(), expected.cpu().numpy())
+    assert torch.equal(first, expected)
     for c in range(1, copies):
         assert torch.equal(out[c * base_docs * dim:(c + 1) * base_docs * dim], first), "repetition %d" % c
     assert torch.equal(out[copies * base_docs * dim:], first[:tail * dim])
-    # a tree sub-range takes the kernels that do not hold the model in registers
+    # a tree sub-range
     half = model.tree_count // 2
     part = torch.zeros_like(out)
     part_base = torch.zeros_like(expected)
