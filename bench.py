@@ -17,9 +17,54 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
-# HBM bytes of one step (both launches, fetched + written), from rocprofv3 FETCH_SIZE / WRITE_SIZE
-# runs scaled by a copy kernel of known size; only known for workloads that were profiled
-MEASURED_TRAFFIC_BYTES = {("C2", 4000000, 1000): 6.12e9}
+# HBM-side bytes of one step (fetched + written) come from rocprofv3 FETCH_SIZE / WRITE_SIZE runs scaled by a copy
+# kernel of known size. They are not measured in this run: the line carries the figure that a profile summary
+# holds for exactly this workload and these kernels (a line "TRAFFIC <config> <docs> <trees> <kernels> <bytes>"
+# in the file below), and null otherwise.
+TRAFFIC_PROFILE = os.path.join("profiles", "c2_hbm_traffic_pmc.txt")
+
+
+def measured_traffic(config, docs, trees, kernels):
+    """(bytes per step, source) from the profile summary, or (None, None) when it holds no matching line."""
+    path = os.path.join(ROOT, TRAFFIC_PROFILE)
+    if not os.path.exists(path):
+        return None, None
+    wanted = "+".join(kernels[k] for k in sorted(kernels))
+    with open(path) as f:
+        for line in f:
+            parts = line.split()
+            if len(parts) == 6 and parts[0] == "TRAFFIC" and parts[1] == config and int(parts[2]) == docs and \
+                    int(parts[3]) == trees and parts[4] == wanted:
+                return float(parts[5]), TRAFFIC_PROFILE
+    return None, None
+
+
+def end_to_end_c_abi(model, info, docs):
+    """CalcModelPredictionFlat (the reference API: one pointer per row, host memory in and out) on a bounded
+    sample: rows gathered into pinned memory, copied over PCIe, evaluated, results copied back."""
+    import numpy as np
+
+    from catboost_amd import synthetic as syn
+
+    docs = int(min(docs, 1_000_000))
+    x = syn.host_features(info, docs, seed=9)
+    model.calc_flat(x[:1000])
+    best = None
+    for _ in range(3):
+        t0 = time.perf_counter()
+        model.calc_flat(x)
+        elapsed = time.perf_counter() - t0
+        best = elapsed if best is None else min(best, elapsed)
+    return {"docs_per_sec": docs / best, "sample": "%d docs of the same workload, best of 3 calls, %.1f ms" % (docs, best * 1e3),
+            "host_to_device_GBps": docs * x.shape[1] * 4 / best / 1e9}
+
+
+def host_threads():
+    """Worker threads for the CPU legs: every host core, unless the machine's environment caps worker pools
+    (OMP_NUM_THREADS: a GPU box gives one GPU's job a share of its cores)."""
+    cap = os.environ.get("OMP_NUM_THREADS", "")
+    cores = os.cpu_count() or 1
+    return max(1, min(cores, int(cap))) if cap.isdigit() else cores
 
 
 def cpu_baseline(model_bytes, info, target_seconds=12.0):
@@ -31,7 +76,7 @@ def cpu_baseline(model_bytes, info, target_seconds=12.0):
     from oracle.oracle import OracleModel
 
     oracle = OracleModel(read_cbm(model_bytes))
-    threads = min(16, os.cpu_count() or 1)
+    threads = host_threads()
     docs = int(min(info["docs"], 400_000))
     x = syn.host_features(info, docs, seed=6)
     t0 = time.perf_counter()
@@ -57,6 +102,7 @@ def cpu_baseline(model_bytes, info, target_seconds=12.0):
         "value": total / elapsed,
         "unit": "docs/sec",
         "cores": threads,
+        "host_cpu_count": os.cpu_count(),
         "kind": "port",
         "sample": "%d docs of the same workload evaluated %d times, %d threads over 128-doc blocks, %.1f s" % (
             docs, repeats, threads, elapsed),
@@ -105,6 +151,7 @@ def main():
     ap.add_argument("--config", default="C2")
     ap.add_argument("--docs", type=int, default=0, help="override the document count of the workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-end-to-end", action="store_true", help="skip the CalcModelPredictionFlat figure")
     ap.add_argument("--check-docs", type=int, default=20000)
     ap.add_argument("--copy-probe-mib", type=int, default=0,
                     help="also run one device-to-device copy of this many MiB (a kernel of known traffic, used to "
@@ -166,18 +213,35 @@ def main():
     idx = torch.randperm(docs, device="cuda:0")[:n_check].sort().values
     sample = x[idx].cpu().numpy()
     got = out.view(docs, dim)[idx].cpu().numpy().ravel()
-    expected = oracle.calc(sample, threads=min(16, os.cpu_count() or 1))
+    expected = oracle.calc(sample, threads=host_threads())
     max_abs = float(np.abs(got - expected).max()) if n_check else 0.0
     ok = bool(np.allclose(got, expected, rtol=1e-9, atol=1e-12))
 
-    used_floats = sum(1 for f in read_cbm(model_bytes)["float_features"] if len(f["borders"]))
-    used_cats = sum(1 for c in read_cbm(model_bytes)["cat_features"] if c["used"])
+    model_dict = read_cbm(model_bytes)
+    used_borders = sorted(len(f["borders"]) for f in model_dict["float_features"] if len(f["borders"]))
+    used_floats = len(used_borders)
+    used_cats = sum(1 for c in model_dict["cat_features"] if c["used"])
     bytes_per_doc = 4 * used_floats + 4 * used_cats + 8 * dim
     step_bytes = bytes_per_doc * docs
     avg_bin, avg_eval = float(np.mean(bin_ms)), float(np.mean(eval_ms))
+    # the kernels of a step run back to back on one stream: the two intervals share their middle event, so
+    # their sum is the time from the step's first event to its last (a fused kernel reports one interval)
     kernels_ms = avg_bin + avg_eval
     achieved = step_bytes / (kernels_ms * 1e-3) / 1e9
     buckets = ev.bucket_count
+    kernel_names = ev.describe_kernels(cb.LAYOUT_FLAT_ROWS)
+    traffic, traffic_source = measured_traffic(args.config, docs, model.tree_count, kernel_names)
+    if "fused" in kernel_names:
+        kernels = {"fused": {"name": kernel_names["fused"], "avg_ms": kernels_ms,
+                             "tree_evals_per_sec": docs * model.tree_count / (kernels_ms * 1e-3)}}
+    else:
+        kernels = {
+            "binarize": {"name": kernel_names["binarize"], "avg_ms": avg_bin,
+                         "GBps": (4 * (used_floats + used_cats) + buckets) * docs / (avg_bin * 1e-3) / 1e9 if avg_bin > 0 else None},
+            "evaluate": {"name": kernel_names["evaluate"], "avg_ms": avg_eval,
+                         "GBps": (buckets + 8 * dim) * docs / (avg_eval * 1e-3) / 1e9,
+                         "tree_evals_per_sec": docs * model.tree_count / (avg_eval * 1e-3)},
+        }
     result = {
         "metric": "docs/sec (binarize + evaluate, %d trees, %d docs)" % (model.tree_count, docs),
         "value": docs * args.steps / elapsed,
@@ -201,18 +265,20 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, docs, model.tree_count)),
+            "traffic": traffic,
+            "traffic_source": traffic_source,
             "algorithmic_bytes_per_doc": bytes_per_doc,
-            "kernel": "binarize + evaluate (the two launches of one step)",
+            "kernel": " + ".join(kernel_names[k] for k in sorted(kernel_names)),
+            "kernel_ms": kernels_ms,
         },
-        "kernels": {
-            "binarize": {"avg_ms": avg_bin, "GBps": (4 * (used_floats + used_cats) + buckets) * docs / (avg_bin * 1e-3) / 1e9
-                         if avg_bin > 0 else None},
-            "evaluate": {"avg_ms": avg_eval, "GBps": (buckets + 8 * dim) * docs / (avg_eval * 1e-3) / 1e9,
-                         "tree_evals_per_sec": docs * model.tree_count / (avg_eval * 1e-3)},
-        },
+        "kernels": kernels,
+        "model": {"buckets": buckets,
+                  "used_borders_per_feature": {"min": used_borders[0], "median": used_borders[len(used_borders) // 2],
+                                               "max": used_borders[-1]} if used_borders else None},
         "parity": {"checked_docs": int(n_check), "max_abs_err": max_abs, "within_1e-9_rel_1e-12_abs": ok},
     }
+    if not args.no_end_to_end:
+        result["end_to_end_c_abi"] = end_to_end_c_abi(model, info, docs)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(model_bytes, info)
         if info["kind"] == "oblivious" and dim == 1 and not info["cat_hashes"]:

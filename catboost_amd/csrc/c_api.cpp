@@ -880,6 +880,15 @@ bool CbHipLastKernelTimes(CbHipEvaluatorHandle* evaluator, float* binarizeMs, fl
     });
 }
 
+bool CbHipDescribeKernels(CbHipEvaluatorHandle* evaluator, int layout, char* buffer, size_t bufferSize) {
+    return Guard([&] {
+        CBAMD_ENSURE(buffer != nullptr && bufferSize > 0, "description buffer is null");
+        const std::string text = E(evaluator)->DescribeKernels(layout);
+        CBAMD_ENSURE(text.size() < bufferSize, "description buffer is too small");
+        std::memcpy(buffer, text.c_str(), text.size() + 1);
+    });
+}
+
 CbHipEvaluatorHandle* CbHipGetEvaluator(void* modelHandle) {
     try {
         return &H(modelHandle)->GetEvaluator();

@@ -9,6 +9,7 @@
 
 #include <memory>
 #include <mutex>
+#include <string>
 
 namespace cbamd {
 
@@ -79,6 +80,9 @@ public:
                            double* results, void* stream);
     void Synchronize(void* stream);
     TKernelTimes LastKernelTimes() const { return LastTimes; }
+    // which kernels a whole-model call on a batch of the given layout (TFeatureBatch::ELayout) launches:
+    // "fused=<kernel>" or "binarize=<kernel>;evaluate=<kernel>"
+    std::string DescribeKernels(int layout) const;
 
     // ---- host-resident data: stage -> binarize -> evaluate -> copy back, in document chunks.
     // rows[doc] points at rowLen floats (FlatRows / SplitRows) or columns[f] at docCount floats.

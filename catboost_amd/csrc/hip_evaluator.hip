@@ -799,6 +799,8 @@ struct THipEvaluator::TImpl {
     TFused Fused[2];
     hipFunction_t FusedFunction = nullptr;
     uint32_t FusedWaves = 0;
+    const char* RegKernelName = "";
+    const char* FusedKernelName = "";
 
     // scratch (grow-only, guarded by THipEvaluator::Lock)
     TDeviceVec<uint8_t> ScratchBins;
@@ -1220,6 +1222,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
     if (regEnabled && variant && regTableAddressable) {
         HIP_CHECK(hipModuleLoadData(&m.RegModule, kEvalRegCodeObject));
         HIP_CHECK(hipModuleGetFunction(&m.RegFunction, m.RegModule, variant->Name));
+        m.RegKernelName = variant->Name;
         const uint32_t block = RegTreeBlock(*variant);
         const size_t pitch = variant->Pitch, rowsPerTree = variant->Leaves;
         const size_t rowDwords = variant->Mixed ? 32 : 16;
@@ -1453,6 +1456,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
             if (!m.FusedFunction) {
                 HIP_CHECK(hipModuleGetFunction(&m.FusedFunction, m.RegModule, fused->Name));
                 m.FusedWaves = fused->Waves;
+                m.FusedKernelName = fused->Name;
             }
             TImpl::TFused& f = m.Fused[layoutIndex];
             f.UnitCount = static_cast<uint32_t>(unitStart.size());
@@ -1969,6 +1973,43 @@ bool THipEvaluator::EvalRowsFusedDevice(const TFeatureBatch& batch, size_t docCo
     void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &argSize, HIP_LAUNCH_PARAM_END};
     HIP_CHECK(hipModuleLaunchKernel(m.FusedFunction, grid, 1, 1, 64 * m.FusedWaves, 1, 1, 0, m.Pick(stream), nullptr, config));
     return true;
+}
+
+std::string THipEvaluator::DescribeKernels(int layout) const {
+    const TImpl& m = *Impl;
+    const int fusedIndex = layout == TFeatureBatch::FlatRows ? 0 : layout == TFeatureBatch::SplitRows ? 1 : -1;
+    if (fusedIndex >= 0 && m.Fused[fusedIndex].Usable) {
+        return std::string("fused=") + m.FusedKernelName;
+    }
+    std::string binarize = m.BinarizeBuckets == 0 ? "none"
+                           : layout == TFeatureBatch::FlatColumns
+                               ? "BinarizeColumnsKernel"
+                               : "BinarizeRowsKernel<" + std::to_string(BinarizeLog2Slots(m.MaxBucketValues)) + ">";
+    if (m.CtrCount > 0) {
+        binarize += m.CtrTileUsable ? "+CtrBinarizeTileKernel" : "+CtrBinarizeKernel";
+    }
+    const int dchunk = TileChunk(m.Dim);
+    std::string evaluate;
+    if (TreeCount == 0) {
+        evaluate = "FillBiasKernel";
+    } else if (m.RegKernelUsable) {
+        evaluate = m.RegKernelName;
+    } else if (m.Oblivious && m.MaxDepth <= 8 && TileLdsBytes(m.LayoutBuckets, dchunk) <= kMaxTileLdsBytes) {
+        evaluate = "EvalObliviousTileKernel";
+    } else if (m.Oblivious && m.MaxDepth <= 8 && m.Dim == 1 && m.HalfTileLeaves.Get() != nullptr &&
+               TileLdsBytes(m.LayoutBuckets, 1) > kMaxTileLdsBytes) {
+        evaluate = "EvalObliviousHalfTileKernel";
+    } else if (m.Oblivious) {
+        evaluate = "EvalObliviousKernel";
+    } else if (m.NsLdsUsable &&
+               TileLdsBytes(m.LayoutBuckets, 1) + dev::kTileWaves * dev::kNsLdsEntries * 4 <= kMaxTileLdsBytes) {
+        evaluate = "EvalNonSymmetricLdsKernel";
+    } else if (m.NsTileUsable && TileLdsBytes(m.LayoutBuckets, m.Dim == 1 ? 1 : m.Dim <= 4 ? 4 : 16) <= kMaxTileLdsBytes) {
+        evaluate = "EvalNonSymmetricTileKernel";
+    } else {
+        evaluate = "EvalNonSymmetricKernel";
+    }
+    return "binarize=" + binarize + ";evaluate=" + evaluate;
 }
 
 void THipEvaluator::LeafIndexesQuantizedDevice(const uint8_t* bins, size_t docCount, size_t treeStart, size_t treeEnd,
