@@ -79,7 +79,7 @@ public:
     void CalcDeviceNoAlloc(const TFeatureBatch& batch, size_t docCount, size_t treeStart, size_t treeEnd,
                            double* results, void* stream);
     void Synchronize(void* stream);
-    TKernelTimes LastKernelTimes() const { return LastTimes; }
+    TKernelTimes LastKernelTimes() const;
     // which kernels a whole-model call on a batch of the given layout (TFeatureBatch::ELayout) launches:
     // "fused=<kernel>" or "binarize=<kernel>;evaluate=<kernel>"
     std::string DescribeKernels(int layout) const;
@@ -101,12 +101,13 @@ public:
     struct TImpl;
 
 private:
+    void SetLastTimes(const TKernelTimes& times);
     std::unique_ptr<TImpl> Impl;
     size_t TreeCount = 0;
     int ApproxDimension = 1;
     uint32_t BucketCount = 0;
     TKernelTimes LastTimes;
-    std::mutex Lock;  // one batch at a time per evaluator (scratch buffers are shared)
+    mutable std::mutex TimesLock;  // callers of one evaluator run side by side; the last one to finish leaves its times
 };
 
 // Number of HIP devices visible; throws TModelError when the runtime reports an error.

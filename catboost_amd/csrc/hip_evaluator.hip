@@ -5,6 +5,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <condition_variable>
 #include <cstdlib>
 #include <cstring>
 #include <limits>
@@ -724,7 +725,6 @@ int GetHipDeviceCount() {
 struct THipEvaluator::TImpl {
     int DeviceId = 0;
     hipStream_t Stream = nullptr;
-    hipEvent_t Ev[3] = {nullptr, nullptr, nullptr};
     uint8_t* NoAllocScratch = nullptr;  // this device's copy of the file-scope array `scratch`
     bool Oblivious = true;
     uint32_t RealBucketCount = 0;  // buckets of the model; the device layout uses max(1, this)
@@ -802,27 +802,108 @@ struct THipEvaluator::TImpl {
     const char* RegKernelName = "";
     const char* FusedKernelName = "";
 
-    // scratch (grow-only, guarded by THipEvaluator::Lock)
-    TDeviceVec<uint8_t> ScratchBins;
-    TDeviceVec<float> StageFloats;
-    TDeviceVec<int32_t> StageCats;
-    TDeviceVec<double> StageResults;
-    TDeviceVec<uint32_t> StageIndexes;
-    TDeviceVec<uint8_t> StageExport;
-    TPinnedVec<float> PinnedFloats;
-    TPinnedVec<int32_t> PinnedCats;
-    TPinnedVec<double> PinnedResults;
-    // second slot of the row staging pipeline (CalcHostRows) and the events of both slots:
-    // binarize start, binarize end, evaluate end, results on the host
-    TPinnedVec<float> PinnedFloats2;
-    TPinnedVec<int32_t> PinnedCats2;
-    TPinnedVec<double> PinnedResults2;
-    TDeviceVec<float> StageFloats2;
-    TDeviceVec<int32_t> StageCats2;
-    TDeviceVec<double> StageResults2;
-    hipEvent_t SlotEv[2][4] = {{nullptr, nullptr, nullptr, nullptr}, {nullptr, nullptr, nullptr, nullptr}};
-    TPinnedVec<uint32_t> PinnedIndexes;
-    TPinnedVec<uint8_t> PinnedExport;
+    // Staging of the calls that own their buffers (CalcDevice and the host entry points): a call borrows a
+    // context - a stream, a bin buffer and two slots of pinned and device staging memory - from a small pool,
+    // so that a few callers of one evaluator run side by side and later ones wait for a free context.
+    struct THostSlot {
+        TPinnedVec<float> PinnedFloats;
+        TPinnedVec<int32_t> PinnedCats;
+        TPinnedVec<double> PinnedResults;
+        TPinnedVec<uint32_t> PinnedIndexes;
+        TPinnedVec<uint8_t> PinnedExport;
+        TDeviceVec<float> StageFloats;
+        TDeviceVec<int32_t> StageCats;
+        TDeviceVec<double> StageResults;
+        TDeviceVec<uint32_t> StageIndexes;
+        TDeviceVec<uint8_t> StageExport;
+        // binarize start, binarize end, evaluate end, results on the host
+        hipEvent_t Ev[4] = {nullptr, nullptr, nullptr, nullptr};
+    };
+    struct THostContext {
+        hipStream_t Stream = nullptr;
+        TDeviceVec<uint8_t> ScratchBins;
+        THostSlot Slots[2];
+        hipEvent_t Ev[3] = {nullptr, nullptr, nullptr};
+        bool Busy = false;
+
+        THostContext() {
+            HIP_CHECK(hipStreamCreateWithFlags(&Stream, hipStreamNonBlocking));
+            for (auto& e : Ev) {
+                HIP_CHECK(hipEventCreate(&e));
+            }
+            for (auto& slot : Slots) {
+                for (auto& e : slot.Ev) {
+                    HIP_CHECK(hipEventCreate(&e));
+                }
+            }
+        }
+        ~THostContext() {
+            if (Stream) {
+                (void)hipStreamSynchronize(Stream);
+            }
+            for (auto& e : Ev) {
+                if (e) {
+                    (void)hipEventDestroy(e);
+                }
+            }
+            for (auto& slot : Slots) {
+                for (auto& e : slot.Ev) {
+                    if (e) {
+                        (void)hipEventDestroy(e);
+                    }
+                }
+            }
+            if (Stream) {
+                (void)hipStreamDestroy(Stream);
+            }
+        }
+        THostContext(const THostContext&) = delete;
+        THostContext& operator=(const THostContext&) = delete;
+    };
+    static constexpr size_t kMaxHostContexts = 4;
+    std::mutex ContextLock;
+    std::condition_variable ContextFree;
+    std::vector<std::unique_ptr<THostContext>> Contexts;
+
+    // A context of the pool for the time of one call.
+    class TContextLease {
+    public:
+        explicit TContextLease(TImpl& impl)
+            : Impl(impl)
+        {
+            std::unique_lock<std::mutex> guard(Impl.ContextLock);
+            for (;;) {
+                for (auto& c : Impl.Contexts) {
+                    if (!c->Busy) {
+                        Context = c.get();
+                        break;
+                    }
+                }
+                if (!Context && Impl.Contexts.size() < kMaxHostContexts) {
+                    Impl.Contexts.emplace_back(new THostContext);
+                    Context = Impl.Contexts.back().get();
+                }
+                if (Context) {
+                    Context->Busy = true;
+                    return;
+                }
+                Impl.ContextFree.wait(guard);
+            }
+        }
+        ~TContextLease() {
+            {
+                std::lock_guard<std::mutex> guard(Impl.ContextLock);
+                Context->Busy = false;
+            }
+            Impl.ContextFree.notify_one();
+        }
+        THostContext& operator*() const { return *Context; }
+        THostContext* operator->() const { return Context; }
+
+    private:
+        TImpl& Impl;
+        THostContext* Context = nullptr;
+    };
 
     dev::TBinarizeTables BinarizeTables(bool flat) const {
         dev::TBinarizeTables t;
@@ -871,18 +952,7 @@ struct THipEvaluator::TImpl {
         if (Stream) {
             (void)hipStreamSynchronize(Stream);
         }
-        for (auto& e : Ev) {
-            if (e) {
-                (void)hipEventDestroy(e);
-            }
-        }
-        for (auto& slot : SlotEv) {
-            for (auto& e : slot) {
-                if (e) {
-                    (void)hipEventDestroy(e);
-                }
-            }
-        }
+        Contexts.clear();
         if (Stream) {
             (void)hipStreamDestroy(Stream);
         }
@@ -906,14 +976,6 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
     m.DeviceId = deviceId;
     m.NoAllocScratch = NoAllocScratchOfCurrentDevice(deviceId);
     HIP_CHECK(hipStreamCreateWithFlags(&m.Stream, hipStreamNonBlocking));
-    for (auto& e : m.Ev) {
-        HIP_CHECK(hipEventCreate(&e));
-    }
-    for (auto& slot : m.SlotEv) {
-        for (auto& e : slot) {
-            HIP_CHECK(hipEventCreate(&e));
-        }
-    }
     TreeCount = trees.GetTreeCount();
     ApproxDimension = trees.ApproxDimension;
     BucketCount = trees.EffectiveBinFeaturesBucketCount;
@@ -2071,27 +2133,28 @@ void THipEvaluator::ApplyPredictionTypeDevice(int predictionType, size_t firstDo
 
 void THipEvaluator::CalcDevice(const TFeatureBatch& batch, size_t docCount, size_t treeStart, size_t treeEnd,
                                double* results, void* stream) {
-    std::lock_guard<std::mutex> guard(Lock);
     TImpl& m = *Impl;
     HIP_CHECK(hipSetDevice(m.DeviceId));
-    hipStream_t s = m.Pick(stream);
-    HIP_CHECK(hipEventRecord(m.Ev[0], s));
+    TImpl::TContextLease ctx(m);
+    hipStream_t s = stream ? static_cast<hipStream_t>(stream) : m.Stream;
+    TKernelTimes times;
+    HIP_CHECK(hipEventRecord(ctx->Ev[0], s));
     if (EvalRowsFusedDevice(batch, docCount, treeStart, treeEnd, results, s)) {
         // one launch does both: its whole duration is reported as the evaluate time
-        HIP_CHECK(hipEventRecord(m.Ev[2], s));
+        HIP_CHECK(hipEventRecord(ctx->Ev[2], s));
         HIP_CHECK(hipStreamSynchronize(s));
-        LastTimes.BinarizeMs = 0.0f;
-        HIP_CHECK(hipEventElapsedTime(&LastTimes.EvalMs, m.Ev[0], m.Ev[2]));
-        return;
+        HIP_CHECK(hipEventElapsedTime(&times.EvalMs, ctx->Ev[0], ctx->Ev[2]));
+    } else {
+        ctx->ScratchBins.Reserve(QuantizedBytes(docCount));
+        QuantizeDevice(batch, docCount, ctx->ScratchBins.Get(), s);
+        HIP_CHECK(hipEventRecord(ctx->Ev[1], s));
+        EvalQuantizedDevice(ctx->ScratchBins.Get(), docCount, treeStart, treeEnd, results, s);
+        HIP_CHECK(hipEventRecord(ctx->Ev[2], s));
+        HIP_CHECK(hipStreamSynchronize(s));
+        HIP_CHECK(hipEventElapsedTime(&times.BinarizeMs, ctx->Ev[0], ctx->Ev[1]));
+        HIP_CHECK(hipEventElapsedTime(&times.EvalMs, ctx->Ev[1], ctx->Ev[2]));
     }
-    m.ScratchBins.Reserve(QuantizedBytes(docCount));
-    QuantizeDevice(batch, docCount, m.ScratchBins.Get(), s);
-    HIP_CHECK(hipEventRecord(m.Ev[1], s));
-    EvalQuantizedDevice(m.ScratchBins.Get(), docCount, treeStart, treeEnd, results, s);
-    HIP_CHECK(hipEventRecord(m.Ev[2], s));
-    HIP_CHECK(hipStreamSynchronize(s));
-    HIP_CHECK(hipEventElapsedTime(&LastTimes.BinarizeMs, m.Ev[0], m.Ev[1]));
-    HIP_CHECK(hipEventElapsedTime(&LastTimes.EvalMs, m.Ev[1], m.Ev[2]));
+    SetLastTimes(times);
 }
 
 void THipEvaluator::CalcDeviceNoAlloc(const TFeatureBatch& batch, size_t docCount, size_t treeStart, size_t treeEnd,
@@ -2113,60 +2176,46 @@ void THipEvaluator::CalcDeviceNoAlloc(const TFeatureBatch& batch, size_t docCoun
 
 namespace {
 
-// documents staged per round trip; bounds pinned and device staging memory
-size_t ChunkDocs(size_t rowFloats, size_t rowCats) {
-    const size_t bytesPerDoc = std::max<size_t>(1, (rowFloats + rowCats) * 4);
-    const size_t budget = size_t(512) << 20;
-    size_t docs = budget / bytesPerDoc;
-    docs = std::max<size_t>(docs, 1024);
-    docs = std::min<size_t>(docs, size_t(1) << 22);
-    return docs / dev::kDocsPerBlock * dev::kDocsPerBlock;
-}
-
-}  // namespace
-
-namespace {
-
-// Copies `count` rows of `rowLen` elements each, given by pointer, into a dense matrix; large
-// batches are split over a few threads (the copy is what bounds the pointer-per-row entry points).
-template <typename T>
-void GatherRows(const T* const* rows, size_t count, size_t rowLen, T* dst) {
-    const size_t bytes = count * rowLen * sizeof(T);
-    size_t threads = std::min<size_t>(std::max(1u, std::thread::hardware_concurrency()), 16);
-    threads = std::min(threads, bytes / (size_t(4) << 20) + 1);
-    const auto copy = [=](size_t begin, size_t end) {
-        for (size_t d = begin; d < end; ++d) {
-            std::memcpy(dst + d * rowLen, rows[d], rowLen * sizeof(T));
-        }
-    };
-    if (threads <= 1) {
-        copy(0, count);
-        return;
-    }
-    std::vector<std::thread> pool;
-    const size_t per = (count + threads - 1) / threads;
-    for (size_t t = 1; t < threads; ++t) {
-        pool.emplace_back(copy, std::min(count, t * per), std::min(count, (t + 1) * per));
-    }
-    copy(0, std::min(count, per));
-    for (auto& th : pool) {
-        th.join();
-    }
-}
-
-// documents per slot of the row staging pipeline: small enough that gathering the next slot on
-// the host overlaps the transfer and the kernels of the current one
-size_t PipelineDocs(size_t rowFloats, size_t rowCats) {
-    const size_t bytesPerDoc = std::max<size_t>(1, (rowFloats + rowCats) * 4);
-    size_t docs = (size_t(64) << 20) / bytesPerDoc;
+// documents per slot of the staging pipeline: small enough that gathering the next slot on the host
+// overlaps the transfer and the kernels of the current one
+size_t PipelineDocs(size_t bytesPerDoc) {
+    size_t docs = (size_t(64) << 20) / std::max<size_t>(1, bytesPerDoc);
     docs = std::max<size_t>(docs, 4096);
     docs = std::min<size_t>(docs, size_t(1) << 20);
     return docs / dev::kDocsPerBlock * dev::kDocsPerBlock;
 }
 
-}  // namespace
+// Runs `work(begin, end)` over [0, count) on a few threads when the bytes to move make it worthwhile.
+template <typename TWork>
+void ParallelCopy(size_t count, size_t bytes, const TWork& work) {
+    size_t threads = std::min<size_t>(std::max(1u, std::thread::hardware_concurrency()), 16);
+    threads = std::min(threads, bytes / (size_t(4) << 20) + 1);
+    threads = std::min(threads, std::max<size_t>(count, 1));
+    if (threads <= 1) {
+        work(size_t(0), count);
+        return;
+    }
+    std::vector<std::thread> pool;
+    const size_t per = (count + threads - 1) / threads;
+    for (size_t t = 1; t < threads; ++t) {
+        pool.emplace_back(work, std::min(count, t * per), std::min(count, (t + 1) * per));
+    }
+    work(size_t(0), std::min(count, per));
+    for (auto& th : pool) {
+        th.join();
+    }
+}
 
-namespace {
+// Copies `count` rows of `rowLen` elements each, given by pointer, into a dense matrix (the copy is
+// what bounds the pointer-per-row entry points).
+template <typename T>
+void GatherRows(const T* const* rows, size_t count, size_t rowLen, T* dst) {
+    ParallelCopy(count, count * rowLen * sizeof(T), [=](size_t begin, size_t end) {
+        for (size_t d = begin; d < end; ++d) {
+            std::memcpy(dst + d * rowLen, rows[d], rowLen * sizeof(T));
+        }
+    });
+}
 
 // A model without trees answers with its bias whatever the prediction type: the reference fills the result
 // array with the bias values in turn and returns before any post-processing (cpu/formula_evaluator.cpp:29-41).
@@ -2176,19 +2225,104 @@ void FillBiasOnly(const std::vector<double>& bias, size_t count, double* results
     }
 }
 
+// The two-slot pipeline of the host entry points: documents go in chunks; while the GPU copies in, runs and
+// copies out the chunk of one slot, the host fills the other slot. stage(slot, begin, n) fills the slot's
+// pinned memory and enqueues everything up to the event Ev[3] of the slot; collect(slot, begin, n) runs once
+// that event has passed.
+template <typename TStage, typename TCollect>
+void RunPipeline(size_t docCount, size_t chunk, hipEvent_t (&done)[2], const TStage& stage, const TCollect& collect) {
+    size_t pendingBegin[2] = {0, 0}, pendingDocs[2] = {0, 0};
+    size_t index = 0;
+    const auto finish = [&](int slot) {
+        if (pendingDocs[slot]) {
+            HIP_CHECK(hipEventSynchronize(done[slot]));
+            collect(slot, pendingBegin[slot], pendingDocs[slot]);
+            pendingDocs[slot] = 0;
+        }
+    };
+    for (size_t begin = 0; begin < docCount; begin += chunk, ++index) {
+        const int slot = static_cast<int>(index & 1);
+        const size_t n = std::min(chunk, docCount - begin);
+        finish(slot);  // the slot's previous chunk must be out before its buffers are reused
+        stage(slot, begin, n);
+        pendingBegin[slot] = begin;
+        pendingDocs[slot] = n;
+    }
+    // the (up to) two chunks still in flight, older first
+    finish(static_cast<int>(index & 1));
+    finish(static_cast<int>((index + 1) & 1));
+}
+
 }  // namespace
 
-// Rows by pointer (the reference API's float** / hashed int**): two slots of pinned and device
-// staging memory; while the GPU copies in, binarizes, evaluates and copies out slot k, the host
-// gathers the rows of slot k + 1.
+void THipEvaluator::SetLastTimes(const TKernelTimes& times) {
+    std::lock_guard<std::mutex> guard(TimesLock);
+    LastTimes = times;
+}
+
+TKernelTimes THipEvaluator::LastKernelTimes() const {
+    std::lock_guard<std::mutex> guard(TimesLock);
+    return LastTimes;
+}
+
+// Stages one chunk of rows given by pointer (the reference API's float** / hashed int**) and returns the
+// batch that describes it on the device.
+static TFeatureBatch StageRowChunk(THipEvaluator::TImpl::THostSlot& slot, hipStream_t s, const float* const* rows,
+                                   const int32_t* const* catRows, size_t begin, size_t n, size_t needFloats,
+                                   size_t needCats, bool flat) {
+    if (needFloats) {
+        GatherRows(rows + begin, n, needFloats, slot.PinnedFloats.Get());
+        HIP_CHECK(hipMemcpyAsync(slot.StageFloats.Get(), slot.PinnedFloats.Get(), n * needFloats * sizeof(float),
+                                 hipMemcpyHostToDevice, s));
+    }
+    if (needCats) {
+        GatherRows(catRows + begin, n, needCats, slot.PinnedCats.Get());
+        HIP_CHECK(hipMemcpyAsync(slot.StageCats.Get(), slot.PinnedCats.Get(), n * needCats * sizeof(int32_t),
+                                 hipMemcpyHostToDevice, s));
+    }
+    TFeatureBatch batch;
+    batch.Layout = flat ? TFeatureBatch::FlatRows : TFeatureBatch::SplitRows;
+    batch.Floats = slot.StageFloats.Get();
+    batch.Stride = needFloats;
+    batch.Cats = needCats ? slot.StageCats.Get() : nullptr;
+    batch.CatStride = needCats;
+    return batch;
+}
+
+// What the prediction entry points share once a chunk's features are on the device: binarize, evaluate,
+// prediction type, copy back; the slot's events bracket the kernels.
+static void RunPredictionChunk(THipEvaluator& ev, THipEvaluator::TImpl::THostContext& ctx, int slotIndex,
+                               const TFeatureBatch& batch, size_t begin, size_t n, size_t docCount, size_t stageDocs,
+                               size_t treeStart, size_t treeEnd, int predictionType) {
+    THipEvaluator::TImpl::THostSlot& slot = ctx.Slots[slotIndex];
+    hipStream_t s = ctx.Stream;
+    const size_t dim = static_cast<size_t>(ev.GetApproxDimension());
+    const size_t outDim = predictionType == dev::kPredClass ? 1 : dim;
+    HIP_CHECK(hipEventRecord(slot.Ev[0], s));
+    if (ev.EvalRowsFusedDevice(batch, n, treeStart, treeEnd, slot.StageResults.Get(), s)) {
+        HIP_CHECK(hipEventRecord(slot.Ev[1], s));
+    } else {
+        ev.QuantizeDevice(batch, n, ctx.ScratchBins.Get(), s);
+        HIP_CHECK(hipEventRecord(slot.Ev[1], s));
+        ev.EvalQuantizedDevice(ctx.ScratchBins.Get(), n, treeStart, treeEnd, slot.StageResults.Get(), s);
+    }
+    HIP_CHECK(hipEventRecord(slot.Ev[2], s));
+    const double* final = slot.StageResults.Get();
+    if (predictionType != dev::kPredRaw) {
+        // raw values, and behind them room for a prediction type that cannot be computed in place
+        double* processed = slot.StageResults.Get() + (outDim == dim ? 0 : stageDocs * dim);
+        ev.ApplyPredictionTypeDevice(predictionType, begin, docCount, n, slot.StageResults.Get(), processed, s);
+        final = processed;
+    }
+    HIP_CHECK(hipMemcpyAsync(slot.PinnedResults.Get(), final, n * outDim * sizeof(double), hipMemcpyDeviceToHost, s));
+    HIP_CHECK(hipEventRecord(slot.Ev[3], s));
+}
+
 void THipEvaluator::CalcHostRows(const float* const* rows, size_t rowLen, bool flat, const int32_t* const* catRows,
                                  size_t catRowLen, size_t docCount, size_t treeStart, size_t treeEnd, double* results,
                                  int predictionType) {
-    std::lock_guard<std::mutex> guard(Lock);
     TImpl& m = *Impl;
     const size_t outDim = predictionType == dev::kPredClass ? 1 : static_cast<size_t>(m.Dim);
-    HIP_CHECK(hipSetDevice(m.DeviceId));
-    hipStream_t s = m.Stream;
     // only the columns the model can address are staged
     const size_t needFloats = flat ? m.FlatVectorSize : m.MinFloatSize;
     const size_t needCats = (!flat && m.HasCats) ? m.MinCatSize : 0;
@@ -2202,100 +2336,48 @@ void THipEvaluator::CalcHostRows(const float* const* rows, size_t rowLen, bool f
         FillBiasOnly(m.HostBias, docCount * outDim, results);
         return;
     }
-    const size_t chunk = PipelineDocs(needFloats, needCats);
+    HIP_CHECK(hipSetDevice(m.DeviceId));
+    TImpl::TContextLease ctx(m);
+    const size_t chunk = PipelineDocs((needFloats + needCats) * 4);
     const size_t stageDocs = std::min(chunk, docCount);
-    const bool twoSlots = docCount > chunk;
-    TPinnedVec<float>* pinnedFloats[2] = {&m.PinnedFloats, &m.PinnedFloats2};
-    TPinnedVec<int32_t>* pinnedCats[2] = {&m.PinnedCats, &m.PinnedCats2};
-    TPinnedVec<double>* pinnedResults[2] = {&m.PinnedResults, &m.PinnedResults2};
-    TDeviceVec<float>* stageFloats[2] = {&m.StageFloats, &m.StageFloats2};
-    TDeviceVec<int32_t>* stageCats[2] = {&m.StageCats, &m.StageCats2};
-    TDeviceVec<double>* stageResults[2] = {&m.StageResults, &m.StageResults2};
-    for (int slot = 0; slot < (twoSlots ? 2 : 1); ++slot) {
-        pinnedFloats[slot]->Reserve(std::max<size_t>(1, stageDocs * needFloats));
-        stageFloats[slot]->Reserve(std::max<size_t>(1, stageDocs * needFloats));
+    for (int i = 0; i < (docCount > chunk ? 2 : 1); ++i) {
+        TImpl::THostSlot& slot = ctx->Slots[i];
+        slot.PinnedFloats.Reserve(std::max<size_t>(1, stageDocs * needFloats));
+        slot.StageFloats.Reserve(std::max<size_t>(1, stageDocs * needFloats));
         if (needCats) {
-            pinnedCats[slot]->Reserve(stageDocs * needCats);
-            stageCats[slot]->Reserve(stageDocs * needCats);
+            slot.PinnedCats.Reserve(stageDocs * needCats);
+            slot.StageCats.Reserve(stageDocs * needCats);
         }
-        pinnedResults[slot]->Reserve(std::max<size_t>(1, stageDocs * m.Dim));
-        // raw values, and behind them room for a prediction type that cannot be computed in place
-        stageResults[slot]->Reserve(std::max<size_t>(1, stageDocs * (m.Dim + 1)));
+        slot.PinnedResults.Reserve(std::max<size_t>(1, stageDocs * m.Dim));
+        slot.StageResults.Reserve(std::max<size_t>(1, stageDocs * (m.Dim + 1)));
     }
-    m.ScratchBins.Reserve(QuantizedBytes(stageDocs));
-    LastTimes = TKernelTimes();
-    // takes the results of the chunk that went through `slot` and adds its kernel times
-    const auto collect = [&](int slot, size_t begin, size_t n) {
-        HIP_CHECK(hipEventSynchronize(m.SlotEv[slot][3]));
-        std::memcpy(results + begin * outDim, pinnedResults[slot]->Get(), n * outDim * sizeof(double));
-        float a = 0.f, b = 0.f;
-        HIP_CHECK(hipEventElapsedTime(&a, m.SlotEv[slot][0], m.SlotEv[slot][1]));
-        HIP_CHECK(hipEventElapsedTime(&b, m.SlotEv[slot][1], m.SlotEv[slot][2]));
-        LastTimes.BinarizeMs += a;
-        LastTimes.EvalMs += b;
-    };
-    size_t pendingBegin[2] = {0, 0}, pendingDocs[2] = {0, 0};
-    size_t index = 0;
-    for (size_t begin = 0; begin < docCount; begin += chunk, ++index) {
-        const int slot = static_cast<int>(index & 1);
-        const size_t n = std::min(chunk, docCount - begin);
-        if (pendingDocs[slot]) {  // the slot's previous chunk must be out before its buffers are reused
-            collect(slot, pendingBegin[slot], pendingDocs[slot]);
-            pendingDocs[slot] = 0;
-        }
-        if (needFloats) {
-            GatherRows(rows + begin, n, needFloats, pinnedFloats[slot]->Get());
-            HIP_CHECK(hipMemcpyAsync(stageFloats[slot]->Get(), pinnedFloats[slot]->Get(), n * needFloats * sizeof(float),
-                                     hipMemcpyHostToDevice, s));
-        }
-        if (needCats) {
-            GatherRows(catRows + begin, n, needCats, pinnedCats[slot]->Get());
-            HIP_CHECK(hipMemcpyAsync(stageCats[slot]->Get(), pinnedCats[slot]->Get(), n * needCats * sizeof(int32_t),
-                                     hipMemcpyHostToDevice, s));
-        }
-        TFeatureBatch batch;
-        batch.Layout = flat ? TFeatureBatch::FlatRows : TFeatureBatch::SplitRows;
-        batch.Floats = stageFloats[slot]->Get();
-        batch.Stride = needFloats;
-        batch.Cats = needCats ? stageCats[slot]->Get() : nullptr;
-        batch.CatStride = needCats;
-        HIP_CHECK(hipEventRecord(m.SlotEv[slot][0], s));
-        if (EvalRowsFusedDevice(batch, n, treeStart, treeEnd, stageResults[slot]->Get(), s)) {
-            HIP_CHECK(hipEventRecord(m.SlotEv[slot][1], s));
-        } else {
-            QuantizeDevice(batch, n, m.ScratchBins.Get(), s);
-            HIP_CHECK(hipEventRecord(m.SlotEv[slot][1], s));
-            EvalQuantizedDevice(m.ScratchBins.Get(), n, treeStart, treeEnd, stageResults[slot]->Get(), s);
-        }
-        HIP_CHECK(hipEventRecord(m.SlotEv[slot][2], s));
-        const double* final = stageResults[slot]->Get();
-        if (predictionType != dev::kPredRaw) {
-            double* processed = stageResults[slot]->Get() + (outDim == static_cast<size_t>(m.Dim) ? 0 : stageDocs * m.Dim);
-            ApplyPredictionTypeDevice(predictionType, begin, docCount, n, stageResults[slot]->Get(), processed, s);
-            final = processed;
-        }
-        HIP_CHECK(hipMemcpyAsync(pinnedResults[slot]->Get(), final, n * outDim * sizeof(double), hipMemcpyDeviceToHost, s));
-        HIP_CHECK(hipEventRecord(m.SlotEv[slot][3], s));
-        pendingBegin[slot] = begin;
-        pendingDocs[slot] = n;
-    }
-    // the (up to) two chunks still in flight, older first
-    for (size_t k = 0; k < 2; ++k) {
-        const int slot = static_cast<int>((index + k) & 1);
-        if (pendingDocs[slot]) {
-            collect(slot, pendingBegin[slot], pendingDocs[slot]);
-            pendingDocs[slot] = 0;
-        }
-    }
+    ctx->ScratchBins.Reserve(QuantizedBytes(stageDocs));
+    TKernelTimes times;
+    hipEvent_t done[2] = {ctx->Slots[0].Ev[3], ctx->Slots[1].Ev[3]};
+    RunPipeline(
+        docCount, chunk, done,
+        [&](int i, size_t begin, size_t n) {
+            const TFeatureBatch batch = StageRowChunk(ctx->Slots[i], ctx->Stream, rows, catRows, begin, n, needFloats, needCats, flat);
+            RunPredictionChunk(*this, *ctx, i, batch, begin, n, docCount, stageDocs, treeStart, treeEnd, predictionType);
+        },
+        [&](int i, size_t begin, size_t n) {
+            TImpl::THostSlot& slot = ctx->Slots[i];
+            std::memcpy(results + begin * outDim, slot.PinnedResults.Get(), n * outDim * sizeof(double));
+            float a = 0.f, b = 0.f;
+            HIP_CHECK(hipEventElapsedTime(&a, slot.Ev[0], slot.Ev[1]));
+            HIP_CHECK(hipEventElapsedTime(&b, slot.Ev[1], slot.Ev[2]));
+            times.BinarizeMs += a;
+            times.EvalMs += b;
+        });
+    SetLastTimes(times);
 }
 
+// Columns by pointer (CalcModelPredictionFlatTransposed): a chunk is staged as a dense [feature][document]
+// matrix, the columns copied by a few threads, and goes through the same two-slot pipeline.
 void THipEvaluator::CalcHostColumns(const float* const* columns, size_t columnCount, size_t docCount, size_t treeStart,
                                     size_t treeEnd, double* results, int predictionType) {
-    std::lock_guard<std::mutex> guard(Lock);
     TImpl& m = *Impl;
     const size_t outDim = predictionType == dev::kPredClass ? 1 : static_cast<size_t>(m.Dim);
-    HIP_CHECK(hipSetDevice(m.DeviceId));
-    hipStream_t s = m.Stream;
     const size_t need = m.FlatVectorSize;
     CBAMD_ENSURE(columnCount >= need, "Not enough features provided");
     CBAMD_ENSURE(need == 0 || columns != nullptr, "Not enough features provided");
@@ -2303,60 +2385,59 @@ void THipEvaluator::CalcHostColumns(const float* const* columns, size_t columnCo
         FillBiasOnly(m.HostBias, docCount * outDim, results);
         return;
     }
-    const size_t chunk = ChunkDocs(need, 0);
+    HIP_CHECK(hipSetDevice(m.DeviceId));
+    TImpl::TContextLease ctx(m);
+    const size_t chunk = PipelineDocs(need * 4);
     const size_t stageDocs = std::min(chunk, docCount);
-    m.PinnedFloats.Reserve(std::max<size_t>(1, stageDocs * need));
-    m.StageFloats.Reserve(std::max<size_t>(1, stageDocs * need));
-    m.PinnedResults.Reserve(std::max<size_t>(1, stageDocs * m.Dim));
-    m.StageResults.Reserve(std::max<size_t>(1, stageDocs * (m.Dim + 1)));
-    m.ScratchBins.Reserve(QuantizedBytes(stageDocs));
-    LastTimes = TKernelTimes();
-    for (size_t begin = 0; begin < docCount; begin += chunk) {
-        const size_t n = std::min(chunk, docCount - begin);
-        float* dst = m.PinnedFloats.Get();
-        for (size_t f = 0; f < need; ++f) {
-            if (columns[f] != nullptr) {
-                std::memcpy(dst + f * n, columns[f] + begin, n * sizeof(float));
-            } else {
-                std::memset(dst + f * n, 0, n * sizeof(float));
-            }
-        }
-        if (need) {
-            HIP_CHECK(hipMemcpyAsync(m.StageFloats.Get(), dst, n * need * sizeof(float), hipMemcpyHostToDevice, s));
-        }
-        TFeatureBatch batch;
-        batch.Layout = TFeatureBatch::FlatColumns;
-        batch.Floats = m.StageFloats.Get();
-        batch.Stride = n;
-        HIP_CHECK(hipEventRecord(m.Ev[0], s));
-        QuantizeDevice(batch, n, m.ScratchBins.Get(), s);
-        HIP_CHECK(hipEventRecord(m.Ev[1], s));
-        EvalQuantizedDevice(m.ScratchBins.Get(), n, treeStart, treeEnd, m.StageResults.Get(), s);
-        HIP_CHECK(hipEventRecord(m.Ev[2], s));
-        const double* final = m.StageResults.Get();
-        if (predictionType != dev::kPredRaw) {
-            double* processed = m.StageResults.Get() + (outDim == static_cast<size_t>(m.Dim) ? 0 : stageDocs * m.Dim);
-            ApplyPredictionTypeDevice(predictionType, begin, docCount, n, m.StageResults.Get(), processed, s);
-            final = processed;
-        }
-        HIP_CHECK(hipMemcpyAsync(m.PinnedResults.Get(), final, n * outDim * sizeof(double), hipMemcpyDeviceToHost, s));
-        HIP_CHECK(hipStreamSynchronize(s));
-        std::memcpy(results + begin * outDim, m.PinnedResults.Get(), n * outDim * sizeof(double));
-        float a = 0.f, b = 0.f;
-        HIP_CHECK(hipEventElapsedTime(&a, m.Ev[0], m.Ev[1]));
-        HIP_CHECK(hipEventElapsedTime(&b, m.Ev[1], m.Ev[2]));
-        LastTimes.BinarizeMs += a;
-        LastTimes.EvalMs += b;
+    for (int i = 0; i < (docCount > chunk ? 2 : 1); ++i) {
+        TImpl::THostSlot& slot = ctx->Slots[i];
+        slot.PinnedFloats.Reserve(std::max<size_t>(1, stageDocs * need));
+        slot.StageFloats.Reserve(std::max<size_t>(1, stageDocs * need));
+        slot.PinnedResults.Reserve(std::max<size_t>(1, stageDocs * m.Dim));
+        slot.StageResults.Reserve(std::max<size_t>(1, stageDocs * (m.Dim + 1)));
     }
+    ctx->ScratchBins.Reserve(QuantizedBytes(stageDocs));
+    TKernelTimes times;
+    hipEvent_t done[2] = {ctx->Slots[0].Ev[3], ctx->Slots[1].Ev[3]};
+    RunPipeline(
+        docCount, chunk, done,
+        [&](int i, size_t begin, size_t n) {
+            TImpl::THostSlot& slot = ctx->Slots[i];
+            float* dst = slot.PinnedFloats.Get();
+            ParallelCopy(need, need * n * sizeof(float), [=](size_t first, size_t last) {
+                for (size_t f = first; f < last; ++f) {
+                    if (columns[f] != nullptr) {
+                        std::memcpy(dst + f * n, columns[f] + begin, n * sizeof(float));
+                    } else {
+                        std::memset(dst + f * n, 0, n * sizeof(float));
+                    }
+                }
+            });
+            if (need) {
+                HIP_CHECK(hipMemcpyAsync(slot.StageFloats.Get(), dst, n * need * sizeof(float), hipMemcpyHostToDevice, ctx->Stream));
+            }
+            TFeatureBatch batch;
+            batch.Layout = TFeatureBatch::FlatColumns;
+            batch.Floats = slot.StageFloats.Get();
+            batch.Stride = n;
+            RunPredictionChunk(*this, *ctx, i, batch, begin, n, docCount, stageDocs, treeStart, treeEnd, predictionType);
+        },
+        [&](int i, size_t begin, size_t n) {
+            TImpl::THostSlot& slot = ctx->Slots[i];
+            std::memcpy(results + begin * outDim, slot.PinnedResults.Get(), n * outDim * sizeof(double));
+            float a = 0.f, b = 0.f;
+            HIP_CHECK(hipEventElapsedTime(&a, slot.Ev[0], slot.Ev[1]));
+            HIP_CHECK(hipEventElapsedTime(&b, slot.Ev[1], slot.Ev[2]));
+            times.BinarizeMs += a;
+            times.EvalMs += b;
+        });
+    SetLastTimes(times);
 }
 
 void THipEvaluator::LeafIndexesHostRows(const float* const* rows, size_t rowLen, bool flat,
                                         const int32_t* const* catRows, size_t catRowLen, size_t docCount,
                                         size_t treeStart, size_t treeEnd, uint32_t* indexes) {
-    std::lock_guard<std::mutex> guard(Lock);
     TImpl& m = *Impl;
-    HIP_CHECK(hipSetDevice(m.DeviceId));
-    hipStream_t s = m.Stream;
     CBAMD_ENSURE(treeStart <= treeEnd && treeEnd <= TreeCount, "tree range is out of bounds");
     const size_t treeCount = treeEnd - treeStart;
     const size_t needFloats = flat ? m.FlatVectorSize : m.MinFloatSize;
@@ -2366,56 +2447,46 @@ void THipEvaluator::LeafIndexesHostRows(const float* const* rows, size_t rowLen,
                                            " expected: " + std::to_string(needFloats));
     CBAMD_ENSURE(needCats == 0 || catRows != nullptr, "Model has categorical features but no categorical features provided");
     CBAMD_ENSURE(catRowLen >= needCats, "insufficient cat features vector size");
-    size_t chunk = ChunkDocs(needFloats + treeCount, needCats);
+    if (docCount == 0 || treeCount == 0) {
+        return;
+    }
+    HIP_CHECK(hipSetDevice(m.DeviceId));
+    TImpl::TContextLease ctx(m);
+    const size_t chunk = PipelineDocs((needFloats + needCats + treeCount) * 4);
     const size_t stageDocs = std::min(chunk, docCount);
-    m.PinnedFloats.Reserve(std::max<size_t>(1, stageDocs * needFloats));
-    m.StageFloats.Reserve(std::max<size_t>(1, stageDocs * needFloats));
-    if (needCats) {
-        m.PinnedCats.Reserve(stageDocs * needCats);
-        m.StageCats.Reserve(stageDocs * needCats);
-    }
-    m.PinnedIndexes.Reserve(std::max<size_t>(1, stageDocs * treeCount));
-    m.StageIndexes.Reserve(std::max<size_t>(1, stageDocs * treeCount));
-    m.ScratchBins.Reserve(QuantizedBytes(stageDocs));
-    for (size_t begin = 0; begin < docCount; begin += chunk) {
-        const size_t n = std::min(chunk, docCount - begin);
-        if (needFloats) {
-            float* dst = m.PinnedFloats.Get();
-            for (size_t d = 0; d < n; ++d) {
-                std::memcpy(dst + d * needFloats, rows[begin + d], needFloats * sizeof(float));
-            }
-            HIP_CHECK(hipMemcpyAsync(m.StageFloats.Get(), dst, n * needFloats * sizeof(float), hipMemcpyHostToDevice, s));
-        }
+    for (int i = 0; i < (docCount > chunk ? 2 : 1); ++i) {
+        TImpl::THostSlot& slot = ctx->Slots[i];
+        slot.PinnedFloats.Reserve(std::max<size_t>(1, stageDocs * needFloats));
+        slot.StageFloats.Reserve(std::max<size_t>(1, stageDocs * needFloats));
         if (needCats) {
-            int32_t* dst = m.PinnedCats.Get();
-            for (size_t d = 0; d < n; ++d) {
-                std::memcpy(dst + d * needCats, catRows[begin + d], needCats * sizeof(int32_t));
-            }
-            HIP_CHECK(hipMemcpyAsync(m.StageCats.Get(), dst, n * needCats * sizeof(int32_t), hipMemcpyHostToDevice, s));
+            slot.PinnedCats.Reserve(stageDocs * needCats);
+            slot.StageCats.Reserve(stageDocs * needCats);
         }
-        TFeatureBatch batch;
-        batch.Layout = flat ? TFeatureBatch::FlatRows : TFeatureBatch::SplitRows;
-        batch.Floats = m.StageFloats.Get();
-        batch.Stride = needFloats;
-        batch.Cats = needCats ? m.StageCats.Get() : nullptr;
-        batch.CatStride = needCats;
-        QuantizeDevice(batch, n, m.ScratchBins.Get(), s);
-        LeafIndexesQuantizedDevice(m.ScratchBins.Get(), n, treeStart, treeEnd, m.StageIndexes.Get(), s);
-        if (treeCount) {
-            HIP_CHECK(hipMemcpyAsync(m.PinnedIndexes.Get(), m.StageIndexes.Get(), n * treeCount * sizeof(uint32_t),
-                                     hipMemcpyDeviceToHost, s));
-        }
-        HIP_CHECK(hipStreamSynchronize(s));
-        std::memcpy(indexes + begin * treeCount, m.PinnedIndexes.Get(), n * treeCount * sizeof(uint32_t));
+        slot.PinnedIndexes.Reserve(stageDocs * treeCount);
+        slot.StageIndexes.Reserve(stageDocs * treeCount);
     }
+    ctx->ScratchBins.Reserve(QuantizedBytes(stageDocs));
+    hipEvent_t done[2] = {ctx->Slots[0].Ev[3], ctx->Slots[1].Ev[3]};
+    RunPipeline(
+        docCount, chunk, done,
+        [&](int i, size_t begin, size_t n) {
+            TImpl::THostSlot& slot = ctx->Slots[i];
+            hipStream_t s = ctx->Stream;
+            const TFeatureBatch batch = StageRowChunk(slot, s, rows, catRows, begin, n, needFloats, needCats, flat);
+            QuantizeDevice(batch, n, ctx->ScratchBins.Get(), s);
+            LeafIndexesQuantizedDevice(ctx->ScratchBins.Get(), n, treeStart, treeEnd, slot.StageIndexes.Get(), s);
+            HIP_CHECK(hipMemcpyAsync(slot.PinnedIndexes.Get(), slot.StageIndexes.Get(), n * treeCount * sizeof(uint32_t),
+                                     hipMemcpyDeviceToHost, s));
+            HIP_CHECK(hipEventRecord(slot.Ev[3], s));
+        },
+        [&](int i, size_t begin, size_t n) {
+            std::memcpy(indexes + begin * treeCount, ctx->Slots[i].PinnedIndexes.Get(), n * treeCount * sizeof(uint32_t));
+        });
 }
 
 void THipEvaluator::QuantizeHostRows(const float* const* rows, size_t rowLen, bool flat, const int32_t* const* catRows,
                                      size_t catRowLen, size_t docCount, uint8_t* referenceLayout) {
-    std::lock_guard<std::mutex> guard(Lock);
     TImpl& m = *Impl;
-    HIP_CHECK(hipSetDevice(m.DeviceId));
-    hipStream_t s = m.Stream;
     const size_t needFloats = flat ? m.FlatVectorSize : m.MinFloatSize;
     const size_t needCats = (!flat && m.HasCats) ? m.MinCatSize : 0;
     CBAMD_ENSURE(needFloats == 0 || rows != nullptr, "Model has float features but no float features provided");
@@ -2426,46 +2497,39 @@ void THipEvaluator::QuantizeHostRows(const float* const* rows, size_t rowLen, bo
     if (docCount == 0 || m.RealBucketCount == 0) {
         return;
     }
-    // chunks must end on a multiple of 128 documents so that reference blocks do not straddle chunks
-    const size_t chunk = ChunkDocs(needFloats + m.RealBucketCount / 4 + 1, needCats);
+    HIP_CHECK(hipSetDevice(m.DeviceId));
+    TImpl::TContextLease ctx(m);
+    // chunks end on a multiple of 256 documents, so that the reference's blocks of 128 do not straddle them
+    const size_t chunk = PipelineDocs((needFloats + needCats) * 4 + m.RealBucketCount);
     const size_t stageDocs = std::min(chunk, docCount);
-    m.PinnedFloats.Reserve(std::max<size_t>(1, stageDocs * needFloats));
-    m.StageFloats.Reserve(std::max<size_t>(1, stageDocs * needFloats));
-    if (needCats) {
-        m.PinnedCats.Reserve(stageDocs * needCats);
-        m.StageCats.Reserve(stageDocs * needCats);
-    }
-    m.PinnedExport.Reserve(stageDocs * m.RealBucketCount);
-    m.StageExport.Reserve(stageDocs * m.RealBucketCount);
-    m.ScratchBins.Reserve(QuantizedBytes(stageDocs));
-    for (size_t begin = 0; begin < docCount; begin += chunk) {
-        const size_t n = std::min(chunk, docCount - begin);
-        if (needFloats) {
-            float* dst = m.PinnedFloats.Get();
-            for (size_t d = 0; d < n; ++d) {
-                std::memcpy(dst + d * needFloats, rows[begin + d], needFloats * sizeof(float));
-            }
-            HIP_CHECK(hipMemcpyAsync(m.StageFloats.Get(), dst, n * needFloats * sizeof(float), hipMemcpyHostToDevice, s));
-        }
+    for (int i = 0; i < (docCount > chunk ? 2 : 1); ++i) {
+        TImpl::THostSlot& slot = ctx->Slots[i];
+        slot.PinnedFloats.Reserve(std::max<size_t>(1, stageDocs * needFloats));
+        slot.StageFloats.Reserve(std::max<size_t>(1, stageDocs * needFloats));
         if (needCats) {
-            int32_t* dst = m.PinnedCats.Get();
-            for (size_t d = 0; d < n; ++d) {
-                std::memcpy(dst + d * needCats, catRows[begin + d], needCats * sizeof(int32_t));
-            }
-            HIP_CHECK(hipMemcpyAsync(m.StageCats.Get(), dst, n * needCats * sizeof(int32_t), hipMemcpyHostToDevice, s));
+            slot.PinnedCats.Reserve(stageDocs * needCats);
+            slot.StageCats.Reserve(stageDocs * needCats);
         }
-        TFeatureBatch batch;
-        batch.Layout = flat ? TFeatureBatch::FlatRows : TFeatureBatch::SplitRows;
-        batch.Floats = m.StageFloats.Get();
-        batch.Stride = needFloats;
-        batch.Cats = needCats ? m.StageCats.Get() : nullptr;
-        batch.CatStride = needCats;
-        QuantizeDevice(batch, n, m.ScratchBins.Get(), s);
-        ExportQuantizedDevice(m.ScratchBins.Get(), n, m.StageExport.Get(), s);
-        HIP_CHECK(hipMemcpyAsync(m.PinnedExport.Get(), m.StageExport.Get(), n * m.RealBucketCount, hipMemcpyDeviceToHost, s));
-        HIP_CHECK(hipStreamSynchronize(s));
-        std::memcpy(referenceLayout + begin * m.RealBucketCount, m.PinnedExport.Get(), n * m.RealBucketCount);
+        slot.PinnedExport.Reserve(stageDocs * m.RealBucketCount);
+        slot.StageExport.Reserve(stageDocs * m.RealBucketCount);
     }
+    ctx->ScratchBins.Reserve(QuantizedBytes(stageDocs));
+    hipEvent_t done[2] = {ctx->Slots[0].Ev[3], ctx->Slots[1].Ev[3]};
+    RunPipeline(
+        docCount, chunk, done,
+        [&](int i, size_t begin, size_t n) {
+            TImpl::THostSlot& slot = ctx->Slots[i];
+            hipStream_t s = ctx->Stream;
+            const TFeatureBatch batch = StageRowChunk(slot, s, rows, catRows, begin, n, needFloats, needCats, flat);
+            QuantizeDevice(batch, n, ctx->ScratchBins.Get(), s);
+            ExportQuantizedDevice(ctx->ScratchBins.Get(), n, slot.StageExport.Get(), s);
+            HIP_CHECK(hipMemcpyAsync(slot.PinnedExport.Get(), slot.StageExport.Get(), n * m.RealBucketCount,
+                                     hipMemcpyDeviceToHost, s));
+            HIP_CHECK(hipEventRecord(slot.Ev[3], s));
+        },
+        [&](int i, size_t begin, size_t n) {
+            std::memcpy(referenceLayout + begin * m.RealBucketCount, ctx->Slots[i].PinnedExport.Get(), n * m.RealBucketCount);
+        });
 }
 
 }  // namespace cbamd

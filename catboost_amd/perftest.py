@@ -8,11 +8,11 @@ it times the evaluator's entry points block by block over a pool).
 
 Without a pool the documents are random: floats around the model's borders, categorical hashes at random.
 A pool is a tab-separated file of flat feature rows (categorical columns as strings). Reports documents
-per second of the flat host entry point (rows by pointer, PCIe both ways) and of the device entry points
+per second of the host entry points (rows by pointer, columns by pointer, leaf indexes; PCIe both ways) and of the device entry points
 on features that already sit in HBM; with --graph also of a block's quantize + evaluate launches captured
 once into a HIP graph and replayed per block (what a serving loop with small blocks does). With
---threads T above 1 the flat host entry point is also timed from T caller threads at once, each with the
-blocks of its share (one model handle: calls from several threads are allowed and run on streams of their own).
+--threads T above 1 the host entry points are also timed from T caller threads at once, each going through
+all blocks (one model handle: calls from several threads are allowed and run on staging contexts of their own).
 """
 import argparse
 import json
@@ -72,38 +72,50 @@ def run(args):
               "block_size": block, "repetitions": args.repetitions}
 
     model.calc_flat(blocks[0])  # binds the model to the device, uploads its tables
-    start = time.perf_counter()
-    for _ in range(args.repetitions):
-        for b in blocks:
-            model.calc_flat(b)
-    seconds = time.perf_counter() - start
-    report["host_flat_docs_per_sec"] = args.repetitions * len(blocks) * block / seconds
+    # the host entry point families: rows by pointer, columns by pointer, leaf indexes of rows by pointer
+    transposed = [np.ascontiguousarray(b.T) for b in blocks]
+    leaf_docs = max(1, min(block, (64 << 20) // max(1, 4 * model.tree_count)))  # bounds the index matrix of a call
+    entry_points = {
+        "host_flat": (lambda i: model.calc_flat(blocks[i]), block),
+        "host_transposed": (lambda i: model.calc_flat_transposed(transposed[i]), block),
+        "host_leaf_indexes": (lambda i: model.calc_leaf_indexes_flat(blocks[i][:leaf_docs]), leaf_docs),
+    }
+    for name, (call, docs_per_call) in entry_points.items():
+        call(0)
+        start = time.perf_counter()
+        for _ in range(args.repetitions):
+            for i in range(len(blocks)):
+                call(i)
+        seconds = time.perf_counter() - start
+        report[name + "_docs_per_sec"] = args.repetitions * len(blocks) * docs_per_call / seconds
 
     if args.threads > 1:
         import threading
 
-        shares = [blocks[t::args.threads] for t in range(args.threads)]
-        failures = []
+        report["threads"] = args.threads
+        for name, (call, docs_per_call) in entry_points.items():
+            # every caller thread goes through all blocks: the calls of one handle run side by side on
+            # staging contexts of their own
+            failures = []
 
-        def caller(share):
-            try:
-                for _ in range(args.repetitions):
-                    for b in share:
-                        model.calc_flat(b)
-            except Exception as e:  # reported by the main thread
-                failures.append(e)
+            def caller():
+                try:
+                    for _ in range(args.repetitions):
+                        for i in range(len(blocks)):
+                            call(i)
+                except Exception as e:  # reported by the main thread
+                    failures.append(e)
 
-        callers = [threading.Thread(target=caller, args=(share,)) for share in shares if share]
-        start = time.perf_counter()
-        for t in callers:
-            t.start()
-        for t in callers:
-            t.join()
-        seconds = time.perf_counter() - start
-        if failures:
-            raise failures[0]
-        report["threads"] = len(callers)
-        report["host_flat_threads_docs_per_sec"] = args.repetitions * len(blocks) * block / seconds
+            callers = [threading.Thread(target=caller) for _ in range(args.threads)]
+            start = time.perf_counter()
+            for t in callers:
+                t.start()
+            for t in callers:
+                t.join()
+            seconds = time.perf_counter() - start
+            if failures:
+                raise failures[0]
+            report[name + "_threads_docs_per_sec"] = args.threads * args.repetitions * len(blocks) * docs_per_call / seconds
 
     ev = model.evaluator()
     device = "cuda:%d" % args.device_id

@@ -916,8 +916,9 @@ def test_workload_configs_device_path(name, docs):
 
 def test_concurrent_callers():
     """Callers on threads of their own: the device entry points with caller-owned buffers and streams run
-    side by side without sharing state; the host entry points of one handle take turns. Every result must
-    equal the single-threaded one."""
+    side by side without sharing state; the host entry points of one handle borrow one of a few staging contexts
+    each (a stream, pinned and device buffers), so flat, transposed and leaf-index calls overlap too, over several
+    pipeline chunks each. Every result must equal the single-threaded one."""
     import threading
 
     import torch
@@ -958,8 +959,27 @@ def test_concurrent_callers():
         except Exception as e:  # noqa: BLE001
             errors.append("host worker %d: %r" % (k, e))
 
+    # larger host batches (several chunks of the staging pipeline), through three entry point families at once
+    big = np.ascontiguousarray(np.tile(host, (12, 1)))
+    big_expected = np.tile(expected_host, 12)
+    columns = np.ascontiguousarray(big.T)
+    leaf_expected = model.calc_leaf_indexes_flat(host[:5000])
+
+    def big_host_worker(k):
+        try:
+            for _ in range(2):
+                if k % 3 == 0 and not np.array_equal(model.calc_flat(big), big_expected):
+                    errors.append("big flat worker %d differs" % k)
+                if k % 3 == 1 and not np.array_equal(model.calc_flat_transposed(columns), big_expected):
+                    errors.append("big transposed worker %d differs" % k)
+                if k % 3 == 2 and not np.array_equal(model.calc_leaf_indexes_flat(host[:5000]), leaf_expected):
+                    errors.append("leaf index worker %d differs" % k)
+        except Exception as e:  # noqa: BLE001
+            errors.append("big host worker %d: %r" % (k, e))
+
     threads = [threading.Thread(target=device_worker, args=(k,)) for k in range(4)]
     threads += [threading.Thread(target=host_worker, args=(k,)) for k in range(4)]
+    threads += [threading.Thread(target=big_host_worker, args=(k,)) for k in range(6)]
     for t in threads:
         t.start()
     for t in threads:
