@@ -42,8 +42,12 @@ Kernel arguments (80 bytes):
   48 scale       double          56 bias const double* (first dimension of this launch)
   64 bucketCount uint32 (1 .. BUCKETS)                68 dim uint32
   72 first dimension of this launch uint32            76 dimensions to store uint32 (1 .. PITCH)
-grid = ceil(blockCount / WAVES) workgroups of WAVES * 64 threads, LDS = 2 * TREE_BLOCK * LEAVES *
-PITCH * 8 bytes.
+  80 tree blocks per slice uint32 (kernels that are not fused; 88 bytes in all)
+grid = (ceil(blockCount / WAVES), slices) workgroups of WAVES * 64 threads, LDS = 2 * TREE_BLOCK * LEAVES *
+PITCH * 8 bytes. Slice y of the grid takes the tree blocks from y * (tree blocks per slice) on, at most that
+many, and writes to out + y * docCount * dim: a small batch is spread over the chip by giving every slice
+of the trees its own workgroups, which store raw sums (flags bit 2) that a second kernel adds up in slice
+order. One slice (grid.y = 1, tree blocks per slice = treeBlocks) is the plain launch.
 
 Fused variants ("cbamd_fused_..."; one-dimensional float-only models, plain and six-bit forms) take the
 documents' fp32 rows instead of bins and binarize them into the bins registers themselves, so the bins
@@ -492,6 +496,8 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
     e("  s_load_dwordx8 s[4:11], s[0:1], 0x0")
     e("  s_load_dwordx8 s[12:19], s[0:1], 0x20")
     e("  s_load_dwordx4 s[96:99], s[0:1], 0x40")
+    if not fused:
+        e("  s_load_dword s101, s[0:1], 0x50")         # tree blocks per slice
     if fused:
         e("  s_load_dwordx4 s[84:87], s[0:1], 0x50")   # floats, unit records
         e("  s_load_dwordx2 s[88:89], s[0:1], 0x60")   # row stride in bytes, units
@@ -516,6 +522,24 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
     e("  s_sub_u32 s28, s100, %d" % group_step(0))
     e("  v_add_u32_e32 v2, s28, v2")
     e("  s_waitcnt lgkmcnt(0)")
+    if not fused:
+        # the slice of the trees that this row of the grid takes (s3: workgroup id y)
+        e("  s_mul_i32 s24, s3, s101")               # its first tree block
+        e("  s_sub_u32 s25, s14, s24")
+        e("  s_min_u32 s14, s25, s101")              # its tree blocks
+        e("  s_mul_i32 s25, s24, %d" % (block * tree_row_bytes))
+        e("  s_add_u32 s6, s6, s25")
+        e("  s_addc_u32 s7, s7, 0")
+        e("  s_mul_hi_u32 s28, s24, %d" % buf_bytes)
+        e("  s_mul_i32 s25, s24, %d" % buf_bytes)
+        e("  s_add_u32 s8, s8, s25")
+        e("  s_addc_u32 s9, s9, s28")
+        e("  s_mul_i32 s25, s12, s97")               # values of one slice: docCount * dim (below 2^29)
+        e("  s_lshl_b32 s25, s25, 3")
+        e("  s_mul_hi_u32 s28, s25, s3")
+        e("  s_mul_i32 s25, s25, s3")
+        e("  s_add_u32 s10, s10, s25")
+        e("  s_addc_u32 s11, s11, s28")
     # first tree block -> buffer 0
     e("  s_mov_b32 s26, s8")
     e("  s_mov_b32 s27, s9")
@@ -681,15 +705,15 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
     e(".amdhsa_kernel %s" % name)
     e("  .amdhsa_group_segment_fixed_size %d" % lds_bytes)
     e("  .amdhsa_private_segment_fixed_size 0")
-    e("  .amdhsa_kernarg_size %d" % (104 if fused else 80))
+    e("  .amdhsa_kernarg_size %d" % (104 if fused else 88))
     e("  .amdhsa_user_sgpr_count 2")
     e("  .amdhsa_user_sgpr_kernarg_segment_ptr 1")
     e("  .amdhsa_system_sgpr_workgroup_id_x 1")
-    e("  .amdhsa_system_sgpr_workgroup_id_y 0")
+    e("  .amdhsa_system_sgpr_workgroup_id_y 1")
     e("  .amdhsa_system_sgpr_workgroup_id_z 0")
     e("  .amdhsa_system_vgpr_workitem_id 0")
     e("  .amdhsa_next_free_vgpr %d" % vgprs)
-    e("  .amdhsa_next_free_sgpr 101")
+    e("  .amdhsa_next_free_sgpr 102")
     e("  .amdhsa_accum_offset %d" % ((vgprs + 3) // 4 * 4))
     e("  .amdhsa_reserve_vcc 1")
     e("  .amdhsa_float_round_mode_32 0")
@@ -734,7 +758,9 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
       - {.address_space: global, .offset: 88, .size: 8, .value_kind: global_buffer}
       - {.offset: 96, .size: 4, .value_kind: by_value}
       - {.offset: 100, .size: 4, .value_kind: by_value}
-""" if fused else "", lds_bytes, 104 if fused else 80, threads, name, name, vgprs)
+""" if fused else """      - {.offset: 80, .size: 4, .value_kind: by_value}
+      - {.offset: 84, .size: 4, .value_kind: by_value}
+""", lds_bytes, 104 if fused else 88, threads, name, name, vgprs)
     return "\n".join(o), meta
 
 

@@ -56,6 +56,14 @@ public:
     void QuantizeDevice(const TFeatureBatch& batch, size_t docCount, uint8_t* bins, void* stream);
     void EvalQuantizedDevice(const uint8_t* bins, size_t docCount, size_t treeStart, size_t treeEnd,
                              double* results, void* stream);
+    // Small batches on the register-resident kernels: the trees are cut into TreeSlicesFor(docCount) slices that
+    // run on workgroups of their own and store raw sums into `partials` (TreeSliceScratchDoubles(docCount)
+    // doubles, the caller's), which a second kernel adds up in slice order. One slice: the plain launch. The
+    // sums of a slice are in tree order; adding the slices' sums rounds differently from one pass over all
+    // trees (within the 1e-9 relative bar, the same for every call).
+    uint32_t TreeSlicesFor(size_t docCount) const;
+    size_t TreeSliceScratchDoubles(size_t docCount) const;
+    void EvalQuantizedSlicedDevice(const uint8_t* bins, size_t docCount, double* results, double* partials, void* stream);
     // binarize + evaluate in one launch of a fused kernel, the bins in registers only; false (and nothing
     // launched) when the model, the batch layout or the tree range has no fused kernel
     bool EvalRowsFusedDevice(const TFeatureBatch& batch, size_t docCount, size_t treeStart, size_t treeEnd,

@@ -131,7 +131,14 @@ struct TEvalRegArgs {
     uint32_t FirstDim;
     uint32_t StoreDims;
 };
-static_assert(sizeof(TEvalRegArgs) == 80, "kernel argument block of the register-resident kernels");
+static_assert(sizeof(TEvalRegArgs) == 80, "kernel argument block shared by the register-resident and the fused kernels");
+
+struct TEvalRegLaunchArgs {
+    TEvalRegArgs Reg;
+    uint32_t TreeBlocksPerSlice;  // grid.y slices of the trees; one slice: all tree blocks
+    uint32_t Padding;
+};
+static_assert(sizeof(TEvalRegLaunchArgs) == 88, "kernel argument block of the register-resident kernels");
 
 struct TEvalRegVariant {
     uint32_t Buckets;
@@ -239,6 +246,7 @@ struct TKernelSwitches {
     bool CtrTile = true;          // CATBOOST_AMD_CTR_TILE=0: the plain CTR kernel instead of the tile kernel
     uint32_t RegMinBuckets = 0;   // CATBOOST_AMD_REG_MIN_BUCKETS=n: only register kernels that hold n buckets or more
     bool Fused = true;            // CATBOOST_AMD_FUSED=0: binarize and evaluate always as two launches
+    bool SmallBatch = true;       // CATBOOST_AMD_SMALL_BATCH=0: small batches are not spread over slices of the trees
     bool LevelOrder = true;       // CATBOOST_AMD_LEVEL_ORDER=0: register kernels keep the model's order of a tree's levels
 
     static TKernelSwitches FromEnvironment() {
@@ -252,6 +260,7 @@ struct TKernelSwitches {
         k.CtrTile = !off("CATBOOST_AMD_CTR_TILE");
         k.Fused = !off("CATBOOST_AMD_FUSED");
         k.LevelOrder = !off("CATBOOST_AMD_LEVEL_ORDER");
+        k.SmallBatch = !off("CATBOOST_AMD_SMALL_BATCH");
         if (const char* v = std::getenv("CATBOOST_AMD_REG_MIN_BUCKETS")) {
             k.RegMinBuckets = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
         }
@@ -775,6 +784,7 @@ struct THipEvaluator::TImpl {
     // register-resident kernels (one-dimensional 7-bit oblivious models of depth <= 8 whose
     // buckets fit the register file): level rows and leaf values at a fixed pitch per tree
     bool RegKernelUsable = false;
+    bool SmallBatchSlices = true;  // small batches: slices of the trees on workgroups of their own
     hipModule_t RegModule = nullptr;
     hipFunction_t RegFunction = nullptr;
     uint32_t RegWaves = 0;
@@ -799,6 +809,7 @@ struct THipEvaluator::TImpl {
     TFused Fused[2];
     hipFunction_t FusedFunction = nullptr;
     uint32_t FusedWaves = 0;
+    size_t FusedMinDocs = 0;
     const char* RegKernelName = "";
     const char* FusedKernelName = "";
 
@@ -822,6 +833,7 @@ struct THipEvaluator::TImpl {
     struct THostContext {
         hipStream_t Stream = nullptr;
         TDeviceVec<uint8_t> ScratchBins;
+        TDeviceVec<double> SlicePartials;  // raw sums per slice of the trees (small batches)
         THostSlot Slots[2];
         hipEvent_t Ev[3] = {nullptr, nullptr, nullptr};
         bool Busy = false;
@@ -1389,6 +1401,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         m.RegLeaves.Upload(leaves);
         m.RegBias.Upload(biasPadded);
         m.RegKernelUsable = true;
+        m.SmallBatchSlices = switches.SmallBatch;
 
         // ---- fused kernels: float-only one-dimensional models in the 7-bit or six-bit form whose rows are
         // at least sixteen columns wide. The bins registers follow the columns of the rows (a unit = sixteen
@@ -1519,6 +1532,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
                 HIP_CHECK(hipModuleGetFunction(&m.FusedFunction, m.RegModule, fused->Name));
                 m.FusedWaves = fused->Waves;
                 m.FusedKernelName = fused->Name;
+                m.FusedMinDocs = switches.SmallBatch ? size_t(1024) * dev::kDocsPerBlock : 0;
             }
             TImpl::TFused& f = m.Fused[layoutIndex];
             f.UnitCount = static_cast<uint32_t>(unitStart.size());
@@ -1548,8 +1562,12 @@ constexpr uint32_t kBinarizeBlocksPerGroup = 8;
 template <int LOG2P, bool CATS_MATRIX>
 void LaunchBinarizeRowsPC(size_t blocks, const float* floats, size_t stride, const int32_t* cats, size_t catStride,
                           size_t docCount, const dev::TBinarizeTables& tab, uint32_t* bins, hipStream_t s) {
-    const size_t groups = (blocks + kBinarizeBlocksPerGroup - 1) / kBinarizeBlocksPerGroup;
     const size_t tiles = (tab.BucketCount + dev::kBucketTile - 1) / dev::kBucketTile;
+    // a workgroup keeps its tile's borders in LDS over up to kBinarizeBlocksPerGroup document blocks; a small
+    // batch gives each fewer blocks, so that there are still about a thousand workgroups
+    const uint32_t blocksPerGroup = static_cast<uint32_t>(
+        std::max<size_t>(1, std::min<size_t>(kBinarizeBlocksPerGroup, blocks * tiles / 1024)));
+    const size_t groups = (blocks + blocksPerGroup - 1) / blocksPerGroup;
     CBAMD_ENSURE(groups * tiles < (size_t(1) << 31), "batch is too large for one binarize launch");
     const dim3 grid(static_cast<uint32_t>(groups * tiles));
     const size_t lds = (static_cast<size_t>(dev::kBucketTile) << LOG2P) * 4 +
@@ -1561,8 +1579,7 @@ void LaunchBinarizeRowsPC(size_t blocks, const float* floats, size_t stride, con
                                       static_cast<int>(lds)));
     }
     hipLaunchKernelGGL(kernel, grid, dim3(256), lds, s, floats, static_cast<uint32_t>(stride), cats,
-                       static_cast<uint32_t>(catStride), static_cast<uint32_t>(docCount), tab, kBinarizeBlocksPerGroup,
-                       bins);
+                       static_cast<uint32_t>(catStride), static_cast<uint32_t>(docCount), tab, blocksPerGroup, bins);
 }
 
 template <int LOG2P>
@@ -1894,7 +1911,8 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
         if (head) {
             generic(tb, wholeBegin, dev::kEvalRaw);
         }
-        TEvalRegArgs args = {};
+        TEvalRegLaunchArgs launchArgs = {};
+        TEvalRegArgs& args = launchArgs.Reg;
         args.Bins = bins;
         args.Rows = m.RegRows.Get() + static_cast<size_t>(wholeBegin) * m.RegRowDwords;
         args.Out = results;
@@ -1905,14 +1923,15 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
         args.Scale = m.Scale;
         args.BucketCount = m.LayoutBuckets;
         args.Dim = static_cast<uint32_t>(m.Dim);
+        launchArgs.TreeBlocksPerSlice = args.TreeBlocks;
         const uint32_t grid = (args.BlockCount + m.RegWaves - 1) / m.RegWaves;
         for (uint32_t first = 0, launch = 0; first < args.Dim; first += m.RegPitch, ++launch) {
             args.Leaves = m.RegLeaves.Get() + launch * m.RegLaunchLeaves + static_cast<size_t>(wholeBegin) * m.RegTreeLeafDoubles;
             args.Bias = m.RegBias.Get() + first;
             args.FirstDim = first;
             args.StoreDims = std::min(m.RegPitch, args.Dim - first);
-            size_t argSize = sizeof(args);
-            void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &argSize,
+            size_t argSize = sizeof(launchArgs);
+            void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &launchArgs, HIP_LAUNCH_PARAM_BUFFER_SIZE, &argSize,
                               HIP_LAUNCH_PARAM_END};
             HIP_CHECK(hipModuleLaunchKernel(m.RegFunction, grid, 1, 1, 64 * m.RegWaves, 1, 1, 0, s, nullptr, config));
         }
@@ -1998,12 +2017,80 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
     HIP_CHECK(hipGetLastError());
 }
 
+uint32_t THipEvaluator::TreeSlicesFor(size_t docCount) const {
+    const TImpl& m = *Impl;
+    if (!m.RegKernelUsable || !m.SmallBatchSlices || docCount == 0) {
+        return 1;
+    }
+    // Workgroups of a plain launch; below one per CU the launch lasts as long as one wave's walk through the
+    // whole model, so the trees are cut into slices with workgroups of their own. A slice is two tree blocks
+    // whatever the batch, so that a document's value does not depend on how many documents came with it
+    // (as long as the batch is small enough to be sliced at all).
+    const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
+    const size_t groups = (blocks + m.RegWaves - 1) / m.RegWaves;
+    if (groups >= 256 || m.RegTreeBlocks < 4) {
+        return 1;
+    }
+    return (m.RegTreeBlocks + 1) / 2;
+}
+
+size_t THipEvaluator::TreeSliceScratchDoubles(size_t docCount) const {
+    const uint32_t slices = TreeSlicesFor(docCount);
+    return slices > 1 ? static_cast<size_t>(slices) * docCount * Impl->Dim : 0;
+}
+
+void THipEvaluator::EvalQuantizedSlicedDevice(const uint8_t* bins, size_t docCount, double* results, double* partials,
+                                              void* stream) {
+    TImpl& m = *Impl;
+    const uint32_t slices = TreeSlicesFor(docCount);
+    if (slices <= 1) {
+        EvalQuantizedDevice(bins, docCount, 0, TreeCount, results, stream);
+        return;
+    }
+    CBAMD_ENSURE(bins != nullptr && results != nullptr && partials != nullptr, "null pointer passed to the sliced evaluation");
+    hipStream_t s = m.Pick(stream);
+    TEvalRegLaunchArgs launchArgs = {};
+    TEvalRegArgs& args = launchArgs.Reg;
+    args.Bins = bins;
+    args.Rows = m.RegRows.Get();
+    args.Out = partials;
+    args.DocCount = static_cast<uint32_t>(docCount);
+    args.BlockCount = static_cast<uint32_t>((docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock);
+    args.TreeBlocks = m.RegTreeBlocks;
+    args.Flags = 4;  // raw sums per slice
+    args.Scale = m.Scale;
+    args.BucketCount = m.LayoutBuckets;
+    args.Dim = static_cast<uint32_t>(m.Dim);
+    launchArgs.TreeBlocksPerSlice = (m.RegTreeBlocks + slices - 1) / slices;
+    const uint32_t usedSlices = (m.RegTreeBlocks + launchArgs.TreeBlocksPerSlice - 1) / launchArgs.TreeBlocksPerSlice;
+    const uint32_t grid = (args.BlockCount + m.RegWaves - 1) / m.RegWaves;
+    for (uint32_t first = 0, launch = 0; first < args.Dim; first += m.RegPitch, ++launch) {
+        args.Leaves = m.RegLeaves.Get() + launch * m.RegLaunchLeaves;
+        args.Bias = m.RegBias.Get() + first;
+        args.FirstDim = first;
+        args.StoreDims = std::min(m.RegPitch, args.Dim - first);
+        size_t argSize = sizeof(launchArgs);
+        void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &launchArgs, HIP_LAUNCH_PARAM_BUFFER_SIZE, &argSize,
+                          HIP_LAUNCH_PARAM_END};
+        HIP_CHECK(hipModuleLaunchKernel(m.RegFunction, grid, usedSlices, 1, 64 * m.RegWaves, 1, 1, 0, s, nullptr, config));
+    }
+    const size_t count = docCount * m.Dim;
+    hipLaunchKernelGGL(dev::CombineSlicesKernel, dim3(static_cast<uint32_t>((count + 255) / 256)), dim3(256), 0, s, partials,
+                       usedSlices, count, m.Scale, m.Bias.Get(), m.Dim, results);
+    HIP_CHECK(hipGetLastError());
+}
+
 bool THipEvaluator::EvalRowsFusedDevice(const TFeatureBatch& batch, size_t docCount, size_t treeStart, size_t treeEnd,
                                         double* results, void* stream) {
     TImpl& m = *Impl;
     const int layoutIndex = batch.Layout == TFeatureBatch::FlatRows ? 0 : batch.Layout == TFeatureBatch::SplitRows ? 1 : -1;
     if (layoutIndex < 0 || !m.Fused[layoutIndex].Usable || docCount == 0 || treeStart != 0 || treeEnd != TreeCount ||
         docCount >= (size_t(1) << 29) || batch.Stride >= (size_t(1) << 20)) {
+        return false;
+    }
+    // Below about one wave per SIMD a fused launch lasts as long as one wave's binarize phase and tree walk,
+    // and two launches (the binarize kernel spreads a block over many waves) are shorter.
+    if (m.FusedMinDocs > 0 && docCount < m.FusedMinDocs) {
         return false;
     }
     const TImpl::TFused& f = m.Fused[layoutIndex];
@@ -2146,9 +2233,17 @@ void THipEvaluator::CalcDevice(const TFeatureBatch& batch, size_t docCount, size
         HIP_CHECK(hipEventElapsedTime(&times.EvalMs, ctx->Ev[0], ctx->Ev[2]));
     } else {
         ctx->ScratchBins.Reserve(QuantizedBytes(docCount));
+        const bool sliced = treeStart == 0 && treeEnd == TreeCount && TreeSlicesFor(docCount) > 1;
+        if (sliced) {
+            ctx->SlicePartials.Reserve(TreeSliceScratchDoubles(docCount));
+        }
         QuantizeDevice(batch, docCount, ctx->ScratchBins.Get(), s);
         HIP_CHECK(hipEventRecord(ctx->Ev[1], s));
-        EvalQuantizedDevice(ctx->ScratchBins.Get(), docCount, treeStart, treeEnd, results, s);
+        if (sliced) {
+            EvalQuantizedSlicedDevice(ctx->ScratchBins.Get(), docCount, results, ctx->SlicePartials.Get(), s);
+        } else {
+            EvalQuantizedDevice(ctx->ScratchBins.Get(), docCount, treeStart, treeEnd, results, s);
+        }
         HIP_CHECK(hipEventRecord(ctx->Ev[2], s));
         HIP_CHECK(hipStreamSynchronize(s));
         HIP_CHECK(hipEventElapsedTime(&times.BinarizeMs, ctx->Ev[0], ctx->Ev[1]));
@@ -2304,7 +2399,12 @@ static void RunPredictionChunk(THipEvaluator& ev, THipEvaluator::TImpl::THostCon
     } else {
         ev.QuantizeDevice(batch, n, ctx.ScratchBins.Get(), s);
         HIP_CHECK(hipEventRecord(slot.Ev[1], s));
-        ev.EvalQuantizedDevice(ctx.ScratchBins.Get(), n, treeStart, treeEnd, slot.StageResults.Get(), s);
+        if (treeStart == 0 && treeEnd == ev.GetTreeCount() && ev.TreeSlicesFor(n) > 1) {
+            ctx.SlicePartials.Reserve(ev.TreeSliceScratchDoubles(n));
+            ev.EvalQuantizedSlicedDevice(ctx.ScratchBins.Get(), n, slot.StageResults.Get(), ctx.SlicePartials.Get(), s);
+        } else {
+            ev.EvalQuantizedDevice(ctx.ScratchBins.Get(), n, treeStart, treeEnd, slot.StageResults.Get(), s);
+        }
     }
     HIP_CHECK(hipEventRecord(slot.Ev[2], s));
     const double* final = slot.StageResults.Get();

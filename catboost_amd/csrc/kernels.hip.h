@@ -666,6 +666,22 @@ __global__ __launch_bounds__(256) void EvalObliviousKernel(const uint32_t* __res
     }
 }
 
+// Small batches on the register-resident kernels: every slice of the trees left its raw sums in
+// partials[slice][count]; adds them in slice order and finishes like ApplyScaleAndBias. One thread per value.
+__global__ __launch_bounds__(256) void CombineSlicesKernel(const double* __restrict__ partials, uint32_t slices,
+                                                           size_t count, double scale, const double* __restrict__ bias,
+                                                           int dim, double* __restrict__ out) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= count) {
+        return;
+    }
+    double sum = partials[i];
+    for (uint32_t s = 1; s < slices; ++s) {
+        sum = __dadd_rn(sum, partials[s * count + i]);
+    }
+    out[i] = Finish(sum, scale, bias[i % static_cast<size_t>(dim)], true);
+}
+
 // Packed tree table of the tile kernel: 16 dwords per tree. Slots 0..7 hold the tree's levels
 // (slot d = split d, unused levels padded with a split that is false for every bin), slot 8 the
 // index of the tree's first leaf value. A level is

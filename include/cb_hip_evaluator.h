@@ -84,6 +84,8 @@ typedef struct CbHipFeatures {
  *   CATBOOST_AMD_REG_KERNEL=0        no register-resident assembly kernels (the LDS tile kernels instead)
  *   CATBOOST_AMD_REG_SIX=0           no six-bit form of the register-resident kernels
  *   CATBOOST_AMD_REG_MIN_BUCKETS=n   only register-resident kernel shapes that hold n buckets or more
+ *   CATBOOST_AMD_SMALL_BATCH=0       no slices of the trees for small batches, fused kernels for every batch size:
+ *                                    every sum then has the CPU evaluator's order of additions
  *   CATBOOST_AMD_LEVEL_ORDER=0       register-resident kernels keep the model's order of a tree's levels
  *   CATBOOST_AMD_FUSED=0             binarize and evaluate always as two launches (no fused kernels)
  *   CATBOOST_AMD_CTR_TILE=0          the plain CTR kernel instead of the LDS tile one */
