@@ -26,7 +26,7 @@ def test_small_batches_through_tree_slices(cfg, trees):
     ev = model.evaluator()
     oracle = OracleModel(read_cbm(model.save_to_buffer()))
     dim = info["dim"]
-    x = syn.device_features(info, 65_536 + 300_000)
+    x = syn.device_features(info, 530_000)  # more than 256 workgroups of eight 256-document blocks
     host = x.cpu().numpy()
     for docs in (1, 256, 4096, 65_536):
         part = x[:docs].contiguous()
