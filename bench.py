@@ -229,7 +229,7 @@ def main():
     kernels_ms = avg_bin + avg_eval
     achieved = step_bytes / (kernels_ms * 1e-3) / 1e9
     buckets = ev.bucket_count
-    kernel_names = ev.describe_kernels(cb.LAYOUT_FLAT_ROWS)
+    kernel_names = ev.describe_kernels(cb.LAYOUT_FLAT_ROWS, docs)
     traffic, traffic_source = measured_traffic(args.config, docs, model.tree_count, kernel_names)
     if "fused" in kernel_names:
         kernels = {"fused": {"name": kernel_names["fused"], "avg_ms": kernels_ms,

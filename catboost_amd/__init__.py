@@ -150,7 +150,7 @@ def load_library():
         "CbHipApplyPredictionTypeDevice": (ctypes.c_bool, [vp, ctypes.c_int, sz, vp, vp, vp]),
         "CbHipSynchronize": (ctypes.c_bool, [vp, vp]),
         "CbHipLastKernelTimes": (ctypes.c_bool, [vp, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float)]),
-        "CbHipDescribeKernels": (ctypes.c_bool, [vp, ctypes.c_int, ctypes.c_char_p, sz]),
+        "CbHipDescribeKernels": (ctypes.c_bool, [vp, ctypes.c_int, sz, ctypes.c_char_p, sz]),
         "CbHipGetEvaluator": (vp, [vp]),
         "CbHipSetFeatureLayout": (ctypes.c_bool, [vp, vp, sz, vp, sz, vp, sz]),
         "CbHipLoadModelFromArrays": (ctypes.c_bool, [vp, ctypes.POINTER(ModelArrays)]),
@@ -389,10 +389,11 @@ class DeviceEvaluator:
     def synchronize(self, stream=None):
         _check(self._lib.CbHipSynchronize(self._h, stream))
 
-    def describe_kernels(self, layout=LAYOUT_FLAT_ROWS):
-        """The kernels of a whole-model call as a dict: {"fused": name} or {"binarize": name, "evaluate": name}."""
+    def describe_kernels(self, layout=LAYOUT_FLAT_ROWS, doc_count=1 << 24):
+        """The kernels of a whole-model eval_data call on doc_count documents as a dict: {"fused": name} or
+        {"binarize": name, "evaluate": name}."""
         buf = ctypes.create_string_buffer(512)
-        _check(self._lib.CbHipDescribeKernels(self._h, int(layout), buf, len(buf)))
+        _check(self._lib.CbHipDescribeKernels(self._h, int(layout), doc_count, buf, len(buf)))
         return dict(item.split("=", 1) for item in buf.value.decode().split(";"))
 
     def last_kernel_times(self):

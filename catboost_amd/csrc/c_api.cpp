@@ -880,10 +880,10 @@ bool CbHipLastKernelTimes(CbHipEvaluatorHandle* evaluator, float* binarizeMs, fl
     });
 }
 
-bool CbHipDescribeKernels(CbHipEvaluatorHandle* evaluator, int layout, char* buffer, size_t bufferSize) {
+bool CbHipDescribeKernels(CbHipEvaluatorHandle* evaluator, int layout, size_t docCount, char* buffer, size_t bufferSize) {
     return Guard([&] {
         CBAMD_ENSURE(buffer != nullptr && bufferSize > 0, "description buffer is null");
-        const std::string text = E(evaluator)->DescribeKernels(layout);
+        const std::string text = E(evaluator)->DescribeKernels(layout, docCount);
         CBAMD_ENSURE(text.size() < bufferSize, "description buffer is too small");
         std::memcpy(buffer, text.c_str(), text.size() + 1);
     });

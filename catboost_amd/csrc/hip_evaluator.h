@@ -88,9 +88,9 @@ public:
                            double* results, void* stream);
     void Synchronize(void* stream);
     TKernelTimes LastKernelTimes() const;
-    // which kernels a whole-model call on a batch of the given layout (TFeatureBatch::ELayout) launches:
-    // "fused=<kernel>" or "binarize=<kernel>;evaluate=<kernel>"
-    std::string DescribeKernels(int layout) const;
+    // which kernels a whole-model call (CalcDevice, the host entry points) on docCount documents of the given
+    // layout (TFeatureBatch::ELayout) launches: "fused=<kernel>" or "binarize=<kernel>;evaluate=<kernel>"
+    std::string DescribeKernels(int layout, size_t docCount) const;
 
     // ---- host-resident data: stage -> binarize -> evaluate -> copy back, in document chunks.
     // rows[doc] points at rowLen floats (FlatRows / SplitRows) or columns[f] at docCount floats.

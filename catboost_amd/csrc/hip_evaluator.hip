@@ -2124,10 +2124,10 @@ bool THipEvaluator::EvalRowsFusedDevice(const TFeatureBatch& batch, size_t docCo
     return true;
 }
 
-std::string THipEvaluator::DescribeKernels(int layout) const {
+std::string THipEvaluator::DescribeKernels(int layout, size_t docCount) const {
     const TImpl& m = *Impl;
     const int fusedIndex = layout == TFeatureBatch::FlatRows ? 0 : layout == TFeatureBatch::SplitRows ? 1 : -1;
-    if (fusedIndex >= 0 && m.Fused[fusedIndex].Usable) {
+    if (fusedIndex >= 0 && m.Fused[fusedIndex].Usable && docCount >= m.FusedMinDocs) {
         return std::string("fused=") + m.FusedKernelName;
     }
     std::string binarize = m.BinarizeBuckets == 0 ? "none"
@@ -2143,6 +2143,10 @@ std::string THipEvaluator::DescribeKernels(int layout) const {
         evaluate = "FillBiasKernel";
     } else if (m.RegKernelUsable) {
         evaluate = m.RegKernelName;
+        const uint32_t slices = TreeSlicesFor(docCount);
+        if (slices > 1) {
+            evaluate += " x " + std::to_string(slices) + " slices of the trees + CombineSlicesKernel";
+        }
     } else if (m.Oblivious && m.MaxDepth <= 8 && TileLdsBytes(m.LayoutBuckets, dchunk) <= kMaxTileLdsBytes) {
         evaluate = "EvalObliviousTileKernel";
     } else if (m.Oblivious && m.MaxDepth <= 8 && m.Dim == 1 && m.HalfTileLeaves.Get() != nullptr &&

@@ -160,10 +160,10 @@ bool CbHipSynchronize(CbHipEvaluatorHandle* evaluator, void* hipStream);
  * host-level prediction call (summed over its chunks). */
 bool CbHipLastKernelTimes(CbHipEvaluatorHandle* evaluator, float* binarizeMs, float* evalMs);
 
-/* Which kernels a whole-model call on a batch of `layout` (ECbHipFeatureLayout) launches, as text:
- * "fused=<kernel>" or "binarize=<kernel>;evaluate=<kernel>". For logs and benchmarks; no counterpart in
- * the reference. */
-bool CbHipDescribeKernels(CbHipEvaluatorHandle* evaluator, int layout, char* buffer, size_t bufferSize);
+/* Which kernels a whole-model CbHipEvalData (or host entry point) call on docCount documents of `layout`
+ * (ECbHipFeatureLayout) launches, as text: "fused=<kernel>" or "binarize=<kernel>;evaluate=<kernel>". For logs
+ * and benchmarks; no counterpart in the reference. */
+bool CbHipDescribeKernels(CbHipEvaluatorHandle* evaluator, int layout, size_t docCount, char* buffer, size_t bufferSize);
 
 /* ---- extensions on a ModelCalcerHandle (c_api.h) ------------------------------------------ */
 
