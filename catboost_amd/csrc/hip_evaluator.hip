@@ -153,6 +153,7 @@ constexpr TEvalRegVariant kEvalRegVariants[] = {
     {96, 8, 1, 256, false, false, "cbamd_eval_reg_b96_w8_p1_l256"},
     {200, 4, 1, 256, false, false, "cbamd_eval_reg_b200_w4_p1_l256"},
     {208, 4, 1, 256, false, false, "cbamd_eval_reg_b208_w4_p1_l256"},
+    {224, 4, 1, 256, false, false, "cbamd_eval_reg_b224_w4_p1_l256"},
     {192, 4, 2, 64, false, false, "cbamd_eval_reg_b192_w4_p2_l64"},
     {160, 4, 4, 64, false, false, "cbamd_eval_reg_b160_w4_p4_l64"},
     {128, 4, 6, 64, false, false, "cbamd_eval_reg_b128_w4_p6_l64"},
@@ -162,6 +163,7 @@ constexpr TEvalRegVariant kEvalRegVariants[] = {
     {96, 8, 1, 256, true, false, "cbamd_eval_reg_b96_w8_p1_l256_m"},
     {200, 4, 1, 256, true, false, "cbamd_eval_reg_b200_w4_p1_l256_m"},
     {208, 4, 1, 256, true, false, "cbamd_eval_reg_b208_w4_p1_l256_m"},
+    {224, 4, 1, 256, true, false, "cbamd_eval_reg_b224_w4_p1_l256_m"},
     {192, 4, 2, 64, true, false, "cbamd_eval_reg_b192_w4_p2_l64_m"},
     {160, 4, 4, 64, true, false, "cbamd_eval_reg_b160_w4_p4_l64_m"},
     {128, 4, 6, 64, true, false, "cbamd_eval_reg_b128_w4_p6_l64_m"},
@@ -171,6 +173,7 @@ constexpr TEvalRegVariant kEvalRegVariants[] = {
     {96, 8, 1, 256, false, true, "cbamd_eval_reg_b96_w8_p1_l256_s"},
     {200, 4, 1, 256, false, true, "cbamd_eval_reg_b200_w4_p1_l256_s"},
     {208, 4, 1, 256, false, true, "cbamd_eval_reg_b208_w4_p1_l256_s"},
+    {224, 4, 1, 256, false, true, "cbamd_eval_reg_b224_w4_p1_l256_s"},
     {192, 4, 2, 64, false, true, "cbamd_eval_reg_b192_w4_p2_l64_s"},
     {160, 4, 4, 64, false, true, "cbamd_eval_reg_b160_w4_p4_l64_s"},
     {128, 4, 6, 64, false, true, "cbamd_eval_reg_b128_w4_p6_l64_s"},

@@ -129,3 +129,36 @@ def test_fused_shallow_trees_and_mixed_depths(monkeypatch):
     model = mb.build_oblivious(feats, [], 1, trees)
     x = rng.normal(size=(3001, columns)).astype(np.float32)
     _compare(_bytes(model), x, monkeypatch)
+
+
+def test_fused_split_rows_layout(monkeypatch):
+    """Separate float rows (the Index positions of the model's features, which need not be their flat positions)
+    take the fused kernel of their own unit tables."""
+    import torch
+
+    rng = np.random.default_rng(21)
+    columns = 150
+    feats = []
+    for f in range(columns):
+        ff = mb.float_feature(f, flat_index=2 * f + 1)  # flat positions differ from the float positions
+        feats.append(ff)
+    trees = []
+    for _ in range(64):
+        splits = [("float", int(rng.integers(0, columns)), float(np.float32(rng.normal()))) for _ in range(8)]
+        trees.append((splits, rng.normal(0, 0.01, size=256)))
+    model_bytes = _bytes(mb.build_oblivious(feats, [], 1, trees))
+    oracle = OracleModel(read_cbm(model_bytes))
+    x = rng.normal(size=(7001, columns)).astype(np.float32)
+    x[rng.random(x.shape) < 0.03] = np.nan
+    (fm, fev), (tm, tev) = _evaluators(model_bytes, monkeypatch)
+    dx = torch.from_numpy(x).to("cuda:0")
+    a = torch.zeros(x.shape[0], dtype=torch.float64, device="cuda:0")
+    b = torch.zeros_like(a)
+    torch.cuda.synchronize()
+    fev.eval_data(fev.features(cb.LAYOUT_SPLIT_ROWS, dx.data_ptr(), columns), x.shape[0], a.data_ptr())
+    tev.eval_data(tev.features(cb.LAYOUT_SPLIT_ROWS, dx.data_ptr(), columns), x.shape[0], b.data_ptr())
+    torch.cuda.synchronize()
+    assert fev.last_kernel_times()[0] == 0.0 and tev.last_kernel_times()[0] > 0.0
+    assert torch.equal(a, b)
+    np.testing.assert_array_equal(a.cpu().numpy(), oracle.calc(x, layout="split", threads=8))
+    np.testing.assert_array_equal(fm.calc_hashed(x, np.zeros((x.shape[0], 0), np.int32)), a.cpu().numpy())

@@ -760,15 +760,16 @@ def _float_only_model(rng, n_float, trees, max_depth, scale=1.0, bias=None, dim=
 
 
 # Models of this kind (one-dimensional, float features with < 128 borders, depth <= 8, at most
-# 208 buckets) run on the register-resident kernels, which add leaf values in tree order like the
-# CPU evaluator: their predictions are compared bit for bit. 209 buckets fall back to the LDS tile
-# kernel (sums per wave, then across waves), which only meets the tolerance. Models whose features all
+# 224 buckets) run on the register-resident kernels (97 to 208 buckets: on the fused kernel), which add leaf
+# values in tree order like the CPU evaluator: their predictions are compared bit for bit. 225 buckets fall back
+# to the LDS tile kernel (sums per wave, then across waves), which only meets the tolerance. Models whose features all
 # have fewer than 64 borders take the six-bit form of these kernels (two levels share a merge); the
 # switch sends them through the 7-bit form as well.
 @pytest.mark.parametrize("six", ["1", "0"])
 @pytest.mark.parametrize("n_float,trees,max_depth,docs", [
     (1, 1, 1, 1), (1, 1, 8, 255), (3, 15, 8, 256), (5, 16, 8, 257), (7, 17, 6, 2049), (20, 33, 8, 1000),
-    (96, 40, 8, 3000), (97, 40, 8, 3000), (208, 70, 8, 5000), (209, 70, 8, 1500), (50, 200, 4, 70001),
+    (96, 40, 8, 3000), (97, 40, 8, 3000), (208, 70, 8, 5000), (209, 70, 8, 1500), (224, 70, 8, 2000),
+    (225, 70, 8, 1500), (50, 200, 4, 70001),
 ])
 def test_register_kernel_shapes(monkeypatch, n_float, trees, max_depth, docs, six):
     monkeypatch.setenv("CATBOOST_AMD_REG_SIX", six)
@@ -780,12 +781,12 @@ def test_register_kernel_shapes(monkeypatch, n_float, trees, max_depth, docs, si
     g = _gpu_model(model)
     expected = o.calc(x)
     got = g.calc_flat(x)
-    if n_float <= 208:
+    if n_float <= 224:
         np.testing.assert_array_equal(got, expected)
     else:
         _close(got, expected)
     np.testing.assert_array_equal(g.quantize_flat(x), o.binarize(x))
-    # a tree sub-range goes through the tile kernel
+    # a tree sub-range
     if len(model["tree_sizes"]) >= 3:
         _close(g.calc_flat(x, tree_start=1, tree_end=len(model["tree_sizes"]) - 1),
                o.calc(x, tree_start=1, tree_end=len(model["tree_sizes"]) - 1))
@@ -1163,6 +1164,43 @@ def test_tree_ranges_stay_on_the_register_kernels_and_equal_the_oracle(cfg, tree
         np.testing.assert_array_equal(out.cpu().numpy(), expected, err_msg="trees [%d, %d)" % (begin, end))
     np.testing.assert_array_equal(model.calc_flat(host[:700], tree_start=19, tree_end=trees - 20),
                                   oracle.calc(host[:700], tree_start=19, tree_end=trees - 20))
+
+
+def test_c5_full_size_properties():
+    """C5 at its full 10M documents (41 GB of features): a sample of the outputs against the oracle, the same
+    documents at other positions of the batch give the same bits, and tree ranges add up to the whole model."""
+    import torch
+
+    model, info = syn.build_model("C5")
+    ev = model.evaluator()
+    oracle = OracleModel(read_cbm(model.save_to_buffer()))
+    docs = info["docs"]
+    x = syn.device_features(info, docs)
+    out = torch.zeros(docs, dtype=torch.float64, device="cuda:0")
+    feats = ev.features(cb.LAYOUT_FLAT_ROWS, x.data_ptr(), x.shape[1])
+    torch.cuda.synchronize()
+    ev.eval_data(feats, docs, out.data_ptr())
+    torch.cuda.synchronize()
+    sample = torch.randperm(docs, device="cuda:0")[:3000].sort().values
+    _close(out[sample].cpu().numpy(), oracle.calc(x[sample].cpu().numpy(), threads=8))
+    # position independence: the last 70 001 documents moved to the front of a smaller batch
+    tail = 70_001
+    moved = x[docs - tail:].contiguous()
+    out_moved = torch.zeros(tail, dtype=torch.float64, device="cuda:0")
+    torch.cuda.synchronize()
+    ev.eval_data(ev.features(cb.LAYOUT_FLAT_ROWS, moved.data_ptr(), moved.shape[1]), tail, out_moved.data_ptr())
+    torch.cuda.synchronize()
+    assert torch.equal(out_moved, out[docs - tail:])
+    # additivity over tree ranges on a slice of the batch (scale 1, bias 0 in this workload)
+    part_docs = 200_000
+    total = torch.zeros(part_docs, dtype=torch.float64, device="cuda:0")
+    part = torch.zeros(part_docs, dtype=torch.float64, device="cuda:0")
+    for begin, end in ((0, 1700), (1700, 1701), (1701, model.tree_count)):
+        torch.cuda.synchronize()
+        ev.eval_data(feats, part_docs, part.data_ptr(), tree_start=begin, tree_end=end)
+        torch.cuda.synchronize()
+        total += part
+    assert torch.allclose(total, out[:part_docs], rtol=RTOL, atol=ATOL)
 
 
 @pytest.mark.parametrize("name,base_docs,copies", [("C2", 1_000_000, 23), ("C4", 1_000_000, 15), ("C3", 500_000, 110)])
