@@ -91,6 +91,31 @@ private:
     size_t Cap = 0;
 };
 
+// A kernel that uses more than 64 KB of dynamic LDS has to be told so once (per device); the largest size asked
+// for so far is remembered, so that the attribute is not set again on every launch.
+void EnsureDynamicLds(const void* kernel, size_t bytes) {
+    if (bytes <= 64 * 1024) {
+        return;
+    }
+    static std::mutex lock;
+    static std::vector<std::pair<std::pair<int, const void*>, size_t>> granted;
+    int device = 0;
+    HIP_CHECK(hipGetDevice(&device));
+    std::lock_guard<std::mutex> guard(lock);
+    for (auto& item : granted) {
+        if (item.first.first == device && item.first.second == kernel) {
+            if (item.second >= bytes) {
+                return;
+            }
+            HIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)));
+            item.second = bytes;
+            return;
+        }
+    }
+    HIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)));
+    granted.push_back({{device, kernel}, bytes});
+}
+
 // Address of `scratch` on a device, asked for once per device, with that device current.
 uint8_t* NoAllocScratchOfCurrentDevice(int deviceId) {
     static std::mutex lock;
@@ -1577,10 +1602,7 @@ void LaunchBinarizeRowsPC(size_t blocks, const float* floats, size_t stride, con
                        static_cast<size_t>(dev::kBucketTile) * dev::kLutCells +
                        static_cast<size_t>(dev::kBucketTile) * dev::kTilePitch * 4;
     auto kernel = dev::BinarizeRowsKernel<LOG2P, CATS_MATRIX>;
-    if (lds > 64 * 1024) {
-        HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      static_cast<int>(lds)));
-    }
+    EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds);
     hipLaunchKernelGGL(kernel, grid, dim3(256), lds, s, floats, static_cast<uint32_t>(stride), cats,
                        static_cast<uint32_t>(catStride), static_cast<uint32_t>(docCount), tab, blocksPerGroup, bins);
 }
@@ -1742,10 +1764,7 @@ void LaunchEvalTileW(const TTileArgs& a) {
     const size_t blocks = (a.DocCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
     const size_t lds = TileLdsBytes(a.Buckets, DCHUNK) + (LEAF_LDS ? TileLeafLdsBytes(MAXD, DCHUNK, WAVES) : 0);
     auto kernel = dev::EvalObliviousTileKernel<SEVEN_BIT, MAXD, DCHUNK, LEAF_LDS, WAVES>;
-    if (lds > 64 * 1024) {
-        HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      static_cast<int>(lds)));
-    }
+    EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds);
     hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(blocks)), dim3(64 * WAVES), lds, a.Stream,
                        reinterpret_cast<const uint32_t*>(a.Bins), a.DocCount, a.Buckets, a.PackedTrees, a.Leaves, a.Bias,
                        a.Scale, a.Dim, a.TreeBegin, a.TreeEnd, a.Out);
@@ -1805,10 +1824,7 @@ void LaunchEvalNonSymmetricTileX(const uint8_t* bins, size_t docCount, uint32_t 
     const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
     const size_t lds = TileLdsBytes(buckets, DCHUNK);
     auto kernel = dev::EvalNonSymmetricTileKernel<NO_XOR, DCHUNK>;
-    if (lds > 64 * 1024) {
-        HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      static_cast<int>(lds)));
-    }
+    EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds);
     hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(blocks)), dim3(64 * dev::kTileWaves), lds, s,
                        reinterpret_cast<const uint32_t*>(bins), docCount, buckets, entries, rows, leaves, bias, scale, dim,
                        treeBegin, treeEnd, out);
@@ -1964,10 +1980,7 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
         const int maxd = m.MaxDepth <= 6 ? 6 : 8;
         const size_t lds = HalfTileLdsBytes(m.LayoutBuckets, maxd);
         const auto launch = [&](auto kernel) {
-            if (lds > 64 * 1024) {
-                HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-            }
+            EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds);
             hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(2 * blocks)), dim3(64 * dev::kTileWaves), lds, s,
                                reinterpret_cast<const uint16_t*>(bins), docCount, m.LayoutBuckets, m.PackedMixed.Get(),
                                m.HalfTileLeaves.Get(), m.Bias.Get(), m.Scale, tb, te, results);
@@ -1984,10 +1997,7 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
         TileLdsBytes(m.LayoutBuckets, 1) + dev::kTileWaves * dev::kNsLdsEntries * 4 <= kMaxTileLdsBytes) {
         const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
         const size_t lds = TileLdsBytes(m.LayoutBuckets, 1) + dev::kTileWaves * dev::kNsLdsEntries * 4;
-        if (lds > 64 * 1024) {
-            HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(dev::EvalNonSymmetricLdsKernel),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-        }
+        EnsureDynamicLds(reinterpret_cast<const void*>(dev::EvalNonSymmetricLdsKernel), lds);
         hipLaunchKernelGGL(dev::EvalNonSymmetricLdsKernel, dim3(static_cast<uint32_t>(blocks)), dim3(64 * dev::kTileWaves),
                            lds, s, reinterpret_cast<const uint32_t*>(bins), docCount, m.LayoutBuckets,
                            m.NsCompactEntries.Get(), reinterpret_cast<const uint4*>(m.NsCompactRows.Get()),

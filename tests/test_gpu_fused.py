@@ -105,7 +105,7 @@ def test_fused_sparse_columns_clustered_borders_and_nan_as_true(monkeypatch):
             return np.concatenate([c + rng.normal(0, 1e-3, size=rng.integers(3, 12)) for c in centers])
         return rng.normal(0, 1, size=rng.integers(1, 50))
 
-    model = _random_model(rng, columns, used, trees=90, depth=8, borders_of=borders_of, nan_true=set(used[::4]))
+    model = _random_model(rng, columns, used, trees=420, depth=8, borders_of=borders_of, nan_true=set(used[::4]))
     x = rng.normal(0, 2, size=(6000, columns)).astype(np.float32)
     for f in used:
         b = np.asarray(model["float_features"][f]["borders"], np.float32)
