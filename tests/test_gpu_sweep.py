@@ -43,12 +43,12 @@ def _check(tag, g, o, x):
 
 def _tree_model_case(seed, rng, asymmetric):
     dim = int(rng.choice([1, 1, 1, 2, 3, 5, 10, 20]))
-    n_float = int(rng.choice([1, 2, 7, 30, 100, 209, 250]))
+    n_float = int(rng.choice([1, 2, 7, 30, 100, 130, 200, 209, 224, 250]))
     n_cat = int(rng.choice([0, 0, 1, 2, 5]))
     trees = int(rng.choice([1, 2, 17, 40, 150, 400]))
     max_depth = int(rng.choice([1, 3, 6, 8, 10]))
     many = bool(rng.integers(0, 2))
-    docs = int(rng.choice([1, 2, 63, 64, 65, 255, 256, 257, 1000, 3333]))
+    docs = int(rng.choice([1, 2, 63, 64, 65, 255, 256, 257, 1000, 3333, 9000]))
     trees = min(trees, max(1, 40000 // n_float))
     tag = "seed %d dim %d floats %d cats %d trees %d depth<=%d many borders %s docs %d non-symmetric %s" % (
         seed, dim, n_float, n_cat, trees, max_depth, many, docs, asymmetric)
@@ -93,6 +93,10 @@ def test_random_model_shapes(monkeypatch, capsys):
         rng = np.random.default_rng(seed)
         kind = seed % 3
         monkeypatch.setenv("CATBOOST_AMD_REG_SIX", str(int(rng.integers(0, 2))))
+        # fused or two launches, a tree's levels ordered or as in the model, small batches sliced or in one pass
+        monkeypatch.setenv("CATBOOST_AMD_FUSED", str(int(rng.integers(0, 2))))
+        monkeypatch.setenv("CATBOOST_AMD_LEVEL_ORDER", str(int(rng.integers(0, 2))))
+        monkeypatch.setenv("CATBOOST_AMD_SMALL_BATCH", str(int(rng.integers(0, 2))))
         if kind == 2:
             _ctr_model_case(seed, rng, monkeypatch)
         else:
