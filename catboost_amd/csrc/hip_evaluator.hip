@@ -274,6 +274,7 @@ struct TKernelSwitches {
     bool Fused = true;            // CATBOOST_AMD_FUSED=0: binarize and evaluate always as two launches
     bool SmallBatch = true;       // CATBOOST_AMD_SMALL_BATCH=0: small batches are not spread over slices of the trees
     bool LevelOrder = true;       // CATBOOST_AMD_LEVEL_ORDER=0: register kernels keep the model's order of a tree's levels
+    bool PairTile = true;         // CATBOOST_AMD_PAIR_TILE=0: the half-tile kernel with one tree per wave
 
     static TKernelSwitches FromEnvironment() {
         const auto off = [](const char* name) {
@@ -287,6 +288,7 @@ struct TKernelSwitches {
         k.Fused = !off("CATBOOST_AMD_FUSED");
         k.LevelOrder = !off("CATBOOST_AMD_LEVEL_ORDER");
         k.SmallBatch = !off("CATBOOST_AMD_SMALL_BATCH");
+        k.PairTile = !off("CATBOOST_AMD_PAIR_TILE");
         if (const char* v = std::getenv("CATBOOST_AMD_REG_MIN_BUCKETS")) {
             k.RegMinBuckets = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
         }
@@ -361,6 +363,13 @@ constexpr size_t kMaxTileLdsBytes = 160 * 1024;
 size_t TileLdsBytes(uint32_t buckets, int dchunk) {
     return ((static_cast<size_t>(buckets) * dev::kDocsPerBlock + 7) & ~size_t(7)) +
            static_cast<size_t>(dev::kDocsPerBlock) * dchunk * sizeof(double);
+}
+
+// LDS of the pair-tile kernel: 128 documents' bins, then per wave the leaf values of two trees; the same area
+// takes one partial sum per wave, lane group and document at the end
+size_t PairTileLdsBytes(uint32_t buckets, int maxd) {
+    return ((static_cast<size_t>(buckets) * 128 + 15) & ~size_t(15)) +
+           static_cast<size_t>(dev::kTileWaves) * 2 * std::max<size_t>(size_t(1) << maxd, 128) * sizeof(double);
 }
 
 // dimensions the tile kernel accumulates per pass over the trees (and the pitch of its padded leaf rows)
@@ -789,6 +798,7 @@ struct THipEvaluator::TImpl {
     TDeviceVec<uint32_t> PackedTrees;  // tile kernel: 16 dwords per oblivious tree of depth <= 8
     TDeviceVec<uint32_t> PackedMixed;  // half-tile kernel: packed rows in the form chosen per tree
     TDeviceVec<double> HalfTileLeaves; // half-tile kernel: 64 or 256 leaf values per tree at a fixed pitch
+    TDeviceVec<uint32_t> PairRows;     // pair-tile kernel: 16 dwords per tree, empty when the model does not qualify
     TDeviceVec<double> LeavesPadded;   // tile kernel, multi-dimensional: [tree][chunk][leaf][TileChunk(dim)]
     bool PackedSevenBit = false;
     bool LeavesPairAligned = false;  // every tree's first leaf value sits at an even index
@@ -1264,12 +1274,41 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
             m.PackedMixed.Upload(mixed);
             if (TileLdsBytes(m.LayoutBuckets, 1) > kMaxTileLdsBytes) {
                 const size_t pitch = m.MaxDepth <= 6 ? 64 : 256;
-                std::vector<double> fixed(trees.GetTreeCount() * pitch, 0.0);
+                // zeros at the end: the pair-tile kernel fetches ahead of its trees without a bound
+                std::vector<double> fixed((trees.GetTreeCount() + dev::kPairTreePadding) * pitch, 0.0);
                 for (size_t t = 0; t < trees.GetTreeCount(); ++t) {
                     std::copy_n(trees.LeafValues.begin() + trees.TreeFirstLeafOffsets[t], size_t(1) << trees.TreeSizes[t],
                                 fixed.begin() + t * pitch);
                 }
                 m.HalfTileLeaves.Upload(fixed);
+                // two trees per wave: every bin of the model below 128 (the one-hot test then fits 7 bits too)
+                uint32_t maxValues = 0;
+                for (size_t b = 0; b + 1 < offsets.size(); ++b) {
+                    maxValues = std::max(maxValues, offsets[b + 1] - offsets[b]);
+                }
+                if (switches.PairTile && maxValues <= 127 && PairTileLdsBytes(m.LayoutBuckets, 8) <= kMaxTileLdsBytes) {
+                    std::vector<uint32_t> pairRows((trees.GetTreeCount() + dev::kPairTreePadding) * dev::kPackedTreeDwords, 0);
+                    for (size_t t = 0; t < trees.GetTreeCount(); ++t) {
+                        uint32_t* row = pairRows.data() + t * dev::kPackedTreeDwords;
+                        bool anyXor = false;
+                        for (int d = 0; d < trees.TreeSizes[t]; ++d) {
+                            const auto& rb = trees.RepackedBins[trees.TreeStartOffsets[t] + d];
+                            row[d] = static_cast<uint32_t>(rb.FeatureIndex) * 128u;
+                            if (rb.XorMask != 0 || rb.SplitIdx == 0xff) {
+                                // one-hot: bin == value, value = ~XorMask; 7 bits of it are enough below 128
+                                row[d] |= (static_cast<uint32_t>(rb.XorMask) & 0x7fu) << 24;
+                                row[8 + d] = 0x01010101u;
+                                anyXor = true;
+                            } else {
+                                row[8 + d] = (128u - rb.SplitIdx) * 0x01010101u;
+                            }
+                        }
+                        if (anyXor) {
+                            row[0] |= dev::kPairRowXorFlag;
+                        }
+                    }
+                    m.PairRows.Upload(pairRows);
+                }
             }
         }
         m.LeavesPairAligned = true;
@@ -1978,6 +2017,24 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
         // the bins of a block exceed the 256-document tile: half blocks
         const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
         const int maxd = m.MaxDepth <= 6 ? 6 : 8;
+        if (m.PairRows.Get() != nullptr) {
+            const size_t lds = PairTileLdsBytes(m.LayoutBuckets, maxd);
+            const auto launch = [&](auto kernel) {
+                EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds);
+                hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(2 * blocks)), dim3(64 * dev::kTileWaves), lds, s,
+                                   reinterpret_cast<const uint16_t*>(bins), docCount, m.LayoutBuckets,
+                                   reinterpret_cast<const uint4*>(m.PairRows.Get()),
+                                   reinterpret_cast<const double2*>(m.HalfTileLeaves.Get()), m.Bias.Get(), m.Scale, tb, te,
+                                   results);
+            };
+            if (maxd == 6) {
+                launch(dev::EvalObliviousPairTileKernel<6>);
+            } else {
+                launch(dev::EvalObliviousPairTileKernel<8>);
+            }
+            HIP_CHECK(hipGetLastError());
+            return;
+        }
         const size_t lds = HalfTileLdsBytes(m.LayoutBuckets, maxd);
         const auto launch = [&](auto kernel) {
             EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds);
@@ -2164,7 +2221,7 @@ std::string THipEvaluator::DescribeKernels(int layout, size_t docCount) const {
         evaluate = "EvalObliviousTileKernel";
     } else if (m.Oblivious && m.MaxDepth <= 8 && m.Dim == 1 && m.HalfTileLeaves.Get() != nullptr &&
                TileLdsBytes(m.LayoutBuckets, 1) > kMaxTileLdsBytes) {
-        evaluate = "EvalObliviousHalfTileKernel";
+        evaluate = m.PairRows.Get() != nullptr ? "EvalObliviousPairTileKernel" : "EvalObliviousHalfTileKernel";
     } else if (m.Oblivious) {
         evaluate = "EvalObliviousKernel";
     } else if (m.NsLdsUsable &&

@@ -1068,6 +1068,209 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousHalfTileKernel(
     }
 }
 
+// The same half tile with two trees in flight per wave: lanes 0..31 evaluate one tree and lanes 32..63 the
+// next one, each lane for four documents of the tile (one LDS dword: the bins of documents
+// (2 * half + j) * 64 + 2 * m + i, byte 2 * i + j, for lane m of either group), so a level costs one LDS read
+// and one byte-parallel compare for 2 x 128 (tree, document) pairs instead of 128. Needs every bin of the
+// model below 128 (the 7-bit compare; a one-hot level xors first: (bin ^ (~value & 0x7f)) + 1 carries into
+// bit 7 exactly when bin == value).
+// `pairRows` holds 16 dwords per tree: slot d = byte offset of level d's bucket in the tile (bucket * 128)
+// | xor byte << 24, slot 0 also bit 23 when some level of the tree xors; slot 8 + d = the value added to all
+// four bytes. Levels past the tree's depth are zero (bucket 0, add 0: never true). A lane keeps its tree's
+// row in registers (four 16-byte loads, the same addresses for the 32 lanes of a group) and the wave
+// publishes the two trees' leaf values, which are contiguous in `leaves` (1 << MAXD doubles per tree), in its
+// own LDS region. Waves take the pairs round robin; a last tree without a partner is done by wave 0 with both
+// groups on the same tree and only the first one adding. Partial sums (one per wave and group) are added in a
+// fixed order at the end. The fetches run kPairAhead rounds ahead of the walk without looking at the tree range:
+// both tables end with kPairTreePadding trees' worth of zeros.
+// grid = 2 * doc blocks, block = 64 * kTileWaves threads, dynamic LDS = buckets * 128 (rounded up to 16) +
+// kTileWaves * 2 * max(1 << MAXD, 128) * 8 bytes (the leaf regions, later the partial sums).
+constexpr uint32_t kPairRowXorFlag = 1u << 23;  // slot 0 of a tree's row: some level xors
+constexpr int kPairAhead = 3;
+constexpr int kPairTreePadding = 2 * kTileWaves * kPairAhead;
+
+template <bool XOR, int MAXD>
+__device__ __forceinline__ uint32_t PairTreeIndexes(const uint8_t* laneTile, const uint4 (&desc)[4]) {
+    const uint32_t offs[8] = {desc[0].x, desc[0].y, desc[0].z, desc[0].w, desc[1].x, desc[1].y, desc[1].z, desc[1].w};
+    const uint32_t adds[8] = {desc[2].x, desc[2].y, desc[2].z, desc[2].w, desc[3].x, desc[3].y, desc[3].z, desc[3].w};
+    uint32_t idx4 = 0;
+#pragma unroll
+    for (int d = 0; d < MAXD; ++d) {
+        // rows of trees that never xor hold the plain offset
+        uint32_t a = *reinterpret_cast<const uint32_t*>(laneTile + (XOR ? offs[d] & 0x007fffffu : offs[d]));
+        if (XOR) {
+            a ^= __builtin_amdgcn_perm(offs[d], offs[d], 0x03030303u);  // the xor byte four times
+        }
+        // the level's four result bits go to bit 7 of the bytes; earlier levels move down one bit and never
+        // reach the byte below within eight levels
+        idx4 = ((a + adds[d]) & 0x80808080u) | (idx4 >> 1);
+    }
+    return idx4;
+}
+
+template <int MAXD>
+__global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousPairTileKernel(
+    const uint16_t* __restrict__ bins, size_t docCount, uint32_t bucketCount, const uint4* __restrict__ pairRows,
+    const double2* __restrict__ leaves2, const double* __restrict__ bias, double scale, uint32_t treeBegin,
+    uint32_t treeEnd, double* __restrict__ out) {
+    constexpr uint32_t kLeaves = 1u << MAXD;
+    constexpr int kLeafRegs = MAXD == 8 ? 4 : 1;  // 16-byte pieces of a pair's 2 * kLeaves leaf values per lane
+    static_assert(MAXD == 8 || MAXD == 6, "64 or 256 leaves per tree");
+    extern __shared__ uint32_t sTile[];
+    uint16_t* sTile16 = reinterpret_cast<uint16_t*>(sTile);
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const size_t block = blockIdx.x >> 1;
+    const uint32_t half = blockIdx.x & 1;
+    const uint32_t tileWords = bucketCount * kWave;
+    const uint16_t* src = bins + block * tileWords * 2 + half;
+    for (uint32_t i = tid; i < tileWords; i += 64 * kTileWaves) {
+        sTile16[i] = src[2 * i];
+    }
+    const uint32_t group = lane >> 5;
+    const uint32_t tileBytes = (tileWords * 2 + 15) & ~15u;
+    double* leafArea = reinterpret_cast<double*>(reinterpret_cast<uint8_t*>(sTile) + tileBytes);
+    double2* sLeafWave2 = reinterpret_cast<double2*>(leafArea + wave * 2 * kLeaves);
+    const double* sLeafMine = leafArea + wave * 2 * kLeaves + group * kLeaves;
+    const uint8_t* laneTile = reinterpret_cast<const uint8_t*>(sTile) + (lane & 31) * 4;
+    __syncthreads();  // tile is loaded
+
+    const uint32_t treeCount = treeEnd - treeBegin;
+    const uint32_t pairCount = treeCount / 2;
+    double acc[4] = {0.0, 0.0, 0.0, 0.0};
+    constexpr int kAhead = kPairAhead;
+    uint4 rows[kAhead][4];
+    double2 pref[kAhead][kLeafRegs];
+    // what a lane fetches of the pair that starts at tree `first`: its group's row and its pieces of the
+    // two trees' leaf values
+    const uint4* myRows = pairRows + group * 4;
+    const double2* myLeaves = leaves2 + lane;
+#define CBAMD_FETCH_PAIR(k, first)                                                                 \
+    do {                                                                                           \
+        const uint4* row = myRows + static_cast<size_t>(first) * 4;                                \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                            \
+            rows[k][i] = row[i];                                                                   \
+        }                                                                                          \
+        const double2* values = myLeaves + static_cast<size_t>(first) * (kLeaves / 2);             \
+        _Pragma("unroll") for (int i = 0; i < kLeafRegs; ++i) {                                    \
+            pref[k][i] = values[i * kWave];                                                        \
+        }                                                                                          \
+    } while (0)
+    // the pair's leaf values into the wave's LDS region (the previous pair's gathers were issued before these
+    // stores and LDS serves one wave's requests in order), then the levels: four leaf indexes per lane
+#define CBAMD_PUBLISH_AND_WALK(k, idx4)                                                            \
+    do {                                                                                           \
+        _Pragma("unroll") for (int i = 0; i < kLeafRegs; ++i) {                                    \
+            sLeafWave2[i * kWave + lane] = pref[k][i];                                             \
+        }                                                                                          \
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                                     \
+        __builtin_amdgcn_wave_barrier();                                                           \
+        const uint32_t flags =                                                                     \
+            __builtin_amdgcn_readlane(rows[k][0].x, 0) | __builtin_amdgcn_readlane(rows[k][0].x, 32); \
+        if (flags & kPairRowXorFlag) {                                                             \
+            idx4 = PairTreeIndexes<true, MAXD>(laneTile, rows[k]);                                 \
+        } else {                                                                                   \
+            idx4 = PairTreeIndexes<false, MAXD>(laneTile, rows[k]);                                \
+        }                                                                                          \
+    } while (0)
+
+    // One round of a wave: the leaf values that the previous round gathered are added while this round's LDS
+    // reads are under way; the registers of this pair take the pair kAhead rounds ahead as soon as every level
+    // has read them (the loads then land in those registers), and the gathers go out last.
+    double gathered[4] = {0.0, 0.0, 0.0, 0.0};
+#define CBAMD_PAIR_ROUND(k)                                                                        \
+    do {                                                                                           \
+        uint32_t idx4;                                                                             \
+        CBAMD_PUBLISH_AND_WALK(k, idx4);                                                           \
+        _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                            \
+            acc[q] = __dadd_rn(acc[q], gathered[q]);                                               \
+        }                                                                                          \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+        CBAMD_FETCH_PAIR(k, treeBegin + 2 * (p + kAhead * kTileWaves));                            \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+        _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                            \
+            gathered[q] = sLeafMine[(idx4 >> (8 * q + 8 - MAXD)) & (kLeaves - 1)];                 \
+        }                                                                                          \
+        __builtin_amdgcn_wave_barrier();                                                           \
+        p += kTileWaves;                                                                           \
+    } while (0)
+
+    uint32_t p = wave;
+#pragma unroll
+    for (int k = 0; k < kAhead; ++k) {
+        // (written before the loads so that the arrays stay in registers)
+#pragma unroll
+        for (int i = 0; i < kLeafRegs; ++i) {
+            pref[k][i] = {0.0, 0.0};
+        }
+        CBAMD_FETCH_PAIR(k, treeBegin + 2 * (p + k * kTileWaves));
+    }
+    static_assert(kAhead == 3, "the rounds below are written out for three register sets");
+    // whole turns of the three register sets without a branch between the rounds, so that the waits for
+    // the loads count only the loads that are older than the one needed
+    while (p + 2 * kTileWaves < pairCount) {
+        CBAMD_PAIR_ROUND(0);
+        CBAMD_PAIR_ROUND(1);
+        CBAMD_PAIR_ROUND(2);
+    }
+    if (p < pairCount) {
+        CBAMD_PAIR_ROUND(0);
+        if (p < pairCount) {
+            CBAMD_PAIR_ROUND(1);
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        acc[q] = __dadd_rn(acc[q], gathered[q]);
+    }
+    if ((treeCount & 1) && wave == 0) {
+        // the last tree has no partner: both groups walk it (its row and its leaf values twice), the first adds
+        const uint4* row = pairRows + static_cast<size_t>(treeEnd - 1) * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            rows[0][i] = row[i];
+        }
+        const double2* values = leaves2 + static_cast<size_t>(treeEnd - 1) * (kLeaves / 2);
+#pragma unroll
+        for (int i = 0; i < kLeafRegs; ++i) {
+            pref[0][i] = values[(i * kWave + lane) & (kLeaves / 2 - 1)];
+        }
+        uint32_t idx4;
+        CBAMD_PUBLISH_AND_WALK(0, idx4);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const double v = sLeafMine[(idx4 >> (8 * q + 8 - MAXD)) & (kLeaves - 1)];
+            acc[q] = __dadd_rn(acc[q], group == 0 ? v : 0.0);
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+#undef CBAMD_PAIR_ROUND
+#undef CBAMD_FETCH_PAIR
+#undef CBAMD_PUBLISH_AND_WALK
+    __syncthreads();  // every wave is through with its leaf region: the area now takes the partial sums
+    // partial sums as [wave][group][document of the tile], then one thread per document adds the sixteen
+    double* sRed = leafArea;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        // byte q of a lane's dword: document (q & 1) * 64 + 2 * (lane & 31) + (q >> 1) of the tile
+        const uint32_t docInTile = (q & 1) * kWave + 2 * (lane & 31) + (q >> 1);
+        sRed[(wave * 2 + group) * 128 + docInTile] = acc[q];
+    }
+    __syncthreads();
+    if (tid < 128) {
+        double sum = sRed[tid];
+#pragma unroll
+        for (int part = 1; part < 2 * kTileWaves; ++part) {
+            sum = __dadd_rn(sum, sRed[part * 128 + tid]);
+        }
+        const size_t doc = block * kDocsPerBlock + (2 * half + (tid >> 6)) * kWave + (tid & 63);
+        if (doc < docCount) {
+            out[doc] = Finish(sum, scale, bias[0], treeBegin == 0);
+        }
+    }
+}
+
 __device__ __forceinline__ uint32_t BinOfDoc(const uint8_t* bins, size_t doc, uint32_t bucketCount, uint32_t bucket) {
     const size_t block = doc / kDocsPerBlock;
     const uint32_t r = static_cast<uint32_t>(doc % kDocsPerBlock);

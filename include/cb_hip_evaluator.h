@@ -88,6 +88,8 @@ typedef struct CbHipFeatures {
  *                                    every sum then has the CPU evaluator's order of additions
  *   CATBOOST_AMD_LEVEL_ORDER=0       register-resident kernels keep the model's order of a tree's levels
  *   CATBOOST_AMD_FUSED=0             binarize and evaluate always as two launches (no fused kernels)
+ *   CATBOOST_AMD_PAIR_TILE=0         wide one-dimensional models (more buckets than an LDS tile of 256 documents
+ *                                    holds): one tree per wave instead of two
  *   CATBOOST_AMD_CTR_TILE=0          the plain CTR kernel instead of the LDS tile one */
 
 /* Model upload: validates the tables, derives buckets / repacked splits / leaf offsets and

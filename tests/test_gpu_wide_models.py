@@ -1,0 +1,76 @@
+"""One-dimensional oblivious models with more buckets than an LDS tile of 256 documents holds (above ~630):
+the half-tile kernels, one tree or two trees per wave, against the oracle through the C ABI.
+
+The two kernels add the trees of a document in different orders (partial sums per wave, and per lane group
+in the two-tree kernel), so predictions are compared within 1e-9 rel / 1e-12 abs; the bins must be equal.
+"""
+import numpy as np
+import pytest
+
+import catboost_amd as cb
+from oracle.oracle import OracleModel
+from tests.test_oracle import _random_flat_data, _random_oblivious
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-9, 1e-12
+
+
+def _evaluator(model, monkeypatch, pair):
+    monkeypatch.setenv("CATBOOST_AMD_PAIR_TILE", pair)
+    g = cb.ModelCalcer()
+    g.load_from_dict(model)
+    g.enable_gpu_evaluation(0)
+    return g
+
+
+@pytest.mark.parametrize("pair", ["1", "0"])
+@pytest.mark.parametrize("seed,n_float,n_cat,trees,max_depth,docs", [
+    (1, 900, 0, 601, 8, 1000),    # odd tree count: the last tree has no partner
+    (2, 900, 12, 600, 8, 129),    # one-hot levels: the xor form, in some pairs only
+    (3, 800, 40, 450, 6, 1),      # 64 leaves per tree, a single document
+    (4, 1000, 3, 1400, 3, 5000),  # shallow trees in the 64-leaf kernel
+])
+def test_wide_models_against_the_oracle(monkeypatch, pair, seed, n_float, n_cat, trees, max_depth, docs):
+    rng = np.random.default_rng(seed)
+    model, cat_values = _random_oblivious(rng, n_float=n_float, n_cat=n_cat, trees=trees, max_depth=max_depth,
+                                          scale=float(rng.choice([1.0, -0.5])), bias=rng.normal(size=1))
+    x = _random_flat_data(rng, model, cat_values, docs)
+    o = OracleModel(model)
+    g = _evaluator(model, monkeypatch, pair)
+    assert g.bucket_count > 632, "the model must not fit the 256-document tile"
+    kernels = g.evaluator().describe_kernels(cb.LAYOUT_FLAT_ROWS, docs)
+    assert kernels["evaluate"] == ("EvalObliviousPairTileKernel" if pair == "1" else "EvalObliviousHalfTileKernel")
+    np.testing.assert_array_equal(g.quantize_flat(x), o.binarize(x))
+    np.testing.assert_allclose(g.calc_flat(x), o.calc(x), rtol=RTOL, atol=ATOL)
+    # tree ranges of odd and even lengths, from even and odd first trees, down to one pair, one tree and none;
+    # the bias only with tree 0
+    for begin, end in ((0, 1), (1, 2), (0, 2), (7, 9), (0, trees - 1), (1, trees), (3, 3), (trees // 2, trees),
+                       (5, 8), (trees - 1, trees)):
+        if end <= trees and begin <= end:
+            np.testing.assert_allclose(g.calc_flat(x, tree_start=begin, tree_end=end),
+                                       o.calc(x, tree_start=begin, tree_end=end), rtol=RTOL, atol=ATOL,
+                                       err_msg="trees %d..%d" % (begin, end))
+
+
+def test_bins_above_127_keep_the_one_tree_kernel(monkeypatch):
+    """A feature with 300 borders: the byte-parallel compare of the two-tree kernel needs 7-bit bins, so the
+    model stays with the kernel that compares 8 bits in the trees that need it."""
+    rng = np.random.default_rng(11)
+    model, cat_values = _random_oblivious(rng, n_float=800, n_cat=4, trees=500, max_depth=8, many_borders=True)
+    x = _random_flat_data(rng, model, cat_values, 700)
+    g = _evaluator(model, monkeypatch, "1")
+    assert g.evaluator().describe_kernels(cb.LAYOUT_FLAT_ROWS, 700)["evaluate"] == "EvalObliviousHalfTileKernel"
+    np.testing.assert_allclose(g.calc_flat(x), OracleModel(model).calc(x), rtol=RTOL, atol=ATOL)
+
+
+def test_two_kernels_agree_on_a_large_batch(monkeypatch):
+    """66 000 documents (a ragged last block) through both kernels of one model."""
+    rng = np.random.default_rng(12)
+    model, cat_values = _random_oblivious(rng, n_float=950, n_cat=8, trees=301, max_depth=8)
+    x = _random_flat_data(rng, model, cat_values, 66_000)
+    two = _evaluator(model, monkeypatch, "1").calc_flat(x)
+    one = _evaluator(model, monkeypatch, "0").calc_flat(x)
+    np.testing.assert_allclose(two, one, rtol=RTOL, atol=ATOL)
+    sample = np.random.default_rng(0).choice(66_000, size=2000, replace=False)
+    np.testing.assert_allclose(two[sample], OracleModel(model).calc(x[sample]), rtol=RTOL, atol=ATOL)
