@@ -275,6 +275,7 @@ struct TKernelSwitches {
     bool SmallBatch = true;       // CATBOOST_AMD_SMALL_BATCH=0: small batches are not spread over slices of the trees
     bool LevelOrder = true;       // CATBOOST_AMD_LEVEL_ORDER=0: register kernels keep the model's order of a tree's levels
     bool PairTile = true;         // CATBOOST_AMD_PAIR_TILE=0: the half-tile kernel with one tree per wave
+    uint32_t NsWaves = 0;         // CATBOOST_AMD_NS_WAVES=8|12|16: that shape of the non-symmetric LDS kernel or none
 
     static TKernelSwitches FromEnvironment() {
         const auto off = [](const char* name) {
@@ -289,6 +290,9 @@ struct TKernelSwitches {
         k.LevelOrder = !off("CATBOOST_AMD_LEVEL_ORDER");
         k.SmallBatch = !off("CATBOOST_AMD_SMALL_BATCH");
         k.PairTile = !off("CATBOOST_AMD_PAIR_TILE");
+        if (const char* v = std::getenv("CATBOOST_AMD_NS_WAVES")) {
+            k.NsWaves = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
+        }
         if (const char* v = std::getenv("CATBOOST_AMD_REG_MIN_BUCKETS")) {
             k.RegMinBuckets = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
         }
@@ -364,6 +368,20 @@ size_t TileLdsBytes(uint32_t buckets, int dchunk) {
     return ((static_cast<size_t>(buckets) * dev::kDocsPerBlock + 7) & ~size_t(7)) +
            static_cast<size_t>(dev::kDocsPerBlock) * dchunk * sizeof(double);
 }
+
+// LDS of EvalNonSymmetricLdsKernel: the tile and the accumulator, then the waves' entry regions at a multiple
+// of their size
+size_t NsLdsKernelBytes(uint32_t buckets, uint32_t waves, uint32_t entries) {
+    const size_t region = static_cast<size_t>(entries) * 4;
+    return (TileLdsBytes(buckets, 1) + region - 1) / region * region + waves * region;
+}
+
+// The shapes of EvalNonSymmetricLdsKernel, most waves first
+struct TNsLdsShape {
+    uint32_t Waves;
+    uint32_t Entries;
+};
+constexpr TNsLdsShape kNsLdsShapes[] = {{16, 1024}, {12, 1536}, {8, 2048}};
 
 // LDS of the pair-tile kernel: 128 documents' bins, then per wave the leaf values of two trees; the same area
 // takes one partial sum per wave, lane group and document at the end
@@ -815,6 +833,7 @@ struct THipEvaluator::TImpl {
     TDeviceVec<uint32_t> NsCompactEntries;
     TDeviceVec<uint32_t> NsCompactRows;  // 8 dwords per unit of trees
     uint32_t NsUnitCount = 0;
+    TNsLdsShape NsLdsShape{0, 0};    // waves and entries per region of EvalNonSymmetricLdsKernel for this model
     TDeviceVec<double> NsValuesByEntry;
 
     // register-resident kernels (one-dimensional 7-bit oblivious models of depth <= 8 whose
@@ -1323,14 +1342,34 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         BuildLevelOrderTrees(trees, m.Dim, firstLeaf, &m.NsEntries, &m.NsRows, &m.NsTileUsable, &m.NsNoXor,
                              &compactEntries, &compactRows, &valuesByEntry, &m.NsLdsUsable);
         if (m.NsLdsUsable) {
-            // units: consecutive trees, at most kNsUnitTrees of them and kNsLdsEntries entries
+            // the shape with the most waves whose regions hold the largest tree and that fits the LDS
+            uint32_t largestTree = 0;
+            for (size_t t = 0; t < TreeCount; ++t) {
+                largestTree = std::max(largestTree, compactRows[t * 4 + 2]);
+            }
+            m.NsLdsUsable = false;
+            for (const TNsLdsShape& shape : kNsLdsShapes) {
+                if (largestTree <= shape.Entries && (switches.NsWaves == 0 || switches.NsWaves == shape.Waves) &&
+                    NsLdsKernelBytes(m.LayoutBuckets, shape.Waves, shape.Entries) <= kMaxTileLdsBytes) {
+                    m.NsLdsShape = shape;
+                    m.NsLdsUsable = true;
+                    break;
+                }
+            }
+        }
+        if (m.NsLdsUsable) {
+            // units: consecutive trees, at most kNsUnitTrees of them and as many entries as a region holds
             std::vector<uint32_t> units;
             for (size_t t = 0; t < TreeCount;) {
                 const uint32_t first = compactRows[t * 4];
                 uint32_t height = 0, count = 0, n = 0;
                 uint32_t start[dev::kNsUnitTrees] = {};
                 while (t < TreeCount && n < static_cast<uint32_t>(dev::kNsUnitTrees) &&
-                       count + compactRows[t * 4 + 2] <= static_cast<uint32_t>(dev::kNsLdsEntries)) {
+                       count + compactRows[t * 4 + 2] <= m.NsLdsShape.Entries) {
+                    // child indexes (bits 21-31) count from the unit's first entry
+                    for (uint32_t e = 0; e < compactRows[t * 4 + 2]; ++e) {
+                        compactEntries[first + count + e] += count << 21;
+                    }
                     start[n++] = count;
                     height = std::max(height, compactRows[t * 4 + 1]);
                     count += compactRows[t * 4 + 2];
@@ -2050,15 +2089,23 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
         HIP_CHECK(hipGetLastError());
         return;
     }
-    if (!m.Oblivious && m.NsLdsUsable && treeStart == 0 && treeEnd == TreeCount &&
-        TileLdsBytes(m.LayoutBuckets, 1) + dev::kTileWaves * dev::kNsLdsEntries * 4 <= kMaxTileLdsBytes) {
+    if (!m.Oblivious && m.NsLdsUsable && treeStart == 0 && treeEnd == TreeCount) {
         const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
-        const size_t lds = TileLdsBytes(m.LayoutBuckets, 1) + dev::kTileWaves * dev::kNsLdsEntries * 4;
-        EnsureDynamicLds(reinterpret_cast<const void*>(dev::EvalNonSymmetricLdsKernel), lds);
-        hipLaunchKernelGGL(dev::EvalNonSymmetricLdsKernel, dim3(static_cast<uint32_t>(blocks)), dim3(64 * dev::kTileWaves),
-                           lds, s, reinterpret_cast<const uint32_t*>(bins), docCount, m.LayoutBuckets,
-                           m.NsCompactEntries.Get(), reinterpret_cast<const uint4*>(m.NsCompactRows.Get()),
-                           m.NsUnitCount, m.NsValuesByEntry.Get(), m.Bias.Get(), m.Scale, results);
+        const size_t lds = NsLdsKernelBytes(m.LayoutBuckets, m.NsLdsShape.Waves, m.NsLdsShape.Entries);
+        const auto launch = [&](auto kernel) {
+            EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds);
+            hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(blocks)), dim3(64 * m.NsLdsShape.Waves), lds, s,
+                               reinterpret_cast<const uint32_t*>(bins), docCount, m.LayoutBuckets,
+                               m.NsCompactEntries.Get(), reinterpret_cast<const uint4*>(m.NsCompactRows.Get()),
+                               m.NsUnitCount, m.NsValuesByEntry.Get(), m.Bias.Get(), m.Scale, results);
+        };
+        if (m.NsLdsShape.Waves == 16) {
+            launch(dev::EvalNonSymmetricLdsKernel<16, 1024>);
+        } else if (m.NsLdsShape.Waves == 12) {
+            launch(dev::EvalNonSymmetricLdsKernel<12, 1536>);
+        } else {
+            launch(dev::EvalNonSymmetricLdsKernel<8, 2048>);
+        }
         HIP_CHECK(hipGetLastError());
         return;
     }
@@ -2224,9 +2271,9 @@ std::string THipEvaluator::DescribeKernels(int layout, size_t docCount) const {
         evaluate = m.PairRows.Get() != nullptr ? "EvalObliviousPairTileKernel" : "EvalObliviousHalfTileKernel";
     } else if (m.Oblivious) {
         evaluate = "EvalObliviousKernel";
-    } else if (m.NsLdsUsable &&
-               TileLdsBytes(m.LayoutBuckets, 1) + dev::kTileWaves * dev::kNsLdsEntries * 4 <= kMaxTileLdsBytes) {
-        evaluate = "EvalNonSymmetricLdsKernel";
+    } else if (m.NsLdsUsable) {
+        evaluate = "EvalNonSymmetricLdsKernel<" + std::to_string(m.NsLdsShape.Waves) + ", " +
+                   std::to_string(m.NsLdsShape.Entries) + ">";
     } else if (m.NsTileUsable && TileLdsBytes(m.LayoutBuckets, m.Dim == 1 ? 1 : m.Dim <= 4 ? 4 : 16) <= kMaxTileLdsBytes) {
         evaluate = "EvalNonSymmetricTileKernel";
     } else {

@@ -1093,17 +1093,27 @@ template <bool XOR, int MAXD>
 __device__ __forceinline__ uint32_t PairTreeIndexes(const uint8_t* laneTile, const uint4 (&desc)[4]) {
     const uint32_t offs[8] = {desc[0].x, desc[0].y, desc[0].z, desc[0].w, desc[1].x, desc[1].y, desc[1].z, desc[1].w};
     const uint32_t adds[8] = {desc[2].x, desc[2].y, desc[2].z, desc[2].w, desc[3].x, desc[3].y, desc[3].z, desc[3].w};
-    uint32_t idx4 = 0;
+    uint32_t a[MAXD];
 #pragma unroll
     for (int d = 0; d < MAXD; ++d) {
         // rows of trees that never xor hold the plain offset
-        uint32_t a = *reinterpret_cast<const uint32_t*>(laneTile + (XOR ? offs[d] & 0x007fffffu : offs[d]));
+        a[d] = *reinterpret_cast<const uint32_t*>(laneTile + (XOR ? offs[d] & 0x007fffffu : offs[d]));
+    }
+    // one wait for the eight reads instead of one per read: LDS returns them in order a few cycles apart, and
+    // every wait takes an issue slot (lgkmcnt 0, the other counters untouched)
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_sched_barrier(0);
+    uint32_t idx4 = 0;
+#pragma unroll
+    for (int d = 0; d < MAXD; ++d) {
+        uint32_t v = a[d];
         if (XOR) {
-            a ^= __builtin_amdgcn_perm(offs[d], offs[d], 0x03030303u);  // the xor byte four times
+            v ^= __builtin_amdgcn_perm(offs[d], offs[d], 0x03030303u);  // the xor byte four times
         }
         // the level's four result bits go to bit 7 of the bytes; earlier levels move down one bit and never
         // reach the byte below within eight levels
-        idx4 = ((a + adds[d]) & 0x80808080u) | (idx4 >> 1);
+        idx4 = ((v + adds[d]) & 0x80808080u) | (idx4 >> 1);
     }
     return idx4;
 }
@@ -1182,6 +1192,9 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousPairTileKernel(
 #define CBAMD_PAIR_ROUND(k)                                                                        \
     do {                                                                                           \
         uint32_t idx4;                                                                             \
+        /* one wait for this pair's eight loads: the sixteen of the two pairs behind it stay in flight */ \
+        __builtin_amdgcn_s_waitcnt(0x4f70);                                                        \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
         CBAMD_PUBLISH_AND_WALK(k, idx4);                                                           \
         _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                            \
             acc[q] = __dadd_rn(acc[q], gathered[q]);                                               \
@@ -1478,11 +1491,17 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalNonSymmetricTileKernel(
 // One-dimensional non-symmetric models without xor masks whose trees have at most kNsLdsEntries
 // entries, whole model: as EvalNonSymmetricTileKernel, but a wave walks its trees out of a copy in
 // its own LDS region (an LDS gather costs a fraction of a gather from global memory). Consecutive
-// trees are grouped into units of up to kNsUnitTrees trees and kNsLdsEntries entries; a wave takes
+// trees are grouped into units of up to kNsUnitTrees trees and ENTRIES entries; a wave takes
 // a unit at a time and walks its trees side by side (4 documents x kNsUnitTrees chains per lane).
 // A compact entry is one dword:
 //   bits 0-7 splitIdx, bits 8-17 bucket (so entry & 0x3ff00 is the bucket's offset in the tile),
-//   bits 21-31 index of the left child relative to the tree's first entry.
+//   bits 21-31 index of the left child relative to the unit's first entry.
+// The tile starts at LDS address 0 and a wave's region at a multiple of its size, so the bin's address takes one
+// instruction, (entry & 0x3ff00) | lane offset, and so does the pair's with regions of 8 KB: the funnel shift
+// {region number, entry} >> 19.
+// The kernel is bound by the latency of this chain of LDS reads, so the workgroup has as many waves as the
+// regions leave room for: WAVES regions of ENTRIES entries, ENTRIES at least the largest tree of the model
+// (16 x 1024, 12 x 1536 or 8 x 2048).
 // The two children of a node sit side by side at an even index (the root is entry 0, entry 1 is
 // unused), so one 8-byte LDS read, issued together with the read of the node's bin, brings both
 // and the compare only selects: one LDS round trip per level. A terminal entry points at its own
@@ -1493,16 +1512,25 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalNonSymmetricTileKernel(
 // its walk and added after the next unit's walk.
 // unitRows: 8 dwords per unit: first entry, height of the tallest tree, number of entries, first
 // entry of the second and of the third tree relative to the unit's, number of trees, 2 unused.
-// grid = doc blocks, block = 64 * kTileWaves, dynamic LDS = buckets * 256 (rounded up to 8) +
-// 256 * 8 + kTileWaves * kNsLdsEntries * 4 bytes.
+// grid = doc blocks, block = 64 * WAVES, dynamic LDS = buckets * 256 + 256 * 8 rounded up to a multiple
+// of ENTRIES * 4, + WAVES * ENTRIES * 4 bytes; no other LDS in the kernel.
 constexpr int kNsLdsEntries = 2048;
 constexpr int kNsUnitTrees = 3;
 
-__global__ __launch_bounds__(64 * kTileWaves) void EvalNonSymmetricLdsKernel(
+// A load of a scalar from an LDS address given as a number (the dynamic LDS of a kernel without other LDS
+// starts at 0).
+template <class T>
+__device__ __forceinline__ T LdsLoad(uint32_t address) {
+    return *reinterpret_cast<const __attribute__((address_space(3))) T*>(address);
+}
+
+template <int WAVES, int ENTRIES>
+__global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
     const uint32_t* __restrict__ bins, size_t docCount, uint32_t bucketCount, const uint32_t* __restrict__ entries,
     const uint4* __restrict__ unitRows, uint32_t unitCount, const double* __restrict__ valuesByEntry,
     const double* __restrict__ bias, double scale, double* __restrict__ out) {
-    constexpr int kFetch = kNsLdsEntries / kWave;
+    constexpr int kFetch = ENTRIES / kWave;
+    static_assert(ENTRIES <= kNsLdsEntries && ENTRIES % kWave == 0, "a region holds whole rounds of a wave's copy");
     extern __shared__ uint32_t sTile[];
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & (kWave - 1);
@@ -1510,14 +1538,18 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalNonSymmetricLdsKernel(
     const size_t block = blockIdx.x;
     const uint32_t tileDwords = bucketCount * kWave;
     const uint32_t* src = bins + block * tileDwords;
-    for (uint32_t i = tid; i < tileDwords; i += 64 * kTileWaves) {
+    for (uint32_t i = tid; i < tileDwords; i += 64 * WAVES) {
         sTile[i] = src[i];
     }
     const uint8_t* tileBytes = reinterpret_cast<const uint8_t*>(sTile);
     const uint32_t laneOff = lane * 4;
     const uint32_t redBase = (tileDwords + 1) & ~1u;
     double* sRed = reinterpret_cast<double*>(sTile + redBase);
-    uint32_t* sEntries = sTile + redBase + 2 * kDocsPerBlock + wave * kNsLdsEntries;
+    // the waves' regions by number: region r covers LDS bytes [r, r + 1) * ENTRIES * 4
+    const uint32_t region = (redBase + 2 * kDocsPerBlock + ENTRIES - 1) / ENTRIES + wave;
+    uint32_t* sEntries = sTile + region * ENTRIES;
+    const uint32_t regionAddr = region * ENTRIES * 4;
+    const uint32_t bucketMask = 0x3ff00u;
     __syncthreads();  // tile is loaded
 
     uint32_t fetched[kFetch];
@@ -1565,7 +1597,7 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalNonSymmetricLdsKernel(
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        const uint32_t uNext = u + kTileWaves;
+        const uint32_t uNext = u + WAVES;
         uint4 rowNext = make_uint4(0, 0, 0, 0), row2Next = make_uint4(0, 0, 0, 0);
         if (uNext < unitCount) {
             rowNext = unitRows[2 * uNext];
@@ -1582,24 +1614,27 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalNonSymmetricLdsKernel(
             }
         }
         for (uint32_t step = 0; step < height; ++step) {
-            uint2 pair[kNsUnitTrees][4];
+            uint64_t pair[kNsUnitTrees][4];  // the two children of a chain's node, left in the low half
             uint32_t bin[kNsUnitTrees][4];
 #pragma unroll
             for (int g = 0; g < kNsUnitTrees; ++g) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const uint32_t e = entry[g][j];
-                    // bits 18-20 of an entry are clear: e >> 19 is the byte offset of the pair of children
-                    pair[g][j] = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint8_t*>(sEntries + start[g]) +
-                                                                 (e >> 19));
-                    bin[g][j] = tileBytes[((e & 0x3ff00u) | laneOff) + j];
+                    // bits 18-20 of an entry are clear: e >> 19 is the byte offset of the pair of children in
+                    // the wave's region, whose number comes in from above
+                    pair[g][j] = LdsLoad<uint64_t>(ENTRIES * 4 == 1 << 13 ? __builtin_amdgcn_alignbit(region, e, 19)
+                                                                         : (e >> 19) + regionAddr);
+                    uint32_t binAddr;
+                    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(binAddr) : "v"(e), "s"(bucketMask), "v"(laneOff));
+                    bin[g][j] = LdsLoad<uint8_t>(binAddr + j);
                 }
             }
 #pragma unroll
             for (int g = 0; g < kNsUnitTrees; ++g) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    entry[g][j] = bin[g][j] >= (entry[g][j] & 0xffu) ? pair[g][j].y : pair[g][j].x;
+                    entry[g][j] = static_cast<uint32_t>(bin[g][j] >= (entry[g][j] & 0xffu) ? pair[g][j] >> 32 : pair[g][j]);
                 }
             }
         }
@@ -1623,7 +1658,7 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalNonSymmetricLdsKernel(
             if (static_cast<uint32_t>(g) < trees) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    pending[g][j] = valuesByEntry[first + start[g] + idx[g][j]];
+                    pending[g][j] = valuesByEntry[first + idx[g][j]];
                 }
             } else {
 #pragma unroll
@@ -1647,7 +1682,7 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalNonSymmetricLdsKernel(
     }
     // waves add their partial sums in wave order into the LDS accumulator; the last wave
     // finishes the values and writes them out
-    for (uint32_t w = 0; w + 1 < kTileWaves; ++w) {
+    for (uint32_t w = 0; w + 1 < WAVES; ++w) {
         if (wave == w) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -1657,7 +1692,7 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalNonSymmetricLdsKernel(
         }
         __syncthreads();
     }
-    if (wave == kTileWaves - 1) {
+    if (wave == WAVES - 1) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const size_t doc = block * kDocsPerBlock + j * kWave + lane;
