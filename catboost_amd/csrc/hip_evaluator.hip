@@ -369,19 +369,69 @@ size_t TileLdsBytes(uint32_t buckets, int dchunk) {
            static_cast<size_t>(dev::kDocsPerBlock) * dchunk * sizeof(double);
 }
 
-// LDS of EvalNonSymmetricLdsKernel: the tile and the accumulator, then the waves' entry regions at a multiple
-// of their size
+// LDS of EvalNonSymmetricLdsKernel: 8 KB per wave (its entries, then rows of bins), the other rows of bins, the
+// accumulator
 size_t NsLdsKernelBytes(uint32_t buckets, uint32_t waves, uint32_t entries) {
-    const size_t region = static_cast<size_t>(entries) * 4;
-    return (TileLdsBytes(buckets, 1) + region - 1) / region * region + waves * region;
+    return static_cast<size_t>(dev::NsLdsTileRows(buckets, waves, entries)) * 256 + dev::kDocsPerBlock * sizeof(double);
 }
 
 // The shapes of EvalNonSymmetricLdsKernel, most waves first
 struct TNsLdsShape {
     uint32_t Waves;
     uint32_t Entries;
+    double Speed;  // steps of a unit per unit of time, relative to the 8-wave shape
 };
-constexpr TNsLdsShape kNsLdsShapes[] = {{16, 1024}, {12, 1536}, {8, 2048}};
+constexpr TNsLdsShape kNsLdsShapes[] = {{16, 1024, 1.45}, {12, 1536, 1.26}, {8, 2048, 1.0}};
+
+// A unit of EvalNonSymmetricLdsKernel: up to three trees that a wave walks side by side out of its LDS region
+struct TNsUnit {
+    uint32_t Trees[dev::kNsUnitTrees];
+    uint32_t TreeCount;
+    uint32_t Entries;
+    uint32_t Height;
+};
+
+// Groups the trees (rows: first entry, height, entry count, unused) into units of at most `limit` entries.
+// A unit takes as many steps as its tallest tree, so the trees go in by falling height, and every tree joins
+// the fullest of the recently opened units that still has room for it (trees need not be neighbours in the
+// model: the kernel's sums are partial sums per wave anyway). False when a tree exceeds the limit.
+bool PackNsUnits(const std::vector<uint32_t>& rows, size_t treeCount, uint32_t limit, std::vector<TNsUnit>* units) {
+    std::vector<uint32_t> order(treeCount);
+    for (size_t t = 0; t < treeCount; ++t) {
+        if (rows[t * 4 + 2] > limit) {
+            return false;
+        }
+        order[t] = static_cast<uint32_t>(t);
+    }
+    std::stable_sort(order.begin(), order.end(), [&](uint32_t a, uint32_t b) {
+        return rows[a * 4 + 1] != rows[b * 4 + 1] ? rows[a * 4 + 1] > rows[b * 4 + 1] : rows[a * 4 + 2] > rows[b * 4 + 2];
+    });
+    constexpr size_t kWindow = 64;  // open units looked at per tree
+    std::vector<size_t> open;
+    for (const uint32_t t : order) {
+        const uint32_t size = rows[t * 4 + 2];
+        size_t best = open.size();
+        for (size_t i = open.size() > kWindow ? open.size() - kWindow : 0; i < open.size(); ++i) {
+            const TNsUnit& unit = (*units)[open[i]];
+            if (unit.Entries + size <= limit && (best == open.size() || unit.Entries > (*units)[open[best]].Entries)) {
+                best = i;
+            }
+        }
+        if (best == open.size()) {
+            TNsUnit unit{};
+            unit.Height = rows[t * 4 + 1];
+            units->push_back(unit);
+            open.push_back(units->size() - 1);
+        }
+        TNsUnit& unit = (*units)[open[best]];
+        unit.Trees[unit.TreeCount++] = t;
+        unit.Entries += size;
+        if (unit.TreeCount == static_cast<uint32_t>(dev::kNsUnitTrees)) {
+            open.erase(open.begin() + static_cast<std::ptrdiff_t>(best));
+        }
+    }
+    return true;
+}
 
 // LDS of the pair-tile kernel: 128 documents' bins, then per wave the leaf values of two trees; the same area
 // takes one partial sum per wave, lane group and document at the end
@@ -1342,46 +1392,64 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         BuildLevelOrderTrees(trees, m.Dim, firstLeaf, &m.NsEntries, &m.NsRows, &m.NsTileUsable, &m.NsNoXor,
                              &compactEntries, &compactRows, &valuesByEntry, &m.NsLdsUsable);
         if (m.NsLdsUsable) {
-            // the shape with the most waves whose regions hold the largest tree and that fits the LDS
-            uint32_t largestTree = 0;
-            for (size_t t = 0; t < TreeCount; ++t) {
-                largestTree = std::max(largestTree, compactRows[t * 4 + 2]);
-            }
+            // the shape whose units take the least time: more waves hide more of the walk's latency (steps per
+            // unit of time relative to 8 waves, measured on 500 trees of about 430 entries: 12 waves 1.26), smaller
+            // regions hold fewer trees per unit
             m.NsLdsUsable = false;
+            double bestCost = 0.0;
+            std::vector<TNsUnit> bestUnits;
             for (const TNsLdsShape& shape : kNsLdsShapes) {
-                if (largestTree <= shape.Entries && (switches.NsWaves == 0 || switches.NsWaves == shape.Waves) &&
-                    NsLdsKernelBytes(m.LayoutBuckets, shape.Waves, shape.Entries) <= kMaxTileLdsBytes) {
-                    m.NsLdsShape = shape;
+                if ((switches.NsWaves != 0 && switches.NsWaves != shape.Waves) ||
+                    NsLdsKernelBytes(m.LayoutBuckets, shape.Waves, shape.Entries) > kMaxTileLdsBytes) {
+                    continue;
+                }
+                std::vector<TNsUnit> plan;
+                if (!PackNsUnits(compactRows, TreeCount, shape.Entries, &plan)) {
+                    continue;  // a tree larger than a region
+                }
+                uint64_t steps = 0;
+                for (const TNsUnit& unit : plan) {
+                    steps += unit.Height;
+                }
+                const double cost = static_cast<double>(steps) / shape.Speed;
+                if (!m.NsLdsUsable || cost < bestCost) {
                     m.NsLdsUsable = true;
-                    break;
+                    m.NsLdsShape = shape;
+                    bestCost = cost;
+                    bestUnits.swap(plan);
                 }
             }
-        }
-        if (m.NsLdsUsable) {
-            // units: consecutive trees, at most kNsUnitTrees of them and as many entries as a region holds
-            std::vector<uint32_t> units;
-            for (size_t t = 0; t < TreeCount;) {
-                const uint32_t first = compactRows[t * 4];
-                uint32_t height = 0, count = 0, n = 0;
-                uint32_t start[dev::kNsUnitTrees] = {};
-                while (t < TreeCount && n < static_cast<uint32_t>(dev::kNsUnitTrees) &&
-                       count + compactRows[t * 4 + 2] <= m.NsLdsShape.Entries) {
-                    // child indexes (bits 21-31) count from the unit's first entry
-                    for (uint32_t e = 0; e < compactRows[t * 4 + 2]; ++e) {
-                        compactEntries[first + count + e] += count << 21;
+            if (m.NsLdsUsable) {
+                // the entries in the order of the units; child indexes (bits 21-31) count from the unit's first entry
+                std::vector<uint32_t> entries, units;
+                std::vector<double> values;
+                entries.reserve(compactEntries.size());
+                values.reserve(valuesByEntry.size());
+                for (const TNsUnit& unit : bestUnits) {
+                    const uint32_t first = static_cast<uint32_t>(entries.size());
+                    uint32_t start[dev::kNsUnitTrees] = {};
+                    uint32_t count = 0;
+                    for (uint32_t i = 0; i < unit.TreeCount; ++i) {
+                        const uint32_t t = unit.Trees[i];
+                        const uint32_t treeFirst = compactRows[t * 4], treeEntries = compactRows[t * 4 + 2];
+                        start[i] = count;
+                        for (uint32_t e = 0; e < treeEntries; ++e) {
+                            // the bucket (bits 8-17) becomes the LDS row of its bins in this shape
+                            const uint32_t entry = compactEntries[treeFirst + e];
+                            const uint32_t tileRow = dev::NsLdsTileRow((entry >> 8) & 0x3ffu, m.NsLdsShape.Waves, m.NsLdsShape.Entries);
+                            entries.push_back((entry & ~0x3ff00u) + (tileRow << 8) + (count << 21));
+                            values.push_back(valuesByEntry[treeFirst + e]);
+                        }
+                        count += treeEntries;
                     }
-                    start[n++] = count;
-                    height = std::max(height, compactRows[t * 4 + 1]);
-                    count += compactRows[t * 4 + 2];
-                    ++t;
+                    const uint32_t row[8] = {first, unit.Height, count, start[1], start[2], unit.TreeCount, 0, 0};
+                    units.insert(units.end(), row, row + 8);
                 }
-                const uint32_t unit[8] = {first, height, count, start[1], start[2], n, 0, 0};
-                units.insert(units.end(), unit, unit + 8);
+                m.NsUnitCount = static_cast<uint32_t>(bestUnits.size());
+                m.NsCompactEntries.Upload(entries);
+                m.NsCompactRows.Upload(units);
+                m.NsValuesByEntry.Upload(values);
             }
-            m.NsUnitCount = static_cast<uint32_t>(units.size() / 8);
-            m.NsCompactEntries.Upload(compactEntries);
-            m.NsCompactRows.Upload(units);
-            m.NsValuesByEntry.Upload(valuesByEntry);
         }
     }
 

@@ -1494,13 +1494,14 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalNonSymmetricTileKernel(
 // trees are grouped into units of up to kNsUnitTrees trees and ENTRIES entries; a wave takes
 // a unit at a time and walks its trees side by side (4 documents x kNsUnitTrees chains per lane).
 // A compact entry is one dword:
-//   bits 0-7 splitIdx, bits 8-17 bucket (so entry & 0x3ff00 is the bucket's offset in the tile),
-//   bits 21-31 index of the left child relative to the unit's first entry.
-// The tile starts at LDS address 0 and a wave's region at a multiple of its size, so the bin's address takes one
-// instruction, (entry & 0x3ff00) | lane offset, and so does the pair's with regions of 8 KB: the funnel shift
-// {region number, entry} >> 19.
-// The kernel is bound by the latency of this chain of LDS reads, so the workgroup has as many waves as the
-// regions leave room for: WAVES regions of ENTRIES entries, ENTRIES at least the largest tree of the model
+//   bits 0-7 splitIdx, bits 8-17 the 256-byte LDS row that holds the bucket's bins (so entry & 0x3ff00 is its
+//   address), bits 21-31 index of the left child relative to the unit's first entry.
+// Both addresses of a step take one instruction: the bin's is (entry & 0x3ff00) | lane offset, the pair's the
+// funnel shift {wave, entry} >> 19, because wave w keeps its entries at LDS address w * 8 KB. Regions shorter than
+// 8 KB leave gaps, and the rows of the bins fill them: NsLdsTileRow() says where bucket b goes, for the copy of
+// the tile here and for the entries on the host.
+// The kernel is bound by the latency of this chain of LDS reads, so the workgroup has as many waves as LDS has
+// room for: WAVES regions of ENTRIES entries, ENTRIES at least the largest tree of the model
 // (16 x 1024, 12 x 1536 or 8 x 2048).
 // The two children of a node sit side by side at an even index (the root is entry 0, entry 1 is
 // unused), so one 8-byte LDS read, issued together with the read of the node's bin, brings both
@@ -1512,10 +1513,25 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalNonSymmetricTileKernel(
 // its walk and added after the next unit's walk.
 // unitRows: 8 dwords per unit: first entry, height of the tallest tree, number of entries, first
 // entry of the second and of the third tree relative to the unit's, number of trees, 2 unused.
-// grid = doc blocks, block = 64 * WAVES, dynamic LDS = buckets * 256 + 256 * 8 rounded up to a multiple
-// of ENTRIES * 4, + WAVES * ENTRIES * 4 bytes; no other LDS in the kernel.
+// grid = doc blocks, block = 64 * WAVES, dynamic LDS = NsLdsTileRows(buckets, WAVES, ENTRIES) * 256 + 256 * 8 bytes;
+// no other LDS in the kernel.
 constexpr int kNsLdsEntries = 2048;
 constexpr int kNsUnitTrees = 3;
+
+// The 256-byte LDS row of bucket b's bins: the 8 KB of a wave start with its entries (entries / 64 rows) and the
+// rows that are left take bins; the other buckets follow the last wave's 8 KB.
+__host__ __device__ constexpr uint32_t NsLdsTileRow(uint32_t bucket, uint32_t waves, uint32_t entries) {
+    const uint32_t regionRows = entries / 64, gapRows = 32 - regionRows;
+    const uint32_t divisor = gapRows ? gapRows : 1;  // regions of 8 KB leave no gap
+    return bucket < gapRows * waves ? 32 * (bucket / divisor) + regionRows + bucket % divisor
+                                    : 32 * waves + bucket - gapRows * waves;
+}
+
+// Rows of LDS up to the end of the bins
+__host__ __device__ constexpr uint32_t NsLdsTileRows(uint32_t buckets, uint32_t waves, uint32_t entries) {
+    const uint32_t gapRows = (32 - entries / 64) * waves;
+    return 32 * waves + (buckets > gapRows ? buckets - gapRows : 0);
+}
 
 // A load of a scalar from an LDS address given as a number (the dynamic LDS of a kernel without other LDS
 // starts at 0).
@@ -1539,16 +1555,11 @@ __global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
     const uint32_t tileDwords = bucketCount * kWave;
     const uint32_t* src = bins + block * tileDwords;
     for (uint32_t i = tid; i < tileDwords; i += 64 * WAVES) {
-        sTile[i] = src[i];
+        sTile[NsLdsTileRow(i / kWave, WAVES, ENTRIES) * kWave + (i & (kWave - 1))] = src[i];
     }
-    const uint8_t* tileBytes = reinterpret_cast<const uint8_t*>(sTile);
     const uint32_t laneOff = lane * 4;
-    const uint32_t redBase = (tileDwords + 1) & ~1u;
-    double* sRed = reinterpret_cast<double*>(sTile + redBase);
-    // the waves' regions by number: region r covers LDS bytes [r, r + 1) * ENTRIES * 4
-    const uint32_t region = (redBase + 2 * kDocsPerBlock + ENTRIES - 1) / ENTRIES + wave;
-    uint32_t* sEntries = sTile + region * ENTRIES;
-    const uint32_t regionAddr = region * ENTRIES * 4;
+    double* sRed = reinterpret_cast<double*>(sTile + NsLdsTileRows(bucketCount, WAVES, ENTRIES) * kWave);
+    uint32_t* sEntries = sTile + wave * kNsLdsEntries;  // 8 KB per wave, the first ENTRIES * 4 bytes of them
     const uint32_t bucketMask = 0x3ff00u;
     __syncthreads();  // tile is loaded
 
@@ -1622,9 +1633,8 @@ __global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
                 for (int j = 0; j < 4; ++j) {
                     const uint32_t e = entry[g][j];
                     // bits 18-20 of an entry are clear: e >> 19 is the byte offset of the pair of children in
-                    // the wave's region, whose number comes in from above
-                    pair[g][j] = LdsLoad<uint64_t>(ENTRIES * 4 == 1 << 13 ? __builtin_amdgcn_alignbit(region, e, 19)
-                                                                         : (e >> 19) + regionAddr);
+                    // the wave's region, whose number comes in from above (kNsLdsEntries * 4 = 1 << 13)
+                    pair[g][j] = LdsLoad<uint64_t>(__builtin_amdgcn_alignbit(wave, e, 19));
                     uint32_t binAddr;
                     asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(binAddr) : "v"(e), "s"(bucketMask), "v"(laneOff));
                     bin[g][j] = LdsLoad<uint8_t>(binAddr + j);
