@@ -518,7 +518,10 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
         e("  s_mov_b32 s29, 0xc0c0c0c0")
     # byte j of the leaf indexes times s23 = offset of the document's leaf row in a tree's table
     # (a six-level index sits in bits 2..7 of its byte)
-    e("  s_mov_b32 s23, %d" % (pitch * 8 >> (8 - depth)))
+    # (tables of several dimensions hold a tree's values as pieces of two dimensions, each piece an array of
+    # 16 bytes per leaf: a wave's 16-byte gathers then spread over all sixteen groups of four LDS banks, which
+    # leaf rows of 32 bytes would not)
+    e("  s_mov_b32 s23, %d" % ((8 if pitch == 1 else 16) >> (8 - depth)))
     e("  s_mul_i32 s100, s20, %d" % wave_bytes)  # offset of the wave's share of a tree block
     # one step back: every group of copies steps forward first
     e("  s_sub_u32 s28, s100, %d" % group_step(0))
@@ -634,7 +637,7 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
                 else:
                     for k in range(0, pitch, 2):
                         e("  ds_read_b128 v[%d:%d], v%d offset:%d" % (lv(j, k), lv(j, k) + 3, ga0 + j,
-                                                                     tree_offset + 8 * k))
+                                                                     tree_offset + (k // 2) * leaves * 16))
             load_rows(rows, buf * block + i + 2)
             # copy of the next tree block into the other buffer, spread over this block's trees
             staged = False

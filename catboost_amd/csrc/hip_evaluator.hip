@@ -902,6 +902,20 @@ struct THipEvaluator::TImpl {
     TDeviceVec<uint32_t> RegRows;
     TDeviceVec<double> RegLeaves;  // [launch][tree][leaf row][pitch]
     TDeviceVec<double> RegBias;    // the bias, readable for a whole pitch behind every dimension
+    // The launches of a pass over the trees: RegPitch dimensions each, the last one with the narrowest kernel that
+    // holds what is left (ten dimensions: six, then four instead of six of which two are padding).
+    struct TRegLaunch {
+        hipFunction_t Function = nullptr;
+        const char* Name = "";
+        uint32_t Waves = 0;
+        uint32_t FirstDim = 0;
+        uint32_t StoreDims = 1;
+        uint32_t TreeBlock = 16;         // trees per LDS buffer of this kernel
+        size_t TreeLeafDoubles = 0;      // doubles of a tree in Leaves
+        const double* Leaves = nullptr;  // the launch's leaf table
+    };
+    std::vector<TRegLaunch> RegLaunches;
+    TDeviceVec<double> RegTailLeaves;  // leaf table of a last launch that uses another kernel
 
     // fused kernels, per row layout (0: flat rows, 1: split rows of a model without categorical features)
     struct TFused {
@@ -1474,7 +1488,6 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         const size_t rowDwords = variant->Mixed ? 32 : 16;
         m.RegWaves = variant->Waves;
         m.RegPitch = variant->Pitch;
-        m.RegTreeBlockSize = block;
         m.RegRowDwords = static_cast<uint32_t>(rowDwords);
         m.RegTreeLeafDoubles = rowsPerTree * pitch;
         m.RegTreeBlocks = static_cast<uint32_t>((TreeCount + block - 1) / block);
@@ -1482,8 +1495,24 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         const size_t tableTrees = (static_cast<size_t>(m.RegTreeBlocks) + 2) * block;
         const size_t launches = (static_cast<size_t>(m.Dim) + pitch - 1) / pitch;
         m.RegLaunchLeaves = tableTrees * rowsPerTree * pitch;
-        std::vector<uint32_t> rows(tableTrees * rowDwords, 0);  // 7-bit form (bucket 0, add 0): false for every bin
-        std::vector<double> leaves(launches * m.RegLaunchLeaves, 0.0);
+        // the last launch: the kernel of the same form with the smallest pitch that holds the dimensions left
+        const size_t tailFirst = (launches - 1) * pitch, tailDims = static_cast<size_t>(m.Dim) - tailFirst;
+        const TEvalRegVariant* tailVariant = nullptr;
+        for (const auto& v : kEvalRegVariants) {
+            if (m.Dim > 1 && v.Pitch > 1 && v.Pitch >= tailDims && v.Pitch < pitch && v.Leaves == variant->Leaves &&
+                v.Mixed == variant->Mixed && v.Six == variant->Six && v.Waves == variant->Waves &&
+                m.LayoutBuckets <= v.Buckets && (!tailVariant || v.Pitch < tailVariant->Pitch)) {
+                tailVariant = &v;
+            }
+        }
+        const uint32_t tailBlock = tailVariant ? RegTreeBlock(*tailVariant) : block;
+        const size_t tailPitch = tailVariant ? tailVariant->Pitch : pitch;
+        const size_t tailTableTrees = ((TreeCount + tailBlock - 1) / tailBlock + 2) * tailBlock;
+        // tree ranges are cut at blocks of the kernel with the larger block (both are powers of two)
+        m.RegTreeBlockSize = std::max(block, tailBlock);
+        std::vector<uint32_t> rows(std::max(tableTrees, tailTableTrees) * rowDwords, 0);  // 7-bit form (bucket 0, add 0): false for every bin
+        std::vector<double> leaves((tailVariant ? launches - 1 : launches) * m.RegLaunchLeaves, 0.0);
+        std::vector<double> tailLeaves(tailVariant ? tailTableTrees * rowsPerTree * tailPitch : 0, 0.0);
         // Order of a tree's levels in these tables (levelOrder[t][position] = level of the model). The leaf
         // gathers of a wave meet in the LDS banks that the low bits of the leaf indexes choose; lanes with the
         // same index share one access, lanes that differ only in high bits wait for each other. So the levels
@@ -1554,15 +1583,20 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
             }
             const double* values = trees.LeafValues.data() + trees.TreeFirstLeafOffsets[t];
             for (size_t launch = 0; launch < launches; ++launch) {
-                double* table = leaves.data() + launch * m.RegLaunchLeaves + t * rowsPerTree * pitch;
+                const bool tailTable = tailVariant && launch + 1 == launches;
+                const size_t launchPitch = tailTable ? tailPitch : pitch;
+                double* table = tailTable ? tailLeaves.data() + t * rowsPerTree * tailPitch
+                                          : leaves.data() + launch * m.RegLaunchLeaves + t * rowsPerTree * pitch;
                 for (size_t leaf = 0; leaf < (size_t(1) << depth); ++leaf) {
                     // the leaf of the model whose level bits are this table row's position bits
                     size_t modelLeaf = 0;
                     for (int d = 0; d < depth; ++d) {
                         modelLeaf |= ((leaf >> d) & 1) << levelOrder[t][d];
                     }
-                    for (size_t k = 0; k < pitch && launch * pitch + k < static_cast<size_t>(m.Dim); ++k) {
-                        table[leaf * pitch + k] = values[modelLeaf * m.Dim + launch * pitch + k];
+                    // one-dimensional: a value per leaf; else pieces of two dimensions, 16 bytes per leaf and piece
+                    for (size_t k = 0; k < launchPitch && launch * pitch + k < static_cast<size_t>(m.Dim); ++k) {
+                        const size_t slot = launchPitch == 1 ? leaf : (k / 2) * rowsPerTree * 2 + leaf * 2 + k % 2;
+                        table[slot] = values[modelLeaf * m.Dim + launch * pitch + k];
                     }
                 }
             }
@@ -1572,6 +1606,29 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         m.RegRows.Upload(rows);
         m.RegLeaves.Upload(leaves);
         m.RegBias.Upload(biasPadded);
+        if (tailVariant) {
+            m.RegTailLeaves.Upload(tailLeaves);
+        }
+        for (size_t launch = 0; launch < launches; ++launch) {
+            TImpl::TRegLaunch l;
+            l.FirstDim = static_cast<uint32_t>(launch * pitch);
+            l.StoreDims = static_cast<uint32_t>(std::min(pitch, static_cast<size_t>(m.Dim) - launch * pitch));
+            l.Waves = variant->Waves;
+            if (tailVariant && launch + 1 == launches) {
+                HIP_CHECK(hipModuleGetFunction(&l.Function, m.RegModule, tailVariant->Name));
+                l.Name = tailVariant->Name;
+                l.TreeBlock = tailBlock;
+                l.TreeLeafDoubles = rowsPerTree * tailPitch;
+                l.Leaves = m.RegTailLeaves.Get();
+            } else {
+                l.Function = m.RegFunction;
+                l.Name = variant->Name;
+                l.TreeBlock = block;
+                l.TreeLeafDoubles = rowsPerTree * pitch;
+                l.Leaves = m.RegLeaves.Get() + launch * m.RegLaunchLeaves;
+            }
+            m.RegLaunches.push_back(l);
+        }
         m.RegKernelUsable = true;
         m.SmallBatchSlices = switches.SmallBatch;
 
@@ -2083,22 +2140,22 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
         args.Out = results;
         args.DocCount = static_cast<uint32_t>(docCount);
         args.BlockCount = static_cast<uint32_t>((docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock);
-        args.TreeBlocks = (wholeEnd - wholeBegin + block - 1) / block;
         args.Flags = (biased && !tail ? 1u : 0u) | (head ? 2u : 0u) | (tail ? 4u : 0u);
         args.Scale = m.Scale;
         args.BucketCount = m.LayoutBuckets;
         args.Dim = static_cast<uint32_t>(m.Dim);
-        launchArgs.TreeBlocksPerSlice = args.TreeBlocks;
-        const uint32_t grid = (args.BlockCount + m.RegWaves - 1) / m.RegWaves;
-        for (uint32_t first = 0, launch = 0; first < args.Dim; first += m.RegPitch, ++launch) {
-            args.Leaves = m.RegLeaves.Get() + launch * m.RegLaunchLeaves + static_cast<size_t>(wholeBegin) * m.RegTreeLeafDoubles;
-            args.Bias = m.RegBias.Get() + first;
-            args.FirstDim = first;
-            args.StoreDims = std::min(m.RegPitch, args.Dim - first);
+        for (const TImpl::TRegLaunch& l : m.RegLaunches) {
+            args.TreeBlocks = (wholeEnd - wholeBegin + l.TreeBlock - 1) / l.TreeBlock;
+            launchArgs.TreeBlocksPerSlice = args.TreeBlocks;
+            args.Leaves = l.Leaves + static_cast<size_t>(wholeBegin) * l.TreeLeafDoubles;
+            args.Bias = m.RegBias.Get() + l.FirstDim;
+            args.FirstDim = l.FirstDim;
+            args.StoreDims = l.StoreDims;
+            const uint32_t grid = (args.BlockCount + l.Waves - 1) / l.Waves;
             size_t argSize = sizeof(launchArgs);
             void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &launchArgs, HIP_LAUNCH_PARAM_BUFFER_SIZE, &argSize,
                               HIP_LAUNCH_PARAM_END};
-            HIP_CHECK(hipModuleLaunchKernel(m.RegFunction, grid, 1, 1, 64 * m.RegWaves, 1, 1, 0, s, nullptr, config));
+            HIP_CHECK(hipModuleLaunchKernel(l.Function, grid, 1, 1, 64 * l.Waves, 1, 1, 0, s, nullptr, config));
         }
         if (tail) {
             generic(wholeEnd, te, dev::kEvalContinue);
@@ -2213,10 +2270,11 @@ uint32_t THipEvaluator::TreeSlicesFor(size_t docCount) const {
     // (as long as the batch is small enough to be sliced at all).
     const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
     const size_t groups = (blocks + m.RegWaves - 1) / m.RegWaves;
-    if (groups >= 256 || m.RegTreeBlocks < 4) {
+    const size_t sliceTrees = 2 * static_cast<size_t>(m.RegTreeBlockSize);
+    if (groups >= 256 || TreeCount <= 3 * static_cast<size_t>(m.RegTreeBlockSize)) {
         return 1;
     }
-    return (m.RegTreeBlocks + 1) / 2;
+    return static_cast<uint32_t>((TreeCount + sliceTrees - 1) / sliceTrees);
 }
 
 size_t THipEvaluator::TreeSliceScratchDoubles(size_t docCount) const {
@@ -2241,27 +2299,28 @@ void THipEvaluator::EvalQuantizedSlicedDevice(const uint8_t* bins, size_t docCou
     args.Out = partials;
     args.DocCount = static_cast<uint32_t>(docCount);
     args.BlockCount = static_cast<uint32_t>((docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock);
-    args.TreeBlocks = m.RegTreeBlocks;
     args.Flags = 4;  // raw sums per slice
     args.Scale = m.Scale;
     args.BucketCount = m.LayoutBuckets;
     args.Dim = static_cast<uint32_t>(m.Dim);
-    launchArgs.TreeBlocksPerSlice = (m.RegTreeBlocks + slices - 1) / slices;
-    const uint32_t usedSlices = (m.RegTreeBlocks + launchArgs.TreeBlocksPerSlice - 1) / launchArgs.TreeBlocksPerSlice;
-    const uint32_t grid = (args.BlockCount + m.RegWaves - 1) / m.RegWaves;
-    for (uint32_t first = 0, launch = 0; first < args.Dim; first += m.RegPitch, ++launch) {
-        args.Leaves = m.RegLeaves.Get() + launch * m.RegLaunchLeaves;
-        args.Bias = m.RegBias.Get() + first;
-        args.FirstDim = first;
-        args.StoreDims = std::min(m.RegPitch, args.Dim - first);
+    // a slice is the same two (largest) tree blocks' worth of trees in every launch
+    const uint32_t sliceTrees = 2 * m.RegTreeBlockSize;
+    for (const TImpl::TRegLaunch& l : m.RegLaunches) {
+        args.TreeBlocks = static_cast<uint32_t>((TreeCount + l.TreeBlock - 1) / l.TreeBlock);
+        launchArgs.TreeBlocksPerSlice = sliceTrees / l.TreeBlock;
+        args.Leaves = l.Leaves;
+        args.Bias = m.RegBias.Get() + l.FirstDim;
+        args.FirstDim = l.FirstDim;
+        args.StoreDims = l.StoreDims;
+        const uint32_t grid = (args.BlockCount + l.Waves - 1) / l.Waves;
         size_t argSize = sizeof(launchArgs);
         void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &launchArgs, HIP_LAUNCH_PARAM_BUFFER_SIZE, &argSize,
                           HIP_LAUNCH_PARAM_END};
-        HIP_CHECK(hipModuleLaunchKernel(m.RegFunction, grid, usedSlices, 1, 64 * m.RegWaves, 1, 1, 0, s, nullptr, config));
+        HIP_CHECK(hipModuleLaunchKernel(l.Function, grid, slices, 1, 64 * l.Waves, 1, 1, 0, s, nullptr, config));
     }
     const size_t count = docCount * m.Dim;
     hipLaunchKernelGGL(dev::CombineSlicesKernel, dim3(static_cast<uint32_t>((count + 255) / 256)), dim3(256), 0, s, partials,
-                       usedSlices, count, m.Scale, m.Bias.Get(), m.Dim, results);
+                       slices, count, m.Scale, m.Bias.Get(), m.Dim, results);
     HIP_CHECK(hipGetLastError());
 }
 
@@ -2328,6 +2387,15 @@ std::string THipEvaluator::DescribeKernels(int layout, size_t docCount) const {
         evaluate = "FillBiasKernel";
     } else if (m.RegKernelUsable) {
         evaluate = m.RegKernelName;
+        if (m.RegLaunches.size() > 1) {
+            const size_t main = m.RegLaunches.size() - (m.RegTailLeaves.Get() != nullptr ? 1 : 0);
+            if (main > 1) {
+                evaluate += " x " + std::to_string(main) + " launches";
+            }
+            if (main < m.RegLaunches.size()) {
+                evaluate += std::string(" + ") + m.RegLaunches.back().Name;
+            }
+        }
         const uint32_t slices = TreeSlicesFor(docCount);
         if (slices > 1) {
             evaluate += " x " + std::to_string(slices) + " slices of the trees + CombineSlicesKernel";

@@ -809,6 +809,13 @@ def test_register_kernel_multi_dimensional(monkeypatch, dim, max_depth, n_float,
     np.testing.assert_array_equal(g.calc_flat(x), o.calc(x))
     _close(g.calc_flat(x, tree_start=1, tree_end=len(model["tree_sizes"])),
            o.calc(x, tree_start=1, tree_end=len(model["tree_sizes"])))
+    # the last launch takes the narrowest kernel that holds the dimensions left over
+    evaluate = g.evaluator().describe_kernels(cb.LAYOUT_FLAT_ROWS, 1 << 20)["evaluate"]
+    expected_tail = {10: "_p4_", 13: "_p2_", 20: "_p2_"}.get(dim)
+    if expected_tail:
+        assert "_p6_" in evaluate.split(" + ")[0] and expected_tail in evaluate.split(" + ")[1], evaluate
+    else:
+        assert " + " not in evaluate, evaluate
 
 
 @pytest.mark.parametrize("max_borders", [64, 65, 128])
