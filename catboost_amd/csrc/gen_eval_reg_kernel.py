@@ -83,7 +83,10 @@ SHAPES = [
     (192, 4, 2, 64), (160, 4, 4, 64), (128, 4, 6, 64),
     (192, 4, 2, 256), (160, 4, 4, 256), (128, 4, 6, 256),
 ]
+# trees of depth 9 and 10 (1024 leaf rows, one dimension): plain and six-bit forms only
+DEEP_SHAPES = [(208, 4, 1, 1024), (96, 8, 1, 1024)]
 VARIANTS = [shape + (mixed, six) for mixed, six in ((False, False), (False, True), (True, False)) for shape in SHAPES]
+VARIANTS += [shape + (False, six) for six in (False, True) for shape in DEEP_SHAPES]
 # shapes of the fused kernels (one dimension, 256 leaf rows), each in a plain and a six-bit form. Only the
 # wide shape: a model of 96 buckets or fewer runs its separate evaluate kernel at four waves per SIMD, which a
 # fused kernel (more registers: three) does not match; measured, two launches are the faster there.
@@ -124,11 +127,13 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
     assert not (mixed and six)
     assert not fused or (pitch == 1 and leaves == 256 and not mixed and buckets % 16 == 0)
     name = kernel_name(buckets, waves, pitch, leaves, mixed, six, fused)
-    row_dwords = 32 if mixed else 16      # level table of a tree
+    depth = {64: 6, 256: 8, 1024: 10}[leaves]
+    deep = depth > 8                      # levels 8 and 9 go into a second index word
+    assert not deep or (pitch == 1 and not mixed and not fused)
+    row_dwords = 32 if mixed or deep else 16      # level table of a tree
     tree_row_bytes = row_dwords * 4
     rows_a, rows_b = 32, 32 + row_dwords  # the two sets of scalar registers holding level tables
     assert pitch == 1 or pitch % 2 == 0
-    depth = {64: 6, 256: 8}[leaves]
     threads = waves * 64
     row_bytes = threads * 16              # one 16-byte piece per thread of a leaf table copy
     tree_bytes = leaves * pitch * 8
@@ -155,7 +160,8 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
     ac0 = lv0 + 8 * pitch                 # the sums
     ga0 = ac0 + 8 * pitch                 # gather addresses of the four documents
     te0 = ga0 + 4                         # two scratch registers of the epilogue
-    b0 = te0 + 2                          # the bins
+    wd0 = te0 + 2                         # deep kernels: the ten-bit leaf indexes of documents 0, 1 and 2, 3 as words
+    b0 = wd0 + (2 if deep else 0)         # the bins
     vgprs = b0 + buckets
     if fused:
         # registers of the binarize phase: those below the bins except v0 and v2, and 20 above the bins
@@ -211,8 +217,26 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
     # Six-level kernels keep the mask: two of those bits would stay below the index.
     first_level_masked = depth < 8
 
+    def levels_high(rows):
+        """Levels 8 and 9 of a deep tree (constants (128 - splitIdx) in every form): their bits become bits 0 and
+        1 of a second byte per document, and the two bytes of a document one 16-bit word: v[wd0] holds the
+        indexes of documents 0 and 1, v[wd0 + 1] those of 2 and 3. The index register is set to 0 behind the
+        last level, so that the instructions that follow may name vector registers in src0."""
+        e("  s_set_gpr_idx_idx s%d" % (rows + 16))
+        e("  v_add_u32_e64 v4, v%d, s%d" % (b0, rows + 17))
+        e("  s_set_gpr_idx_idx s%d" % (rows + 18))
+        e("  v_add_u32_e64 v5, v%d, s%d" % (b0, rows + 19))
+        e("  s_set_gpr_idx_idx 0")
+        e("  v_lshrrev_b32_e32 v4, 7, v4")
+        e("  v_lshrrev_b32_e32 v5, 6, v5")
+        e("  v_and_b32_e32 v4, 0x01010101, v4")
+        e("  v_and_b32_e32 v5, 0x02020202, v5")
+        e("  v_or_b32_e32 v4, v4, v5")
+        e("  v_perm_b32 v%d, v4, v3, s24" % wd0)        # bytes: index 0 low, high, index 1 low, high
+        e("  v_perm_b32 v%d, v4, v3, s25" % (wd0 + 1))
+
     def levels_seven_bit(rows):
-        for d in range(depth):
+        for d in range(min(depth, 8)):
             e("  s_set_gpr_idx_idx s%d" % (rows + 2 * d))
             if d == 0 and not first_level_masked:
                 e("  v_add_u32_e64 v3, v%d, s%d" % (b0, rows + 2 * d + 1))
@@ -230,7 +254,7 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
         form. A pair of levels is then merged into the index with one shift: five instructions for two
         levels instead of six. What the first pair leaves below its two bits goes the way the 7-bit
         form's first sum goes; six-level kernels mask it."""
-        for pair in range(depth // 2):
+        for pair in range(min(depth, 8) // 2):
             even, odd = rows + 4 * pair, rows + 4 * pair + 2
             e("  s_set_gpr_idx_idx s%d" % even)
             e("  v_add_u32_e64 v4, v%d, s%d" % (b0, even + 1))
@@ -521,7 +545,7 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
     # (tables of several dimensions hold a tree's values as pieces of two dimensions, each piece an array of
     # 16 bytes per leaf: a wave's 16-byte gathers then spread over all sixteen groups of four LDS banks, which
     # leaf rows of 32 bytes would not)
-    e("  s_mov_b32 s23, %d" % ((8 if pitch == 1 else 16) >> (8 - depth)))
+    e("  s_mov_b32 s23, %d" % ((8 if pitch == 1 else 16) >> max(8 - depth, 0)))
     e("  s_mul_i32 s100, s20, %d" % wave_bytes)  # offset of the wave's share of a tree block
     # one step back: every group of copies steps forward first
     e("  s_sub_u32 s28, s100, %d" % group_step(0))
@@ -608,6 +632,10 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
     e("  s_lshl_b32 s28, s28, 6")
     e("  s_add_u32 s30, s6, s28")
     e("  s_addc_u32 s31, s7, 0")
+    if deep:
+        # byte selectors of the two index words (s24 and s25 are free from here to the epilogue)
+        e("  s_mov_b32 s24, 0x05010400")
+        e("  s_mov_b32 s25, 0x07030602")
     e("%s_loop:" % name)
     for buf in range(2):
         for i in range(block):
@@ -625,12 +653,18 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
                 levels_six_bit(rows)
             else:
                 levels_seven_bit(rows)
+            if deep:
+                levels_high(rows)
             # previous tree's leaf values have arrived (and so has the next tree's row)
             e("  s_waitcnt lgkmcnt(0)")
             add_leaf_values()
             for j in range(4):
-                e("  v_mul_u32_u24_sdwa v%d, s23, v3 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_%d"
-                  % (ga0 + j, j))
+                if deep:
+                    e("  v_mul_u32_u24_sdwa v%d, s23, v%d dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_%d"
+                      % (ga0 + j, wd0 + j // 2, j % 2))
+                else:
+                    e("  v_mul_u32_u24_sdwa v%d, s23, v3 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_%d"
+                      % (ga0 + j, j))
                 tree_offset = buf * buf_bytes + i * tree_bytes
                 if pitch == 1:
                     e("  ds_read_b64 v[%d:%d], v%d offset:%d" % (lv(j, 0), lv(j, 0) + 1, ga0 + j, tree_offset))

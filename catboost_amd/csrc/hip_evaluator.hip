@@ -205,7 +205,13 @@ constexpr TEvalRegVariant kEvalRegVariants[] = {
     {192, 4, 2, 256, false, true, "cbamd_eval_reg_b192_w4_p2_l256_s"},
     {160, 4, 4, 256, false, true, "cbamd_eval_reg_b160_w4_p4_l256_s"},
     {128, 4, 6, 256, false, true, "cbamd_eval_reg_b128_w4_p6_l256_s"},
+    // trees of depth 9 and 10 (one dimension, 1024 leaf rows; gen_eval_reg_kernel.py's DEEP_SHAPES)
+    {96, 8, 1, 1024, false, false, "cbamd_eval_reg_b96_w8_p1_l1024"},
+    {208, 4, 1, 1024, false, false, "cbamd_eval_reg_b208_w4_p1_l1024"},
+    {96, 8, 1, 1024, false, true, "cbamd_eval_reg_b96_w8_p1_l1024_s"},
+    {208, 4, 1, 1024, false, true, "cbamd_eval_reg_b208_w4_p1_l1024_s"},
 };
+constexpr int kRegMaxDepth = 10;  // deepest tree of the register kernels (one-dimensional models; 8 otherwise)
 
 // Fused kernels (binarize + evaluate in one launch, bins only ever in registers): shapes of
 // gen_eval_reg_kernel.py's FUSED_SHAPES, each in a plain and a six-bit form.
@@ -234,6 +240,12 @@ struct TEvalFusedArgs {
 };
 static_assert(sizeof(TEvalFusedArgs) == 104, "kernel argument block of the fused kernels");
 
+// Trees of a slice of a small batch: two of the kernels' tree blocks, and not fewer than 32 trees (kernels with
+// large leaf tables have blocks of 2 or 4 trees, and a slice costs a partial sum per document)
+uint32_t RegSliceTrees(uint32_t treeBlock) {
+    return std::max(2 * treeBlock, 32u);
+}
+
 // trees per LDS buffer of a variant: a power of two, at most 16, buffer at most 32 KB
 uint32_t RegTreeBlock(const TEvalRegVariant& v) {
     uint32_t block = 16;
@@ -251,7 +263,8 @@ const TEvalRegVariant* PickRegVariant(uint32_t buckets, uint32_t dim, uint32_t m
     const TEvalRegVariant* best = nullptr;
     uint32_t bestLaunches = 0;
     for (const auto& v : kEvalRegVariants) {
-        if (buckets > v.Buckets || v.Buckets < minVariantBuckets || (dim == 1) != (v.Pitch == 1) || v.Leaves != (dim > 1 && maxDepth <= 6 ? 64u : 256u) ||
+        const uint32_t leaves = maxDepth > 8 ? 1024u : dim > 1 && maxDepth <= 6 ? 64u : 256u;
+        if (buckets > v.Buckets || v.Buckets < minVariantBuckets || (dim == 1) != (v.Pitch == 1) || v.Leaves != leaves ||
             v.Mixed != mixed || v.Six != six) {
             continue;
         }
@@ -1278,9 +1291,9 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
     }
     m.Bias.Upload(trees.Bias);
 
+    // 7-bit compares need every bin and split index to fit 7 bits and no xor mask
+    m.PackedSevenBit = m.Oblivious && !m.HasOneHot && m.MaxBucketValues <= 127;
     if (m.Oblivious && m.MaxDepth <= 8) {
-        // 7-bit compares need every bin and split index to fit 7 bits and no xor mask
-        m.PackedSevenBit = !m.HasOneHot && m.MaxBucketValues <= 127;
         std::vector<uint32_t> packed(trees.GetTreeCount() * dev::kPackedTreeDwords, 0);
         for (size_t t = 0; t < trees.GetTreeCount(); ++t) {
             uint32_t* row = packed.data() + t * dev::kPackedTreeDwords;
@@ -1471,7 +1484,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
     // six-bit form: no one-hot split and no bucket with more than 63 values, so that every bin is below 64
     const bool six = m.PackedSevenBit && m.MaxBucketValues <= 63 && switches.RegSix;
     const TEvalRegVariant* variant =
-        m.Oblivious && m.MaxDepth <= 8 && TreeCount > 0
+        m.Oblivious && m.MaxDepth <= kRegMaxDepth && TreeCount > 0
             ? PickRegVariant(m.LayoutBuckets, static_cast<uint32_t>(m.Dim), m.MaxDepth, !m.PackedSevenBit, six,
                              switches.RegMinBuckets)
             : nullptr;
@@ -1485,7 +1498,8 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         m.RegKernelName = variant->Name;
         const uint32_t block = RegTreeBlock(*variant);
         const size_t pitch = variant->Pitch, rowsPerTree = variant->Leaves;
-        const size_t rowDwords = variant->Mixed ? 32 : 16;
+        const size_t rowDwords = variant->Mixed || variant->Leaves > 256 ? 32 : 16;
+        const int rowLevels = variant->Leaves > 256 ? 10 : 8;
         m.RegWaves = variant->Waves;
         m.RegPitch = variant->Pitch;
         m.RegRowDwords = static_cast<uint32_t>(rowDwords);
@@ -1559,9 +1573,10 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
                     const auto& rb = levelAt(d);
                     row[2 * d] = rb.FeatureIndex;
                     // the level's bit is the carry into bit 7; six-bit kernels want the even levels' in bit 6
-                    row[2 * d + 1] = ((variant->Six && d % 2 == 0 ? 64u : 128u) - rb.SplitIdx) * 0x01010101u;
+                    // (of the first eight levels: levels 8 and 9 of a deep tree are read from bit 7 in every form)
+                    row[2 * d + 1] = ((variant->Six && d % 2 == 0 && d < 8 ? 64u : 128u) - rb.SplitIdx) * 0x01010101u;
                 }
-                for (int d = depth; d < 8 && depth > 0; ++d) {
+                for (int d = depth; d < rowLevels && depth > 0; ++d) {
                     row[2 * d] = row[0];
                 }
             } else {
@@ -1637,7 +1652,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         // consecutive columns = sixteen registers), so the level rows are rewritten per row layout.
         // (models that fit the 96-register shape stay on two launches: their evaluate kernel runs at four waves per
         // SIMD, a fused one at three, and is the faster - measured on 50 and 90 buckets)
-        const bool fusedCandidate = switches.Fused && !variant->Mixed && variant->Pitch == 1 && variant->Waves == 4 && m.Dim == 1 && !m.HasCats &&
+        const bool fusedCandidate = switches.Fused && !variant->Mixed && variant->Pitch == 1 && variant->Waves == 4 && variant->Leaves == 256 && m.Dim == 1 && !m.HasCats &&
                                     m.CtrCount == 0 && m.BinarizeBuckets == BucketCount && BucketCount > 0;
         for (int layoutIndex = 0; layoutIndex < 2 && fusedCandidate; ++layoutIndex) {
             const std::vector<uint32_t>& columns = layoutIndex == 0 ? srcFlat : srcSplit;
@@ -2270,8 +2285,8 @@ uint32_t THipEvaluator::TreeSlicesFor(size_t docCount) const {
     // (as long as the batch is small enough to be sliced at all).
     const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
     const size_t groups = (blocks + m.RegWaves - 1) / m.RegWaves;
-    const size_t sliceTrees = 2 * static_cast<size_t>(m.RegTreeBlockSize);
-    if (groups >= 256 || TreeCount <= 3 * static_cast<size_t>(m.RegTreeBlockSize)) {
+    const size_t sliceTrees = RegSliceTrees(m.RegTreeBlockSize);
+    if (groups >= 256 || TreeCount < 2 * sliceTrees) {
         return 1;
     }
     return static_cast<uint32_t>((TreeCount + sliceTrees - 1) / sliceTrees);
@@ -2303,8 +2318,8 @@ void THipEvaluator::EvalQuantizedSlicedDevice(const uint8_t* bins, size_t docCou
     args.Scale = m.Scale;
     args.BucketCount = m.LayoutBuckets;
     args.Dim = static_cast<uint32_t>(m.Dim);
-    // a slice is the same two (largest) tree blocks' worth of trees in every launch
-    const uint32_t sliceTrees = 2 * m.RegTreeBlockSize;
+    // a slice is the same number of trees in every launch
+    const uint32_t sliceTrees = RegSliceTrees(m.RegTreeBlockSize);
     for (const TImpl::TRegLaunch& l : m.RegLaunches) {
         args.TreeBlocks = static_cast<uint32_t>((TreeCount + l.TreeBlock - 1) / l.TreeBlock);
         launchArgs.TreeBlocksPerSlice = sliceTrees / l.TreeBlock;

@@ -793,6 +793,42 @@ def test_register_kernel_shapes(monkeypatch, n_float, trees, max_depth, docs, si
 
 
 @pytest.mark.parametrize("six", ["1", "0"])
+@pytest.mark.parametrize("n_float,trees,max_depth,docs,small_batch", [
+    (30, 60, 10, 3000, "0"), (96, 37, 9, 700, "0"), (97, 41, 10, 2500, "0"), (208, 45, 10, 1500, "0"),
+    (12, 300, 10, 70001, "0"), (12, 300, 10, 900, "1"), (5, 3, 10, 1, "0"),
+])
+def test_register_kernel_deep_trees(monkeypatch, n_float, trees, max_depth, docs, small_batch, six):
+    """One-dimensional float-only models with trees of depth 9 and 10: register-resident kernels with 1024 leaf
+    rows per tree (the index of a document is a 16-bit word of two byte-parallel index bytes), bit for bit like
+    the shallower ones; small batches in slices of the trees within the tolerance."""
+    monkeypatch.setenv("CATBOOST_AMD_REG_SIX", six)
+    monkeypatch.setenv("CATBOOST_AMD_SMALL_BATCH", small_batch)
+    rng = np.random.default_rng(31 * n_float + trees + max_depth)
+    model = _float_only_model(rng, n_float, trees, max_depth, scale=-0.5, bias=[2.0])
+    assert max(model["tree_sizes"]) > 8
+    x = rng.normal(size=(docs, n_float)).astype(np.float32)
+    x[rng.random(x.shape) < 0.01] = np.nan
+    o = OracleModel(model)
+    g = _gpu_model(model)
+    evaluate = g.evaluator().describe_kernels(cb.LAYOUT_FLAT_ROWS, docs)["evaluate"]
+    kernel = evaluate.split(" ")[0]
+    assert "_l1024" in kernel and kernel.endswith("_s") == (six == "1"), evaluate
+    expected = o.calc(x)
+    got = g.calc_flat(x)
+    if small_batch == "0":
+        np.testing.assert_array_equal(got, expected)
+    else:
+        assert " slices" in evaluate, evaluate
+        _close(got, expected)
+    np.testing.assert_array_equal(g.calc_leaf_indexes_flat(x), o.leaf_indexes(x))
+    n = len(model["tree_sizes"])
+    for begin, end in ((1, n - 1), (0, n // 2), (n // 2, n), (5, 6)):
+        if begin < end <= n:
+            np.testing.assert_array_equal(g.calc_flat(x, tree_start=begin, tree_end=end),
+                                          o.calc(x, tree_start=begin, tree_end=end), err_msg="trees %d..%d" % (begin, end))
+
+
+@pytest.mark.parametrize("six", ["1", "0"])
 @pytest.mark.parametrize("dim,max_depth,n_float,trees,docs", [
     (2, 6, 10, 20, 1000), (3, 6, 30, 33, 3000), (5, 8, 12, 9, 700), (6, 6, 128, 50, 2500), (7, 8, 100, 21, 1300),
     (10, 6, 100, 100, 5000), (13, 8, 60, 18, 900), (20, 6, 40, 30, 2049), (4, 6, 160, 60, 600), (2, 8, 192, 70, 600),
