@@ -1,6 +1,8 @@
 """Writes the gfx950 assembly of the register-resident evaluate kernels.
 
-The kernels evaluate oblivious trees of depth <= 8. The plain variants take models whose bins and
+The kernels evaluate oblivious trees of depth <= 8 (LEAVES = 64 or 256; LEAVES = 1024: depth <= 10, one
+dimension, plain and six-bit forms, level tables of 32 dwords of which the first 20 are used, the two extra
+levels' bits in a second index byte per document). The plain variants take models whose bins and
 split indexes all fit 7 bits (no xor masks), the case of float-feature models with at most 127
 used borders per feature; the "_s" variants take such models when no feature uses more than 63
 borders, which lets two levels share their merge; the "_m" (mixed) variants take any bins and xor masks (one-hot splits)
