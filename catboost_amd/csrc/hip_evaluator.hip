@@ -906,16 +906,14 @@ struct THipEvaluator::TImpl {
     hipModule_t RegModule = nullptr;
     hipFunction_t RegFunction = nullptr;
     uint32_t RegWaves = 0;
-    uint32_t RegPitch = 1;
     uint32_t RegTreeBlocks = 0;
     uint32_t RegTreeBlockSize = 16;   // trees per LDS buffer of the chosen kernel
     uint32_t RegRowDwords = 16;       // dwords of a tree's level table
-    size_t RegTreeLeafDoubles = 256;  // doubles of a tree's leaf table (leaf rows x pitch)
     size_t RegLaunchLeaves = 0;  // doubles of the leaf table of one launch
     TDeviceVec<uint32_t> RegRows;
     TDeviceVec<double> RegLeaves;  // [launch][tree][leaf row][pitch]
     TDeviceVec<double> RegBias;    // the bias, readable for a whole pitch behind every dimension
-    // The launches of a pass over the trees: RegPitch dimensions each, the last one with the narrowest kernel that
+    // The launches of a pass over the trees: the kernel's pitch in dimensions each, the last one with the narrowest kernel that
     // holds what is left (ten dimensions: six, then four instead of six of which two are padding).
     struct TRegLaunch {
         hipFunction_t Function = nullptr;
@@ -1501,9 +1499,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         const size_t rowDwords = variant->Mixed || variant->Leaves > 256 ? 32 : 16;
         const int rowLevels = variant->Leaves > 256 ? 10 : 8;
         m.RegWaves = variant->Waves;
-        m.RegPitch = variant->Pitch;
         m.RegRowDwords = static_cast<uint32_t>(rowDwords);
-        m.RegTreeLeafDoubles = rowsPerTree * pitch;
         m.RegTreeBlocks = static_cast<uint32_t>((TreeCount + block - 1) / block);
         // two blocks of null trees behind the last one: the kernels prefetch that far
         const size_t tableTrees = (static_cast<size_t>(m.RegTreeBlocks) + 2) * block;
@@ -2102,7 +2098,7 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
     const dev::TTreeTables tt = m.TreeTables();
     const uint32_t tb = static_cast<uint32_t>(treeStart), te = static_cast<uint32_t>(treeEnd);
     if (m.RegKernelUsable) {
-        // Bins kept in registers, RegPitch dimensions per launch. A launch addresses its results with 32
+        // Bins kept in registers, a launch per group of dimensions (RegLaunches). A launch addresses its results with 32
         // bits, so a very large batch goes in slices of whole document blocks.
         const size_t sliceDocs = ((size_t(1) << 29) - 1) / m.Dim / dev::kDocsPerBlock * dev::kDocsPerBlock;
         if (docCount > sliceDocs) {
