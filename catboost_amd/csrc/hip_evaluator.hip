@@ -464,14 +464,94 @@ int TileChunk(int dim) {
 // node's own leaf (NonSymmetricNodeIdToLeafId). A zero side becomes a terminal entry of its own.
 // usable = false when a tree does not fit the 16-bit offsets of an entry.
 // The compact tables (EvalNonSymmetricLdsKernel) are filled when the model is one-dimensional,
-// has no xor masks, at most 1023 buckets and no tree above dev::kNsLdsEntries entries.
+// has at most 1023 buckets and no tree above dev::kNsLdsEntries entries (one-hot splits count two).
 void BuildLevelOrderTrees(const TModelTrees& trees, int dim, const std::vector<uint32_t>& firstLeaf,
                           TDeviceVec<uint32_t>* entriesOut, TDeviceVec<uint32_t>* rowsOut, bool* usable, bool* noXor,
                           std::vector<uint32_t>* compactEntries, std::vector<uint32_t>* compactRows,
                           std::vector<double>* valuesByEntry, bool* compactUsable) {
     struct TItem {
-        uint32_t Node;   // model node, or the parent node of a synthetic terminal
+        uint32_t Node;        // model node, or the parent node of a synthetic terminal
         bool Terminal;
+        bool Second = false;     // the second test of a one-hot split taken apart (see unfold)
+        uint32_t LeftEntry = 0;  // of a second test: the entry of the split's left side
+        int64_t CopyOf = -1;     // an entry that repeats an earlier one of the tree: same test, same children
+    };
+    struct TUnfolded {
+        std::vector<TItem> Order;                                // breadth first, the two children of an entry side by side
+        std::vector<uint32_t> Level;
+        std::vector<std::pair<uint32_t, uint32_t>> Children;     // entry index of (false side, true side); terminals: unused
+        uint32_t Height = 0;
+        bool Fits = true;
+    };
+    // Breadth-first order of a tree's entries. A tree whose nodes share children (the loader only checks that
+    // every step stays inside the tree) unfolds into more entries than it has nodes, up to 2^depth: the walk
+    // stops as soon as the entries no longer fit the 16-bit offsets, and the model goes to the kernel that
+    // follows the step nodes.
+    // splitOneHot: the compact entries only know "bin >= splitIdx". A one-hot split, bin == v, becomes two of
+    // them: "bin >= v" (false: the model's left side) and behind its true side "bin >= v + 1" (false: the
+    // model's right side, the bins are equal; true: the left side again). The entry of the left side is
+    // repeated there, not its subtree: the copy names the same pair of children.
+    const auto unfold = [&](uint32_t root, bool splitOneHot) {
+        TUnfolded u;
+        u.Order.push_back({root, false});
+        u.Level.push_back(0);
+        for (size_t i = 0; i < u.Order.size() && u.Order.size() * 8 <= 0xffffu; ++i) {
+            if (u.Order[i].CopyOf >= 0) {
+                const size_t original = static_cast<size_t>(u.Order[i].CopyOf);  // an earlier index: already visited
+                const int64_t keep = u.Order[i].CopyOf;
+                u.Order[i] = u.Order[original];
+                u.Order[i].CopyOf = keep;
+                u.Children.push_back(u.Children[original]);
+                if (u.Order[i].Terminal) {
+                    u.Height = std::max(u.Height, u.Level[i]);
+                }
+                continue;
+            }
+            const TItem item = u.Order[i];
+            const auto& st = trees.NonSymmetricStepNodes[item.Node];
+            const bool terminal = item.Terminal || (!item.Second && st.LeftSubtreeDiff == 0 && st.RightSubtreeDiff == 0);
+            u.Order[i].Terminal = terminal;
+            if (terminal) {
+                u.Height = std::max(u.Height, u.Level[i]);
+                u.Children.emplace_back(0, 0);
+                continue;
+            }
+            const uint32_t diffs[2] = {st.LeftSubtreeDiff, st.RightSubtreeDiff};
+            const auto pushSide = [&](int side) {
+                const uint32_t index = static_cast<uint32_t>(u.Order.size());
+                if (diffs[side] == 0) {
+                    u.Order.push_back({item.Node, true});
+                } else {
+                    u.Order.push_back({item.Node + diffs[side], false});
+                }
+                u.Level.push_back(u.Level[i] + 1);
+                return index;
+            };
+            const bool oneHot = splitOneHot && trees.RepackedBins[item.Node].XorMask != 0;
+            uint32_t child[2];
+            if (!oneHot) {
+                child[0] = pushSide(0);
+                child[1] = pushSide(1);
+            } else if (!item.Second) {
+                child[0] = pushSide(0);
+                child[1] = static_cast<uint32_t>(u.Order.size());
+                TItem second{item.Node, false};
+                second.Second = true;
+                second.LeftEntry = child[0];
+                u.Order.push_back(second);
+                u.Level.push_back(u.Level[i] + 1);
+            } else {
+                child[0] = pushSide(1);
+                child[1] = static_cast<uint32_t>(u.Order.size());
+                TItem copy{item.Node, false};
+                copy.CopyOf = item.LeftEntry;
+                u.Order.push_back(copy);
+                u.Level.push_back(u.Level[i] + 1);
+            }
+            u.Children.emplace_back(child[0], child[1]);
+        }
+        u.Fits = u.Order.size() * 8 <= 0xffffu;
+        return u;
     };
     const size_t treeCount = trees.GetTreeCount();
     *noXor = true;
@@ -480,46 +560,18 @@ void BuildLevelOrderTrees(const TModelTrees& trees, int dim, const std::vector<u
     }
     std::vector<uint32_t> entries, rows(treeCount * 4, 0);
     *usable = true;
-    *compactUsable = *noXor && dim == 1 && trees.EffectiveBinFeaturesBucketCount <= 1023;
+    *compactUsable = dim == 1 && trees.EffectiveBinFeaturesBucketCount <= 1023;
     compactRows->assign(treeCount * 4, 0);
     for (size_t t = 0; t < treeCount && *usable; ++t) {
         const uint32_t root = static_cast<uint32_t>(trees.TreeStartOffsets[t]);
         const size_t firstEntry = entries.size() / 2;
-        std::vector<TItem> order = {{root, false}};
-        std::vector<uint32_t> level = {0};
-        uint32_t height = 0;
-        // first pass: breadth-first order; second pass below fills the entries
-        std::vector<std::pair<uint32_t, uint32_t>> children;  // entry index of (left, right); terminals: unused
-        // A tree whose nodes share children (the loader only checks that every step stays inside the tree)
-        // unfolds into more entries than it has nodes, up to 2^depth: the walk stops as soon as the entries
-        // no longer fit the 16-bit offsets, and the model goes to the kernel that follows the step nodes.
-        for (size_t i = 0; i < order.size() && order.size() * 8 <= 0xffffu; ++i) {
-            const TItem item = order[i];
-            const auto& st = trees.NonSymmetricStepNodes[item.Node];
-            const bool terminal = item.Terminal || (st.LeftSubtreeDiff == 0 && st.RightSubtreeDiff == 0);
-            order[i].Terminal = terminal;
-            if (terminal) {
-                height = std::max(height, level[i]);
-                children.emplace_back(0, 0);
-                continue;
-            }
-            uint32_t child[2];
-            const uint32_t diffs[2] = {st.LeftSubtreeDiff, st.RightSubtreeDiff};
-            for (int side = 0; side < 2; ++side) {
-                child[side] = static_cast<uint32_t>(order.size());
-                if (diffs[side] == 0) {
-                    order.push_back({item.Node, true});
-                } else {
-                    order.push_back({item.Node + diffs[side], false});
-                }
-                level.push_back(level[i] + 1);
-            }
-            children.emplace_back(child[0], child[1]);
-        }
-        if (order.size() * 8 > 0xffffu) {
+        const TUnfolded plain = unfold(root, false);
+        if (!plain.Fits) {
             *usable = false;
             break;
         }
+        const std::vector<TItem>& order = plain.Order;
+        const auto& children = plain.Children;
         for (size_t i = 0; i < order.size(); ++i) {
             const TItem item = order[i];
             uint32_t x, y;
@@ -542,17 +594,23 @@ void BuildLevelOrderTrees(const TModelTrees& trees, int dim, const std::vector<u
             entries.push_back(y);
         }
         rows[t * 4 + 0] = static_cast<uint32_t>(firstEntry);
-        rows[t * 4 + 1] = height;
+        rows[t * 4 + 1] = plain.Height;
         rows[t * 4 + 2] = firstLeaf[t];
         // compact layout: root at 0, entry 1 unused, so that every pair of children starts even
-        *compactUsable = *compactUsable && *usable && order.size() + 1 <= static_cast<size_t>(dev::kNsLdsEntries);
+        if (!*compactUsable || !*usable) {
+            *compactUsable = false;
+            continue;
+        }
+        const TUnfolded split = *noXor ? TUnfolded() : unfold(root, true);
+        const TUnfolded& compact = *noXor ? plain : split;
+        *compactUsable = compact.Fits && compact.Order.size() + 1 <= static_cast<size_t>(dev::kNsLdsEntries);
         if (*compactUsable) {
             const auto compactIndex = [](size_t i) { return static_cast<uint32_t>(i == 0 ? 0 : i + 1); };
             (*compactRows)[t * 4 + 0] = static_cast<uint32_t>(compactEntries->size());
-            (*compactRows)[t * 4 + 1] = height;
-            (*compactRows)[t * 4 + 2] = static_cast<uint32_t>(order.size() + 1);
-            for (size_t i = 0; i < order.size(); ++i) {
-                const TItem item = order[i];
+            (*compactRows)[t * 4 + 1] = compact.Height;
+            (*compactRows)[t * 4 + 2] = static_cast<uint32_t>(compact.Order.size() + 1);
+            for (size_t i = 0; i < compact.Order.size(); ++i) {
+                const TItem item = compact.Order[i];
                 const uint32_t self = compactIndex(i);
                 if (item.Terminal) {
                     const bool odd = (self & 1u) != 0;
@@ -560,10 +618,16 @@ void BuildLevelOrderTrees(const TModelTrees& trees, int dim, const std::vector<u
                     valuesByEntry->push_back(trees.LeafValues[trees.NonSymmetricNodeIdToLeafId[item.Node]]);
                 } else {
                     const auto& rb = trees.RepackedBins[item.Node];
-                    // the right child always follows the left one in `order`
-                    compactEntries->push_back(static_cast<uint32_t>(rb.SplitIdx) |
-                                              (static_cast<uint32_t>(rb.FeatureIndex) << 8) |
-                                              (compactIndex(children[i].first) << 21));
+                    // a one-hot split holds ~value in its xor mask (and 255 as its split index)
+                    uint32_t splitIdx = rb.SplitIdx;
+                    if (rb.XorMask != 0) {
+                        const uint32_t value = (~static_cast<uint32_t>(rb.XorMask)) & 0xffu;
+                        splitIdx = item.Second ? value + 1 : value;
+                        *compactUsable = *compactUsable && splitIdx <= 255;
+                    }
+                    // the true side always follows the false side in the order
+                    compactEntries->push_back(splitIdx | (static_cast<uint32_t>(rb.FeatureIndex) << 8) |
+                                              (compactIndex(compact.Children[i].first) << 21));
                     valuesByEntry->push_back(0.0);
                 }
                 if (i == 0) {

@@ -103,6 +103,28 @@ def test_simple_asymmetric_model():
     np.testing.assert_array_equal(r.calc_flat(rm.DATA), rm.ASYMMETRIC_PREDICTIONS)
 
 
+@pytest.mark.parametrize("seed,n_float,n_cat,trees,max_depth,docs", [
+    (1, 20, 6, 90, 8, 3000), (2, 150, 3, 40, 9, 1000), (3, 4, 10, 25, 6, 257), (4, 30, 2, 300, 5, 5000),
+])
+def test_non_symmetric_models_with_one_hot_splits(seed, n_float, n_cat, trees, max_depth, docs):
+    """One-dimensional non-symmetric models with one-hot splits walk out of LDS like float-only ones: the tables
+    of that kernel hold a one-hot split (bin == v) as two tests, bin >= v and behind it bin >= v + 1, with the
+    left side's entry repeated. Bins and leaf indexes equal the oracle's, predictions within the tolerance
+    (partial sums per wave)."""
+    rng = np.random.default_rng(seed)
+    model, cat_values = _random_oblivious(rng, n_float=n_float, n_cat=n_cat, trees=trees, max_depth=max_depth,
+                                          scale=0.5, bias=rng.normal(size=1))
+    model = mb.convert_oblivious_to_asymmetric(model)
+    assert any(len(f["values"]) for f in model["one_hot_features"]), "the model needs one-hot splits"
+    x = _random_flat_data(rng, model, cat_values, docs)
+    o = OracleModel(model)
+    g = _gpu_model(model)
+    assert "EvalNonSymmetricLdsKernel" in g.evaluator().describe_kernels(cb.LAYOUT_FLAT_ROWS, docs)["evaluate"]
+    np.testing.assert_array_equal(g.quantize_flat(x), o.binarize(x))
+    np.testing.assert_array_equal(g.calc_leaf_indexes_flat(x), o.leaf_indexes(x))
+    _close(g.calc_flat(x), o.calc(x))
+
+
 def test_non_symmetric_tree_whose_nodes_share_children():
     """A chain of 60 nodes in which both steps of every node lead to the next one passes the loader's
     range checks; unfolded level by level it would have 2^60 entries. The level-order tables give up
