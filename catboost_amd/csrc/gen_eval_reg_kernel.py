@@ -44,7 +44,9 @@ Kernel arguments (80 bytes):
   48 scale       double          56 bias const double* (first dimension of this launch)
   64 bucketCount uint32 (1 .. BUCKETS)                68 dim uint32
   72 first dimension of this launch uint32            76 dimensions to store uint32 (1 .. PITCH)
-  80 tree blocks per slice uint32 (kernels that are not fused; 88 bytes in all)
+  80 tree blocks per slice uint32 (kernels that are not fused)
+  88 map of the bins registers const uint32* (plain and six-bit kernels that are not fused, read when
+     flags bit 3 is set; 96 bytes in all)
 grid = (ceil(blockCount / WAVES), slices) workgroups of WAVES * 64 threads, LDS = 2 * TREE_BLOCK * LEAVES *
 PITCH * 8 bytes. Slice y of the grid takes the tree blocks from y * (tree blocks per slice) on, at most that
 many, and writes to out + y * docCount * dim: a small batch is spread over the chip by giving every slice
@@ -591,6 +593,9 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
         e("  s_add_u32 s32, s4, s30")
         e("  s_addc_u32 s33, s5, s31")
         e("  s_add_u32 s28, s96, -1")
+        if not mixed:
+            e("  s_bitcmp1_b32 s15, 3")
+            e("  s_cbranch_scc1 %s_mapped" % name)
         for i in range(buckets):
             # registers past the model's bucket count reload the last bucket and are never indexed
             e("  s_min_u32 s24, %d, s28" % i)
@@ -598,6 +603,58 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
             e("  s_add_u32 s34, s32, s24")
             e("  s_addc_u32 s35, s33, 0")
             e("  global_load_dword v%d, v1, s[34:35]" % (b0 + i))
+        if not mixed:
+            # Flags bit 3: the bins registers follow a map, one dword per register: bits 0..15 the bucket it
+            # is loaded from, bits 16.. what becomes of the bins there: 0 as they are, 1 min(bin, 127), 2
+            # max(bin - 127, 0). A bucket with more than 127 values then takes two registers, and a level
+            # "bin >= s" reads the first (s <= 127) or the second (with s - 127): every model without xor
+            # masks runs in the 7-bit form. The map has ceil(BUCKETS / 16) * 16 entries.
+            e("  s_branch %s_loaded" % name)
+            e("%s_mapped:" % name)
+            e("  s_load_dwordx2 s[52:53], s[0:1], 0x58")
+            e("  s_mov_b32 s25, 0x7f7f7f7f")
+            batches = (buckets + 15) // 16
+            for batch in range(batches):
+                e("  s_waitcnt lgkmcnt(0)")
+                e("  s_load_dwordx16 s[36:51], s[52:53], 0x%x" % (64 * batch))
+                e("  s_waitcnt lgkmcnt(0)")
+                for k in range(16):
+                    i = 16 * batch + k
+                    if i >= buckets:
+                        break
+                    e("  s_and_b32 s24, s%d, 0xffff" % (36 + k))
+                    e("  s_lshl_b32 s24, s24, 8")
+                    e("  s_add_u32 s34, s32, s24")
+                    e("  s_addc_u32 s35, s33, 0")
+                    e("  global_load_dword v%d, v1, s[34:35]" % (b0 + i))
+            e("  s_waitcnt vmcnt(0)")
+            for batch in range(batches):
+                e("  s_load_dwordx16 s[36:51], s[52:53], 0x%x" % (64 * batch))
+                e("  s_waitcnt lgkmcnt(0)")
+                for k in range(16):
+                    i = 16 * batch + k
+                    if i >= buckets:
+                        break
+                    reg = b0 + i
+                    label = "%s_map%d" % (name, i)
+                    e("  s_lshr_b32 s24, s%d, 16" % (36 + k))
+                    e("  s_cmp_eq_u32 s24, 0")
+                    e("  s_cbranch_scc1 %s" % label)
+                    # bytes of 128 and more -> 0xff
+                    e("  v_and_b32_e32 v4, 0x80808080, v%d" % reg)
+                    e("  v_lshrrev_b32_e32 v5, 7, v4")
+                    e("  v_sub_u32_e32 v5, v4, v5")
+                    e("  v_or_b32_e32 v4, v4, v5")
+                    e("  s_cmp_eq_u32 s24, 1")
+                    e("  s_cbranch_scc1 %s_low" % label)
+                    e("  v_and_b32_e32 v5, 0x7f7f7f7f, v%d" % reg)      # those bytes: (bin & 127) + 1 = bin - 127
+                    e("  v_add_u32_e32 v5, 0x1010101, v5")
+                    e("  v_and_b32_e32 v%d, v4, v5" % reg)
+                    e("  s_branch %s" % label)
+                    e("%s_low:" % label)
+                    e("  v_bfi_b32 v%d, v4, s25, v%d" % (reg, reg))      # those bytes: 127
+                    e("%s:" % label)
+            e("%s_loaded:" % name)
     load_rows(rows_a, 0)
     load_rows(rows_b, 1)
     for r in range(lv0, ga0):
@@ -746,7 +803,7 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
     e(".amdhsa_kernel %s" % name)
     e("  .amdhsa_group_segment_fixed_size %d" % lds_bytes)
     e("  .amdhsa_private_segment_fixed_size 0")
-    e("  .amdhsa_kernarg_size %d" % (104 if fused else 88))
+    e("  .amdhsa_kernarg_size %d" % (104 if fused else 96))
     e("  .amdhsa_user_sgpr_count 2")
     e("  .amdhsa_user_sgpr_kernarg_segment_ptr 1")
     e("  .amdhsa_system_sgpr_workgroup_id_x 1")
@@ -801,7 +858,8 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
       - {.offset: 100, .size: 4, .value_kind: by_value}
 """ if fused else """      - {.offset: 80, .size: 4, .value_kind: by_value}
       - {.offset: 84, .size: 4, .value_kind: by_value}
-""", lds_bytes, 104 if fused else 88, threads, name, name, vgprs)
+      - {.address_space: global, .offset: 88, .size: 8, .value_kind: global_buffer}
+""", lds_bytes, 104 if fused else 96, threads, name, name, vgprs)
     return "\n".join(o), meta
 
 

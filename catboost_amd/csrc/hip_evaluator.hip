@@ -162,8 +162,12 @@ struct TEvalRegLaunchArgs {
     TEvalRegArgs Reg;
     uint32_t TreeBlocksPerSlice;  // grid.y slices of the trees; one slice: all tree blocks
     uint32_t Padding;
+    const uint32_t* RegMap;       // read when Reg.Flags has kRegFlagMapped: where each bins register comes from
 };
-static_assert(sizeof(TEvalRegLaunchArgs) == 88, "kernel argument block of the register-resident kernels");
+static_assert(sizeof(TEvalRegLaunchArgs) == 96, "kernel argument block of the register-resident kernels");
+constexpr uint32_t kRegFlagMapped = 8;
+// what a mapped bins register holds of its bucket's bins (bits 16.. of a map entry)
+constexpr uint32_t kRegMapAsIs = 0, kRegMapLow = 1, kRegMapHigh = 2;  // bin, min(bin, 127), max(bin - 127, 0)
 
 struct TEvalRegVariant {
     uint32_t Buckets;
@@ -288,6 +292,7 @@ struct TKernelSwitches {
     bool SmallBatch = true;       // CATBOOST_AMD_SMALL_BATCH=0: small batches are not spread over slices of the trees
     bool LevelOrder = true;       // CATBOOST_AMD_LEVEL_ORDER=0: register kernels keep the model's order of a tree's levels
     bool PairTile = true;         // CATBOOST_AMD_PAIR_TILE=0: the half-tile kernel with one tree per wave
+    bool RegSplit = true;         // CATBOOST_AMD_REG_SPLIT=0: buckets of more than 127 values send a model to the mixed kernels
     uint32_t NsWaves = 0;         // CATBOOST_AMD_NS_WAVES=8|12|16: that shape of the non-symmetric LDS kernel or none
 
     static TKernelSwitches FromEnvironment() {
@@ -303,6 +308,7 @@ struct TKernelSwitches {
         k.LevelOrder = !off("CATBOOST_AMD_LEVEL_ORDER");
         k.SmallBatch = !off("CATBOOST_AMD_SMALL_BATCH");
         k.PairTile = !off("CATBOOST_AMD_PAIR_TILE");
+        k.RegSplit = !off("CATBOOST_AMD_REG_SPLIT");
         if (const char* v = std::getenv("CATBOOST_AMD_NS_WAVES")) {
             k.NsWaves = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
         }
@@ -991,6 +997,9 @@ struct THipEvaluator::TImpl {
     };
     std::vector<TRegLaunch> RegLaunches;
     TDeviceVec<double> RegTailLeaves;  // leaf table of a last launch that uses another kernel
+    // Models without xor masks whose buckets hold more than 127 values: such a bucket takes two bins registers,
+    // min(bin, 127) and max(bin - 127, 0), so that every level is a 7-bit compare (the kernels' register map)
+    TDeviceVec<uint32_t> RegMap;
 
     // fused kernels, per row layout (0: flat rows, 1: split rows of a model without categorical features)
     struct TFused {
@@ -1550,6 +1559,28 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
             ? PickRegVariant(m.LayoutBuckets, static_cast<uint32_t>(m.Dim), m.MaxDepth, !m.PackedSevenBit, six,
                              switches.RegMinBuckets)
             : nullptr;
+    // bins registers: one per bucket, or two for the buckets of more than 127 values when that keeps a model
+    // without xor masks off the 8-bit compare
+    std::vector<uint32_t> firstRegOfBucket(offsets.size(), 0), regMap;
+    bool regMapped = false;
+    if (m.Oblivious && m.MaxDepth <= kRegMaxDepth && TreeCount > 0 && !m.PackedSevenBit && !m.HasOneHot && switches.RegSplit) {
+        for (size_t b = 0; b + 1 < offsets.size(); ++b) {
+            firstRegOfBucket[b] = static_cast<uint32_t>(regMap.size());
+            if (offsets[b + 1] - offsets[b] <= 127) {
+                regMap.push_back(static_cast<uint32_t>(b) | (kRegMapAsIs << 16));
+            } else {
+                regMap.push_back(static_cast<uint32_t>(b) | (kRegMapLow << 16));
+                regMap.push_back(static_cast<uint32_t>(b) | (kRegMapHigh << 16));
+            }
+        }
+        const TEvalRegVariant* sevenBitVariant = PickRegVariant(static_cast<uint32_t>(regMap.size()), static_cast<uint32_t>(m.Dim),
+                                                                m.MaxDepth, false, false, switches.RegMinBuckets);
+        if (sevenBitVariant != nullptr) {
+            variant = sevenBitVariant;
+            regMapped = true;
+        }
+    }
+    const uint32_t regCount = regMapped ? static_cast<uint32_t>(regMap.size()) : m.LayoutBuckets;
     // a thread's 32-bit offset walks through the leaf table of a launch while it is copied to LDS
     const bool regTableAddressable =
         variant && (TreeCount / RegTreeBlock(*variant) + 3) * RegTreeBlock(*variant) * variant->Leaves * variant->Pitch * 8 <
@@ -1575,7 +1606,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         for (const auto& v : kEvalRegVariants) {
             if (m.Dim > 1 && v.Pitch > 1 && v.Pitch >= tailDims && v.Pitch < pitch && v.Leaves == variant->Leaves &&
                 v.Mixed == variant->Mixed && v.Six == variant->Six && v.Waves == variant->Waves &&
-                m.LayoutBuckets <= v.Buckets && (!tailVariant || v.Pitch < tailVariant->Pitch)) {
+                regCount <= v.Buckets && (!tailVariant || v.Pitch < tailVariant->Pitch)) {
                 tailVariant = &v;
             }
         }
@@ -1620,7 +1651,8 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
             bool sevenBit = true;
             for (int d = 0; d < depth; ++d) {
                 const auto& rb = levelAt(d);
-                sevenBit = sevenBit && rb.XorMask == 0 && offsets[rb.FeatureIndex + 1] - offsets[rb.FeatureIndex] <= 127;
+                sevenBit = sevenBit && rb.XorMask == 0 &&
+                           (regMapped || offsets[rb.FeatureIndex + 1] - offsets[rb.FeatureIndex] <= 127);
             }
             CBAMD_ENSURE(sevenBit || variant->Mixed, "internal error: tree needs the 8-bit compare");
             // a mixed model's bucket 0 may hold bins above 127, which the 7-bit padding level
@@ -1631,10 +1663,20 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
             if (sevenBit) {
                 for (int d = 0; d < depth; ++d) {
                     const auto& rb = levelAt(d);
-                    row[2 * d] = rb.FeatureIndex;
+                    // the register of the level's bins and the split index there: a bucket that takes two
+                    // registers answers "bin >= s" in the first for s <= 127 and as "bin - 127 >= s - 127" in the second
+                    uint32_t reg = rb.FeatureIndex, splitIdx = rb.SplitIdx;
+                    if (regMapped) {
+                        reg = firstRegOfBucket[rb.FeatureIndex];
+                        if (splitIdx > 127) {
+                            reg += 1;
+                            splitIdx -= 127;
+                        }
+                    }
+                    row[2 * d] = reg;
                     // the level's bit is the carry into bit 7; six-bit kernels want the even levels' in bit 6
                     // (of the first eight levels: levels 8 and 9 of a deep tree are read from bit 7 in every form)
-                    row[2 * d + 1] = ((variant->Six && d % 2 == 0 && d < 8 ? 64u : 128u) - rb.SplitIdx) * 0x01010101u;
+                    row[2 * d + 1] = ((variant->Six && d % 2 == 0 && d < 8 ? 64u : 128u) - splitIdx) * 0x01010101u;
                 }
                 for (int d = depth; d < rowLevels && depth > 0; ++d) {
                     row[2 * d] = row[0];
@@ -1684,6 +1726,11 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         if (tailVariant) {
             m.RegTailLeaves.Upload(tailLeaves);
         }
+        if (regMapped) {
+            // an entry per register of the largest kernel, in whole batches of sixteen; the spare ones load bucket 0
+            regMap.resize((224 + 15) / 16 * 16, 0);
+            m.RegMap.Upload(regMap);
+        }
         for (size_t launch = 0; launch < launches; ++launch) {
             TImpl::TRegLaunch l;
             l.FirstDim = static_cast<uint32_t>(launch * pitch);
@@ -1712,7 +1759,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         // consecutive columns = sixteen registers), so the level rows are rewritten per row layout.
         // (models that fit the 96-register shape stay on two launches: their evaluate kernel runs at four waves per
         // SIMD, a fused one at three, and is the faster - measured on 50 and 90 buckets)
-        const bool fusedCandidate = switches.Fused && !variant->Mixed && variant->Pitch == 1 && variant->Waves == 4 && variant->Leaves == 256 && m.Dim == 1 && !m.HasCats &&
+        const bool fusedCandidate = switches.Fused && !regMapped && !variant->Mixed && variant->Pitch == 1 && variant->Waves == 4 && variant->Leaves == 256 && m.Dim == 1 && !m.HasCats &&
                                     m.CtrCount == 0 && m.BinarizeBuckets == BucketCount && BucketCount > 0;
         for (int layoutIndex = 0; layoutIndex < 2 && fusedCandidate; ++layoutIndex) {
             const std::vector<uint32_t>& columns = layoutIndex == 0 ? srcFlat : srcSplit;
@@ -2215,7 +2262,8 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
         args.Out = results;
         args.DocCount = static_cast<uint32_t>(docCount);
         args.BlockCount = static_cast<uint32_t>((docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock);
-        args.Flags = (biased && !tail ? 1u : 0u) | (head ? 2u : 0u) | (tail ? 4u : 0u);
+        args.Flags = (biased && !tail ? 1u : 0u) | (head ? 2u : 0u) | (tail ? 4u : 0u) | (m.RegMap.Get() != nullptr ? kRegFlagMapped : 0u);
+        launchArgs.RegMap = m.RegMap.Get();
         args.Scale = m.Scale;
         args.BucketCount = m.LayoutBuckets;
         args.Dim = static_cast<uint32_t>(m.Dim);
@@ -2374,7 +2422,8 @@ void THipEvaluator::EvalQuantizedSlicedDevice(const uint8_t* bins, size_t docCou
     args.Out = partials;
     args.DocCount = static_cast<uint32_t>(docCount);
     args.BlockCount = static_cast<uint32_t>((docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock);
-    args.Flags = 4;  // raw sums per slice
+    args.Flags = 4 | (m.RegMap.Get() != nullptr ? kRegFlagMapped : 0u);  // raw sums per slice
+    launchArgs.RegMap = m.RegMap.Get();
     args.Scale = m.Scale;
     args.BucketCount = m.LayoutBuckets;
     args.Dim = static_cast<uint32_t>(m.Dim);

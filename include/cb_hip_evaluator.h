@@ -84,6 +84,8 @@ typedef struct CbHipFeatures {
  *   CATBOOST_AMD_REG_KERNEL=0        no register-resident assembly kernels (the LDS tile kernels instead)
  *   CATBOOST_AMD_REG_SIX=0           no six-bit form of the register-resident kernels
  *   CATBOOST_AMD_REG_MIN_BUCKETS=n   only register-resident kernel shapes that hold n buckets or more
+ *   CATBOOST_AMD_REG_SPLIT=0         a float feature with more than 127 used borders sends the model to the mixed
+ *                                    (8-bit compare) kernels instead of taking two bins registers
  *   CATBOOST_AMD_SMALL_BATCH=0       no slices of the trees for small batches, fused kernels for every batch size:
  *                                    every sum then has the CPU evaluator's order of additions
  *   CATBOOST_AMD_LEVEL_ORDER=0       register-resident kernels keep the model's order of a tree's levels

@@ -896,6 +896,44 @@ def test_register_kernel_border_counts(max_borders):
         np.testing.assert_array_equal(_gpu_model(m).quantize_flat(xx), OracleModel(m).binarize(xx))
 
 
+@pytest.mark.parametrize("split", ["1", "0"])
+@pytest.mark.parametrize("borders,n_float,dim,depth", [(128, 6, 1, 8), (200, 20, 1, 8), (254, 3, 1, 6), (254, 40, 3, 6),
+                                                       (300, 10, 1, 10)])
+def test_register_kernel_buckets_of_many_values(monkeypatch, split, borders, n_float, dim, depth):
+    """Float features with 128 and more used borders (values on the borders included, around the 127th above
+    all): a bucket of more than 127 values takes two bins registers, min(bin, 127) and max(bin - 127, 0), and the
+    model keeps the 7-bit compare; with the switch off it takes the 8-bit one of the mixed kernels. Bit for bit
+    either way (trees of depth 10 have no mixed kernel: those fall back to the plain evaluate kernel)."""
+    monkeypatch.setenv("CATBOOST_AMD_REG_SPLIT", split)
+    rng = np.random.default_rng(borders + n_float)
+    ffs = [mb.float_feature(i, i) for i in range(n_float)]
+    cands = [np.unique(rng.normal(size=4 * borders).astype(np.float32))[:borders] for _ in range(n_float)]
+    trees = []
+    for f in range(n_float):  # every border of every feature is used by some tree
+        for start in range(0, borders, depth):
+            splits = [("float", f, float(b)) for b in cands[f][start:start + depth]]
+            trees.append((splits, rng.normal(size=(1 << len(splits)) * dim)))
+    model = mb.build_oblivious(ffs, [], dim, trees, scale=0.5, bias=list(rng.normal(size=dim)))
+    assert max(len(f["borders"]) for f in model["float_features"]) == borders
+    x = rng.normal(size=(2500, n_float)).astype(np.float32)
+    for f in range(n_float):
+        x[:600, f] = rng.choice(cands[f][max(0, 120):min(borders, 135)], size=600)  # on the borders around the 127th
+    x[rng.random(x.shape) < 0.01] = np.nan
+    o = OracleModel(model)
+    g = _gpu_model(model)
+    evaluate = g.evaluator().describe_kernels(cb.LAYOUT_FLAT_ROWS, 2500)["evaluate"]
+    if depth <= 8 or split == "1":
+        assert evaluate.startswith("cbamd_eval_reg_"), evaluate
+        assert ("_m" in evaluate.split(" ")[0]) == (split == "0"), evaluate
+    np.testing.assert_array_equal(g.quantize_flat(x), o.binarize(x))
+    if evaluate.startswith("cbamd_eval_reg_"):
+        np.testing.assert_array_equal(g.calc_flat(x), o.calc(x))
+    else:
+        _close(g.calc_flat(x), o.calc(x))
+    n = len(model["tree_sizes"])
+    np.testing.assert_array_equal(g.calc_flat(x, tree_start=3, tree_end=n - 2), o.calc(x, tree_start=3, tree_end=n - 2))
+
+
 def test_register_kernel_against_tile_kernel():
     """The same model with the register-resident kernels switched off: both paths agree."""
     rng = np.random.default_rng(5)
