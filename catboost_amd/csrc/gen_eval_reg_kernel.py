@@ -45,8 +45,8 @@ Kernel arguments (80 bytes):
   64 bucketCount uint32 (1 .. BUCKETS)                68 dim uint32
   72 first dimension of this launch uint32            76 dimensions to store uint32 (1 .. PITCH)
   80 tree blocks per slice uint32 (kernels that are not fused)
-  88 map of the bins registers const uint32* (plain and six-bit kernels that are not fused, read when
-     flags bit 3 is set; 96 bytes in all)
+  88 map of the bins registers const uint32* (kernels that are not fused, read when flags bit 3 is set;
+     96 bytes in all)
 grid = (ceil(blockCount / WAVES), slices) workgroups of WAVES * 64 threads, LDS = 2 * TREE_BLOCK * LEAVES *
 PITCH * 8 bytes. Slice y of the grid takes the tree blocks from y * (tree blocks per slice) on, at most that
 many, and writes to out + y * docCount * dim: a small batch is spread over the chip by giving every slice
@@ -593,9 +593,8 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
         e("  s_add_u32 s32, s4, s30")
         e("  s_addc_u32 s33, s5, s31")
         e("  s_add_u32 s28, s96, -1")
-        if not mixed:
-            e("  s_bitcmp1_b32 s15, 3")
-            e("  s_cbranch_scc1 %s_mapped" % name)
+        e("  s_bitcmp1_b32 s15, 3")
+        e("  s_cbranch_scc1 %s_mapped" % name)
         for i in range(buckets):
             # registers past the model's bucket count reload the last bucket and are never indexed
             e("  s_min_u32 s24, %d, s28" % i)
@@ -603,11 +602,11 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
             e("  s_add_u32 s34, s32, s24")
             e("  s_addc_u32 s35, s33, 0")
             e("  global_load_dword v%d, v1, s[34:35]" % (b0 + i))
-        if not mixed:
+        if True:
             # Flags bit 3: the bins registers follow a map, one dword per register: bits 0..15 the bucket it
             # is loaded from, bits 16.. what becomes of the bins there: 0 as they are, 1 min(bin, 127), 2
-            # max(bin - 127, 0). A bucket with more than 127 values then takes two registers, and a level
-            # "bin >= s" reads the first (s <= 127) or the second (with s - 127): every model without xor
+            # max(bin - 127, 0). A float bucket with more than 127 values then takes two registers, and a level
+            # "bin >= s" reads the first (s <= 127) or the second (with s - 127): every tree without xor
             # masks runs in the 7-bit form. The map has ceil(BUCKETS / 16) * 16 entries.
             e("  s_branch %s_loaded" % name)
             e("%s_mapped:" % name)

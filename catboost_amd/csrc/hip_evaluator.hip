@@ -11,6 +11,7 @@
 #include <limits>
 #include <string>
 #include <thread>
+#include <tuple>
 #include <vector>
 
 // Bin buffer of the entry point that allocates nothing (THipEvaluator::CalcDeviceNoAlloc): every GPU the
@@ -1563,20 +1564,27 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
     // without xor masks off the 8-bit compare
     std::vector<uint32_t> firstRegOfBucket(offsets.size(), 0), regMap;
     bool regMapped = false;
-    if (m.Oblivious && m.MaxDepth <= kRegMaxDepth && TreeCount > 0 && !m.PackedSevenBit && !m.HasOneHot && switches.RegSplit) {
+    uint32_t maxFloatBucketValues = 0;
+    for (size_t b = 0; b + 1 < offsets.size(); ++b) {
+        if (!(flags[b] & dev::kBucketFlagOneHot)) {
+            maxFloatBucketValues = std::max(maxFloatBucketValues, offsets[b + 1] - offsets[b]);
+        }
+    }
+    if (m.Oblivious && m.MaxDepth <= kRegMaxDepth && TreeCount > 0 && maxFloatBucketValues > 127 && switches.RegSplit) {
         for (size_t b = 0; b + 1 < offsets.size(); ++b) {
             firstRegOfBucket[b] = static_cast<uint32_t>(regMap.size());
-            if (offsets[b + 1] - offsets[b] <= 127) {
+            if ((flags[b] & dev::kBucketFlagOneHot) || offsets[b + 1] - offsets[b] <= 127) {
                 regMap.push_back(static_cast<uint32_t>(b) | (kRegMapAsIs << 16));
             } else {
                 regMap.push_back(static_cast<uint32_t>(b) | (kRegMapLow << 16));
                 regMap.push_back(static_cast<uint32_t>(b) | (kRegMapHigh << 16));
             }
         }
-        const TEvalRegVariant* sevenBitVariant = PickRegVariant(static_cast<uint32_t>(regMap.size()), static_cast<uint32_t>(m.Dim),
-                                                                m.MaxDepth, false, false, switches.RegMinBuckets);
-        if (sevenBitVariant != nullptr) {
-            variant = sevenBitVariant;
+        // without one-hot splits the model is all 7-bit now; with them the trees that have none are
+        const TEvalRegVariant* splitVariant = PickRegVariant(static_cast<uint32_t>(regMap.size()), static_cast<uint32_t>(m.Dim),
+                                                             m.MaxDepth, m.HasOneHot, false, switches.RegMinBuckets);
+        if (splitVariant != nullptr) {
+            variant = splitVariant;
             regMapped = true;
         }
     }
@@ -1642,6 +1650,19 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
                 levelOrder[t].push_back(item.second);
             }
         }
+        // The register of a level's bins and the split index there: a float bucket that takes two registers answers
+        // "bin >= s" in the first for s <= 127 and as "bin - 127 >= s - 127" in the second.
+        const auto registerOf = [&](const TRepackedBin& rb) -> std::pair<uint32_t, uint32_t> {
+            uint32_t reg = rb.FeatureIndex, splitIdx = rb.SplitIdx;
+            if (regMapped) {
+                reg = firstRegOfBucket[rb.FeatureIndex];
+                if (rb.XorMask == 0 && splitIdx > 127 && !(flags[rb.FeatureIndex] & dev::kBucketFlagOneHot)) {
+                    reg += 1;
+                    splitIdx -= 127;
+                }
+            }
+            return {reg, splitIdx};
+        };
         for (size_t t = 0; t < TreeCount; ++t) {
             const int depth = trees.TreeSizes[t];
             const auto levelAt = [&](int position) -> const TRepackedBin& {
@@ -1663,16 +1684,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
             if (sevenBit) {
                 for (int d = 0; d < depth; ++d) {
                     const auto& rb = levelAt(d);
-                    // the register of the level's bins and the split index there: a bucket that takes two
-                    // registers answers "bin >= s" in the first for s <= 127 and as "bin - 127 >= s - 127" in the second
-                    uint32_t reg = rb.FeatureIndex, splitIdx = rb.SplitIdx;
-                    if (regMapped) {
-                        reg = firstRegOfBucket[rb.FeatureIndex];
-                        if (splitIdx > 127) {
-                            reg += 1;
-                            splitIdx -= 127;
-                        }
-                    }
+                    const auto [reg, splitIdx] = registerOf(rb);
                     row[2 * d] = reg;
                     // the level's bit is the carry into bit 7; six-bit kernels want the even levels' in bit 6
                     // (of the first eight levels: levels 8 and 9 of a deep tree are read from bit 7 in every form)
@@ -1687,9 +1699,8 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
                     uint32_t bucket = 0, xorMask = 0, splitIdx = 255;
                     if (d < depth) {
                         const auto& rb = levelAt(d);
-                        bucket = rb.FeatureIndex;
+                        std::tie(bucket, splitIdx) = registerOf(rb);
                         xorMask = rb.XorMask;
-                        splitIdx = rb.SplitIdx;
                     }
                     row[4 * d] = bucket;
                     row[4 * d + 1] = xorMask * 0x01010101u;
