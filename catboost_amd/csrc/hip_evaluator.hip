@@ -94,6 +94,25 @@ private:
 
 // A kernel that uses more than 64 KB of dynamic LDS has to be told so once (per device); the largest size asked
 // for so far is remembered, so that the attribute is not set again on every launch.
+// The code object of the assembly kernels, loaded once per device and kept for the life of the process: every
+// evaluator of a device shares it (a few megabytes of code and some milliseconds of loading otherwise per model).
+hipModule_t SharedRegModule(const void* image) {
+    static std::mutex lock;
+    static std::vector<std::pair<int, hipModule_t>> loaded;
+    int device = 0;
+    HIP_CHECK(hipGetDevice(&device));
+    std::lock_guard<std::mutex> guard(lock);
+    for (const auto& item : loaded) {
+        if (item.first == device) {
+            return item.second;
+        }
+    }
+    hipModule_t module = nullptr;
+    HIP_CHECK(hipModuleLoadData(&module, image));
+    loaded.emplace_back(device, module);
+    return module;
+}
+
 void EnsureDynamicLds(const void* kernel, size_t bytes) {
     if (bytes <= 64 * 1024) {
         return;
@@ -974,7 +993,7 @@ struct THipEvaluator::TImpl {
     // buckets fit the register file): level rows and leaf values at a fixed pitch per tree
     bool RegKernelUsable = false;
     bool SmallBatchSlices = true;  // small batches: slices of the trees on workgroups of their own
-    hipModule_t RegModule = nullptr;
+    hipModule_t RegModule = nullptr;  // the device's shared module (SharedRegModule), not owned
     hipFunction_t RegFunction = nullptr;
     uint32_t RegWaves = 0;
     uint32_t RegTreeBlocks = 0;
@@ -1171,9 +1190,6 @@ struct THipEvaluator::TImpl {
         Contexts.clear();
         if (Stream) {
             (void)hipStreamDestroy(Stream);
-        }
-        if (RegModule) {
-            (void)hipModuleUnload(RegModule);
         }
     }
 };
@@ -1594,7 +1610,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         variant && (TreeCount / RegTreeBlock(*variant) + 3) * RegTreeBlock(*variant) * variant->Leaves * variant->Pitch * 8 <
                        (uint64_t(1) << 32) - (1u << 20);
     if (regEnabled && variant && regTableAddressable) {
-        HIP_CHECK(hipModuleLoadData(&m.RegModule, kEvalRegCodeObject));
+        m.RegModule = SharedRegModule(kEvalRegCodeObject);
         HIP_CHECK(hipModuleGetFunction(&m.RegFunction, m.RegModule, variant->Name));
         m.RegKernelName = variant->Name;
         const uint32_t block = RegTreeBlock(*variant);
