@@ -2579,6 +2579,22 @@ void THipEvaluator::LeafIndexesQuantizedDevice(const uint8_t* bins, size_t docCo
     CBAMD_ENSURE(bins != nullptr && indexes != nullptr, "null pointer passed to leaf index calculation");
     hipStream_t s = m.Pick(stream);
     const size_t blocks = (docCount + 255) / 256;
+    const size_t tileLds = static_cast<size_t>(m.LayoutBuckets) * dev::kDocsPerBlock + dev::kWave * dev::kLeafIndexPitch * 4;
+    if (m.Oblivious && m.MaxDepth <= 8 && m.PackedTrees.Get() != nullptr && tileLds <= kMaxTileLdsBytes) {
+        const auto launch = [&](auto kernel) {
+            EnsureDynamicLds(reinterpret_cast<const void*>(kernel), tileLds);
+            hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(blocks)), dim3(256), tileLds, s,
+                               reinterpret_cast<const uint32_t*>(bins), docCount, m.LayoutBuckets, m.PackedTrees.Get(),
+                               static_cast<uint32_t>(treeStart), static_cast<uint32_t>(treeEnd), indexes);
+        };
+        if (m.PackedSevenBit) {
+            launch(dev::LeafIndexesTileKernel<true>);
+        } else {
+            launch(dev::LeafIndexesTileKernel<false>);
+        }
+        HIP_CHECK(hipGetLastError());
+        return;
+    }
     hipLaunchKernelGGL(dev::LeafIndexesKernel, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0, s, bins, docCount,
                        m.LayoutBuckets, m.TreeTables(), m.Oblivious ? 1 : 0, static_cast<uint32_t>(treeStart),
                        static_cast<uint32_t>(treeEnd), indexes);
@@ -2988,7 +3004,12 @@ void THipEvaluator::LeafIndexesHostRows(const float* const* rows, size_t rowLen,
             HIP_CHECK(hipEventRecord(slot.Ev[3], s));
         },
         [&](int i, size_t begin, size_t n) {
-            std::memcpy(indexes + begin * treeCount, ctx->Slots[i].PinnedIndexes.Get(), n * treeCount * sizeof(uint32_t));
+            // 4 bytes per document and tree: the copy out of the pinned buffer bounds this call, so it is shared out
+            uint32_t* dst = indexes + begin * treeCount;
+            const uint32_t* src = ctx->Slots[i].PinnedIndexes.Get();
+            ParallelCopy(n, n * treeCount * sizeof(uint32_t), [=](size_t first, size_t last) {
+                std::memcpy(dst + first * treeCount, src + first * treeCount, (last - first) * treeCount * sizeof(uint32_t));
+            });
         });
 }
 

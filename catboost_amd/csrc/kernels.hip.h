@@ -1744,6 +1744,58 @@ __global__ __launch_bounds__(256) void LeafIndexesKernel(const uint8_t* __restri
     }
 }
 
+// Leaf indexes of oblivious trees of depth <= 8 whose 256-document tile of bins fits LDS: the byte-parallel walk of
+// the tile kernel (four documents per lane, a tree per wave and turn), and rows of the output written whole. A
+// workgroup of four waves takes a block of 256 documents and the trees in groups of 64: wave w walks trees
+// 16 w .. 16 w + 15 of the group and leaves each tree's four index bytes per lane in LDS ([lane][tree], 65 dwords
+// per lane); then wave j writes, document by document, the 64 indexes of documents 64 j .. 64 j + 63: one 256-byte
+// store per document and group where the plain kernel stores four bytes per (document, tree) a row apart.
+// packedTrees as in EvalObliviousTileKernel. grid = doc blocks, block = 256, dynamic LDS = buckets * 256 + 64 * 65 * 4.
+constexpr int kLeafIndexGroup = 64;
+constexpr int kLeafIndexPitch = kLeafIndexGroup + 1;
+
+template <bool SEVEN_BIT>
+__global__ __launch_bounds__(256) void LeafIndexesTileKernel(const uint32_t* __restrict__ bins, size_t docCount,
+                                                             uint32_t bucketCount, const uint32_t* __restrict__ packedTrees,
+                                                             uint32_t treeBegin, uint32_t treeEnd,
+                                                             uint32_t* __restrict__ out) {
+    extern __shared__ uint32_t sTile[];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const size_t block = blockIdx.x;
+    const uint32_t tileDwords = bucketCount * kWave;
+    const uint32_t* src = bins + block * tileDwords;
+    for (uint32_t i = tid; i < tileDwords; i += 256) {
+        sTile[i] = src[i];
+    }
+    uint32_t* stage = sTile + tileDwords;
+    const uint8_t* laneTile = reinterpret_cast<const uint8_t*>(sTile) + lane * 4;
+    const uint32_t slot = lane & (kPackedTreeDwords - 1);
+    const size_t treeCount = treeEnd - treeBegin;
+    const size_t firstDoc = block * kDocsPerBlock + wave * kWave;  // of the 64 documents this wave writes
+    for (uint32_t group = treeBegin; group < treeEnd; group += kLeafIndexGroup) {
+        __syncthreads();  // the tile is loaded; the previous group's indexes are written
+        constexpr int kPerWave = kLeafIndexGroup / 4;
+#pragma unroll 4
+        for (int k = 0; k < kPerWave; ++k) {
+            const uint32_t t = group + wave * kPerWave + k;
+            if (t < treeEnd) {
+                const uint32_t row = packedTrees[static_cast<size_t>(t) * kPackedTreeDwords + slot];
+                stage[lane * kLeafIndexPitch + wave * kPerWave + k] = TreeIndexes<SEVEN_BIT, 8>(laneTile, row);
+            }
+        }
+        __syncthreads();
+        const uint32_t tree = group + lane;
+        for (uint32_t d = 0; d < kWave; ++d) {
+            const size_t doc = firstDoc + d;
+            if (doc < docCount && tree < treeEnd) {
+                out[doc * treeCount + (tree - treeBegin)] = (stage[d * kLeafIndexPitch + lane] >> (8 * wave)) & 0xffu;
+            }
+        }
+    }
+}
+
 // Re-lays bins out as the reference does: blocks of 128 documents, [block][bucket][doc in block],
 // the last block packed with its own document count (cpu/quantization.h:357-365).
 __global__ __launch_bounds__(256) void ExportBinsKernel(const uint8_t* __restrict__ bins, size_t docCount,
