@@ -450,6 +450,44 @@ __device__ __forceinline__ float CtrValue(const TCtrTablesDev& ctr, const TCtrFe
     return CtrCalc(f, static_cast<float>(n1), static_cast<float>(n0 + n1));
 }
 
+// Tables whose row is one or two dwords (all but the class histograms of more than two classes): the dwords of
+// a row, read once for all the features of the table, and the value of a feature from them (as CtrValue).
+__device__ __forceinline__ bool CtrRowIsShort(const TCtrFeatureDev& f) {
+    return (f.Type >= 2 && f.Type <= 5) || (f.Type != 1 && f.TargetClassesCount <= 2);
+}
+
+__device__ __forceinline__ uint2 CtrShortRow(const TCtrTablesDev& ctr, const TCtrFeatureDev& f, uint32_t row) {
+    const uint32_t* blob = ctr.Blob + f.BlobOffset;
+    if (row == kCtrNotFound) {
+        return make_uint2(0u, 0u);
+    }
+    if (f.Type == 4 || f.Type == 5) {
+        return make_uint2(blob[row], 0u);
+    }
+    return make_uint2(blob[2 * static_cast<size_t>(row)], blob[2 * static_cast<size_t>(row) + 1]);
+}
+
+__device__ __forceinline__ float CtrValueOfShortRow(const TCtrFeatureDev& f, uint32_t row, uint2 dwords) {
+    if (f.Type == 2 || f.Type == 3) {
+        if (row == kCtrNotFound) {
+            return CtrCalc(f, 0.f, 0.f);
+        }
+        return CtrCalc(f, __uint_as_float(dwords.x), static_cast<float>(static_cast<int32_t>(dwords.y)));
+    }
+    if (f.Type == 4 || f.Type == 5) {
+        const float denominator = static_cast<float>(f.CounterDenominator);
+        if (row == kCtrNotFound) {
+            return CtrCalc(f, 0.f, denominator);
+        }
+        return CtrCalc(f, static_cast<float>(static_cast<int32_t>(dwords.x)), denominator);
+    }
+    if (row == kCtrNotFound) {
+        return CtrCalc(f, 0.f, 0.f);
+    }
+    const int32_t n0 = static_cast<int32_t>(dwords.x), n1 = static_cast<int32_t>(dwords.y);
+    return CtrCalc(f, static_cast<float>(n1), static_cast<float>(n0 + n1));
+}
+
 // grid = (document blocks, CTR features), one wave per workgroup: lane l computes the CTR of documents
 // l, l + 64, l + 128, l + 192 of the block from the block's float / one-hot bins (already written)
 // and the hashed categorical values, and writes the bins of the CTR's buckets.
@@ -527,6 +565,9 @@ __global__ __launch_bounds__(256) void CtrBinarizeTileKernel(TCatSource cats, ui
     constexpr uint32_t kPerWave = kCtrGroup / 4;
     const uint32_t first = blockIdx.y * kCtrGroup + wave * kPerWave;
     uint64_t hash[4] = {0, 0, 0, 0};
+    uint32_t row[4] = {kCtrNotFound, kCtrNotFound, kCtrNotFound, kCtrNotFound};
+    uint2 rowDwords[4] = {};
+    uint32_t tableOfRows = 0;  // HashBuckets of the table that row[] was looked up in
     for (uint32_t k = 0; k < kPerWave && first + k < ctr.FeatureCount; ++k) {
         const TCtrFeatureDev f = ctr.Features[first + k];
         if (k == 0 || !f.SameProjectionAsPrevious) {
@@ -554,10 +595,25 @@ __global__ __launch_bounds__(256) void CtrBinarizeTileKernel(TCatSource cats, ui
                 }
             }
         }
+        // features that differ only in prior, target border, shift or scale read the same row of the same table
+        const bool shortRow = CtrRowIsShort(f);
+        if (k == 0 || !f.SameProjectionAsPrevious || f.HashBuckets != tableOfRows) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                row[j] = CtrTableRow(ctr, f, hash[j]);
+            }
+            if (shortRow) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    rowDwords[j] = CtrShortRow(ctr, f, row[j]);
+                }
+            }
+            tableOfRows = f.HashBuckets;
+        }
         float value[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            value[j] = CtrValue(ctr, f, CtrTableRow(ctr, f, hash[j]));
+            value[j] = shortRow ? CtrValueOfShortRow(f, row[j], rowDwords[j]) : CtrValue(ctr, f, row[j]);
         }
         for (uint32_t b = 0; b < f.BucketCount; ++b) {
             const uint32_t bucket = f.FirstBucket + b;
