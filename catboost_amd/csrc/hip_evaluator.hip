@@ -1990,6 +1990,38 @@ void LaunchBinarizeRows(uint32_t maxBucketValues, size_t blocks, const float* fl
     }
 }
 
+template <int LOG2P>
+void LaunchBinarizeColumnsP(size_t blocks, const float* floats, size_t stride, size_t docCount,
+                            const dev::TBinarizeTables& tab, uint32_t* bins, hipStream_t s) {
+    const size_t tiles = (tab.BucketCount + dev::kBucketTile - 1) / dev::kBucketTile;
+    const uint32_t blocksPerGroup = static_cast<uint32_t>(
+        std::max<size_t>(1, std::min<size_t>(kBinarizeBlocksPerGroup, blocks * tiles / 1024)));
+    const size_t groups = (blocks + blocksPerGroup - 1) / blocksPerGroup;
+    CBAMD_ENSURE(groups * tiles < (size_t(1) << 31), "batch is too large for one binarize launch");
+    const size_t lds = (static_cast<size_t>(dev::kBucketTile) << LOG2P) * 4 +
+                       static_cast<size_t>(dev::kBucketTile) * dev::kLutCells;
+    auto kernel = dev::BinarizeColumnsKernel<LOG2P>;
+    EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds);
+    hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(groups * tiles)), dim3(256), lds, s, floats, stride,
+                       static_cast<uint32_t>(docCount), tab, blocksPerGroup, bins);
+}
+
+// column-major documents: the same choice of LDS slots as for rows
+void LaunchBinarizeColumns(uint32_t maxBucketValues, size_t blocks, const float* floats, size_t stride,
+                           size_t docCount, const dev::TBinarizeTables& tab, uint32_t* bins, hipStream_t s) {
+    CBAMD_ENSURE(docCount < (size_t(1) << 31), "batch is too large for one binarize launch");
+    const int log2Slots = BinarizeLog2Slots(maxBucketValues);
+    if (log2Slots == 5) {
+        LaunchBinarizeColumnsP<5>(blocks, floats, stride, docCount, tab, bins, s);
+    } else if (log2Slots == 6) {
+        LaunchBinarizeColumnsP<6>(blocks, floats, stride, docCount, tab, bins, s);
+    } else if (log2Slots == 7) {
+        LaunchBinarizeColumnsP<7>(blocks, floats, stride, docCount, tab, bins, s);
+    } else {
+        LaunchBinarizeColumnsP<8>(blocks, floats, stride, docCount, tab, bins, s);
+    }
+}
+
 }  // namespace
 
 void THipEvaluator::QuantizeDevice(const TFeatureBatch& batch, size_t docCount, uint8_t* bins, void* stream) {
@@ -2039,9 +2071,8 @@ void THipEvaluator::QuantizeDevice(const TFeatureBatch& batch, size_t docCount, 
         case TFeatureBatch::FlatColumns: {
             CBAMD_ENSURE(batch.Stride >= docCount, "column stride is shorter than the document count");
             if (m.BinarizeBuckets > 0) {
-                const dim3 grid(static_cast<uint32_t>(blocks), (m.BinarizeBuckets + 3) / 4);
-                hipLaunchKernelGGL(dev::BinarizeColumnsKernel, grid, dim3(256), 0, s, batch.Floats, batch.Stride, docCount,
-                                   m.BinarizeTables(true), reinterpret_cast<uint32_t*>(bins));
+                LaunchBinarizeColumns(m.MaxBucketValues, blocks, batch.Floats, batch.Stride, docCount,
+                                      m.BinarizeTables(true), reinterpret_cast<uint32_t*>(bins), s);
             }
             break;
         }

@@ -272,53 +272,125 @@ __global__ __launch_bounds__(256) void BinarizeRowsKernel(const float* __restric
 #undef CBAMD_LOAD_BLOCK
 }
 
-// Column-major input: floats[column * stride + doc] (categorical hashes bit-cast in their column).
-// grid = (doc blocks, ceil(buckets / 4)), block = 256 threads: one wave per bucket.
+// Column-major input: floats[column * stride + doc] (categorical hashes bit-cast in their column). The work of a
+// workgroup is that of BinarizeRowsKernel - kBucketTile buckets, their borders and search tables in LDS,
+// `blocksPerGroup` consecutive 256-document blocks, every wave a bucket at a time for the block's 256 documents,
+// a lane its four documents side by side - without the tile: a lane's values are neighbours of the other lanes' in
+// the column, so they are loaded straight into registers, all buckets of the wave's turn before the first search.
+// grid = ceil(doc blocks / blocksPerGroup) * ceil(buckets / kBucketTile), block = 256 threads,
+// dynamic LDS = (kBucketTile << LOG2P) * 4 + kBucketTile * kLutCells bytes.
+template <int LOG2P>
 __global__ __launch_bounds__(256) void BinarizeColumnsKernel(const float* __restrict__ floats, size_t stride,
-                                                             size_t docCount, TBinarizeTables tab,
-                                                             uint32_t* __restrict__ bins) {
-    __shared__ uint32_t sValues[4][kMaxBucketValues];
+                                                             uint32_t docCount, TBinarizeTables tab,
+                                                             uint32_t blocksPerGroup, uint32_t* __restrict__ bins) {
+    constexpr uint32_t kSlots = 1u << LOG2P;
+    extern __shared__ uint32_t sBinarize[];
+    uint32_t* sValues = sBinarize;                      // [kBucketTile][kSlots]
+    uint32_t* sLut = sBinarize + kBucketTile * kSlots;  // [kBucketTile][kLutCells / 4]
     const uint32_t tid = threadIdx.x;
-    const uint32_t lane = tid & (kWave - 1);
-    const uint32_t wave = tid / kWave;
-    const size_t block = blockIdx.x;
-    const uint32_t bucket = blockIdx.y * 4 + wave;
-    const bool active = bucket < tab.BucketCount;
-    uint32_t off = 0, cnt = 0, flags = 0, src = 0;
-    if (active) {
-        off = tab.BucketOffset[bucket];
-        cnt = tab.BucketOffset[bucket + 1] - off;
-        flags = tab.BucketFlags[bucket];
-        src = tab.BucketSrc[bucket];
-    }
-    for (uint32_t k = lane; k < kMaxBucketValues; k += kWave) {
-        sValues[wave][k] = (k < cnt) ? tab.Values[off + k] : 0x7f800000u;
-    }
-    __syncthreads();
-    if (!active) {
-        return;
-    }
-    uint32_t packed = 0;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const size_t doc = block * kDocsPerBlock + j * kWave + lane;
-        uint32_t raw = 0;
-        if (doc < docCount) {
-            raw = __float_as_uint(floats[static_cast<size_t>(src) * stride + doc]);
-        }
-        uint32_t bin;
-        if (flags & kBucketFlagOneHot) {
-            bin = OneHotBin(sValues[wave], cnt, raw);
-        } else {
-            float v = __uint_as_float(raw);
-            if ((flags & kBucketFlagNanToInf) && isnan(v)) {
-                v = __uint_as_float(0x7f800000u);
+    const uint32_t tileCount = (tab.BucketCount + kBucketTile - 1) / kBucketTile;
+    const uint32_t b0 = (blockIdx.x % tileCount) * kBucketTile;
+    const uint32_t nb = min(static_cast<uint32_t>(kBucketTile), tab.BucketCount - b0);
+    const uint32_t blockCount = (docCount + kDocsPerBlock - 1) / kDocsPerBlock;
+    const uint32_t blockBegin = (blockIdx.x / tileCount) * blocksPerGroup;
+    const uint32_t blockEnd = min(blockBegin + blocksPerGroup, blockCount);
+    for (uint32_t i = tid; i < kBucketTile * kSlots; i += 256) {
+        const uint32_t bb = i >> LOG2P, k = i & (kSlots - 1);
+        uint32_t v = 0x7f800000u;  // +inf
+        if (bb < nb) {
+            const uint32_t off = tab.BucketOffset[b0 + bb];
+            const uint32_t cnt = tab.BucketOffset[b0 + bb + 1] - off;
+            if (k < cnt) {
+                v = tab.Values[off + k];
             }
-            bin = CountBelow<8>(sValues[wave], v);
         }
-        packed |= bin << (8 * j);
+        sValues[i] = v;
     }
-    bins[(block * tab.BucketPitch + bucket) * kWave + lane] = packed;
+    for (uint32_t i = tid; i < kBucketTile * (kLutCells / 4); i += 256) {
+        const uint32_t bb = i / (kLutCells / 4);
+        sLut[i] = bb < nb ? tab.Lut[static_cast<size_t>(b0) * (kLutCells / 4) + i] : 0u;
+    }
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    constexpr int kBucketsPerWave = kBucketTile / (256 / kWave);
+    uint32_t myFlags[kBucketsPerWave], myTopStep[kBucketsPerWave], myCount[kBucketsPerWave];
+    float myLo[kBucketsPerWave], myScale[kBucketsPerWave];
+    const uint32_t* myColumn[kBucketsPerWave];
+#pragma unroll
+    for (int k = 0; k < kBucketsPerWave; ++k) {
+        const uint32_t bucket = b0 + min(wave + k * (256 / kWave), nb - 1);
+        const uint4 grid = tab.Grid[bucket];
+        myFlags[k] = __builtin_amdgcn_readfirstlane(tab.BucketFlags[bucket]);
+        myLo[k] = __uint_as_float(__builtin_amdgcn_readfirstlane(grid.x));
+        myScale[k] = __uint_as_float(__builtin_amdgcn_readfirstlane(grid.y));
+        const uint32_t steps = __builtin_amdgcn_readfirstlane(grid.z);
+        myTopStep[k] = steps ? 1u << (steps - 1) : 0u;
+        myCount[k] = __builtin_amdgcn_readfirstlane(tab.BucketOffset[bucket + 1] - tab.BucketOffset[bucket]);
+        myColumn[k] = reinterpret_cast<const uint32_t*>(floats) +
+                      static_cast<size_t>(__builtin_amdgcn_readfirstlane(tab.BucketSrc[bucket])) * stride;
+    }
+    __syncthreads();  // the tables are in LDS
+    for (uint32_t block = blockBegin; block < blockEnd; ++block) {
+        // documents past the last one are read as the last one (their bins are never used)
+        uint32_t doc[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            doc[j] = min(block * kDocsPerBlock + j * kWave + lane, docCount - 1);
+        }
+        uint32_t raw[kBucketsPerWave][4];
+#pragma unroll
+        for (int k = 0; k < kBucketsPerWave; ++k) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                raw[k][j] = myColumn[k][doc[j]];
+            }
+        }
+        uint32_t* blockBins = bins + (static_cast<size_t>(block) * tab.BucketPitch + b0) * kWave + lane;
+#pragma unroll
+        for (int k = 0; k < kBucketsPerWave; ++k) {
+            const uint32_t bb = wave + k * (256 / kWave);
+            if (bb >= nb) {
+                break;
+            }
+            const uint32_t* values = sValues + bb * kSlots;
+            uint32_t packed = 0;
+            if (myFlags[k] & kBucketFlagOneHot) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    packed |= OneHotBin(values, myCount[k], raw[k][j]) << (8 * j);
+                }
+            } else {
+                const uint8_t* lut = reinterpret_cast<const uint8_t*>(sLut + bb * (kLutCells / 4));
+                float v[4];
+                uint32_t below[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    v[j] = __uint_as_float(raw[k][j]);
+                }
+                if (myFlags[k] & kBucketFlagNanToInf) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        v[j] = isnan(v[j]) ? __uint_as_float(0x7f800000u) : v[j];
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    below[j] = static_cast<uint32_t>(lut[GridCell(v[j], myLo[k], myScale[k])]) * 4;  // byte offsets
+                }
+                const uint8_t* valueBytes = reinterpret_cast<const uint8_t*>(values);
+                for (uint32_t step4 = __builtin_amdgcn_readfirstlane(myTopStep[k]) * 4; step4 >= 4; step4 >>= 1) {
+                    const uint8_t* probe = valueBytes + step4 - 4;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float b = *reinterpret_cast<const float*>(probe + below[j]);
+                        below[j] += (b < v[j]) ? step4 : 0u;
+                    }
+                }
+                packed = (below[0] >> 2) | (below[1] << 6) | (below[2] << 14) | (below[3] << 22);
+            }
+            blockBins[bb * kWave] = packed;
+        }
+    }
 }
 
 // ---- CTR (target statistics) features -------------------------------------------------------
