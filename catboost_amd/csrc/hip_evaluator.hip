@@ -313,7 +313,7 @@ struct TKernelSwitches {
     bool LevelOrder = true;       // CATBOOST_AMD_LEVEL_ORDER=0: register kernels keep the model's order of a tree's levels
     bool PairTile = true;         // CATBOOST_AMD_PAIR_TILE=0: the half-tile kernel with one tree per wave
     bool RegSplit = true;         // CATBOOST_AMD_REG_SPLIT=0: buckets of more than 127 values send a model to the mixed kernels
-    uint32_t NsWaves = 0;         // CATBOOST_AMD_NS_WAVES=8|12|16: that shape of the non-symmetric LDS kernel or none
+    uint32_t NsWaves = 0;         // CATBOOST_AMD_NS_WAVES=4|6|8|12|16: that shape of the non-symmetric LDS kernel or none
 
     static TKernelSwitches FromEnvironment() {
         const auto off = [](const char* name) {
@@ -410,17 +410,22 @@ size_t TileLdsBytes(uint32_t buckets, int dchunk) {
 
 // LDS of EvalNonSymmetricLdsKernel: 8 KB per wave (its entries, then rows of bins), the other rows of bins, the
 // accumulator
-size_t NsLdsKernelBytes(uint32_t buckets, uint32_t waves, uint32_t entries) {
-    return static_cast<size_t>(dev::NsLdsTileRows(buckets, waves, entries)) * 256 + dev::kDocsPerBlock * sizeof(double);
+size_t NsLdsKernelBytes(uint32_t buckets, uint32_t waves, uint32_t entries, uint32_t dims) {
+    return static_cast<size_t>(dev::NsLdsTileRows(buckets, waves, entries)) * 256 + dev::kDocsPerBlock * sizeof(double) * dims;
 }
 
 // The shapes of EvalNonSymmetricLdsKernel, most waves first
+// dimensions that one workgroup of EvalNonSymmetricLdsKernel sums (a model of more walks its trees once per slice)
+uint32_t NsLdsDims(int dim) {
+    return dim == 1 ? 1 : dim == 2 ? 2 : 4;
+}
+
 struct TNsLdsShape {
     uint32_t Waves;
     uint32_t Entries;
     double Speed;  // steps of a unit per unit of time, relative to the 8-wave shape
 };
-constexpr TNsLdsShape kNsLdsShapes[] = {{16, 1024, 1.45}, {12, 1536, 1.26}, {8, 2048, 1.0}};
+constexpr TNsLdsShape kNsLdsShapes[] = {{16, 1024, 1.45}, {12, 1536, 1.26}, {8, 2048, 1.0}, {6, 2048, 0.8}, {4, 2048, 0.55}};
 
 // A unit of EvalNonSymmetricLdsKernel: up to three trees that a wave walks side by side out of its LDS region
 struct TNsUnit {
@@ -586,7 +591,7 @@ void BuildLevelOrderTrees(const TModelTrees& trees, int dim, const std::vector<u
     }
     std::vector<uint32_t> entries, rows(treeCount * 4, 0);
     *usable = true;
-    *compactUsable = dim == 1 && trees.EffectiveBinFeaturesBucketCount <= 1023;
+    *compactUsable = trees.EffectiveBinFeaturesBucketCount <= 1023;
     compactRows->assign(treeCount * 4, 0);
     for (size_t t = 0; t < treeCount && *usable; ++t) {
         const uint32_t root = static_cast<uint32_t>(trees.TreeStartOffsets[t]);
@@ -641,7 +646,8 @@ void BuildLevelOrderTrees(const TModelTrees& trees, int dim, const std::vector<u
                 if (item.Terminal) {
                     const bool odd = (self & 1u) != 0;
                     compactEntries->push_back((odd ? 0u : 255u) | ((self & ~1u) << 21));
-                    valuesByEntry->push_back(trees.LeafValues[trees.NonSymmetricNodeIdToLeafId[item.Node]]);
+                    const double* leaf = trees.LeafValues.data() + trees.NonSymmetricNodeIdToLeafId[item.Node];
+                    valuesByEntry->insert(valuesByEntry->end(), leaf, leaf + dim);
                 } else {
                     const auto& rb = trees.RepackedBins[item.Node];
                     // a one-hot split holds ~value in its xor mask (and 255 as its split index)
@@ -654,11 +660,11 @@ void BuildLevelOrderTrees(const TModelTrees& trees, int dim, const std::vector<u
                     // the true side always follows the false side in the order
                     compactEntries->push_back(splitIdx | (static_cast<uint32_t>(rb.FeatureIndex) << 8) |
                                               (compactIndex(compact.Children[i].first) << 21));
-                    valuesByEntry->push_back(0.0);
+                    valuesByEntry->insert(valuesByEntry->end(), static_cast<size_t>(dim), 0.0);
                 }
                 if (i == 0) {
                     compactEntries->push_back(255u);  // the unused entry
-                    valuesByEntry->push_back(0.0);
+                    valuesByEntry->insert(valuesByEntry->end(), static_cast<size_t>(dim), 0.0);
                 }
             }
         }
@@ -986,6 +992,7 @@ struct THipEvaluator::TImpl {
     TDeviceVec<uint32_t> NsCompactEntries;
     TDeviceVec<uint32_t> NsCompactRows;  // 8 dwords per unit of trees
     uint32_t NsUnitCount = 0;
+    uint32_t NsEntryCount = 0;       // entries of all units: rows of NsValuesByEntry per slice of the dimensions
     TNsLdsShape NsLdsShape{0, 0};    // waves and entries per region of EvalNonSymmetricLdsKernel for this model
     TDeviceVec<double> NsValuesByEntry;
 
@@ -1515,7 +1522,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
             std::vector<TNsUnit> bestUnits;
             for (const TNsLdsShape& shape : kNsLdsShapes) {
                 if ((switches.NsWaves != 0 && switches.NsWaves != shape.Waves) ||
-                    NsLdsKernelBytes(m.LayoutBuckets, shape.Waves, shape.Entries) > kMaxTileLdsBytes) {
+                    NsLdsKernelBytes(m.LayoutBuckets, shape.Waves, shape.Entries, NsLdsDims(m.Dim)) > kMaxTileLdsBytes) {
                     continue;
                 }
                 std::vector<TNsUnit> plan;
@@ -1553,7 +1560,8 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
                             const uint32_t entry = compactEntries[treeFirst + e];
                             const uint32_t tileRow = dev::NsLdsTileRow((entry >> 8) & 0x3ffu, m.NsLdsShape.Waves, m.NsLdsShape.Entries);
                             entries.push_back((entry & ~0x3ff00u) + (tileRow << 8) + (count << 21));
-                            values.push_back(valuesByEntry[treeFirst + e]);
+                            const double* value = valuesByEntry.data() + static_cast<size_t>(treeFirst + e) * m.Dim;
+                            values.insert(values.end(), value, value + m.Dim);
                         }
                         count += treeEntries;
                     }
@@ -1563,6 +1571,20 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
                 m.NsUnitCount = static_cast<uint32_t>(bestUnits.size());
                 m.NsCompactEntries.Upload(entries);
                 m.NsCompactRows.Upload(units);
+                m.NsEntryCount = static_cast<uint32_t>(entries.size());
+                if (m.Dim > 1) {
+                    // [slice of the dimensions][entry][dimension of the slice], zeros past the last dimension
+                    const uint32_t dims = NsLdsDims(m.Dim), slices = (static_cast<uint32_t>(m.Dim) + dims - 1) / dims;
+                    std::vector<double> bySlice(static_cast<size_t>(slices) * entries.size() * dims, 0.0);
+                    for (uint32_t slice = 0; slice < slices; ++slice) {
+                        for (size_t e = 0; e < entries.size(); ++e) {
+                            for (uint32_t k = 0; k < dims && slice * dims + k < static_cast<uint32_t>(m.Dim); ++k) {
+                                bySlice[(slice * entries.size() + e) * dims + k] = values[e * m.Dim + slice * dims + k];
+                            }
+                        }
+                    }
+                    values.swap(bySlice);
+                }
                 m.NsValuesByEntry.Upload(values);
             }
         }
@@ -2397,20 +2419,41 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
     }
     if (!m.Oblivious && m.NsLdsUsable && treeStart == 0 && treeEnd == TreeCount) {
         const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
-        const size_t lds = NsLdsKernelBytes(m.LayoutBuckets, m.NsLdsShape.Waves, m.NsLdsShape.Entries);
+        const uint32_t dims = NsLdsDims(m.Dim);
+        const size_t lds = NsLdsKernelBytes(m.LayoutBuckets, m.NsLdsShape.Waves, m.NsLdsShape.Entries, dims);
         const auto launch = [&](auto kernel) {
             EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds);
-            hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(blocks)), dim3(64 * m.NsLdsShape.Waves), lds, s,
+            const dim3 grid(static_cast<uint32_t>(blocks), (static_cast<uint32_t>(m.Dim) + dims - 1) / dims);
+            hipLaunchKernelGGL(kernel, grid, dim3(64 * m.NsLdsShape.Waves), lds, s,
                                reinterpret_cast<const uint32_t*>(bins), docCount, m.LayoutBuckets,
                                m.NsCompactEntries.Get(), reinterpret_cast<const uint4*>(m.NsCompactRows.Get()),
-                               m.NsUnitCount, m.NsValuesByEntry.Get(), m.Bias.Get(), m.Scale, results);
+                               m.NsUnitCount, m.NsValuesByEntry.Get(), m.Bias.Get(), m.Scale,
+                               static_cast<uint32_t>(m.Dim), m.NsEntryCount, results);
+        };
+        const auto launchDims = [&](auto one, auto two, auto four) {
+            if (dims == 1) {
+                launch(one);
+            } else if (dims == 2) {
+                launch(two);
+            } else {
+                launch(four);
+            }
         };
         if (m.NsLdsShape.Waves == 16) {
-            launch(dev::EvalNonSymmetricLdsKernel<16, 1024>);
+            launchDims(dev::EvalNonSymmetricLdsKernel<16, 1024, 1>, dev::EvalNonSymmetricLdsKernel<16, 1024, 2>,
+                       dev::EvalNonSymmetricLdsKernel<16, 1024, 4>);
         } else if (m.NsLdsShape.Waves == 12) {
-            launch(dev::EvalNonSymmetricLdsKernel<12, 1536>);
+            launchDims(dev::EvalNonSymmetricLdsKernel<12, 1536, 1>, dev::EvalNonSymmetricLdsKernel<12, 1536, 2>,
+                       dev::EvalNonSymmetricLdsKernel<12, 1536, 4>);
+        } else if (m.NsLdsShape.Waves == 6) {
+            launchDims(dev::EvalNonSymmetricLdsKernel<6, 2048, 1>, dev::EvalNonSymmetricLdsKernel<6, 2048, 2>,
+                       dev::EvalNonSymmetricLdsKernel<6, 2048, 4>);
+        } else if (m.NsLdsShape.Waves == 4) {
+            launchDims(dev::EvalNonSymmetricLdsKernel<4, 2048, 1>, dev::EvalNonSymmetricLdsKernel<4, 2048, 2>,
+                       dev::EvalNonSymmetricLdsKernel<4, 2048, 4>);
         } else {
-            launch(dev::EvalNonSymmetricLdsKernel<8, 2048>);
+            launchDims(dev::EvalNonSymmetricLdsKernel<8, 2048, 1>, dev::EvalNonSymmetricLdsKernel<8, 2048, 2>,
+                       dev::EvalNonSymmetricLdsKernel<8, 2048, 4>);
         }
         HIP_CHECK(hipGetLastError());
         return;
@@ -2591,7 +2634,7 @@ std::string THipEvaluator::DescribeKernels(int layout, size_t docCount) const {
         evaluate = "EvalObliviousKernel";
     } else if (m.NsLdsUsable) {
         evaluate = "EvalNonSymmetricLdsKernel<" + std::to_string(m.NsLdsShape.Waves) + ", " +
-                   std::to_string(m.NsLdsShape.Entries) + ">";
+                   std::to_string(m.NsLdsShape.Entries) + (m.Dim > 1 ? ", " + std::to_string(NsLdsDims(m.Dim)) : "") + ">";
     } else if (m.NsTileUsable && TileLdsBytes(m.LayoutBuckets, m.Dim == 1 ? 1 : m.Dim <= 4 ? 4 : 16) <= kMaxTileLdsBytes) {
         evaluate = "EvalNonSymmetricTileKernel";
     } else {

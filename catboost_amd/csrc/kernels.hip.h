@@ -15,6 +15,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <type_traits>
 
 namespace cbamd::dev {
 
@@ -1641,8 +1642,12 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalNonSymmetricTileKernel(
 // its walk and added after the next unit's walk.
 // unitRows: 8 dwords per unit: first entry, height of the tallest tree, number of entries, first
 // entry of the second and of the third tree relative to the unit's, number of trees, 2 unused.
-// grid = doc blocks, block = 64 * WAVES, dynamic LDS = NsLdsTileRows(buckets, WAVES, ENTRIES) * 256 + 256 * 8 bytes;
-// no other LDS in the kernel.
+// Models of several dimensions: a workgroup sums DIMS of them, those from blockIdx.y * DIMS on (every slice of
+// the dimensions walks the trees again), and valuesByEntry is [slice][entryCount] rows of DIMS values (zeros past
+// the last dimension), so that a leaf's values come with one aligned load; they are read and added right behind
+// the unit's walk, with the other waves of the SIMD to cover the wait.
+// grid = (doc blocks, ceil(dim / DIMS)), block = 64 * WAVES, dynamic LDS = NsLdsTileRows(buckets, WAVES, ENTRIES) * 256
+// + 256 * 8 * DIMS bytes; no other LDS in the kernel.
 constexpr int kNsLdsEntries = 2048;
 constexpr int kNsUnitTrees = 3;
 
@@ -1668,11 +1673,19 @@ __device__ __forceinline__ T LdsLoad(uint32_t address) {
     return *reinterpret_cast<const __attribute__((address_space(3))) T*>(address);
 }
 
-template <int WAVES, int ENTRIES>
+__device__ __forceinline__ double LeafRowValue(const double2& row, int k) {
+    return k == 0 ? row.x : row.y;
+}
+
+__device__ __forceinline__ double LeafRowValue(const double4& row, int k) {
+    return k == 0 ? row.x : k == 1 ? row.y : k == 2 ? row.z : row.w;
+}
+
+template <int WAVES, int ENTRIES, int DIMS>
 __global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
     const uint32_t* __restrict__ bins, size_t docCount, uint32_t bucketCount, const uint32_t* __restrict__ entries,
     const uint4* __restrict__ unitRows, uint32_t unitCount, const double* __restrict__ valuesByEntry,
-    const double* __restrict__ bias, double scale, double* __restrict__ out) {
+    const double* __restrict__ bias, double scale, uint32_t dim, uint32_t entryCount, double* __restrict__ out) {
     constexpr int kFetch = ENTRIES / kWave;
     static_assert(ENTRIES <= kNsLdsEntries && ENTRIES % kWave == 0, "a region holds whole rounds of a wave's copy");
     extern __shared__ uint32_t sTile[];
@@ -1703,7 +1716,15 @@ __global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
         }                                                                            \
     } while (0)
 
-    double acc[4] = {0.0, 0.0, 0.0, 0.0};
+    double acc[4][DIMS];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int k = 0; k < DIMS; ++k) {
+            acc[j][k] = 0.0;
+        }
+    }
+    // one dimension: a unit's values are requested behind its walk and added after the next unit's
     double pending[kNsUnitTrees][4];
 #pragma unroll
     for (int g = 0; g < kNsUnitTrees; ++g) {
@@ -1712,6 +1733,8 @@ __global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
             pending[g][j] = 0.0;
         }
     }
+    const uint32_t d0 = blockIdx.y * DIMS;
+    const double* sliceValues = valuesByEntry + static_cast<size_t>(blockIdx.y) * entryCount * DIMS;
     uint32_t u = wave;
     uint4 row = make_uint4(0, 0, 0, 0), row2 = make_uint4(0, 0, 0, 0);
     if (u < unitCount) {
@@ -1784,24 +1807,45 @@ __global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
                 idx[g][j] = (entry[g][j] >> 21) + ((entry[g][j] & 0xffu) == 0 ? 1u : 0u);
             }
         }
+        if constexpr (DIMS == 1) {
 #pragma unroll
-        for (int g = 0; g < kNsUnitTrees; ++g) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                acc[j] = __dadd_rn(acc[j], pending[g][j]);
-            }
-        }
-#pragma unroll
-        for (int g = 0; g < kNsUnitTrees; ++g) {
-            if (static_cast<uint32_t>(g) < trees) {
+            for (int g = 0; g < kNsUnitTrees; ++g) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    pending[g][j] = valuesByEntry[first + idx[g][j]];
+                    acc[j][0] = __dadd_rn(acc[j][0], pending[g][j]);
                 }
-            } else {
+            }
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    pending[g][j] = 0.0;
+            for (int g = 0; g < kNsUnitTrees; ++g) {
+                if (static_cast<uint32_t>(g) < trees) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        pending[g][j] = valuesByEntry[first + idx[g][j]];
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        pending[g][j] = 0.0;
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int g = 0; g < kNsUnitTrees; ++g) {
+                if (static_cast<uint32_t>(g) < trees) {
+                    using TLeafRow = typename std::conditional<DIMS == 2, double2, double4>::type;
+                    TLeafRow value[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        value[j] = reinterpret_cast<const TLeafRow*>(sliceValues)[first + idx[g][j]];
+                    }
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                        for (int k = 0; k < DIMS; ++k) {
+                            acc[j][k] = __dadd_rn(acc[j][k], LeafRowValue(value[j], k));
+                        }
+                    }
                 }
             }
         }
@@ -1811,11 +1855,13 @@ __global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
         row2 = row2Next;
     }
 #undef CBAMD_FETCH_UNIT
+    if constexpr (DIMS == 1) {
 #pragma unroll
-    for (int g = 0; g < kNsUnitTrees; ++g) {
+        for (int g = 0; g < kNsUnitTrees; ++g) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            acc[j] = __dadd_rn(acc[j], pending[g][j]);
+            for (int j = 0; j < 4; ++j) {
+                acc[j][0] = __dadd_rn(acc[j][0], pending[g][j]);
+            }
         }
     }
     // waves add their partial sums in wave order into the LDS accumulator; the last wave
@@ -1824,8 +1870,11 @@ __global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
         if (wave == w) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                double* cell = sRed + j * kWave + lane;
-                *cell = (w == 0) ? acc[j] : __dadd_rn(*cell, acc[j]);
+#pragma unroll
+                for (int k = 0; k < DIMS; ++k) {
+                    double* cell = sRed + (k * 4 + j) * kWave + lane;
+                    *cell = (w == 0) ? acc[j][k] : __dadd_rn(*cell, acc[j][k]);
+                }
             }
         }
         __syncthreads();
@@ -1834,8 +1883,12 @@ __global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const size_t doc = block * kDocsPerBlock + j * kWave + lane;
-            if (doc < docCount) {
-                out[doc] = Finish(__dadd_rn(sRed[j * kWave + lane], acc[j]), scale, bias[0], true);
+#pragma unroll
+            for (int k = 0; k < DIMS; ++k) {
+                if (doc < docCount && d0 + k < dim) {
+                    out[doc * dim + d0 + k] =
+                        Finish(__dadd_rn(sRed[(k * 4 + j) * kWave + lane], acc[j][k]), scale, bias[d0 + k], true);
+                }
             }
         }
     }

@@ -125,6 +125,29 @@ def test_non_symmetric_models_with_one_hot_splits(seed, n_float, n_cat, trees, m
     _close(g.calc_flat(x), o.calc(x))
 
 
+@pytest.mark.parametrize("seed,dim,n_float,n_cat,trees,max_depth,docs", [
+    (1, 2, 30, 0, 120, 8, 3000), (2, 3, 150, 3, 60, 9, 1000), (3, 4, 8, 4, 25, 6, 257), (4, 5, 40, 0, 200, 5, 5000),
+    (5, 10, 60, 2, 90, 7, 2049), (6, 13, 12, 0, 33, 10, 64),
+])
+def test_non_symmetric_models_of_several_dimensions(seed, dim, n_float, n_cat, trees, max_depth, docs):
+    """Non-symmetric models of several dimensions walk out of LDS as well: a workgroup sums two or four
+    dimensions (a slice), the model's slices are rows of the grid. Two dimensions, one slice with a dimension
+    to spare, and several slices the last of which is short; with and without one-hot splits."""
+    rng = np.random.default_rng(seed)
+    model, cat_values = _random_oblivious(rng, n_float=n_float, n_cat=n_cat, trees=trees, max_depth=max_depth, dim=dim,
+                                          scale=-0.5, bias=rng.normal(size=dim))
+    model = mb.convert_oblivious_to_asymmetric(model)
+    x = _random_flat_data(rng, model, cat_values, docs)
+    o = OracleModel(model)
+    g = _gpu_model(model)
+    kernels = g.evaluator().describe_kernels(cb.LAYOUT_FLAT_ROWS, docs)
+    assert "EvalNonSymmetricLdsKernel" in kernels["evaluate"] and kernels["evaluate"].endswith(", %d>" % (2 if dim == 2 else 4))
+    np.testing.assert_array_equal(g.calc_leaf_indexes_flat(x), o.leaf_indexes(x))
+    _close(g.calc_flat(x), o.calc(x))
+    # a range of the trees goes to the kernel that takes ranges; both must agree with the oracle
+    _close(g.calc_flat(x, tree_start=1, tree_end=trees - 1), o.calc(x, tree_start=1, tree_end=trees - 1))
+
+
 def test_non_symmetric_tree_whose_nodes_share_children():
     """A chain of 60 nodes in which both steps of every node lead to the next one passes the loader's
     range checks; unfolded level by level it would have 2^60 entries. The level-order tables give up
