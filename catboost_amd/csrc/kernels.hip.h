@@ -1640,8 +1640,10 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalNonSymmetricTileKernel(
 // are fetched into registers while the current unit is walked. valuesByEntry holds the leaf
 // value of every terminal entry, indexed like `entries`; a unit's values are requested behind
 // its walk and added after the next unit's walk.
-// unitRows: 8 dwords per unit: first entry, height of the tallest tree, number of entries, first
-// entry of the second and of the third tree relative to the unit's, number of trees, 2 unused.
+// unitRows: 8 dwords per unit: first entry, height of the tallest tree, number of entries, first entry of the
+// second tree relative to the unit's, that of the third tree | number of trees << 16, and the model's numbers
+// of the three trees: a call for the trees [treeBegin, treeEnd) adds the values of those only and passes over
+// the units that hold none of them.
 // Models of several dimensions: a workgroup sums DIMS of them, those from blockIdx.y * DIMS on (every slice of
 // the dimensions walks the trees again), and valuesByEntry is [slice][entryCount] rows of DIMS values (zeros past
 // the last dimension), so that a leaf's values come with one aligned load; they are read and added right behind
@@ -1685,7 +1687,8 @@ template <int WAVES, int ENTRIES, int DIMS>
 __global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
     const uint32_t* __restrict__ bins, size_t docCount, uint32_t bucketCount, const uint32_t* __restrict__ entries,
     const uint4* __restrict__ unitRows, uint32_t unitCount, const double* __restrict__ valuesByEntry,
-    const double* __restrict__ bias, double scale, uint32_t dim, uint32_t entryCount, double* __restrict__ out) {
+    const double* __restrict__ bias, double scale, uint32_t dim, uint32_t entryCount, uint32_t treeBegin,
+    uint32_t treeEnd, double* __restrict__ out) {
     constexpr int kFetch = ENTRIES / kWave;
     static_assert(ENTRIES <= kNsLdsEntries && ENTRIES % kWave == 0, "a region holds whole rounds of a wave's copy");
     extern __shared__ uint32_t sTile[];
@@ -1746,19 +1749,32 @@ __global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
         const uint32_t first = __builtin_amdgcn_readfirstlane(row.x);
         const uint32_t height = __builtin_amdgcn_readfirstlane(row.y);
         const uint32_t count = __builtin_amdgcn_readfirstlane(row.z);
-        const uint32_t trees = __builtin_amdgcn_readfirstlane(row2.y);
+        const uint32_t packed = __builtin_amdgcn_readfirstlane(row2.x);
+        const uint32_t trees = packed >> 16;
         // trees the unit does not have walk its first tree again; their values are not added
         const uint32_t start[kNsUnitTrees] = {0u, trees > 1 ? __builtin_amdgcn_readfirstlane(row.w) : 0u,
-                                              trees > 2 ? __builtin_amdgcn_readfirstlane(row2.x) : 0u};
-        // the previous unit's reads were issued before these stores and LDS serves one wave in order
+                                              trees > 2 ? (packed & 0xffffu) : 0u};
+        const uint32_t treeOf[kNsUnitTrees] = {static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(row2.y)),
+                                               static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(row2.z)),
+                                               static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(row2.w))};
+        bool wanted[kNsUnitTrees];
+        bool anyWanted = false;
 #pragma unroll
-        for (int i = 0; i < kFetch; ++i) {
-            if (static_cast<uint32_t>(i) * kWave < count) {
-                sEntries[i * kWave + lane] = fetched[i];
-            }
+        for (int g = 0; g < kNsUnitTrees; ++g) {
+            wanted[g] = static_cast<uint32_t>(g) < trees && treeOf[g] - treeBegin < treeEnd - treeBegin;
+            anyWanted = anyWanted || wanted[g];
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
+        if (anyWanted) {
+            // the previous unit's reads were issued before these stores and LDS serves one wave in order
+#pragma unroll
+            for (int i = 0; i < kFetch; ++i) {
+                if (static_cast<uint32_t>(i) * kWave < count) {
+                    sEntries[i * kWave + lane] = fetched[i];
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+        }
         const uint32_t uNext = u + WAVES;
         uint4 rowNext = make_uint4(0, 0, 0, 0), row2Next = make_uint4(0, 0, 0, 0);
         if (uNext < unitCount) {
@@ -1769,13 +1785,13 @@ __global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
         uint32_t entry[kNsUnitTrees][4];
 #pragma unroll
         for (int g = 0; g < kNsUnitTrees; ++g) {
-            const uint32_t rootEntry = sEntries[start[g]];
+            const uint32_t rootEntry = anyWanted ? sEntries[start[g]] : 0u;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 entry[g][j] = rootEntry;
             }
         }
-        for (uint32_t step = 0; step < height; ++step) {
+        for (uint32_t step = 0; step < (anyWanted ? height : 0u); ++step) {
             uint64_t pair[kNsUnitTrees][4];  // the two children of a chain's node, left in the low half
             uint32_t bin[kNsUnitTrees][4];
 #pragma unroll
@@ -1817,7 +1833,7 @@ __global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
             }
 #pragma unroll
             for (int g = 0; g < kNsUnitTrees; ++g) {
-                if (static_cast<uint32_t>(g) < trees) {
+                if (wanted[g]) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         pending[g][j] = valuesByEntry[first + idx[g][j]];
@@ -1832,7 +1848,7 @@ __global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
         } else {
 #pragma unroll
             for (int g = 0; g < kNsUnitTrees; ++g) {
-                if (static_cast<uint32_t>(g) < trees) {
+                if (wanted[g]) {
                     using TLeafRow = typename std::conditional<DIMS == 2, double2, double4>::type;
                     TLeafRow value[4];
 #pragma unroll
@@ -1887,7 +1903,7 @@ __global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
             for (int k = 0; k < DIMS; ++k) {
                 if (doc < docCount && d0 + k < dim) {
                     out[doc * dim + d0 + k] =
-                        Finish(__dadd_rn(sRed[(k * 4 + j) * kWave + lane], acc[j][k]), scale, bias[d0 + k], true);
+                        Finish(__dadd_rn(sRed[(k * 4 + j) * kWave + lane], acc[j][k]), scale, bias[d0 + k], treeBegin == 0);
                 }
             }
         }
