@@ -312,6 +312,7 @@ struct TKernelSwitches {
     bool SmallBatch = true;       // CATBOOST_AMD_SMALL_BATCH=0: small batches are not spread over slices of the trees
     bool LevelOrder = true;       // CATBOOST_AMD_LEVEL_ORDER=0: register kernels keep the model's order of a tree's levels
     bool PairTile = true;         // CATBOOST_AMD_PAIR_TILE=0: the half-tile kernel with one tree per wave
+    bool RowTile = true;          // CATBOOST_AMD_ROW_TILE=0: the tile kernel that broadcasts a tree's levels from a lane
     bool RegSplit = true;         // CATBOOST_AMD_REG_SPLIT=0: buckets of more than 127 values send a model to the mixed kernels
     uint32_t NsWaves = 0;         // CATBOOST_AMD_NS_WAVES=4|6|8|12|16: that shape of the non-symmetric LDS kernel or none
 
@@ -328,6 +329,7 @@ struct TKernelSwitches {
         k.LevelOrder = !off("CATBOOST_AMD_LEVEL_ORDER");
         k.SmallBatch = !off("CATBOOST_AMD_SMALL_BATCH");
         k.PairTile = !off("CATBOOST_AMD_PAIR_TILE");
+        k.RowTile = !off("CATBOOST_AMD_ROW_TILE");
         k.RegSplit = !off("CATBOOST_AMD_REG_SPLIT");
         if (const char* v = std::getenv("CATBOOST_AMD_NS_WAVES")) {
             k.NsWaves = static_cast<uint32_t>(std::strtoul(v, nullptr, 10));
@@ -475,6 +477,24 @@ bool PackNsUnits(const std::vector<uint32_t>& rows, size_t treeCount, uint32_t l
         }
     }
     return true;
+}
+
+// LDS of the row-tile kernel: 256 documents' bins, then a region of 256 doubles per wave (a tree's leaf values,
+// at the end the wave's partial sums)
+size_t RowTileLdsBytes(uint32_t buckets, uint32_t waves) {
+    return ((static_cast<size_t>(buckets) * 256 + 15) & ~size_t(15)) + static_cast<size_t>(waves) * 256 * sizeof(double);
+}
+
+// Waves per workgroup of the row-tile kernel: eight when two workgroups then share a CU, else sixteen if LDS
+// has room for their regions, else eight; 0 when the tile leaves no room for eight regions.
+uint32_t RowTileWaves(uint32_t buckets) {
+    if (2 * RowTileLdsBytes(buckets, dev::kTileWaves) <= kMaxTileLdsBytes) {
+        return dev::kTileWaves;
+    }
+    if (RowTileLdsBytes(buckets, dev::kWideTileWaves) <= kMaxTileLdsBytes) {
+        return dev::kWideTileWaves;
+    }
+    return RowTileLdsBytes(buckets, dev::kTileWaves) <= kMaxTileLdsBytes ? dev::kTileWaves : 0;
 }
 
 // LDS of the pair-tile kernel: 128 documents' bins, then per wave the leaf values of two trees; the same area
@@ -976,6 +996,7 @@ struct THipEvaluator::TImpl {
     TDeviceVec<uint32_t> PackedMixed;  // half-tile kernel: packed rows in the form chosen per tree
     TDeviceVec<double> HalfTileLeaves; // half-tile kernel: 64 or 256 leaf values per tree at a fixed pitch
     TDeviceVec<uint32_t> PairRows;     // pair-tile kernel: 16 dwords per tree, empty when the model does not qualify
+    TDeviceVec<uint32_t> TileRows;     // row-tile kernel (whole tile, one tree per wave): the same with 256 bytes per bucket
     TDeviceVec<double> LeavesPadded;   // tile kernel, multi-dimensional: [tree][chunk][leaf][TileChunk(dim)]
     bool PackedSevenBit = false;
     bool LeavesPairAligned = false;  // every tree's first leaf value sits at an even index
@@ -1463,43 +1484,50 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
                 }
             }
             m.PackedMixed.Upload(mixed);
-            if (TileLdsBytes(m.LayoutBuckets, 1) > kMaxTileLdsBytes) {
+            // The kernels that keep a tree's row in registers (two trees per wave on half a tile, one on a whole
+            // tile) need every bin of the model below 128 (the one-hot test then fits 7 bits too); their rows name a
+            // bucket by its byte offset in the tile.
+            uint32_t maxValues = 0;
+            for (size_t b = 0; b + 1 < offsets.size(); ++b) {
+                maxValues = std::max(maxValues, offsets[b + 1] - offsets[b]);
+            }
+            const bool wholeTile = TileLdsBytes(m.LayoutBuckets, 1) <= kMaxTileLdsBytes;
+            const bool rowsInRegisters =
+                maxValues <= 127 && (wholeTile ? switches.RowTile && RowTileWaves(m.LayoutBuckets) != 0
+                                               : switches.PairTile && PairTileLdsBytes(m.LayoutBuckets, 8) <= kMaxTileLdsBytes);
+            if (!wholeTile || rowsInRegisters) {
                 const size_t pitch = m.MaxDepth <= 6 ? 64 : 256;
-                // zeros at the end: the pair-tile kernel fetches ahead of its trees without a bound
+                // zeros at the end: those kernels fetch ahead of their trees without a bound
                 std::vector<double> fixed((trees.GetTreeCount() + dev::kPairTreePadding) * pitch, 0.0);
                 for (size_t t = 0; t < trees.GetTreeCount(); ++t) {
                     std::copy_n(trees.LeafValues.begin() + trees.TreeFirstLeafOffsets[t], size_t(1) << trees.TreeSizes[t],
                                 fixed.begin() + t * pitch);
                 }
                 m.HalfTileLeaves.Upload(fixed);
-                // two trees per wave: every bin of the model below 128 (the one-hot test then fits 7 bits too)
-                uint32_t maxValues = 0;
-                for (size_t b = 0; b + 1 < offsets.size(); ++b) {
-                    maxValues = std::max(maxValues, offsets[b + 1] - offsets[b]);
-                }
-                if (switches.PairTile && maxValues <= 127 && PairTileLdsBytes(m.LayoutBuckets, 8) <= kMaxTileLdsBytes) {
-                    std::vector<uint32_t> pairRows((trees.GetTreeCount() + dev::kPairTreePadding) * dev::kPackedTreeDwords, 0);
-                    for (size_t t = 0; t < trees.GetTreeCount(); ++t) {
-                        uint32_t* row = pairRows.data() + t * dev::kPackedTreeDwords;
-                        bool anyXor = false;
-                        for (int d = 0; d < trees.TreeSizes[t]; ++d) {
-                            const auto& rb = trees.RepackedBins[trees.TreeStartOffsets[t] + d];
-                            row[d] = static_cast<uint32_t>(rb.FeatureIndex) * 128u;
-                            if (rb.XorMask != 0 || rb.SplitIdx == 0xff) {
-                                // one-hot: bin == value, value = ~XorMask; 7 bits of it are enough below 128
-                                row[d] |= (static_cast<uint32_t>(rb.XorMask) & 0x7fu) << 24;
-                                row[8 + d] = 0x01010101u;
-                                anyXor = true;
-                            } else {
-                                row[8 + d] = (128u - rb.SplitIdx) * 0x01010101u;
-                            }
-                        }
-                        if (anyXor) {
-                            row[0] |= dev::kPairRowXorFlag;
+            }
+            if (rowsInRegisters) {
+                const uint32_t bucketBytes = wholeTile ? 256u : 128u;
+                std::vector<uint32_t> pairRows((trees.GetTreeCount() + dev::kPairTreePadding) * dev::kPackedTreeDwords, 0);
+                for (size_t t = 0; t < trees.GetTreeCount(); ++t) {
+                    uint32_t* row = pairRows.data() + t * dev::kPackedTreeDwords;
+                    bool anyXor = false;
+                    for (int d = 0; d < trees.TreeSizes[t]; ++d) {
+                        const auto& rb = trees.RepackedBins[trees.TreeStartOffsets[t] + d];
+                        row[d] = static_cast<uint32_t>(rb.FeatureIndex) * bucketBytes;
+                        if (rb.XorMask != 0 || rb.SplitIdx == 0xff) {
+                            // one-hot: bin == value, value = ~XorMask; 7 bits of it are enough below 128
+                            row[d] |= (static_cast<uint32_t>(rb.XorMask) & 0x7fu) << 24;
+                            row[8 + d] = 0x01010101u;
+                            anyXor = true;
+                        } else {
+                            row[8 + d] = (128u - rb.SplitIdx) * 0x01010101u;
                         }
                     }
-                    m.PairRows.Upload(pairRows);
+                    if (anyXor) {
+                        row[0] |= dev::kPairRowXorFlag;
+                    }
                 }
+                (wholeTile ? m.TileRows : m.PairRows).Upload(pairRows);
             }
         }
         m.LeavesPairAligned = true;
@@ -2367,6 +2395,33 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
         return;
     }
     const int dchunk = TileChunk(m.Dim);
+    if (m.TileRows.Get() != nullptr) {
+        // one-dimensional, 7-bit bins, the tile fits: a tree's row in registers
+        const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
+        const uint32_t waves = RowTileWaves(m.LayoutBuckets);
+        const size_t lds = RowTileLdsBytes(m.LayoutBuckets, waves);
+        const auto launch = [&](auto kernel) {
+            EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds);
+            hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(blocks)), dim3(64 * waves), lds, s,
+                               reinterpret_cast<const uint32_t*>(bins), docCount, m.LayoutBuckets,
+                               reinterpret_cast<const uint4*>(m.TileRows.Get()),
+                               reinterpret_cast<const double2*>(m.HalfTileLeaves.Get()), m.Bias.Get(), m.Scale, tb, te,
+                               results);
+        };
+        if (m.MaxDepth <= 6) {
+            if (waves == dev::kTileWaves) {
+                launch(dev::EvalObliviousRowTileKernel<6, dev::kTileWaves>);
+            } else {
+                launch(dev::EvalObliviousRowTileKernel<6, dev::kWideTileWaves>);
+            }
+        } else if (waves == dev::kTileWaves) {
+            launch(dev::EvalObliviousRowTileKernel<8, dev::kTileWaves>);
+        } else {
+            launch(dev::EvalObliviousRowTileKernel<8, dev::kWideTileWaves>);
+        }
+        HIP_CHECK(hipGetLastError());
+        return;
+    }
     if (m.Oblivious && m.MaxDepth <= 8 && TileLdsBytes(m.LayoutBuckets, dchunk) <= kMaxTileLdsBytes) {
         // byte-parallel kernel over an LDS tile of bins
         const TTileArgs args{bins, docCount, m.LayoutBuckets, m.PackedTrees.Get(),
@@ -2629,6 +2684,8 @@ std::string THipEvaluator::DescribeKernels(int layout, size_t docCount) const {
         if (slices > 1) {
             evaluate += " x " + std::to_string(slices) + " slices of the trees + CombineSlicesKernel";
         }
+    } else if (m.TileRows.Get() != nullptr) {
+        evaluate = "EvalObliviousRowTileKernel";
     } else if (m.Oblivious && m.MaxDepth <= 8 && TileLdsBytes(m.LayoutBuckets, dchunk) <= kMaxTileLdsBytes) {
         evaluate = "EvalObliviousTileKernel";
     } else if (m.Oblivious && m.MaxDepth <= 8 && m.Dim == 1 && m.HalfTileLeaves.Get() != nullptr &&

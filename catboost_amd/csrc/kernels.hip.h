@@ -1413,6 +1413,154 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousPairTileKernel(
     }
 }
 
+// One-dimensional models of 7-bit bins whose 256-document tile fits LDS, one tree per wave: the walk of
+// EvalObliviousPairTileKernel on the whole tile. A tree's row is `tileRows` (the format of pairRows with
+// bucket * 256 as the byte offset) and sits in registers, the same in every lane, so a level is an LDS read
+// and three vector instructions with no lane reads and no scalar arithmetic; the leaf values (1 << MAXD per
+// tree at a fixed pitch in `leaves2`) go through the wave's LDS region; rows and values are fetched
+// kPairAhead rounds ahead without looking at the tree range (both tables end with kRowTilePadding trees' worth
+// of zeros). Waves take the trees round robin; their partial sums are added in wave order at the end.
+// grid = doc blocks, block = 64 * WAVES, dynamic LDS = buckets * 256 (rounded up to 16) + WAVES * 256 * 8 bytes
+// (the leaf regions, later the partial sums).
+constexpr int kRowTilePadding = kWideTileWaves * kPairAhead;
+static_assert(kRowTilePadding <= kPairTreePadding, "the two kernels share the padded leaf table");
+
+template <int MAXD, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void EvalObliviousRowTileKernel(
+    const uint32_t* __restrict__ bins, size_t docCount, uint32_t bucketCount, const uint4* __restrict__ tileRows,
+    const double2* __restrict__ leaves2, const double* __restrict__ bias, double scale, uint32_t treeBegin,
+    uint32_t treeEnd, double* __restrict__ out) {
+    constexpr uint32_t kLeaves = 1u << MAXD;
+    constexpr uint32_t kRegion = 256;                    // doubles of a wave's region: its tree's values, its sums
+    constexpr int kLeafRegs = MAXD == 8 ? 2 : 1;         // 16-byte pieces of a tree's leaf values per lane
+    constexpr uint32_t kPieceMask = kLeaves / 2 - 1;     // 64 leaves: the upper lanes repeat the lower lanes' pieces
+    static_assert(MAXD == 8 || MAXD == 6, "64 or 256 leaves per tree");
+    static_assert(WAVES <= kWideTileWaves, "the tables are padded for that many waves");
+    extern __shared__ uint32_t sTile[];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const size_t block = blockIdx.x;
+    const uint32_t tileDwords = bucketCount * kWave;
+    const uint32_t* src = bins + block * tileDwords;
+    for (uint32_t i = tid; i < tileDwords; i += 64 * WAVES) {
+        sTile[i] = src[i];
+    }
+    const uint32_t tileBytes = (tileDwords * 4 + 15) & ~15u;
+    double* leafArea = reinterpret_cast<double*>(reinterpret_cast<uint8_t*>(sTile) + tileBytes);
+    double2* sLeafWave2 = reinterpret_cast<double2*>(leafArea + wave * kRegion);
+    const double* sLeafMine = leafArea + wave * kRegion;
+    const uint8_t* laneTile = reinterpret_cast<const uint8_t*>(sTile) + lane * 4;
+    __syncthreads();  // tile is loaded
+
+    const uint32_t treeCount = treeEnd - treeBegin;
+    double acc[4] = {0.0, 0.0, 0.0, 0.0};
+    constexpr int kAhead = kPairAhead;
+    uint4 rows[kAhead][4];
+    double2 pref[kAhead][kLeafRegs];
+    const double2* myLeaves = leaves2 + (lane & kPieceMask);
+#define CBAMD_FETCH_TREE(k, tree)                                                                  \
+    do {                                                                                           \
+        const uint4* row = tileRows + static_cast<size_t>(tree) * 4;                               \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                            \
+            rows[k][i] = row[i];                                                                   \
+        }                                                                                          \
+        const double2* values = myLeaves + static_cast<size_t>(tree) * (kLeaves / 2);              \
+        _Pragma("unroll") for (int i = 0; i < kLeafRegs; ++i) {                                    \
+            pref[k][i] = values[i * kWave];                                                        \
+        }                                                                                          \
+    } while (0)
+    // the tree's leaf values into the wave's LDS region (the previous tree's gathers were issued before these
+    // stores and LDS serves one wave's requests in order), then the levels: four leaf indexes per lane
+#define CBAMD_PUBLISH_AND_WALK(k, idx4)                                                            \
+    do {                                                                                           \
+        _Pragma("unroll") for (int i = 0; i < kLeafRegs; ++i) {                                    \
+            sLeafWave2[(i * kWave + lane) & kPieceMask] = pref[k][i];                              \
+        }                                                                                          \
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                                     \
+        __builtin_amdgcn_wave_barrier();                                                           \
+        if (__builtin_amdgcn_readfirstlane(rows[k][0].x) & kPairRowXorFlag) {                      \
+            idx4 = PairTreeIndexes<true, MAXD>(laneTile, rows[k]);                                 \
+        } else {                                                                                   \
+            idx4 = PairTreeIndexes<false, MAXD>(laneTile, rows[k]);                                \
+        }                                                                                          \
+    } while (0)
+    // One round of a wave, as in the two-tree kernel: the values that the previous round gathered are added
+    // while this round's LDS reads are under way, the registers of this tree take the tree kAhead rounds ahead
+    // as soon as every level has read them, and the gathers go out last.
+    constexpr int kLoadsBehind = 2 * (4 + kLeafRegs);  // loads of the two rounds behind the one that is waited for
+    constexpr int kWaitLoads = 0x0f70 | (kLoadsBehind & 15) | ((kLoadsBehind >> 4) << 14);  // vmcnt(kLoadsBehind)
+    double gathered[4] = {0.0, 0.0, 0.0, 0.0};
+#define CBAMD_TREE_ROUND(k)                                                                        \
+    do {                                                                                           \
+        uint32_t idx4;                                                                             \
+        __builtin_amdgcn_s_waitcnt(kWaitLoads);                                                    \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+        CBAMD_PUBLISH_AND_WALK(k, idx4);                                                           \
+        _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                            \
+            acc[q] = __dadd_rn(acc[q], gathered[q]);                                               \
+        }                                                                                          \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+        CBAMD_FETCH_TREE(k, treeBegin + p + kAhead * WAVES);                                       \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+        _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                            \
+            gathered[q] = sLeafMine[(idx4 >> (8 * q + 8 - MAXD)) & (kLeaves - 1)];                 \
+        }                                                                                          \
+        __builtin_amdgcn_wave_barrier();                                                           \
+        p += WAVES;                                                                                \
+    } while (0)
+
+    uint32_t p = wave;
+#pragma unroll
+    for (int k = 0; k < kAhead; ++k) {
+        // (written before the loads so that the arrays stay in registers)
+#pragma unroll
+        for (int i = 0; i < kLeafRegs; ++i) {
+            pref[k][i] = {0.0, 0.0};
+        }
+        CBAMD_FETCH_TREE(k, treeBegin + p + k * WAVES);
+    }
+    static_assert(kAhead == 3, "the rounds below are written out for three register sets");
+    // whole turns of the three register sets without a branch between the rounds, so that the waits for
+    // the loads count only the loads that are older than the one needed
+    while (p + 2 * WAVES < treeCount) {
+        CBAMD_TREE_ROUND(0);
+        CBAMD_TREE_ROUND(1);
+        CBAMD_TREE_ROUND(2);
+    }
+    if (p < treeCount) {
+        CBAMD_TREE_ROUND(0);
+        if (p < treeCount) {
+            CBAMD_TREE_ROUND(1);
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        acc[q] = __dadd_rn(acc[q], gathered[q]);
+    }
+#undef CBAMD_TREE_ROUND
+#undef CBAMD_FETCH_TREE
+#undef CBAMD_PUBLISH_AND_WALK
+    __syncthreads();  // every wave is through with its leaf region: the area now takes the partial sums
+    double* sRed = leafArea;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        sRed[wave * kRegion + q * kWave + lane] = acc[q];  // byte q of a lane's dword: document q * 64 + lane
+    }
+    __syncthreads();
+    if (tid < kDocsPerBlock) {
+        double sum = sRed[tid];
+#pragma unroll
+        for (int part = 1; part < WAVES; ++part) {
+            sum = __dadd_rn(sum, sRed[part * kRegion + tid]);
+        }
+        const size_t doc = block * kDocsPerBlock + tid;
+        if (doc < docCount) {
+            out[doc] = Finish(sum, scale, bias[0], treeBegin == 0);
+        }
+    }
+}
+
 __device__ __forceinline__ uint32_t BinOfDoc(const uint8_t* bins, size_t doc, uint32_t bucketCount, uint32_t bucket) {
     const size_t block = doc / kDocsPerBlock;
     const uint32_t r = static_cast<uint32_t>(doc % kDocsPerBlock);

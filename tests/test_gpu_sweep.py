@@ -98,6 +98,7 @@ def test_random_model_shapes(monkeypatch, capsys):
         monkeypatch.setenv("CATBOOST_AMD_LEVEL_ORDER", str(int(rng.integers(0, 2))))
         monkeypatch.setenv("CATBOOST_AMD_SMALL_BATCH", str(int(rng.integers(0, 2))))
         monkeypatch.setenv("CATBOOST_AMD_REG_SPLIT", str(int(rng.integers(0, 2))))
+        monkeypatch.setenv("CATBOOST_AMD_ROW_TILE", str(int(rng.integers(0, 2))))
         # the shape of the non-symmetric LDS kernel: chosen by the model, or one of the five
         monkeypatch.setenv("CATBOOST_AMD_NS_WAVES", str(int(rng.choice([0, 4, 6, 8, 12, 16]))))
         if kind == 2:

@@ -1,5 +1,6 @@
-"""One-dimensional oblivious models with more buckets than an LDS tile of 256 documents holds (above ~630):
-the half-tile kernels, one tree or two trees per wave, against the oracle through the C ABI.
+"""One-dimensional oblivious models with more buckets than the register kernels take: the tile kernels with a
+tree's row in registers or broadcast from a lane (the 256-document tile fits LDS, up to ~630 buckets), and
+above that the half-tile kernels, one tree or two trees per wave; against the oracle through the C ABI.
 
 The two kernels add the trees of a document in different orders (partial sums per wave, and per lane group
 in the two-tree kernel), so predictions are compared within 1e-9 rel / 1e-12 abs; the bins must be equal.
@@ -74,3 +75,34 @@ def test_two_kernels_agree_on_a_large_batch(monkeypatch):
     np.testing.assert_allclose(two, one, rtol=RTOL, atol=ATOL)
     sample = np.random.default_rng(0).choice(66_000, size=2000, replace=False)
     np.testing.assert_allclose(two[sample], OracleModel(model).calc(x[sample]), rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("rows_in_registers", ["1", "0"])
+@pytest.mark.parametrize("seed,n_float,n_cat,trees,max_depth,docs", [
+    (21, 230, 0, 301, 8, 1000),   # two workgroups of eight waves share a CU
+    (22, 400, 6, 200, 8, 513),    # sixteen waves; one-hot levels in some trees
+    (23, 560, 0, 500, 8, 255),    # 552 buckets: the tile leaves room for eight regions only
+    (24, 300, 20, 333, 6, 1),     # 64 leaves per tree, a single document
+    (25, 560, 2, 400, 3, 4097),   # shallow trees in the 64-leaf kernel
+])
+def test_tile_models_against_the_oracle(monkeypatch, rows_in_registers, seed, n_float, n_cat, trees, max_depth, docs):
+    rng = np.random.default_rng(seed)
+    model, cat_values = _random_oblivious(rng, n_float=n_float, n_cat=n_cat, trees=trees, max_depth=max_depth,
+                                          scale=float(rng.choice([1.0, -0.5])), bias=rng.normal(size=1))
+    x = _random_flat_data(rng, model, cat_values, docs)
+    o = OracleModel(model)
+    monkeypatch.setenv("CATBOOST_AMD_ROW_TILE", rows_in_registers)
+    g = cb.ModelCalcer()
+    g.load_from_dict(model)
+    g.enable_gpu_evaluation(0)
+    assert 224 < g.bucket_count <= 632, "the model must take a tile kernel"
+    kernels = g.evaluator().describe_kernels(cb.LAYOUT_FLAT_ROWS, docs)
+    assert kernels["evaluate"] == ("EvalObliviousRowTileKernel" if rows_in_registers == "1" else "EvalObliviousTileKernel")
+    np.testing.assert_array_equal(g.quantize_flat(x), o.binarize(x))
+    np.testing.assert_allclose(g.calc_flat(x), o.calc(x), rtol=RTOL, atol=ATOL)
+    for begin, end in ((0, 1), (1, 2), (0, 17), (7, 9), (0, trees - 1), (1, trees), (3, 3), (trees // 2, trees),
+                       (trees - 1, trees)):
+        if end <= trees and begin <= end:
+            np.testing.assert_allclose(g.calc_flat(x, tree_start=begin, tree_end=end),
+                                       o.calc(x, tree_start=begin, tree_end=end), rtol=RTOL, atol=ATOL,
+                                       err_msg="trees %d..%d" % (begin, end))
