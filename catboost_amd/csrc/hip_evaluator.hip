@@ -286,16 +286,24 @@ const TEvalRegVariant* PickRegVariant(uint32_t buckets, uint32_t dim, uint32_t m
                                       uint32_t minVariantBuckets = 0) {
     const TEvalRegVariant* best = nullptr;
     uint32_t bestLaunches = 0;
-    for (const auto& v : kEvalRegVariants) {
-        const uint32_t leaves = maxDepth > 8 ? 1024u : dim > 1 && maxDepth <= 6 ? 64u : 256u;
-        if (buckets > v.Buckets || v.Buckets < minVariantBuckets || (dim == 1) != (v.Pitch == 1) || v.Leaves != leaves ||
-            v.Mixed != mixed || v.Six != six) {
-            continue;
+    // A model of several dimensions with more buckets than the kernels of two and more dimensions hold (they
+    // need registers for their sums) takes the one-dimensional kernels, a launch per dimension: every launch
+    // walks the trees again, which still is several times faster than leaving the registers.
+    for (int onePerLaunch = 0; onePerLaunch < 2 && !best; ++onePerLaunch) {
+        if (onePerLaunch && dim == 1) {
+            break;
         }
-        const uint32_t launches = (dim + v.Pitch - 1) / v.Pitch;
-        if (!best || launches < bestLaunches || (launches == bestLaunches && dim > 1 && v.Pitch < best->Pitch)) {
-            best = &v;
-            bestLaunches = launches;
+        for (const auto& v : kEvalRegVariants) {
+            const uint32_t leaves = maxDepth > 8 ? 1024u : dim > 1 && maxDepth <= 6 && !onePerLaunch ? 64u : 256u;
+            if (buckets > v.Buckets || v.Buckets < minVariantBuckets || (dim == 1 || onePerLaunch) != (v.Pitch == 1) ||
+                v.Leaves != leaves || v.Mixed != mixed || v.Six != six) {
+                continue;
+            }
+            const uint32_t launches = (dim + v.Pitch - 1) / v.Pitch;
+            if (!best || launches < bestLaunches || (launches == bestLaunches && dim > 1 && v.Pitch < best->Pitch)) {
+                best = &v;
+                bestLaunches = launches;
+            }
         }
     }
     return best;
@@ -479,22 +487,30 @@ bool PackNsUnits(const std::vector<uint32_t>& rows, size_t treeCount, uint32_t l
     return true;
 }
 
-// LDS of the row-tile kernel: 256 documents' bins, then a region of 256 doubles per wave (a tree's leaf values,
-// at the end the wave's partial sums)
-size_t RowTileLdsBytes(uint32_t buckets, uint32_t waves) {
-    return ((static_cast<size_t>(buckets) * 256 + 15) & ~size_t(15)) + static_cast<size_t>(waves) * 256 * sizeof(double);
+// Dimensions that a workgroup of the row-tile kernel sums at a time: two keep the sums, the values in flight and
+// the three trees' worth of values fetched ahead within a wave's registers at sixteen waves (four spill)
+uint32_t RowTileDims(uint32_t /*maxDepth*/, int dim) {
+    return dim == 1 ? 1 : 2;
+}
+
+// LDS of the row-tile kernel: 256 documents' bins, the accumulator, a tree's leaf values per wave
+size_t RowTileLdsBytes(uint32_t buckets, uint32_t maxDepth, uint32_t dims, uint32_t waves) {
+    const size_t leaves = maxDepth <= 6 ? 64 : 256;
+    return ((static_cast<size_t>(buckets) * 256 + 15) & ~size_t(15)) + dev::kDocsPerBlock * dims * sizeof(double) +
+           static_cast<size_t>(waves) * leaves * dims * sizeof(double);
 }
 
 // Waves per workgroup of the row-tile kernel: eight when two workgroups then share a CU, else sixteen if LDS
 // has room for their regions, else eight; 0 when the tile leaves no room for eight regions.
-uint32_t RowTileWaves(uint32_t buckets) {
-    if (2 * RowTileLdsBytes(buckets, dev::kTileWaves) <= kMaxTileLdsBytes) {
+uint32_t RowTileWaves(uint32_t buckets, uint32_t maxDepth, int dim) {
+    const uint32_t dims = RowTileDims(maxDepth, dim);
+    if (2 * RowTileLdsBytes(buckets, maxDepth, dims, dev::kTileWaves) <= kMaxTileLdsBytes) {
         return dev::kTileWaves;
     }
-    if (RowTileLdsBytes(buckets, dev::kWideTileWaves) <= kMaxTileLdsBytes) {
+    if (RowTileLdsBytes(buckets, maxDepth, dims, dev::kWideTileWaves) <= kMaxTileLdsBytes) {
         return dev::kWideTileWaves;
     }
-    return RowTileLdsBytes(buckets, dev::kTileWaves) <= kMaxTileLdsBytes ? dev::kTileWaves : 0;
+    return RowTileLdsBytes(buckets, maxDepth, dims, dev::kTileWaves) <= kMaxTileLdsBytes ? dev::kTileWaves : 0;
 }
 
 // LDS of the pair-tile kernel: 128 documents' bins, then per wave the leaf values of two trees; the same area
@@ -997,6 +1013,8 @@ struct THipEvaluator::TImpl {
     TDeviceVec<double> HalfTileLeaves; // half-tile kernel: 64 or 256 leaf values per tree at a fixed pitch
     TDeviceVec<uint32_t> PairRows;     // pair-tile kernel: 16 dwords per tree, empty when the model does not qualify
     TDeviceVec<uint32_t> TileRows;     // row-tile kernel (whole tile, one tree per wave): the same with 256 bytes per bucket
+    TDeviceVec<double> TileLeaves;     // its leaf values: [slice of the dimensions][tree][pair of dimensions][leaf][2]
+    size_t TileSliceStride = 0;        // 16-byte pairs of TileLeaves per slice
     TDeviceVec<double> LeavesPadded;   // tile kernel, multi-dimensional: [tree][chunk][leaf][TileChunk(dim)]
     bool PackedSevenBit = false;
     bool LeavesPairAligned = false;  // every tree's first leaf value sits at an even index
@@ -1407,6 +1425,37 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
     }
     m.Bias.Upload(trees.Bias);
 
+    uint32_t maxBucketValues = 0;  // one-hot buckets included
+    for (size_t b = 0; b + 1 < offsets.size(); ++b) {
+        maxBucketValues = std::max(maxBucketValues, offsets[b + 1] - offsets[b]);
+    }
+    // Rows of the kernels that keep a tree's row in registers (two trees per wave on half a tile, one on a whole
+    // tile; every bin of the model below 128): 16 dwords per tree, slot d the byte offset of level d's bucket in
+    // the tile | xor byte << 24, slot 8 + d the value added to the four bins of a dword.
+    const auto rowsInRegisters = [&](uint32_t bucketBytes) {
+        std::vector<uint32_t> rows((trees.GetTreeCount() + dev::kPairTreePadding) * dev::kPackedTreeDwords, 0);
+        for (size_t t = 0; t < trees.GetTreeCount(); ++t) {
+            uint32_t* row = rows.data() + t * dev::kPackedTreeDwords;
+            bool anyXor = false;
+            for (int d = 0; d < trees.TreeSizes[t]; ++d) {
+                const auto& rb = trees.RepackedBins[trees.TreeStartOffsets[t] + d];
+                row[d] = static_cast<uint32_t>(rb.FeatureIndex) * bucketBytes;
+                if (rb.XorMask != 0 || rb.SplitIdx == 0xff) {
+                    // one-hot: bin == value, value = ~XorMask; 7 bits of it are enough below 128
+                    row[d] |= (static_cast<uint32_t>(rb.XorMask) & 0x7fu) << 24;
+                    row[8 + d] = 0x01010101u;
+                    anyXor = true;
+                } else {
+                    row[8 + d] = (128u - rb.SplitIdx) * 0x01010101u;
+                }
+            }
+            if (anyXor) {
+                row[0] |= dev::kPairRowXorFlag;
+            }
+        }
+        return rows;
+    };
+
     // 7-bit compares need every bin and split index to fit 7 bits and no xor mask
     m.PackedSevenBit = m.Oblivious && !m.HasOneHot && m.MaxBucketValues <= 127;
     if (m.Oblivious && m.MaxDepth <= 8) {
@@ -1484,50 +1533,19 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
                 }
             }
             m.PackedMixed.Upload(mixed);
-            // The kernels that keep a tree's row in registers (two trees per wave on half a tile, one on a whole
-            // tile) need every bin of the model below 128 (the one-hot test then fits 7 bits too); their rows name a
-            // bucket by its byte offset in the tile.
-            uint32_t maxValues = 0;
-            for (size_t b = 0; b + 1 < offsets.size(); ++b) {
-                maxValues = std::max(maxValues, offsets[b + 1] - offsets[b]);
-            }
-            const bool wholeTile = TileLdsBytes(m.LayoutBuckets, 1) <= kMaxTileLdsBytes;
-            const bool rowsInRegisters =
-                maxValues <= 127 && (wholeTile ? switches.RowTile && RowTileWaves(m.LayoutBuckets) != 0
-                                               : switches.PairTile && PairTileLdsBytes(m.LayoutBuckets, 8) <= kMaxTileLdsBytes);
-            if (!wholeTile || rowsInRegisters) {
+            if (TileLdsBytes(m.LayoutBuckets, 1) > kMaxTileLdsBytes) {
                 const size_t pitch = m.MaxDepth <= 6 ? 64 : 256;
-                // zeros at the end: those kernels fetch ahead of their trees without a bound
+                // zeros at the end: the pair-tile kernel fetches ahead of its trees without a bound
                 std::vector<double> fixed((trees.GetTreeCount() + dev::kPairTreePadding) * pitch, 0.0);
                 for (size_t t = 0; t < trees.GetTreeCount(); ++t) {
                     std::copy_n(trees.LeafValues.begin() + trees.TreeFirstLeafOffsets[t], size_t(1) << trees.TreeSizes[t],
                                 fixed.begin() + t * pitch);
                 }
                 m.HalfTileLeaves.Upload(fixed);
-            }
-            if (rowsInRegisters) {
-                const uint32_t bucketBytes = wholeTile ? 256u : 128u;
-                std::vector<uint32_t> pairRows((trees.GetTreeCount() + dev::kPairTreePadding) * dev::kPackedTreeDwords, 0);
-                for (size_t t = 0; t < trees.GetTreeCount(); ++t) {
-                    uint32_t* row = pairRows.data() + t * dev::kPackedTreeDwords;
-                    bool anyXor = false;
-                    for (int d = 0; d < trees.TreeSizes[t]; ++d) {
-                        const auto& rb = trees.RepackedBins[trees.TreeStartOffsets[t] + d];
-                        row[d] = static_cast<uint32_t>(rb.FeatureIndex) * bucketBytes;
-                        if (rb.XorMask != 0 || rb.SplitIdx == 0xff) {
-                            // one-hot: bin == value, value = ~XorMask; 7 bits of it are enough below 128
-                            row[d] |= (static_cast<uint32_t>(rb.XorMask) & 0x7fu) << 24;
-                            row[8 + d] = 0x01010101u;
-                            anyXor = true;
-                        } else {
-                            row[8 + d] = (128u - rb.SplitIdx) * 0x01010101u;
-                        }
-                    }
-                    if (anyXor) {
-                        row[0] |= dev::kPairRowXorFlag;
-                    }
+                // two trees per wave: every bin of the model below 128 (the one-hot test then fits 7 bits too)
+                if (switches.PairTile && maxBucketValues <= 127 && PairTileLdsBytes(m.LayoutBuckets, 8) <= kMaxTileLdsBytes) {
+                    m.PairRows.Upload(rowsInRegisters(128));
                 }
-                (wholeTile ? m.TileRows : m.PairRows).Upload(pairRows);
             }
         }
         m.LeavesPairAligned = true;
@@ -1973,6 +1991,30 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
             f.Usable = true;
         }
     }
+
+    // Models that the register kernels do not take, every bin below 128, the 256-document tile and the leaf
+    // regions of eight waves in LDS: a tree's row in registers (EvalObliviousRowTileKernel).
+    if (!m.RegKernelUsable && m.Oblivious && m.MaxDepth <= 8 && TreeCount > 0 && switches.RowTile && maxBucketValues <= 127 &&
+        RowTileWaves(m.LayoutBuckets, m.MaxDepth, m.Dim) != 0) {
+        const size_t leavesPerTree = m.MaxDepth <= 6 ? 64 : 256;
+        const size_t dims = RowTileDims(m.MaxDepth, m.Dim), slices = (static_cast<size_t>(m.Dim) + dims - 1) / dims;
+        const size_t tableTrees = TreeCount + dev::kPairTreePadding;  // zeros at the end: the kernel fetches ahead of its trees
+        std::vector<double> values(slices * tableTrees * leavesPerTree * dims, 0.0);
+        for (size_t t = 0; t < TreeCount; ++t) {
+            const double* leaf = trees.LeafValues.data() + trees.TreeFirstLeafOffsets[t];
+            for (size_t l = 0; l < (size_t(1) << trees.TreeSizes[t]); ++l) {
+                for (size_t d = 0; d < static_cast<size_t>(m.Dim); ++d) {
+                    // [slice][tree][pair of dimensions][leaf][dimension of the pair]; one dimension: [tree][leaf]
+                    const size_t slice = d / dims, k = d % dims;
+                    const size_t slot = dims == 1 ? l : ((k / 2) * leavesPerTree + l) * 2 + k % 2;
+                    values[(slice * tableTrees + t) * leavesPerTree * dims + slot] = leaf[l * m.Dim + d];
+                }
+            }
+        }
+        m.TileLeaves.Upload(values);
+        m.TileSliceStride = tableTrees * leavesPerTree * dims / 2;
+        m.TileRows.Upload(rowsInRegisters(256));
+    }
 }
 
 THipEvaluator::~THipEvaluator() = default;
@@ -2396,28 +2438,34 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
     }
     const int dchunk = TileChunk(m.Dim);
     if (m.TileRows.Get() != nullptr) {
-        // one-dimensional, 7-bit bins, the tile fits: a tree's row in registers
+        // 7-bit bins, the tile fits: a tree's row in registers
         const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
-        const uint32_t waves = RowTileWaves(m.LayoutBuckets);
-        const size_t lds = RowTileLdsBytes(m.LayoutBuckets, waves);
+        const uint32_t waves = RowTileWaves(m.LayoutBuckets, m.MaxDepth, m.Dim);
+        const uint32_t dims = RowTileDims(m.MaxDepth, m.Dim);
+        const size_t lds = RowTileLdsBytes(m.LayoutBuckets, m.MaxDepth, dims, waves);
         const auto launch = [&](auto kernel) {
             EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds);
             hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(blocks)), dim3(64 * waves), lds, s,
                                reinterpret_cast<const uint32_t*>(bins), docCount, m.LayoutBuckets,
                                reinterpret_cast<const uint4*>(m.TileRows.Get()),
-                               reinterpret_cast<const double2*>(m.HalfTileLeaves.Get()), m.Bias.Get(), m.Scale, tb, te,
-                               results);
+                               reinterpret_cast<const double2*>(m.TileLeaves.Get()), m.Bias.Get(), m.Scale,
+                               static_cast<uint32_t>(m.Dim), m.TileSliceStride, tb, te, results);
         };
+        const bool wide = waves == dev::kWideTileWaves;
         if (m.MaxDepth <= 6) {
-            if (waves == dev::kTileWaves) {
-                launch(dev::EvalObliviousRowTileKernel<6, dev::kTileWaves>);
+            if (dims == 1) {
+                wide ? launch(dev::EvalObliviousRowTileKernel<6, dev::kWideTileWaves, 1>)
+                     : launch(dev::EvalObliviousRowTileKernel<6, dev::kTileWaves, 1>);
             } else {
-                launch(dev::EvalObliviousRowTileKernel<6, dev::kWideTileWaves>);
+                wide ? launch(dev::EvalObliviousRowTileKernel<6, dev::kWideTileWaves, 2>)
+                     : launch(dev::EvalObliviousRowTileKernel<6, dev::kTileWaves, 2>);
             }
-        } else if (waves == dev::kTileWaves) {
-            launch(dev::EvalObliviousRowTileKernel<8, dev::kTileWaves>);
+        } else if (dims == 1) {
+            wide ? launch(dev::EvalObliviousRowTileKernel<8, dev::kWideTileWaves, 1>)
+                 : launch(dev::EvalObliviousRowTileKernel<8, dev::kTileWaves, 1>);
         } else {
-            launch(dev::EvalObliviousRowTileKernel<8, dev::kWideTileWaves>);
+            wide ? launch(dev::EvalObliviousRowTileKernel<8, dev::kWideTileWaves, 2>)
+                 : launch(dev::EvalObliviousRowTileKernel<8, dev::kTileWaves, 2>);
         }
         HIP_CHECK(hipGetLastError());
         return;

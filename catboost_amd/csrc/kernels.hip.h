@@ -1413,28 +1413,36 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousPairTileKernel(
     }
 }
 
-// One-dimensional models of 7-bit bins whose 256-document tile fits LDS, one tree per wave: the walk of
+// Models of 7-bit bins whose 256-document tile fits LDS, one tree per wave: the walk of
 // EvalObliviousPairTileKernel on the whole tile. A tree's row is `tileRows` (the format of pairRows with
-// bucket * 256 as the byte offset) and sits in registers, the same in every lane, so a level is an LDS read
-// and three vector instructions with no lane reads and no scalar arithmetic; the leaf values (1 << MAXD per
-// tree at a fixed pitch in `leaves2`) go through the wave's LDS region; rows and values are fetched
-// kPairAhead rounds ahead without looking at the tree range (both tables end with kRowTilePadding trees' worth
-// of zeros). Waves take the trees round robin; their partial sums are added in wave order at the end.
-// grid = doc blocks, block = 64 * WAVES, dynamic LDS = buckets * 256 (rounded up to 16) + WAVES * 256 * 8 bytes
-// (the leaf regions, later the partial sums).
+// bucket * 256 as the byte offset); its address is the same in every lane, so it comes through scalar loads
+// and a level is an LDS read and three vector instructions with no lane reads and no scalar arithmetic. The
+// leaf values go through the wave's LDS region; rows and values are fetched kPairAhead rounds ahead without
+// looking at the tree range (both tables end with kRowTilePadding trees' worth of zeros). Waves take the trees
+// round robin; their partial sums are added in wave order through an accumulator in LDS at the end.
+// Leaf values: one dimension: (1 << MAXD) values per tree. Several dimensions: a workgroup sums DIMS (2; 4 is
+// written out but spills at sixteen waves) of them at a time, slice after slice of the model's dimensions over the same tile, every slice with another
+// walk of the trees; `leaves2` is [slice][tree][piece][leaf] pairs of values (16 bytes: dimensions 2 * piece and
+// 2 * piece + 1 of the slice, zeros past the model's last dimension), sliceStride pairs per slice. A wave's
+// 16-byte gathers of one piece then spread over all groups of four LDS banks, which leaf rows of 32 bytes would
+// not.
+// grid = doc blocks, block = 64 * WAVES, dynamic LDS = buckets * 256 (rounded up to 16) + 256 * DIMS * 8 (the
+// accumulator) + WAVES * (1 << MAXD) * DIMS * 8 bytes (the leaf regions).
 constexpr int kRowTilePadding = kWideTileWaves * kPairAhead;
 static_assert(kRowTilePadding <= kPairTreePadding, "the two kernels share the padded leaf table");
 
-template <int MAXD, int WAVES>
+template <int MAXD, int WAVES, int DIMS>
 __global__ __launch_bounds__(64 * WAVES) void EvalObliviousRowTileKernel(
     const uint32_t* __restrict__ bins, size_t docCount, uint32_t bucketCount, const uint4* __restrict__ tileRows,
-    const double2* __restrict__ leaves2, const double* __restrict__ bias, double scale, uint32_t treeBegin,
-    uint32_t treeEnd, double* __restrict__ out) {
+    const double2* __restrict__ leaves2, const double* __restrict__ bias, double scale, uint32_t dim,
+    size_t sliceStride, uint32_t treeBegin, uint32_t treeEnd, double* __restrict__ out) {
     constexpr uint32_t kLeaves = 1u << MAXD;
-    constexpr uint32_t kRegion = 256;                    // doubles of a wave's region: its tree's values, its sums
-    constexpr int kLeafRegs = MAXD == 8 ? 2 : 1;         // 16-byte pieces of a tree's leaf values per lane
-    constexpr uint32_t kPieceMask = kLeaves / 2 - 1;     // 64 leaves: the upper lanes repeat the lower lanes' pieces
+    constexpr uint32_t kTreePieces = kLeaves * DIMS / 2;     // 16-byte pieces of a tree's leaf values (of a slice)
+    constexpr int kLeafRegs = kTreePieces > kWave ? static_cast<int>(kTreePieces / kWave) : 1;
+    constexpr uint32_t kPieceMask = kTreePieces - 1;         // 32 pieces: the upper lanes repeat the lower lanes' pieces
+    constexpr int kPairsPerLeaf = DIMS > 1 ? DIMS / 2 : 1;
     static_assert(MAXD == 8 || MAXD == 6, "64 or 256 leaves per tree");
+    static_assert(DIMS == 1 || DIMS == 2 || DIMS == 4, "one value or whole pairs per leaf");
     static_assert(WAVES <= kWideTileWaves, "the tables are padded for that many waves");
     extern __shared__ uint32_t sTile[];
     const uint32_t tid = threadIdx.x;
@@ -1447,25 +1455,22 @@ __global__ __launch_bounds__(64 * WAVES) void EvalObliviousRowTileKernel(
         sTile[i] = src[i];
     }
     const uint32_t tileBytes = (tileDwords * 4 + 15) & ~15u;
-    double* leafArea = reinterpret_cast<double*>(reinterpret_cast<uint8_t*>(sTile) + tileBytes);
-    double2* sLeafWave2 = reinterpret_cast<double2*>(leafArea + wave * kRegion);
-    const double* sLeafMine = leafArea + wave * kRegion;
+    double* sRed = reinterpret_cast<double*>(reinterpret_cast<uint8_t*>(sTile) + tileBytes);  // [DIMS][256 documents]
+    double* leafArea = sRed + kDocsPerBlock * DIMS;
+    double2* sLeafWave2 = reinterpret_cast<double2*>(leafArea + wave * kLeaves * DIMS);
+    const double* sLeafMine = leafArea + wave * kLeaves * DIMS;
     const uint8_t* laneTile = reinterpret_cast<const uint8_t*>(sTile) + lane * 4;
-    __syncthreads();  // tile is loaded
-
     const uint32_t treeCount = treeEnd - treeBegin;
-    double acc[4] = {0.0, 0.0, 0.0, 0.0};
     constexpr int kAhead = kPairAhead;
-    uint4 rows[kAhead][4];
-    double2 pref[kAhead][kLeafRegs];
-    const double2* myLeaves = leaves2 + (lane & kPieceMask);
+    static_assert(kAhead == 3, "the rounds below are written out for three register sets");
+
 #define CBAMD_FETCH_TREE(k, tree)                                                                  \
     do {                                                                                           \
         const uint4* row = tileRows + static_cast<size_t>(tree) * 4;                               \
         _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                            \
             rows[k][i] = row[i];                                                                   \
         }                                                                                          \
-        const double2* values = myLeaves + static_cast<size_t>(tree) * (kLeaves / 2);              \
+        const double2* values = myLeaves + static_cast<size_t>(tree) * kTreePieces;                \
         _Pragma("unroll") for (int i = 0; i < kLeafRegs; ++i) {                                    \
             pref[k][i] = values[i * kWave];                                                        \
         }                                                                                          \
@@ -1488,9 +1493,8 @@ __global__ __launch_bounds__(64 * WAVES) void EvalObliviousRowTileKernel(
     // One round of a wave, as in the two-tree kernel: the values that the previous round gathered are added
     // while this round's LDS reads are under way, the registers of this tree take the tree kAhead rounds ahead
     // as soon as every level has read them, and the gathers go out last.
-    constexpr int kLoadsBehind = 2 * (4 + kLeafRegs);  // loads of the two rounds behind the one that is waited for
+    constexpr int kLoadsBehind = 2 * kLeafRegs;  // vector loads of the two rounds behind the one that is waited for
     constexpr int kWaitLoads = 0x0f70 | (kLoadsBehind & 15) | ((kLoadsBehind >> 4) << 14);  // vmcnt(kLoadsBehind)
-    double gathered[4] = {0.0, 0.0, 0.0, 0.0};
 #define CBAMD_TREE_ROUND(k)                                                                        \
     do {                                                                                           \
         uint32_t idx4;                                                                             \
@@ -1498,67 +1502,107 @@ __global__ __launch_bounds__(64 * WAVES) void EvalObliviousRowTileKernel(
         __builtin_amdgcn_sched_barrier(0);                                                         \
         CBAMD_PUBLISH_AND_WALK(k, idx4);                                                           \
         _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                            \
-            acc[q] = __dadd_rn(acc[q], gathered[q]);                                               \
+            _Pragma("unroll") for (int c = 0; c < DIMS; ++c) {                                     \
+                acc[q][c] = __dadd_rn(acc[q][c], gathered[q][c]);                                  \
+            }                                                                                      \
         }                                                                                          \
         __builtin_amdgcn_sched_barrier(0);                                                         \
         CBAMD_FETCH_TREE(k, treeBegin + p + kAhead * WAVES);                                       \
         __builtin_amdgcn_sched_barrier(0);                                                         \
         _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                            \
-            gathered[q] = sLeafMine[(idx4 >> (8 * q + 8 - MAXD)) & (kLeaves - 1)];                 \
+            const uint32_t leaf = (idx4 >> (8 * q + 8 - MAXD)) & (kLeaves - 1);                    \
+            if constexpr (DIMS == 1) {                                                             \
+                gathered[q][0] = sLeafMine[leaf];                                                  \
+            } else {                                                                               \
+                _Pragma("unroll") for (int piece = 0; piece < kPairsPerLeaf; ++piece) {            \
+                    const double2 pair = reinterpret_cast<const double2*>(sLeafMine)[piece * kLeaves + leaf]; \
+                    gathered[q][2 * piece] = pair.x;                                               \
+                    gathered[q][2 * piece + 1] = pair.y;                                           \
+                }                                                                                  \
+            }                                                                                      \
         }                                                                                          \
         __builtin_amdgcn_wave_barrier();                                                           \
         p += WAVES;                                                                                \
     } while (0)
 
-    uint32_t p = wave;
+    const uint32_t slices = (dim + DIMS - 1) / DIMS;
+    for (uint32_t slice = 0; slice < slices; ++slice) {
+        __syncthreads();  // tile is loaded / the previous slice's accumulator has been read
+        double acc[4][DIMS], gathered[4][DIMS];
 #pragma unroll
-    for (int k = 0; k < kAhead; ++k) {
-        // (written before the loads so that the arrays stay in registers)
+        for (int q = 0; q < 4; ++q) {
 #pragma unroll
-        for (int i = 0; i < kLeafRegs; ++i) {
-            pref[k][i] = {0.0, 0.0};
+            for (int c = 0; c < DIMS; ++c) {
+                acc[q][c] = 0.0;
+                gathered[q][c] = 0.0;
+            }
         }
-        CBAMD_FETCH_TREE(k, treeBegin + p + k * WAVES);
-    }
-    static_assert(kAhead == 3, "the rounds below are written out for three register sets");
-    // whole turns of the three register sets without a branch between the rounds, so that the waits for
-    // the loads count only the loads that are older than the one needed
-    while (p + 2 * WAVES < treeCount) {
-        CBAMD_TREE_ROUND(0);
-        CBAMD_TREE_ROUND(1);
-        CBAMD_TREE_ROUND(2);
-    }
-    if (p < treeCount) {
-        CBAMD_TREE_ROUND(0);
-        if (p < treeCount) {
+        uint4 rows[kAhead][4];
+        double2 pref[kAhead][kLeafRegs];
+        const double2* myLeaves = leaves2 + slice * sliceStride + (lane & kPieceMask);
+        uint32_t p = wave;
+#pragma unroll
+        for (int k = 0; k < kAhead; ++k) {
+            // (written before the loads so that the arrays stay in registers)
+#pragma unroll
+            for (int i = 0; i < kLeafRegs; ++i) {
+                pref[k][i] = {0.0, 0.0};
+            }
+            CBAMD_FETCH_TREE(k, treeBegin + p + k * WAVES);
+        }
+        // whole turns of the three register sets without a branch between the rounds, so that the waits for
+        // the loads count only the loads that are older than the one needed
+        while (p + 2 * WAVES < treeCount) {
+            CBAMD_TREE_ROUND(0);
             CBAMD_TREE_ROUND(1);
+            CBAMD_TREE_ROUND(2);
         }
-    }
+        if (p < treeCount) {
+            CBAMD_TREE_ROUND(0);
+            if (p < treeCount) {
+                CBAMD_TREE_ROUND(1);
+            }
+        }
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        acc[q] = __dadd_rn(acc[q], gathered[q]);
+        for (int q = 0; q < 4; ++q) {
+#pragma unroll
+            for (int c = 0; c < DIMS; ++c) {
+                acc[q][c] = __dadd_rn(acc[q][c], gathered[q][c]);
+            }
+        }
+        // waves add their partial sums in wave order into the LDS accumulator; the last wave finishes the values
+        // and writes them out (byte q of a lane's dword: document q * 64 + lane)
+        for (uint32_t w = 0; w + 1 < WAVES; ++w) {
+            if (wave == w) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+#pragma unroll
+                    for (int c = 0; c < DIMS; ++c) {
+                        double* cell = sRed + c * kDocsPerBlock + q * kWave + lane;
+                        *cell = (w == 0) ? acc[q][c] : __dadd_rn(*cell, acc[q][c]);
+                    }
+                }
+            }
+            __syncthreads();
+        }
+        if (wave == WAVES - 1) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const size_t doc = block * kDocsPerBlock + q * kWave + lane;
+#pragma unroll
+                for (int c = 0; c < DIMS; ++c) {
+                    const uint32_t d = slice * DIMS + c;
+                    if (doc < docCount && d < dim) {
+                        const double sum = __dadd_rn(sRed[c * kDocsPerBlock + q * kWave + lane], acc[q][c]);
+                        out[doc * dim + d] = Finish(sum, scale, bias[d], treeBegin == 0);
+                    }
+                }
+            }
+        }
     }
 #undef CBAMD_TREE_ROUND
 #undef CBAMD_FETCH_TREE
 #undef CBAMD_PUBLISH_AND_WALK
-    __syncthreads();  // every wave is through with its leaf region: the area now takes the partial sums
-    double* sRed = leafArea;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        sRed[wave * kRegion + q * kWave + lane] = acc[q];  // byte q of a lane's dword: document q * 64 + lane
-    }
-    __syncthreads();
-    if (tid < kDocsPerBlock) {
-        double sum = sRed[tid];
-#pragma unroll
-        for (int part = 1; part < WAVES; ++part) {
-            sum = __dadd_rn(sum, sRed[part * kRegion + tid]);
-        }
-        const size_t doc = block * kDocsPerBlock + tid;
-        if (doc < docCount) {
-            out[doc] = Finish(sum, scale, bias[0], treeBegin == 0);
-        }
-    }
 }
 
 __device__ __forceinline__ uint32_t BinOfDoc(const uint8_t* bins, size_t doc, uint32_t bucketCount, uint32_t bucket) {

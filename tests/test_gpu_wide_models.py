@@ -106,3 +106,32 @@ def test_tile_models_against_the_oracle(monkeypatch, rows_in_registers, seed, n_
             np.testing.assert_allclose(g.calc_flat(x, tree_start=begin, tree_end=end),
                                        o.calc(x, tree_start=begin, tree_end=end), rtol=RTOL, atol=ATOL,
                                        err_msg="trees %d..%d" % (begin, end))
+
+
+@pytest.mark.parametrize("seed,dim,n_float,n_cat,trees,max_depth,docs,registers", [
+    (31, 2, 300, 0, 300, 8, 1000, "1"),   # two dimensions: one slice
+    (32, 3, 280, 6, 300, 6, 513, "1"),    # 64 leaves; two slices, the second with a dimension to spare; one-hot levels
+    (33, 10, 420, 0, 400, 6, 255, "1"),   # five slices
+    (34, 5, 300, 2, 200, 8, 4097, "1"),   # 256 leaves, three slices
+    (35, 3, 30, 2, 50, 8, 700, "0"),      # a small tile: two workgroups of eight waves per CU
+    (36, 13, 520, 0, 450, 5, 129, "1"),   # 494 buckets: room for eight leaf regions only
+])
+def test_tile_models_of_several_dimensions(monkeypatch, seed, dim, n_float, n_cat, trees, max_depth, docs, registers):
+    """Models of several dimensions on the tile kernel with a tree's row in registers: a workgroup sums two
+    dimensions at a time over the same tile, slice after slice."""
+    rng = np.random.default_rng(seed)
+    model, cat_values = _random_oblivious(rng, n_float=n_float, n_cat=n_cat, trees=trees, max_depth=max_depth, dim=dim,
+                                          scale=float(rng.choice([1.0, -0.5])), bias=rng.normal(size=dim))
+    x = _random_flat_data(rng, model, cat_values, docs)
+    o = OracleModel(model)
+    monkeypatch.setenv("CATBOOST_AMD_REG_KERNEL", registers)
+    g = cb.ModelCalcer()
+    g.load_from_dict(model)
+    g.enable_gpu_evaluation(0)
+    kernels = g.evaluator().describe_kernels(cb.LAYOUT_FLAT_ROWS, docs)
+    assert kernels["evaluate"] == "EvalObliviousRowTileKernel", kernels
+    np.testing.assert_allclose(g.calc_flat(x), o.calc(x), rtol=RTOL, atol=ATOL)
+    for begin, end in ((0, 1), (1, 2), (0, 17), (0, trees - 1), (1, trees), (3, 3), (trees // 2, trees)):
+        np.testing.assert_allclose(g.calc_flat(x, tree_start=begin, tree_end=end),
+                                   o.calc(x, tree_start=begin, tree_end=end), rtol=RTOL, atol=ATOL,
+                                   err_msg="trees %d..%d" % (begin, end))
