@@ -1015,6 +1015,9 @@ struct THipEvaluator::TImpl {
     TDeviceVec<uint32_t> TileRows;     // row-tile kernel (whole tile, one tree per wave): the same with 256 bytes per bucket
     TDeviceVec<double> TileLeaves;     // its leaf values: [slice of the dimensions][tree][pair of dimensions][leaf][2]
     size_t TileSliceStride = 0;        // 16-byte pairs of TileLeaves per slice
+    TDeviceVec<uint32_t> TileMap;      // rows of the tile of the row-tile or pair-tile kernel when buckets of more than
+                                       // 127 values take two; empty: a row per bucket
+    uint32_t TileRowCount = 0;
     TDeviceVec<double> LeavesPadded;   // tile kernel, multi-dimensional: [tree][chunk][leaf][TileChunk(dim)]
     bool PackedSevenBit = false;
     bool LeavesPairAligned = false;  // every tree's first leaf value sits at an even index
@@ -1425,13 +1428,27 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
     }
     m.Bias.Upload(trees.Bias);
 
-    uint32_t maxBucketValues = 0;  // one-hot buckets included
+    // The kernels that keep a tree's row in registers (two trees per wave on half a tile, one on a whole tile)
+    // compare 7 bits. Their tile has a row per bucket, and two for a float bucket of more than 127 values:
+    // min(bin, 127) and max(bin - 127, 0), which the kernel makes while it copies the bins to LDS (tileMap). A
+    // one-hot bucket of more than 127 values keeps the model off these kernels.
+    std::vector<uint32_t> tileRowOfBucket(offsets.size(), 0), tileMap;
+    bool tileRowsUsable = true, tileRowsSplit = false;
     for (size_t b = 0; b + 1 < offsets.size(); ++b) {
-        maxBucketValues = std::max(maxBucketValues, offsets[b + 1] - offsets[b]);
+        tileRowOfBucket[b] = static_cast<uint32_t>(tileMap.size());
+        if (offsets[b + 1] - offsets[b] <= 127) {
+            tileMap.push_back(static_cast<uint32_t>(b));
+        } else if (!(flags[b] & dev::kBucketFlagOneHot)) {
+            tileMap.push_back(static_cast<uint32_t>(b) | (dev::kTileMapLow << 16));
+            tileMap.push_back(static_cast<uint32_t>(b) | (dev::kTileMapHigh << 16));
+            tileRowsSplit = true;
+        } else {
+            tileRowsUsable = false;
+        }
     }
-    // Rows of the kernels that keep a tree's row in registers (two trees per wave on half a tile, one on a whole
-    // tile; every bin of the model below 128): 16 dwords per tree, slot d the byte offset of level d's bucket in
-    // the tile | xor byte << 24, slot 8 + d the value added to the four bins of a dword.
+    const uint32_t tileRowCount = static_cast<uint32_t>(tileMap.size());
+    // Their rows: 16 dwords per tree, slot d the byte offset of level d's row in the tile | xor byte << 24, slot
+    // 8 + d the value added to the four bins of a dword.
     const auto rowsInRegisters = [&](uint32_t bucketBytes) {
         std::vector<uint32_t> rows((trees.GetTreeCount() + dev::kPairTreePadding) * dev::kPackedTreeDwords, 0);
         for (size_t t = 0; t < trees.GetTreeCount(); ++t) {
@@ -1439,12 +1456,15 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
             bool anyXor = false;
             for (int d = 0; d < trees.TreeSizes[t]; ++d) {
                 const auto& rb = trees.RepackedBins[trees.TreeStartOffsets[t] + d];
-                row[d] = static_cast<uint32_t>(rb.FeatureIndex) * bucketBytes;
+                row[d] = tileRowOfBucket[rb.FeatureIndex] * bucketBytes;
                 if (rb.XorMask != 0 || rb.SplitIdx == 0xff) {
                     // one-hot: bin == value, value = ~XorMask; 7 bits of it are enough below 128
                     row[d] |= (static_cast<uint32_t>(rb.XorMask) & 0x7fu) << 24;
                     row[8 + d] = 0x01010101u;
                     anyXor = true;
+                } else if (rb.SplitIdx > 127) {
+                    row[d] += bucketBytes;  // the bucket's second row holds max(bin - 127, 0)
+                    row[8 + d] = (128u - (rb.SplitIdx - 127u)) * 0x01010101u;
                 } else {
                     row[8 + d] = (128u - rb.SplitIdx) * 0x01010101u;
                 }
@@ -1543,8 +1563,12 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
                 }
                 m.HalfTileLeaves.Upload(fixed);
                 // two trees per wave: every bin of the model below 128 (the one-hot test then fits 7 bits too)
-                if (switches.PairTile && maxBucketValues <= 127 && PairTileLdsBytes(m.LayoutBuckets, 8) <= kMaxTileLdsBytes) {
+                if (switches.PairTile && tileRowsUsable && PairTileLdsBytes(tileRowCount, 8) <= kMaxTileLdsBytes) {
                     m.PairRows.Upload(rowsInRegisters(128));
+                    m.TileRowCount = tileRowCount;
+                    if (tileRowsSplit) {
+                        m.TileMap.Upload(tileMap);
+                    }
                 }
             }
         }
@@ -1994,8 +2018,8 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
 
     // Models that the register kernels do not take, every bin below 128, the 256-document tile and the leaf
     // regions of eight waves in LDS: a tree's row in registers (EvalObliviousRowTileKernel).
-    if (!m.RegKernelUsable && m.Oblivious && m.MaxDepth <= 8 && TreeCount > 0 && switches.RowTile && maxBucketValues <= 127 &&
-        RowTileWaves(m.LayoutBuckets, m.MaxDepth, m.Dim) != 0) {
+    if (!m.RegKernelUsable && m.Oblivious && m.MaxDepth <= 8 && TreeCount > 0 && switches.RowTile && tileRowsUsable &&
+        RowTileWaves(tileRowCount, m.MaxDepth, m.Dim) != 0) {
         const size_t leavesPerTree = m.MaxDepth <= 6 ? 64 : 256;
         const size_t dims = RowTileDims(m.MaxDepth, m.Dim), slices = (static_cast<size_t>(m.Dim) + dims - 1) / dims;
         const size_t tableTrees = TreeCount + dev::kPairTreePadding;  // zeros at the end: the kernel fetches ahead of its trees
@@ -2014,6 +2038,10 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         m.TileLeaves.Upload(values);
         m.TileSliceStride = tableTrees * leavesPerTree * dims / 2;
         m.TileRows.Upload(rowsInRegisters(256));
+        m.TileRowCount = tileRowCount;
+        if (tileRowsSplit) {
+            m.TileMap.Upload(tileMap);
+        }
     }
 }
 
@@ -2440,14 +2468,14 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
     if (m.TileRows.Get() != nullptr) {
         // 7-bit bins, the tile fits: a tree's row in registers
         const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
-        const uint32_t waves = RowTileWaves(m.LayoutBuckets, m.MaxDepth, m.Dim);
+        const uint32_t waves = RowTileWaves(m.TileRowCount, m.MaxDepth, m.Dim);
         const uint32_t dims = RowTileDims(m.MaxDepth, m.Dim);
-        const size_t lds = RowTileLdsBytes(m.LayoutBuckets, m.MaxDepth, dims, waves);
+        const size_t lds = RowTileLdsBytes(m.TileRowCount, m.MaxDepth, dims, waves);
         const auto launch = [&](auto kernel) {
             EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds);
             hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(blocks)), dim3(64 * waves), lds, s,
-                               reinterpret_cast<const uint32_t*>(bins), docCount, m.LayoutBuckets,
-                               reinterpret_cast<const uint4*>(m.TileRows.Get()),
+                               reinterpret_cast<const uint32_t*>(bins), docCount, m.LayoutBuckets, m.TileMap.Get(),
+                               m.TileRowCount, reinterpret_cast<const uint4*>(m.TileRows.Get()),
                                reinterpret_cast<const double2*>(m.TileLeaves.Get()), m.Bias.Get(), m.Scale,
                                static_cast<uint32_t>(m.Dim), m.TileSliceStride, tb, te, results);
         };
@@ -2489,12 +2517,12 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
         const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
         const int maxd = m.MaxDepth <= 6 ? 6 : 8;
         if (m.PairRows.Get() != nullptr) {
-            const size_t lds = PairTileLdsBytes(m.LayoutBuckets, maxd);
+            const size_t lds = PairTileLdsBytes(m.TileRowCount, maxd);
             const auto launch = [&](auto kernel) {
                 EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds);
                 hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(2 * blocks)), dim3(64 * dev::kTileWaves), lds, s,
-                                   reinterpret_cast<const uint16_t*>(bins), docCount, m.LayoutBuckets,
-                                   reinterpret_cast<const uint4*>(m.PairRows.Get()),
+                                   reinterpret_cast<const uint16_t*>(bins), docCount, m.LayoutBuckets, m.TileMap.Get(),
+                                   m.TileRowCount, reinterpret_cast<const uint4*>(m.PairRows.Get()),
                                    reinterpret_cast<const double2*>(m.HalfTileLeaves.Get()), m.Bias.Get(), m.Scale, tb, te,
                                    results);
             };

@@ -1212,11 +1212,29 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousHalfTileKernel(
 // groups on the same tree and only the first one adding. Partial sums (one per wave and group) are added in a
 // fixed order at the end. The fetches run kPairAhead rounds ahead of the walk without looking at the tree range:
 // both tables end with kPairTreePadding trees' worth of zeros.
-// grid = 2 * doc blocks, block = 64 * kTileWaves threads, dynamic LDS = buckets * 128 (rounded up to 16) +
+// With `tileMap` the tile has rowCount rows (MapTileBins) and the offsets in pairRows name rows, not buckets.
+// grid = 2 * doc blocks, block = 64 * kTileWaves threads, dynamic LDS = rows * 128 (rounded up to 16) +
 // kTileWaves * 2 * max(1 << MAXD, 128) * 8 bytes (the leaf regions, later the partial sums).
 constexpr uint32_t kPairRowXorFlag = 1u << 23;  // slot 0 of a tree's row: some level xors
 constexpr int kPairAhead = 3;
 constexpr int kPairTreePadding = 2 * kTileWaves * kPairAhead;
+
+// Rows of a tile that splits the buckets of more than 127 values in two (`tileMap`, a dword per row: bits 0-15 the
+// bucket, bits 16.. what becomes of its bins: 0 as they are, 1 min(bin, 127), 2 max(bin - 127, 0)), byte-parallel.
+// A split "bin >= s" of such a bucket then reads the first row (s <= 127) or the second (with s - 127), and every
+// level of the model is a 7-bit compare.
+constexpr uint32_t kTileMapLow = 1, kTileMapHigh = 2;
+
+__device__ __forceinline__ uint32_t MapTileBins(uint32_t bins4, uint32_t mode) {
+    const uint32_t high = bins4 & 0x80808080u;  // bytes above 127
+    if (mode == kTileMapLow) {
+        return (bins4 | (high - (high >> 7))) & 0x7f7f7f7fu;
+    }
+    if (mode == kTileMapHigh) {
+        return ((bins4 & 0x7f7f7f7fu) + 0x01010101u) & ((high >> 7) * 0xffu);
+    }
+    return bins4;
+}
 
 template <bool XOR, int MAXD>
 __device__ __forceinline__ uint32_t PairTreeIndexes(const uint8_t* laneTile, const uint4 (&desc)[4]) {
@@ -1249,9 +1267,9 @@ __device__ __forceinline__ uint32_t PairTreeIndexes(const uint8_t* laneTile, con
 
 template <int MAXD>
 __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousPairTileKernel(
-    const uint16_t* __restrict__ bins, size_t docCount, uint32_t bucketCount, const uint4* __restrict__ pairRows,
-    const double2* __restrict__ leaves2, const double* __restrict__ bias, double scale, uint32_t treeBegin,
-    uint32_t treeEnd, double* __restrict__ out) {
+    const uint16_t* __restrict__ bins, size_t docCount, uint32_t bucketCount, const uint32_t* __restrict__ tileMap,
+    uint32_t rowCount, const uint4* __restrict__ pairRows, const double2* __restrict__ leaves2,
+    const double* __restrict__ bias, double scale, uint32_t treeBegin, uint32_t treeEnd, double* __restrict__ out) {
     constexpr uint32_t kLeaves = 1u << MAXD;
     constexpr int kLeafRegs = MAXD == 8 ? 4 : 1;  // 16-byte pieces of a pair's 2 * kLeaves leaf values per lane
     static_assert(MAXD == 8 || MAXD == 6, "64 or 256 leaves per tree");
@@ -1262,10 +1280,18 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousPairTileKernel(
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kWave);
     const size_t block = blockIdx.x >> 1;
     const uint32_t half = blockIdx.x & 1;
-    const uint32_t tileWords = bucketCount * kWave;
-    const uint16_t* src = bins + block * tileWords * 2 + half;
-    for (uint32_t i = tid; i < tileWords; i += 64 * kTileWaves) {
-        sTile16[i] = src[2 * i];
+    const uint32_t tileWords = rowCount * kWave;  // rowCount = bucketCount without a map
+    const uint16_t* src = bins + block * (bucketCount * kWave) * 2 + half;
+    if (tileMap == nullptr) {
+        for (uint32_t i = tid; i < tileWords; i += 64 * kTileWaves) {
+            sTile16[i] = src[2 * i];
+        }
+    } else {
+        for (uint32_t row = wave; row < rowCount; row += kTileWaves) {
+            const uint32_t entry = tileMap[row];
+            const uint32_t bins2 = src[2 * ((entry & 0xffffu) * kWave + lane)];
+            sTile16[row * kWave + lane] = static_cast<uint16_t>(MapTileBins(bins2, entry >> 16));
+        }
     }
     const uint32_t group = lane >> 5;
     const uint32_t tileBytes = (tileWords * 2 + 15) & ~15u;
@@ -1426,16 +1452,18 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousPairTileKernel(
 // 2 * piece + 1 of the slice, zeros past the model's last dimension), sliceStride pairs per slice. A wave's
 // 16-byte gathers of one piece then spread over all groups of four LDS banks, which leaf rows of 32 bytes would
 // not.
-// grid = doc blocks, block = 64 * WAVES, dynamic LDS = buckets * 256 (rounded up to 16) + 256 * DIMS * 8 (the
+// With `tileMap` the tile has rowCount rows (MapTileBins) and the offsets in tileRows name rows, not buckets.
+// grid = doc blocks, block = 64 * WAVES, dynamic LDS = rows * 256 (rounded up to 16) + 256 * DIMS * 8 (the
 // accumulator) + WAVES * (1 << MAXD) * DIMS * 8 bytes (the leaf regions).
 constexpr int kRowTilePadding = kWideTileWaves * kPairAhead;
 static_assert(kRowTilePadding <= kPairTreePadding, "the two kernels share the padded leaf table");
 
 template <int MAXD, int WAVES, int DIMS>
 __global__ __launch_bounds__(64 * WAVES) void EvalObliviousRowTileKernel(
-    const uint32_t* __restrict__ bins, size_t docCount, uint32_t bucketCount, const uint4* __restrict__ tileRows,
-    const double2* __restrict__ leaves2, const double* __restrict__ bias, double scale, uint32_t dim,
-    size_t sliceStride, uint32_t treeBegin, uint32_t treeEnd, double* __restrict__ out) {
+    const uint32_t* __restrict__ bins, size_t docCount, uint32_t bucketCount, const uint32_t* __restrict__ tileMap,
+    uint32_t rowCount, const uint4* __restrict__ tileRows, const double2* __restrict__ leaves2,
+    const double* __restrict__ bias, double scale, uint32_t dim, size_t sliceStride, uint32_t treeBegin,
+    uint32_t treeEnd, double* __restrict__ out) {
     constexpr uint32_t kLeaves = 1u << MAXD;
     constexpr uint32_t kTreePieces = kLeaves * DIMS / 2;     // 16-byte pieces of a tree's leaf values (of a slice)
     constexpr int kLeafRegs = kTreePieces > kWave ? static_cast<int>(kTreePieces / kWave) : 1;
@@ -1449,10 +1477,17 @@ __global__ __launch_bounds__(64 * WAVES) void EvalObliviousRowTileKernel(
     const uint32_t lane = tid & (kWave - 1);
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kWave);
     const size_t block = blockIdx.x;
-    const uint32_t tileDwords = bucketCount * kWave;
-    const uint32_t* src = bins + block * tileDwords;
-    for (uint32_t i = tid; i < tileDwords; i += 64 * WAVES) {
-        sTile[i] = src[i];
+    const uint32_t tileDwords = rowCount * kWave;  // rowCount = bucketCount without a map
+    const uint32_t* src = bins + block * (bucketCount * kWave);
+    if (tileMap == nullptr) {
+        for (uint32_t i = tid; i < tileDwords; i += 64 * WAVES) {
+            sTile[i] = src[i];
+        }
+    } else {
+        for (uint32_t row = wave; row < rowCount; row += WAVES) {
+            const uint32_t entry = tileMap[row];
+            sTile[row * kWave + lane] = MapTileBins(src[(entry & 0xffffu) * kWave + lane], entry >> 16);
+        }
     }
     const uint32_t tileBytes = (tileDwords * 4 + 15) & ~15u;
     double* sRed = reinterpret_cast<double*>(reinterpret_cast<uint8_t*>(sTile) + tileBytes);  // [DIMS][256 documents]

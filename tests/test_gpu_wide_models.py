@@ -54,15 +54,24 @@ def test_wide_models_against_the_oracle(monkeypatch, pair, seed, n_float, n_cat,
                                        err_msg="trees %d..%d" % (begin, end))
 
 
-def test_bins_above_127_keep_the_one_tree_kernel(monkeypatch):
-    """A feature with 300 borders: the byte-parallel compare of the two-tree kernel needs 7-bit bins, so the
-    model stays with the kernel that compares 8 bits in the trees that need it."""
+@pytest.mark.parametrize("n_float,trees,docs,kernel", [
+    (800, 500, 700, "EvalObliviousPairTileKernel"),    # 717 rows of 128 bytes and the leaf regions fit LDS
+    (1100, 900, 300, "EvalObliviousHalfTileKernel"),   # 1045 rows do not: one tree per wave, 8-bit compares
+])
+def test_wide_models_with_bins_above_127(monkeypatch, n_float, trees, docs, kernel):
+    """A feature with 300 borders: its bucket of more than 127 values takes two rows of the tile, min(bin, 127)
+    and max(bin - 127, 0), and the two-tree kernel compares 7 bits as before; when the rows no longer fit LDS
+    the model stays with the kernel that compares 8 bits in the trees that need it."""
     rng = np.random.default_rng(11)
-    model, cat_values = _random_oblivious(rng, n_float=800, n_cat=4, trees=500, max_depth=8, many_borders=True)
-    x = _random_flat_data(rng, model, cat_values, 700)
+    model, cat_values = _random_oblivious(rng, n_float=n_float, n_cat=4, trees=trees, max_depth=8, many_borders=True)
+    assert max(len(f["borders"]) for f in model["float_features"]) > 127
+    x = _random_flat_data(rng, model, cat_values, docs)
+    o = OracleModel(model)
     g = _evaluator(model, monkeypatch, "1")
-    assert g.evaluator().describe_kernels(cb.LAYOUT_FLAT_ROWS, 700)["evaluate"] == "EvalObliviousHalfTileKernel"
-    np.testing.assert_allclose(g.calc_flat(x), OracleModel(model).calc(x), rtol=RTOL, atol=ATOL)
+    assert g.evaluator().describe_kernels(cb.LAYOUT_FLAT_ROWS, docs)["evaluate"] == kernel
+    np.testing.assert_allclose(g.calc_flat(x), o.calc(x), rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(g.calc_flat(x, tree_start=3, tree_end=trees - 2), o.calc(x, tree_start=3, tree_end=trees - 2),
+                               rtol=RTOL, atol=ATOL)
 
 
 def test_two_kernels_agree_on_a_large_batch(monkeypatch):
@@ -84,11 +93,14 @@ def test_two_kernels_agree_on_a_large_batch(monkeypatch):
     (23, 560, 0, 500, 8, 255),    # 552 buckets: the tile leaves room for eight regions only
     (24, 300, 20, 333, 6, 1),     # 64 leaves per tree, a single document
     (25, 560, 2, 400, 3, 4097),   # shallow trees in the 64-leaf kernel
+    (41, 300, 2, 300, 8, 777),    # (seeds from 41: a feature of 300 borders, whose large bucket takes two rows)
+    (43, 500, 0, 800, 8, 64),
 ])
 def test_tile_models_against_the_oracle(monkeypatch, rows_in_registers, seed, n_float, n_cat, trees, max_depth, docs):
     rng = np.random.default_rng(seed)
     model, cat_values = _random_oblivious(rng, n_float=n_float, n_cat=n_cat, trees=trees, max_depth=max_depth,
-                                          scale=float(rng.choice([1.0, -0.5])), bias=rng.normal(size=1))
+                                          many_borders=seed >= 41, scale=float(rng.choice([1.0, -0.5])),
+                                          bias=rng.normal(size=1))
     x = _random_flat_data(rng, model, cat_values, docs)
     o = OracleModel(model)
     monkeypatch.setenv("CATBOOST_AMD_ROW_TILE", rows_in_registers)
@@ -115,13 +127,15 @@ def test_tile_models_against_the_oracle(monkeypatch, rows_in_registers, seed, n_
     (34, 5, 300, 2, 200, 8, 4097, "1"),   # 256 leaves, three slices
     (35, 3, 30, 2, 50, 8, 700, "0"),      # a small tile: two workgroups of eight waves per CU
     (36, 13, 520, 0, 450, 5, 129, "1"),   # 494 buckets: room for eight leaf regions only
+    (42, 3, 350, 3, 200, 6, 900, "1"),    # (seeds from 41: a feature of 300 borders, whose large bucket takes two rows)
 ])
 def test_tile_models_of_several_dimensions(monkeypatch, seed, dim, n_float, n_cat, trees, max_depth, docs, registers):
     """Models of several dimensions on the tile kernel with a tree's row in registers: a workgroup sums two
     dimensions at a time over the same tile, slice after slice."""
     rng = np.random.default_rng(seed)
     model, cat_values = _random_oblivious(rng, n_float=n_float, n_cat=n_cat, trees=trees, max_depth=max_depth, dim=dim,
-                                          scale=float(rng.choice([1.0, -0.5])), bias=rng.normal(size=dim))
+                                          many_borders=seed >= 41, scale=float(rng.choice([1.0, -0.5])),
+                                          bias=rng.normal(size=dim))
     x = _random_flat_data(rng, model, cat_values, docs)
     o = OracleModel(model)
     monkeypatch.setenv("CATBOOST_AMD_REG_KERNEL", registers)
