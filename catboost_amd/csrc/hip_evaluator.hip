@@ -1565,7 +1565,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
                 // two trees per wave: every bin of the model below 128 (the one-hot test then fits 7 bits too)
                 if (switches.PairTile && tileRowsUsable && PairTileLdsBytes(tileRowCount, 8) <= kMaxTileLdsBytes) {
                     m.PairRows.Upload(rowsInRegisters(128));
-                    m.TileRowCount = tileRowCount;
+                    m.TileRowCount = tileRowsSplit ? tileRowCount : m.LayoutBuckets;  // (a model without splits: its one zero bucket)
                     if (tileRowsSplit) {
                         m.TileMap.Upload(tileMap);
                     }
@@ -2038,7 +2038,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         m.TileLeaves.Upload(values);
         m.TileSliceStride = tableTrees * leavesPerTree * dims / 2;
         m.TileRows.Upload(rowsInRegisters(256));
-        m.TileRowCount = tileRowCount;
+        m.TileRowCount = tileRowsSplit ? tileRowCount : m.LayoutBuckets;  // (a model without splits: its one zero bucket)
         if (tileRowsSplit) {
             m.TileMap.Upload(tileMap);
         }

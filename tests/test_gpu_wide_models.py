@@ -149,3 +149,24 @@ def test_tile_models_of_several_dimensions(monkeypatch, seed, dim, n_float, n_ca
         np.testing.assert_allclose(g.calc_flat(x, tree_start=begin, tree_end=end),
                                    o.calc(x, tree_start=begin, tree_end=end), rtol=RTOL, atol=ATOL,
                                    err_msg="trees %d..%d" % (begin, end))
+
+
+@pytest.mark.parametrize("dim", [1, 3])
+@pytest.mark.parametrize("row_tile", ["1", "0"])
+def test_trees_without_splits_on_the_tile_kernels(monkeypatch, row_tile, dim):
+    """A model whose trees have no splits has no buckets; its documents keep one all-zero bucket, which is the
+    row that the padding levels of the tile kernels read. Every document gets the sum of the trees' only leaves."""
+    monkeypatch.setenv("CATBOOST_AMD_REG_KERNEL", "0")
+    monkeypatch.setenv("CATBOOST_AMD_ROW_TILE", row_tile)
+    leaves = [([], [0.25 + k for k in range(dim)]), ([], [0.5 - k for k in range(dim)]), ([], [2.0] * dim)]
+    g = cb.ModelCalcer()
+    g.build_oblivious([dict(index=0, flat_index=0)], [], dim, leaves, bias=[1.0] * dim)
+    g.enable_gpu_evaluation(0)
+    kernels = g.evaluator().describe_kernels(cb.LAYOUT_FLAT_ROWS, 700)
+    assert kernels["evaluate"] == ("EvalObliviousRowTileKernel" if row_tile == "1" else "EvalObliviousTileKernel")
+    x = np.random.default_rng(0).normal(size=(700, 1)).astype(np.float32)
+    expected = np.array([1.0 + sum(leaf[1][k] for leaf in leaves) for k in range(dim)])
+    np.testing.assert_allclose(g.calc_flat(x).reshape(700, dim), np.tile(expected, (700, 1)), rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(g.calc_flat(x, tree_start=1, tree_end=3).reshape(700, dim),
+                               np.tile(expected - 1.0 - np.array([leaves[0][1][k] for k in range(dim)]), (700, 1)),
+                               rtol=RTOL, atol=ATOL)
