@@ -513,6 +513,11 @@ uint32_t RowTileWaves(uint32_t buckets, uint32_t maxDepth, int dim) {
     return RowTileLdsBytes(buckets, maxDepth, dims, dev::kTileWaves) <= kMaxTileLdsBytes ? dev::kTileWaves : 0;
 }
 
+// LDS of the deep-tile kernel: 256 documents' bins and the accumulator
+size_t DeepTileLdsBytes(uint32_t rows) {
+    return ((static_cast<size_t>(rows) * 256 + 15) & ~size_t(15)) + dev::kDocsPerBlock * sizeof(double);
+}
+
 // LDS of the pair-tile kernel: 128 documents' bins, then per wave the leaf values of two trees; the same area
 // takes one partial sum per wave, lane group and document at the end
 size_t PairTileLdsBytes(uint32_t buckets, int maxd) {
@@ -1015,6 +1020,8 @@ struct THipEvaluator::TImpl {
     TDeviceVec<uint32_t> TileRows;     // row-tile kernel (whole tile, one tree per wave): the same with 256 bytes per bucket
     TDeviceVec<double> TileLeaves;     // its leaf values: [slice of the dimensions][tree][pair of dimensions][leaf][2]
     size_t TileSliceStride = 0;        // 16-byte pairs of TileLeaves per slice
+    TDeviceVec<uint32_t> DeepRows;     // deep-tile kernel (depth 9 to 16): 32 dwords per tree, two halves of the row-tile form
+    TDeviceVec<uint32_t> DeepFirstLeaf;  // and the trees' first leaf values in Leaves
     TDeviceVec<uint32_t> TileMap;      // rows of the tile of the row-tile or pair-tile kernel when buckets of more than
                                        // 127 values take two; empty: a row per bucket
     uint32_t TileRowCount = 0;
@@ -2043,6 +2050,45 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
             m.TileMap.Upload(tileMap);
         }
     }
+
+    // One-dimensional models of depth 9 to 16 that the register kernels do not take (deeper than 10, one-hot
+    // splits, more registers than they have): the same tile, a tree's levels in two halves of eight, leaf values
+    // gathered from the model's own table (EvalObliviousDeepTileKernel).
+    if (!m.RegKernelUsable && m.Oblivious && m.Dim == 1 && m.MaxDepth > 8 && m.MaxDepth <= 16 && TreeCount > 0 &&
+        switches.RowTile && tileRowsUsable && DeepTileLdsBytes(tileRowsSplit ? tileRowCount : m.LayoutBuckets) <= kMaxTileLdsBytes) {
+        const size_t tableTrees = TreeCount + dev::kPairTreePadding;
+        std::vector<uint32_t> rows(tableTrees * 32, 0), first(tableTrees, 0);
+        for (size_t t = 0; t < TreeCount; ++t) {
+            uint32_t* row = rows.data() + t * 32;
+            bool anyXor = false;
+            for (int d = 0; d < trees.TreeSizes[t]; ++d) {
+                const auto& rb = trees.RepackedBins[trees.TreeStartOffsets[t] + d];
+                uint32_t* half = row + (d < 8 ? 0 : 16);
+                const int slot = d % 8;
+                half[slot] = tileRowOfBucket[rb.FeatureIndex] * 256u;
+                if (rb.XorMask != 0 || rb.SplitIdx == 0xff) {
+                    half[slot] |= (static_cast<uint32_t>(rb.XorMask) & 0x7fu) << 24;
+                    half[8 + slot] = 0x01010101u;
+                    anyXor = true;
+                } else if (rb.SplitIdx > 127) {
+                    half[slot] += 256u;
+                    half[8 + slot] = (128u - (rb.SplitIdx - 127u)) * 0x01010101u;
+                } else {
+                    half[8 + slot] = (128u - rb.SplitIdx) * 0x01010101u;
+                }
+            }
+            if (anyXor) {
+                row[0] |= dev::kPairRowXorFlag;
+            }
+            first[t] = firstLeaf[t];
+        }
+        m.DeepRows.Upload(rows);
+        m.DeepFirstLeaf.Upload(first);
+        m.TileRowCount = tileRowsSplit ? tileRowCount : m.LayoutBuckets;
+        if (tileRowsSplit) {
+            m.TileMap.Upload(tileMap);
+        }
+    }
 }
 
 THipEvaluator::~THipEvaluator() = default;
@@ -2604,6 +2650,27 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
             return;
         }
     }
+    if (m.DeepRows.Get() != nullptr) {
+        const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
+        const size_t lds = DeepTileLdsBytes(m.TileRowCount);
+        const bool wide = 2 * lds > kMaxTileLdsBytes;  // one workgroup per CU: sixteen waves
+        const auto launch = [&](auto kernel) {
+            EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds);
+            hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(blocks)), dim3(64 * (wide ? dev::kWideTileWaves : dev::kTileWaves)),
+                               lds, s, reinterpret_cast<const uint32_t*>(bins), docCount, m.LayoutBuckets, m.TileMap.Get(),
+                               m.TileRowCount, reinterpret_cast<const uint4*>(m.DeepRows.Get()), m.DeepFirstLeaf.Get(),
+                               m.Leaves.Get(), m.Bias.Get(), m.Scale, tb, te, results);
+        };
+        if (m.MaxDepth <= 12) {
+            wide ? launch(dev::EvalObliviousDeepTileKernel<4, dev::kWideTileWaves>)
+                 : launch(dev::EvalObliviousDeepTileKernel<4, dev::kTileWaves>);
+        } else {
+            wide ? launch(dev::EvalObliviousDeepTileKernel<8, dev::kWideTileWaves>)
+                 : launch(dev::EvalObliviousDeepTileKernel<8, dev::kTileWaves>);
+        }
+        HIP_CHECK(hipGetLastError());
+        return;
+    }
     if (m.Dim == 1) {
         LaunchEval<1>(m.Oblivious, bins, docCount, m.LayoutBuckets, tt, tb, te, results, s);
     } else if (m.Dim == 2) {
@@ -2767,6 +2834,8 @@ std::string THipEvaluator::DescribeKernels(int layout, size_t docCount) const {
     } else if (m.Oblivious && m.MaxDepth <= 8 && m.Dim == 1 && m.HalfTileLeaves.Get() != nullptr &&
                TileLdsBytes(m.LayoutBuckets, 1) > kMaxTileLdsBytes) {
         evaluate = m.PairRows.Get() != nullptr ? "EvalObliviousPairTileKernel" : "EvalObliviousHalfTileKernel";
+    } else if (m.DeepRows.Get() != nullptr) {
+        evaluate = "EvalObliviousDeepTileKernel";
     } else if (m.Oblivious) {
         evaluate = "EvalObliviousKernel";
     } else if (m.NsLdsUsable) {

@@ -1640,6 +1640,118 @@ __global__ __launch_bounds__(64 * WAVES) void EvalObliviousRowTileKernel(
 #undef CBAMD_PUBLISH_AND_WALK
 }
 
+// One-dimensional models of depth 9 to 16 on the same tile, one tree per wave: the walk of the row-tile kernel
+// in two halves. `deepRows` holds 32 dwords per tree: the first sixteen as in tileRows for the levels 0..7, the
+// second sixteen for the levels 8..8 + HIGH - 1 (levels past the tree's depth: row 0, add 0, never true; the
+// flag of slot 0 says whether any level of the tree xors). The two halves give a byte per document each,
+// together the leaf index; a tree's table has up to 512 KB, so the leaf values are gathered from global memory,
+// `leaves` + firstLeaf[tree], and added one round later. Rows come two rounds ahead (scalar loads: the address
+// is the same in every lane). Both tables end with kRowTilePadding null trees.
+// grid = doc blocks, block = 64 * WAVES, dynamic LDS = rows * 256 (rounded up to 16) + 256 * 8 bytes.
+template <int HIGH, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void EvalObliviousDeepTileKernel(
+    const uint32_t* __restrict__ bins, size_t docCount, uint32_t bucketCount, const uint32_t* __restrict__ tileMap,
+    uint32_t rowCount, const uint4* __restrict__ deepRows, const uint32_t* __restrict__ firstLeaf,
+    const double* __restrict__ leaves, const double* __restrict__ bias, double scale, uint32_t treeBegin,
+    uint32_t treeEnd, double* __restrict__ out) {
+    static_assert(HIGH == 4 || HIGH == 8, "levels 8..11 or 8..15 in the second half");
+    extern __shared__ uint32_t sTile[];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const size_t block = blockIdx.x;
+    const uint32_t tileDwords = rowCount * kWave;  // rowCount = bucketCount without a map
+    const uint32_t* src = bins + block * (bucketCount * kWave);
+    if (tileMap == nullptr) {
+        for (uint32_t i = tid; i < tileDwords; i += 64 * WAVES) {
+            sTile[i] = src[i];
+        }
+    } else {
+        for (uint32_t row = wave; row < rowCount; row += WAVES) {
+            const uint32_t entry = tileMap[row];
+            sTile[row * kWave + lane] = MapTileBins(src[(entry & 0xffffu) * kWave + lane], entry >> 16);
+        }
+    }
+    const uint32_t tileBytes = (tileDwords * 4 + 15) & ~15u;
+    double* sRed = reinterpret_cast<double*>(reinterpret_cast<uint8_t*>(sTile) + tileBytes);  // [256 documents]
+    const uint8_t* laneTile = reinterpret_cast<const uint8_t*>(sTile) + lane * 4;
+    const uint32_t treeCount = treeEnd - treeBegin;
+    __syncthreads();  // tile is loaded
+
+    double acc[4] = {0.0, 0.0, 0.0, 0.0}, gathered[4] = {0.0, 0.0, 0.0, 0.0};
+    uint4 rows[2][2][4];
+    uint32_t first[2];
+#define CBAMD_FETCH_DEEP(k, tree)                                                                  \
+    do {                                                                                           \
+        const uint4* row = deepRows + static_cast<size_t>(tree) * 8;                               \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                            \
+            rows[k][0][i] = row[i];                                                                \
+            rows[k][1][i] = row[4 + i];                                                            \
+        }                                                                                          \
+        first[k] = firstLeaf[tree];                                                                \
+    } while (0)
+#define CBAMD_DEEP_ROUND(k)                                                                        \
+    do {                                                                                           \
+        uint32_t low4, high4;                                                                      \
+        if (__builtin_amdgcn_readfirstlane(rows[k][0][0].x) & kPairRowXorFlag) {                   \
+            low4 = PairTreeIndexes<true, 8>(laneTile, rows[k][0]);                                 \
+            high4 = PairTreeIndexes<true, HIGH>(laneTile, rows[k][1]);                             \
+        } else {                                                                                   \
+            low4 = PairTreeIndexes<false, 8>(laneTile, rows[k][0]);                                \
+            high4 = PairTreeIndexes<false, HIGH>(laneTile, rows[k][1]);                            \
+        }                                                                                          \
+        const double* treeLeaves = leaves + __builtin_amdgcn_readfirstlane(first[k]);              \
+        _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                            \
+            acc[q] = __dadd_rn(acc[q], gathered[q]);                                               \
+        }                                                                                          \
+        _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                            \
+            const uint32_t leaf = ((low4 >> (8 * q)) & 0xffu) |                                    \
+                                  (((high4 >> (8 * q + 8 - HIGH)) & ((1u << HIGH) - 1)) << 8);     \
+            gathered[q] = treeLeaves[leaf];                                                        \
+        }                                                                                          \
+        CBAMD_FETCH_DEEP(k, treeBegin + p + 2 * WAVES);                                            \
+        p += WAVES;                                                                                \
+    } while (0)
+
+    uint32_t p = wave;
+    CBAMD_FETCH_DEEP(0, treeBegin + p);
+    CBAMD_FETCH_DEEP(1, treeBegin + p + WAVES);
+    while (p + WAVES < treeCount) {
+        CBAMD_DEEP_ROUND(0);
+        CBAMD_DEEP_ROUND(1);
+    }
+    if (p < treeCount) {
+        CBAMD_DEEP_ROUND(0);
+    }
+#undef CBAMD_DEEP_ROUND
+#undef CBAMD_FETCH_DEEP
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        acc[q] = __dadd_rn(acc[q], gathered[q]);
+    }
+    // waves add their partial sums in wave order into the LDS accumulator; the last wave finishes the values
+    // and writes them out (byte q of a lane's dword: document q * 64 + lane)
+    for (uint32_t w = 0; w + 1 < WAVES; ++w) {
+        if (wave == w) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                double* cell = sRed + q * kWave + lane;
+                *cell = (w == 0) ? acc[q] : __dadd_rn(*cell, acc[q]);
+            }
+        }
+        __syncthreads();
+    }
+    if (wave == WAVES - 1) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const size_t doc = block * kDocsPerBlock + q * kWave + lane;
+            if (doc < docCount) {
+                out[doc] = Finish(__dadd_rn(sRed[q * kWave + lane], acc[q]), scale, bias[0], treeBegin == 0);
+            }
+        }
+    }
+}
+
 __device__ __forceinline__ uint32_t BinOfDoc(const uint8_t* bins, size_t doc, uint32_t bucketCount, uint32_t bucket) {
     const size_t block = doc / kDocsPerBlock;
     const uint32_t r = static_cast<uint32_t>(doc % kDocsPerBlock);

@@ -928,7 +928,8 @@ def test_register_kernel_buckets_of_many_values(monkeypatch, split, borders, n_f
     """Float features with 128 and more used borders (values on the borders included, around the 127th above
     all): a bucket of more than 127 values takes two bins registers, min(bin, 127) and max(bin - 127, 0), and the
     model keeps the 7-bit compare; with the switch off it takes the 8-bit one of the mixed kernels. Bit for bit
-    either way (trees of depth 10 have no mixed kernel: those fall back to the plain evaluate kernel)."""
+    either way (trees of depth 10 have no mixed kernel: those go to the tile kernel for deep trees, whose waves
+    add partial sums: within the tolerance)."""
     monkeypatch.setenv("CATBOOST_AMD_REG_SPLIT", split)
     rng = np.random.default_rng(borders + n_float)
     ffs = [mb.float_feature(i, i) for i in range(n_float)]
@@ -956,7 +957,10 @@ def test_register_kernel_buckets_of_many_values(monkeypatch, split, borders, n_f
     else:
         _close(g.calc_flat(x), o.calc(x))
     n = len(model["tree_sizes"])
-    np.testing.assert_array_equal(g.calc_flat(x, tree_start=3, tree_end=n - 2), o.calc(x, tree_start=3, tree_end=n - 2))
+    if evaluate.startswith("cbamd_eval_reg_"):
+        np.testing.assert_array_equal(g.calc_flat(x, tree_start=3, tree_end=n - 2), o.calc(x, tree_start=3, tree_end=n - 2))
+    else:
+        _close(g.calc_flat(x, tree_start=3, tree_end=n - 2), o.calc(x, tree_start=3, tree_end=n - 2))
 
 
 def test_register_kernel_against_tile_kernel():

@@ -46,7 +46,7 @@ def _tree_model_case(seed, rng, asymmetric):
     n_float = int(rng.choice([1, 2, 7, 30, 100, 130, 200, 209, 224, 250, 400]))
     n_cat = int(rng.choice([0, 0, 1, 2, 5]))
     trees = int(rng.choice([1, 2, 17, 40, 150, 400]))
-    max_depth = int(rng.choice([1, 3, 6, 8, 10]))
+    max_depth = int(rng.choice([1, 3, 6, 8, 10, 12]))
     many = bool(rng.integers(0, 2))
     docs = int(rng.choice([1, 2, 63, 64, 65, 255, 256, 257, 1000, 3333, 9000]))
     trees = min(trees, max(1, 40000 // n_float))

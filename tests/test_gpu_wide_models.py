@@ -170,3 +170,33 @@ def test_trees_without_splits_on_the_tile_kernels(monkeypatch, row_tile, dim):
     np.testing.assert_allclose(g.calc_flat(x, tree_start=1, tree_end=3).reshape(700, dim),
                                np.tile(expected - 1.0 - np.array([leaves[0][1][k] for k in range(dim)]), (700, 1)),
                                rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("seed,n_float,n_cat,trees,max_depth,many,docs", [
+    (51, 40, 0, 60, 12, False, 1000),   # twelve levels: four in the second half; two workgroups of eight waves per CU
+    (52, 30, 5, 25, 16, False, 513),    # sixteen levels, one-hot levels in either half
+    (53, 300, 3, 40, 11, True, 255),    # a feature of 300 borders: two rows of the tile for its large bucket
+    (54, 20, 4, 80, 10, False, 4097),   # depth 10 with one-hot splits, which the register kernels do not take
+    (55, 500, 0, 30, 14, False, 64),    # a tile of which one fits a CU: sixteen waves
+])
+def test_deep_trees_on_the_tile_kernel(seed, n_float, n_cat, trees, max_depth, many, docs):
+    """One-dimensional models of depth 9 to 16 outside the register kernels: the tile kernel that walks a tree's
+    levels in two halves and gathers the leaf values from the model's table. Bins and leaf indexes equal the
+    oracle's, predictions within the tolerance (partial sums per wave)."""
+    rng = np.random.default_rng(seed)
+    model, cat_values = _random_oblivious(rng, n_float=n_float, n_cat=n_cat, trees=trees, max_depth=max_depth,
+                                          many_borders=many, scale=float(rng.choice([1.0, -0.5])),
+                                          bias=rng.normal(size=1))
+    x = _random_flat_data(rng, model, cat_values, docs)
+    o = OracleModel(model)
+    g = cb.ModelCalcer()
+    g.load_from_dict(model)
+    g.enable_gpu_evaluation(0)
+    kernels = g.evaluator().describe_kernels(cb.LAYOUT_FLAT_ROWS, docs)
+    assert kernels["evaluate"] == "EvalObliviousDeepTileKernel", kernels
+    np.testing.assert_array_equal(g.calc_leaf_indexes_flat(x), o.leaf_indexes(x))
+    np.testing.assert_allclose(g.calc_flat(x), o.calc(x), rtol=RTOL, atol=ATOL)
+    for begin, end in ((0, 1), (1, 2), (0, 17), (0, trees - 1), (1, trees), (3, 3), (trees // 2, trees)):
+        np.testing.assert_allclose(g.calc_flat(x, tree_start=begin, tree_end=end),
+                                   o.calc(x, tree_start=begin, tree_end=end), rtol=RTOL, atol=ATOL,
+                                   err_msg="trees %d..%d" % (begin, end))
