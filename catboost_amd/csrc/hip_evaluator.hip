@@ -1569,7 +1569,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
                                 fixed.begin() + t * pitch);
                 }
                 m.HalfTileLeaves.Upload(fixed);
-                // two trees per wave: every bin of the model below 128 (the one-hot test then fits 7 bits too)
+                // two trees per wave: every bin of the tile's rows below 128 (the one-hot test then fits 7 bits too)
                 if (switches.PairTile && tileRowsUsable && PairTileLdsBytes(tileRowCount, 8) <= kMaxTileLdsBytes) {
                     m.PairRows.Upload(rowsInRegisters(128));
                     m.TileRowCount = tileRowsSplit ? tileRowCount : m.LayoutBuckets;  // (a model without splits: its one zero bucket)
@@ -2023,7 +2023,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         }
     }
 
-    // Models that the register kernels do not take, every bin below 128, the 256-document tile and the leaf
+    // Models that the register kernels do not take, every bin of the tile's rows below 128, the 256-document tile and the leaf
     // regions of eight waves in LDS: a tree's row in registers (EvalObliviousRowTileKernel).
     if (!m.RegKernelUsable && m.Oblivious && m.MaxDepth <= 8 && TreeCount > 0 && switches.RowTile && tileRowsUsable &&
         RowTileWaves(tileRowCount, m.MaxDepth, m.Dim) != 0) {

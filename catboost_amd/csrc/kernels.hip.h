@@ -1201,7 +1201,7 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousHalfTileKernel(
 // next one, each lane for four documents of the tile (one LDS dword: the bins of documents
 // (2 * half + j) * 64 + 2 * m + i, byte 2 * i + j, for lane m of either group), so a level costs one LDS read
 // and one byte-parallel compare for 2 x 128 (tree, document) pairs instead of 128. Needs every bin of the
-// model below 128 (the 7-bit compare; a one-hot level xors first: (bin ^ (~value & 0x7f)) + 1 carries into
+// tile below 128 (the 7-bit compare; a one-hot level xors first: (bin ^ (~value & 0x7f)) + 1 carries into
 // bit 7 exactly when bin == value).
 // `pairRows` holds 16 dwords per tree: slot d = byte offset of level d's bucket in the tile (bucket * 128)
 // | xor byte << 24, slot 0 also bit 23 when some level of the tree xors; slot 8 + d = the value added to all
