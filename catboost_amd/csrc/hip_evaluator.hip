@@ -487,10 +487,12 @@ bool PackNsUnits(const std::vector<uint32_t>& rows, size_t treeCount, uint32_t l
     return true;
 }
 
-// Dimensions that a workgroup of the row-tile kernel sums at a time: two keep the sums, the values in flight and
-// the three trees' worth of values fetched ahead within a wave's registers at sixteen waves (four spill)
-uint32_t RowTileDims(uint32_t /*maxDepth*/, int dim) {
-    return dim == 1 ? 1 : 2;
+// Dimensions that a workgroup of the row-tile kernel sums at a time. Two: the sums, the values in flight and three
+// trees' worth of values fetched ahead then fit a wave's registers at sixteen waves. A walk for four dimensions takes
+// 1.8 times as long (C3's trees over 300 features: 3.6 against 2.06 ms), so only models of three or four dimensions
+// with 64 leaves per tree take it, for one walk instead of two.
+uint32_t RowTileDims(uint32_t maxDepth, int dim) {
+    return dim == 1 ? 1 : maxDepth <= 6 && (dim == 3 || dim == 4) ? 4 : 2;
 }
 
 // LDS of the row-tile kernel: 256 documents' bins, the accumulator, a tree's leaf values per wave
@@ -2530,9 +2532,12 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
             if (dims == 1) {
                 wide ? launch(dev::EvalObliviousRowTileKernel<6, dev::kWideTileWaves, 1>)
                      : launch(dev::EvalObliviousRowTileKernel<6, dev::kTileWaves, 1>);
-            } else {
+            } else if (dims == 2) {
                 wide ? launch(dev::EvalObliviousRowTileKernel<6, dev::kWideTileWaves, 2>)
                      : launch(dev::EvalObliviousRowTileKernel<6, dev::kTileWaves, 2>);
+            } else {
+                wide ? launch(dev::EvalObliviousRowTileKernel<6, dev::kWideTileWaves, 4>)
+                     : launch(dev::EvalObliviousRowTileKernel<6, dev::kTileWaves, 4>);
             }
         } else if (dims == 1) {
             wide ? launch(dev::EvalObliviousRowTileKernel<8, dev::kWideTileWaves, 1>)

@@ -1446,8 +1446,8 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousPairTileKernel(
 // leaf values go through the wave's LDS region; rows and values are fetched kPairAhead rounds ahead without
 // looking at the tree range (both tables end with kRowTilePadding trees' worth of zeros). Waves take the trees
 // round robin; their partial sums are added in wave order through an accumulator in LDS at the end.
-// Leaf values: one dimension: (1 << MAXD) values per tree. Several dimensions: a workgroup sums DIMS (2; 4 is
-// written out but spills at sixteen waves) of them at a time, slice after slice of the model's dimensions over the same tile, every slice with another
+// Leaf values: one dimension: (1 << MAXD) values per tree. Several dimensions: a workgroup sums DIMS (2 or 4)
+// of them at a time, slice after slice of the model's dimensions over the same tile, every slice with another
 // walk of the trees; `leaves2` is [slice][tree][piece][leaf] pairs of values (16 bytes: dimensions 2 * piece and
 // 2 * piece + 1 of the slice, zeros past the model's last dimension), sliceStride pairs per slice. A wave's
 // 16-byte gathers of one piece then spread over all groups of four LDS banks, which leaf rows of 32 bytes would
@@ -1469,6 +1469,7 @@ __global__ __launch_bounds__(64 * WAVES) void EvalObliviousRowTileKernel(
     constexpr int kLeafRegs = kTreePieces > kWave ? static_cast<int>(kTreePieces / kWave) : 1;
     constexpr uint32_t kPieceMask = kTreePieces - 1;         // 32 pieces: the upper lanes repeat the lower lanes' pieces
     constexpr int kPairsPerLeaf = DIMS > 1 ? DIMS / 2 : 1;
+    constexpr bool kPipelined = DIMS <= 2;  // the values gathered in a round are added during the next one
     static_assert(MAXD == 8 || MAXD == 6, "64 or 256 leaves per tree");
     static_assert(DIMS == 1 || DIMS == 2 || DIMS == 4, "one value or whole pairs per leaf");
     static_assert(WAVES <= kWideTileWaves, "the tables are padded for that many waves");
@@ -1536,9 +1537,11 @@ __global__ __launch_bounds__(64 * WAVES) void EvalObliviousRowTileKernel(
         __builtin_amdgcn_s_waitcnt(kWaitLoads);                                                    \
         __builtin_amdgcn_sched_barrier(0);                                                         \
         CBAMD_PUBLISH_AND_WALK(k, idx4);                                                           \
-        _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                            \
-            _Pragma("unroll") for (int c = 0; c < DIMS; ++c) {                                     \
-                acc[q][c] = __dadd_rn(acc[q][c], gathered[q][c]);                                  \
+        if constexpr (kPipelined) {                                                                \
+            _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                        \
+                _Pragma("unroll") for (int c = 0; c < DIMS; ++c) {                                 \
+                    acc[q][c] = __dadd_rn(acc[q][c], gathered[q][c]);                              \
+                }                                                                                  \
             }                                                                                      \
         }                                                                                          \
         __builtin_amdgcn_sched_barrier(0);                                                         \
@@ -1553,6 +1556,15 @@ __global__ __launch_bounds__(64 * WAVES) void EvalObliviousRowTileKernel(
                     const double2 pair = reinterpret_cast<const double2*>(sLeafMine)[piece * kLeaves + leaf]; \
                     gathered[q][2 * piece] = pair.x;                                               \
                     gathered[q][2 * piece + 1] = pair.y;                                           \
+                }                                                                                  \
+            }                                                                                      \
+        }                                                                                          \
+        if constexpr (!kPipelined) {                                                               \
+            /* four dimensions: no registers for values in flight across a round */               \
+            _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                        \
+                _Pragma("unroll") for (int c = 0; c < DIMS; ++c) {                                 \
+                    acc[q][c] = __dadd_rn(acc[q][c], gathered[q][c]);                              \
+                    gathered[q][c] = 0.0;                                                          \
                 }                                                                                  \
             }                                                                                      \
         }                                                                                          \

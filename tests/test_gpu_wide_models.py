@@ -122,7 +122,7 @@ def test_tile_models_against_the_oracle(monkeypatch, rows_in_registers, seed, n_
 
 @pytest.mark.parametrize("seed,dim,n_float,n_cat,trees,max_depth,docs,registers", [
     (31, 2, 300, 0, 300, 8, 1000, "1"),   # two dimensions: one slice
-    (32, 3, 280, 6, 300, 6, 513, "1"),    # 64 leaves; two slices, the second with a dimension to spare; one-hot levels
+    (32, 3, 280, 6, 300, 6, 513, "1"),    # 64 leaves and three dimensions: one slice of four; one-hot levels
     (33, 10, 420, 0, 400, 6, 255, "1"),   # five slices
     (34, 5, 300, 2, 200, 8, 4097, "1"),   # 256 leaves, three slices
     (35, 3, 30, 2, 50, 8, 700, "0"),      # a small tile: two workgroups of eight waves per CU
@@ -131,7 +131,7 @@ def test_tile_models_against_the_oracle(monkeypatch, rows_in_registers, seed, n_
 ])
 def test_tile_models_of_several_dimensions(monkeypatch, seed, dim, n_float, n_cat, trees, max_depth, docs, registers):
     """Models of several dimensions on the tile kernel with a tree's row in registers: a workgroup sums two
-    dimensions at a time over the same tile, slice after slice."""
+    dimensions at a time over the same tile, slice after slice (four when that is the whole model)."""
     rng = np.random.default_rng(seed)
     model, cat_values = _random_oblivious(rng, n_float=n_float, n_cat=n_cat, trees=trees, max_depth=max_depth, dim=dim,
                                           many_borders=seed >= 41, scale=float(rng.choice([1.0, -0.5])),
