@@ -2837,7 +2837,7 @@ std::string THipEvaluator::DescribeKernels(int layout, size_t docCount) const {
     } else if (m.Oblivious && m.MaxDepth <= 8 && TileLdsBytes(m.LayoutBuckets, dchunk) <= kMaxTileLdsBytes) {
         evaluate = "EvalObliviousTileKernel";
     } else if (m.Oblivious && m.MaxDepth <= 8 && m.Dim == 1 && m.HalfTileLeaves.Get() != nullptr &&
-               TileLdsBytes(m.LayoutBuckets, 1) > kMaxTileLdsBytes) {
+               TileLdsBytes(m.LayoutBuckets, 1) > kMaxTileLdsBytes && HalfTileLdsBytes(m.LayoutBuckets, 8) <= kMaxTileLdsBytes) {
         evaluate = m.PairRows.Get() != nullptr ? "EvalObliviousPairTileKernel" : "EvalObliviousHalfTileKernel";
     } else if (m.DeepRows.Get() != nullptr) {
         evaluate = "EvalObliviousDeepTileKernel";
