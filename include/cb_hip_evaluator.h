@@ -92,9 +92,9 @@ typedef struct CbHipFeatures {
  *   CATBOOST_AMD_FUSED=0             binarize and evaluate always as two launches (no fused kernels)
  *   CATBOOST_AMD_PAIR_TILE=0         wide one-dimensional models (more buckets than an LDS tile of 256 documents
  *                                    holds): one tree per wave instead of two
- *   CATBOOST_AMD_ROW_TILE=0          one-dimensional models of 7-bit bins whose 256-document tile fits LDS: the tile
+ *   CATBOOST_AMD_ROW_TILE=0          models outside the register kernels whose 256-document tile fits LDS: the tile
  *                                    kernel that broadcasts a tree's levels from a lane instead of the one that
- *                                    keeps a tree's row in every lane's registers
+ *                                    keeps a tree's row in registers (depth 9 to 16: the plain kernel)
  *   CATBOOST_AMD_NS_WAVES=4|6|8|12|16 non-symmetric models walked out of LDS: only that many waves per workgroup
  *                                    (regions of 2048, 1536 or 1024 tree entries) instead of the most that hold
  *                                    the model's largest tree
