@@ -520,6 +520,12 @@ size_t DeepTileLdsBytes(uint32_t rows) {
     return ((static_cast<size_t>(rows) * 256 + 15) & ~size_t(15)) + dev::kDocsPerBlock * sizeof(double);
 }
 
+// LDS of the quad-tile kernel: 64 documents' bins, then per wave the leaf values of four trees (later the partial sums)
+size_t QuadTileLdsBytes(uint32_t rows, int maxd) {
+    return ((static_cast<size_t>(rows) * 64 + 15) & ~size_t(15)) +
+           static_cast<size_t>(dev::kTileWaves) * 4 * (size_t(1) << maxd) * sizeof(double);
+}
+
 // LDS of the pair-tile kernel: 128 documents' bins, then per wave the leaf values of two trees; the same area
 // takes one partial sum per wave, lane group and document at the end
 size_t PairTileLdsBytes(uint32_t buckets, int maxd) {
@@ -1019,6 +1025,7 @@ struct THipEvaluator::TImpl {
     TDeviceVec<uint32_t> PackedMixed;  // half-tile kernel: packed rows in the form chosen per tree
     TDeviceVec<double> HalfTileLeaves; // half-tile kernel: 64 or 256 leaf values per tree at a fixed pitch
     TDeviceVec<uint32_t> PairRows;     // pair-tile kernel: 16 dwords per tree, empty when the model does not qualify
+    TDeviceVec<uint32_t> QuadRows;     // quad-tile kernel: the same with 64 bytes per row of the tile
     TDeviceVec<uint32_t> TileRows;     // row-tile kernel (whole tile, one tree per wave): the same with 256 bytes per bucket
     TDeviceVec<double> TileLeaves;     // its leaf values: [slice of the dimensions][tree][pair of dimensions][leaf][2]
     size_t TileSliceStride = 0;        // 16-byte pairs of TileLeaves per slice
@@ -1459,7 +1466,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
     // Their rows: 16 dwords per tree, slot d the byte offset of level d's row in the tile | xor byte << 24, slot
     // 8 + d the value added to the four bins of a dword.
     const auto rowsInRegisters = [&](uint32_t bucketBytes) {
-        std::vector<uint32_t> rows((trees.GetTreeCount() + dev::kPairTreePadding) * dev::kPackedTreeDwords, 0);
+        std::vector<uint32_t> rows((trees.GetTreeCount() + dev::kQuadTreePadding) * dev::kPackedTreeDwords, 0);
         for (size_t t = 0; t < trees.GetTreeCount(); ++t) {
             uint32_t* row = rows.data() + t * dev::kPackedTreeDwords;
             bool anyXor = false;
@@ -1564,16 +1571,20 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
             m.PackedMixed.Upload(mixed);
             if (TileLdsBytes(m.LayoutBuckets, 1) > kMaxTileLdsBytes) {
                 const size_t pitch = m.MaxDepth <= 6 ? 64 : 256;
-                // zeros at the end: the pair-tile kernel fetches ahead of its trees without a bound
-                std::vector<double> fixed((trees.GetTreeCount() + dev::kPairTreePadding) * pitch, 0.0);
+                // zeros at the end: the pair-tile and quad-tile kernels fetch ahead of their trees without a bound
+                std::vector<double> fixed((trees.GetTreeCount() + dev::kQuadTreePadding) * pitch, 0.0);
                 for (size_t t = 0; t < trees.GetTreeCount(); ++t) {
                     std::copy_n(trees.LeafValues.begin() + trees.TreeFirstLeafOffsets[t], size_t(1) << trees.TreeSizes[t],
                                 fixed.begin() + t * pitch);
                 }
                 m.HalfTileLeaves.Upload(fixed);
                 // two trees per wave: every bin of the tile's rows below 128 (the one-hot test then fits 7 bits too)
-                if (switches.PairTile && tileRowsUsable && PairTileLdsBytes(tileRowCount, 8) <= kMaxTileLdsBytes) {
-                    m.PairRows.Upload(rowsInRegisters(128));
+                const int maxd = m.MaxDepth <= 6 ? 6 : 8;
+                const bool pairFits = PairTileLdsBytes(tileRowCount, 8) <= kMaxTileLdsBytes;
+                // four trees per wave on a quarter of a block when the rows do not fit the half tile
+                const bool quadFits = !pairFits && QuadTileLdsBytes(tileRowCount, maxd) <= kMaxTileLdsBytes;
+                if (switches.PairTile && tileRowsUsable && (pairFits || quadFits)) {
+                    (pairFits ? m.PairRows : m.QuadRows).Upload(rowsInRegisters(pairFits ? 128 : 64));
                     m.TileRowCount = tileRowsSplit ? tileRowCount : m.LayoutBuckets;  // (a model without splits: its one zero bucket)
                     if (tileRowsSplit) {
                         m.TileMap.Upload(tileMap);
@@ -2562,6 +2573,28 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
         HIP_CHECK(hipGetLastError());
         return;
     }
+    if (m.QuadRows.Get() != nullptr) {
+        // the rows do not fit the half tile: quarter blocks, four trees per wave
+        const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
+        const int maxd = m.MaxDepth <= 6 ? 6 : 8;
+        const size_t lds = QuadTileLdsBytes(m.TileRowCount, maxd);
+        CBAMD_ENSURE(4 * blocks < (size_t(1) << 31), "batch is too large for one evaluate launch");
+        const auto launch = [&](auto kernel) {
+            EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds);
+            hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(4 * blocks)), dim3(64 * dev::kTileWaves), lds, s, bins,
+                               docCount, m.LayoutBuckets, m.TileMap.Get(), m.TileRowCount,
+                               reinterpret_cast<const uint4*>(m.QuadRows.Get()),
+                               reinterpret_cast<const double2*>(m.HalfTileLeaves.Get()), m.Bias.Get(), m.Scale, tb, te,
+                               results);
+        };
+        if (maxd == 6) {
+            launch(dev::EvalObliviousQuadTileKernel<6>);
+        } else {
+            launch(dev::EvalObliviousQuadTileKernel<8>);
+        }
+        HIP_CHECK(hipGetLastError());
+        return;
+    }
     if (m.Oblivious && m.MaxDepth <= 8 && m.Dim == 1 && m.HalfTileLeaves.Get() != nullptr &&
         HalfTileLdsBytes(m.LayoutBuckets, 8) <= kMaxTileLdsBytes) {
         // the bins of a block exceed the 256-document tile: half blocks
@@ -2836,6 +2869,8 @@ std::string THipEvaluator::DescribeKernels(int layout, size_t docCount) const {
         evaluate = "EvalObliviousRowTileKernel";
     } else if (m.Oblivious && m.MaxDepth <= 8 && TileLdsBytes(m.LayoutBuckets, dchunk) <= kMaxTileLdsBytes) {
         evaluate = "EvalObliviousTileKernel";
+    } else if (m.QuadRows.Get() != nullptr) {
+        evaluate = "EvalObliviousQuadTileKernel";
     } else if (m.Oblivious && m.MaxDepth <= 8 && m.Dim == 1 && m.HalfTileLeaves.Get() != nullptr &&
                TileLdsBytes(m.LayoutBuckets, 1) > kMaxTileLdsBytes && HalfTileLdsBytes(m.LayoutBuckets, 8) <= kMaxTileLdsBytes) {
         evaluate = m.PairRows.Get() != nullptr ? "EvalObliviousPairTileKernel" : "EvalObliviousHalfTileKernel";

@@ -1439,6 +1439,194 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousPairTileKernel(
     }
 }
 
+// The same with four trees per wave on a quarter of a block, for models whose rows do not fit the half tile: the
+// tile holds the bins of 64 documents (documents quarter * 64 + l of the block in byte l of a row), lanes 16 g ..
+// 16 g + 15 walk tree g of a quad of trees, each lane for the four documents of one dword. The rows are pairRows
+// with 64 bytes per row of the tile; rows and leaf values are fetched three rounds ahead, so both tables end with
+// kQuadTreePadding null trees.
+// grid = 4 * doc blocks, block = 64 * kTileWaves threads, dynamic LDS = rows * 64 (rounded up to 16) +
+// kTileWaves * 4 * (1 << MAXD) * 8 bytes (the leaf regions, later the partial sums).
+constexpr int kQuadTreePadding = 4 * kTileWaves * kPairAhead;
+
+template <int MAXD>
+__global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousQuadTileKernel(
+    const uint8_t* __restrict__ bins, size_t docCount, uint32_t bucketCount, const uint32_t* __restrict__ tileMap,
+    uint32_t rowCount, const uint4* __restrict__ pairRows, const double2* __restrict__ leaves2,
+    const double* __restrict__ bias, double scale, uint32_t treeBegin, uint32_t treeEnd, double* __restrict__ out) {
+    constexpr uint32_t kLeaves = 1u << MAXD;
+    constexpr int kLeafRegs = MAXD == 8 ? 8 : 2;  // 16-byte pieces of a quad's 4 * kLeaves leaf values per lane
+    static_assert(MAXD == 8 || MAXD == 6, "64 or 256 leaves per tree");
+    extern __shared__ uint32_t sTile[];
+    uint8_t* sTile8 = reinterpret_cast<uint8_t*>(sTile);
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const size_t block = blockIdx.x >> 2;
+    const uint32_t quarter = blockIdx.x & 3;
+    const uint32_t tileBytesUsed = rowCount * kWave;  // rowCount = bucketCount without a map
+    const uint8_t* src = bins + block * (bucketCount * kWave) * 4 + quarter;
+    if (tileMap == nullptr) {
+        for (uint32_t i = tid; i < tileBytesUsed; i += 64 * kTileWaves) {
+            sTile8[i] = src[4 * i];
+        }
+    } else {
+        for (uint32_t row = wave; row < rowCount; row += kTileWaves) {
+            const uint32_t entry = tileMap[row];
+            const uint32_t bin = src[4 * ((entry & 0xffffu) * kWave + lane)];
+            sTile8[row * kWave + lane] = static_cast<uint8_t>(MapTileBins(bin, entry >> 16));
+        }
+    }
+    const uint32_t group = lane >> 4;
+    const uint32_t tileBytes = (tileBytesUsed + 15) & ~15u;
+    double* leafArea = reinterpret_cast<double*>(reinterpret_cast<uint8_t*>(sTile) + tileBytes);
+    double2* sLeafWave2 = reinterpret_cast<double2*>(leafArea + wave * 4 * kLeaves);
+    const double* sLeafMine = leafArea + wave * 4 * kLeaves + group * kLeaves;
+    const uint8_t* laneTile = reinterpret_cast<const uint8_t*>(sTile) + (lane & 15) * 4;
+    __syncthreads();  // tile is loaded
+
+    const uint32_t treeCount = treeEnd - treeBegin;
+    const uint32_t pairCount = treeCount / 4;  // whole quads of trees
+    double acc[4] = {0.0, 0.0, 0.0, 0.0};
+    constexpr int kAhead = kPairAhead;
+    uint4 rows[kAhead][4];
+    double2 pref[kAhead][kLeafRegs];
+    // what a lane fetches of the quad that starts at tree `first`: its group's row and its pieces of the
+    // four trees' leaf values
+    const uint4* myRows = pairRows + group * 4;
+    const double2* myLeaves = leaves2 + lane;
+#define CBAMD_FETCH_PAIR(k, first)                                                                 \
+    do {                                                                                           \
+        const uint4* row = myRows + static_cast<size_t>(first) * 4;                                \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                            \
+            rows[k][i] = row[i];                                                                   \
+        }                                                                                          \
+        const double2* values = myLeaves + static_cast<size_t>(first) * (kLeaves / 2);             \
+        _Pragma("unroll") for (int i = 0; i < kLeafRegs; ++i) {                                    \
+            pref[k][i] = values[i * kWave];                                                        \
+        }                                                                                          \
+    } while (0)
+    // the quad's leaf values into the wave's LDS region (the previous quad's gathers were issued before these
+    // stores and LDS serves one wave's requests in order), then the levels: four leaf indexes per lane
+#define CBAMD_PUBLISH_AND_WALK(k, idx4)                                                            \
+    do {                                                                                           \
+        _Pragma("unroll") for (int i = 0; i < kLeafRegs; ++i) {                                    \
+            sLeafWave2[i * kWave + lane] = pref[k][i];                                             \
+        }                                                                                          \
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                                     \
+        __builtin_amdgcn_wave_barrier();                                                           \
+        const uint32_t flags =                                                                     \
+            __builtin_amdgcn_readlane(rows[k][0].x, 0) | __builtin_amdgcn_readlane(rows[k][0].x, 16) | \
+            __builtin_amdgcn_readlane(rows[k][0].x, 32) | __builtin_amdgcn_readlane(rows[k][0].x, 48); \
+        if (flags & kPairRowXorFlag) {                                                             \
+            idx4 = PairTreeIndexes<true, MAXD>(laneTile, rows[k]);                                 \
+        } else {                                                                                   \
+            idx4 = PairTreeIndexes<false, MAXD>(laneTile, rows[k]);                                \
+        }                                                                                          \
+    } while (0)
+
+    // One round of a wave: the leaf values that the previous round gathered are added while this round's LDS
+    // reads are under way; the registers of this quad take the quad kAhead rounds ahead as soon as every level
+    // has read them (the loads then land in those registers), and the gathers go out last.
+    constexpr int kLoadsBehind = 2 * (4 + kLeafRegs);
+    constexpr int kWaitLoads = 0x0f70 | (kLoadsBehind & 15) | ((kLoadsBehind >> 4) << 14);  // vmcnt(kLoadsBehind)
+    double gathered[4] = {0.0, 0.0, 0.0, 0.0};
+#define CBAMD_PAIR_ROUND(k)                                                                        \
+    do {                                                                                           \
+        uint32_t idx4;                                                                             \
+        /* one wait for this quad's loads: those of the two quads behind it stay in flight */       \
+        __builtin_amdgcn_s_waitcnt(kWaitLoads);                                                    \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+        CBAMD_PUBLISH_AND_WALK(k, idx4);                                                           \
+        _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                            \
+            acc[q] = __dadd_rn(acc[q], gathered[q]);                                               \
+        }                                                                                          \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+        CBAMD_FETCH_PAIR(k, treeBegin + 4 * (p + kAhead * kTileWaves));                            \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+        _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                            \
+            gathered[q] = sLeafMine[(idx4 >> (8 * q + 8 - MAXD)) & (kLeaves - 1)];                 \
+        }                                                                                          \
+        __builtin_amdgcn_wave_barrier();                                                           \
+        p += kTileWaves;                                                                           \
+    } while (0)
+
+    uint32_t p = wave;
+#pragma unroll
+    for (int k = 0; k < kAhead; ++k) {
+        // (written before the loads so that the arrays stay in registers)
+#pragma unroll
+        for (int i = 0; i < kLeafRegs; ++i) {
+            pref[k][i] = {0.0, 0.0};
+        }
+        CBAMD_FETCH_PAIR(k, treeBegin + 4 * (p + k * kTileWaves));
+    }
+    static_assert(kAhead == 3, "the rounds below are written out for three register sets");
+    // whole turns of the three register sets without a branch between the rounds, so that the waits for
+    // the loads count only the loads that are older than the one needed
+    while (p + 2 * kTileWaves < pairCount) {
+        CBAMD_PAIR_ROUND(0);
+        CBAMD_PAIR_ROUND(1);
+        CBAMD_PAIR_ROUND(2);
+    }
+    if (p < pairCount) {
+        CBAMD_PAIR_ROUND(0);
+        if (p < pairCount) {
+            CBAMD_PAIR_ROUND(1);
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        acc[q] = __dadd_rn(acc[q], gathered[q]);
+    }
+    const uint32_t rest = treeCount & 3;
+    if (rest && wave == 0) {
+        // the last one to three trees: a group without a tree of its own walks the last one and adds nothing
+        const uint32_t base = treeEnd - rest;
+        const uint4* row = pairRows + static_cast<size_t>(base + min(group, rest - 1)) * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            rows[0][i] = row[i];
+        }
+#pragma unroll
+        for (int i = 0; i < kLeafRegs; ++i) {
+            const uint32_t piece = i * kWave + lane;  // of the four trees' regions, kLeaves / 2 pieces each
+            const uint32_t tree = base + min(piece / (kLeaves / 2), rest - 1);
+            pref[0][i] = leaves2[static_cast<size_t>(tree) * (kLeaves / 2) + piece % (kLeaves / 2)];
+        }
+        uint32_t idx4;
+        CBAMD_PUBLISH_AND_WALK(0, idx4);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const double v = sLeafMine[(idx4 >> (8 * q + 8 - MAXD)) & (kLeaves - 1)];
+            acc[q] = __dadd_rn(acc[q], group < rest ? v : 0.0);
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+#undef CBAMD_PAIR_ROUND
+#undef CBAMD_FETCH_PAIR
+#undef CBAMD_PUBLISH_AND_WALK
+    __syncthreads();  // every wave is through with its leaf region: the area now takes the partial sums
+    // partial sums as [wave][group][document of the tile], then one thread per document adds the thirty-two
+    double* sRed = leafArea;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        // byte q of a lane's dword: document 4 * (lane & 15) + q of the tile
+        sRed[(wave * 4 + group) * kWave + 4 * (lane & 15) + q] = acc[q];
+    }
+    __syncthreads();
+    if (tid < kWave) {
+        double sum = sRed[tid];
+#pragma unroll
+        for (int part = 1; part < 4 * kTileWaves; ++part) {
+            sum = __dadd_rn(sum, sRed[part * kWave + tid]);
+        }
+        const size_t doc = block * kDocsPerBlock + quarter * kWave + tid;
+        if (doc < docCount) {
+            out[doc] = Finish(sum, scale, bias[0], treeBegin == 0);
+        }
+    }
+}
+
 // Models of 7-bit bins whose 256-document tile fits LDS, one tree per wave: the walk of
 // EvalObliviousPairTileKernel on the whole tile. A tree's row is `tileRows` (the format of pairRows with
 // bucket * 256 as the byte offset); its address is the same in every lane, so it comes through scalar loads

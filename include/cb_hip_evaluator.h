@@ -91,7 +91,7 @@ typedef struct CbHipFeatures {
  *   CATBOOST_AMD_LEVEL_ORDER=0       register-resident kernels keep the model's order of a tree's levels
  *   CATBOOST_AMD_FUSED=0             binarize and evaluate always as two launches (no fused kernels)
  *   CATBOOST_AMD_PAIR_TILE=0         wide one-dimensional models (more buckets than an LDS tile of 256 documents
- *                                    holds): one tree per wave instead of two
+ *                                    holds): one tree per wave instead of two or four
  *   CATBOOST_AMD_ROW_TILE=0          models outside the register kernels whose 256-document tile fits LDS: the tile
  *                                    kernel that broadcasts a tree's levels from a lane instead of the one that
  *                                    keeps a tree's row in registers (depth 9 to 16: the plain kernel)

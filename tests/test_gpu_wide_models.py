@@ -56,12 +56,11 @@ def test_wide_models_against_the_oracle(monkeypatch, pair, seed, n_float, n_cat,
 
 @pytest.mark.parametrize("n_float,trees,docs,kernel", [
     (800, 500, 700, "EvalObliviousPairTileKernel"),    # 717 rows of 128 bytes and the leaf regions fit LDS
-    (1100, 900, 300, "EvalObliviousHalfTileKernel"),   # 1045 rows do not: one tree per wave, 8-bit compares
+    (1100, 900, 300, "EvalObliviousQuadTileKernel"),   # 1045 rows do not: rows of 64 bytes, four trees per wave
 ])
 def test_wide_models_with_bins_above_127(monkeypatch, n_float, trees, docs, kernel):
     """A feature with 300 borders: its bucket of more than 127 values takes two rows of the tile, min(bin, 127)
-    and max(bin - 127, 0), and the two-tree kernel compares 7 bits as before; when the rows no longer fit LDS
-    the model stays with the kernel that compares 8 bits in the trees that need it."""
+    and max(bin - 127, 0), and the kernels with two or four trees per wave compare 7 bits as before."""
     rng = np.random.default_rng(11)
     model, cat_values = _random_oblivious(rng, n_float=n_float, n_cat=4, trees=trees, max_depth=8, many_borders=True)
     assert max(len(f["borders"]) for f in model["float_features"]) > 127
@@ -197,6 +196,37 @@ def test_deep_trees_on_the_tile_kernel(seed, n_float, n_cat, trees, max_depth, m
     np.testing.assert_array_equal(g.calc_leaf_indexes_flat(x), o.leaf_indexes(x))
     np.testing.assert_allclose(g.calc_flat(x), o.calc(x), rtol=RTOL, atol=ATOL)
     for begin, end in ((0, 1), (1, 2), (0, 17), (0, trees - 1), (1, trees), (3, 3), (trees // 2, trees)):
+        np.testing.assert_allclose(g.calc_flat(x, tree_start=begin, tree_end=end),
+                                   o.calc(x, tree_start=begin, tree_end=end), rtol=RTOL, atol=ATOL,
+                                   err_msg="trees %d..%d" % (begin, end))
+
+
+@pytest.mark.parametrize("quad", ["1", "0"])
+@pytest.mark.parametrize("seed,n_float,n_cat,trees,max_depth,many,docs", [
+    (61, 1300, 0, 901, 8, False, 700),    # 1241 buckets; a last tree without partners
+    (62, 1500, 6, 602, 8, False, 129),    # one-hot levels; two trees left over
+    (63, 1700, 10, 1503, 6, False, 65),   # 64 leaves per tree, 1541 buckets; three trees left over
+    (64, 1250, 3, 700, 8, True, 1),       # a feature of 300 borders: two rows for its large bucket; a single document
+])
+def test_very_wide_models_against_the_oracle(monkeypatch, quad, seed, n_float, n_cat, trees, max_depth, many, docs):
+    """More rows than the half tile holds: a tile of 64 documents with four trees per wave, or (switched off) the
+    half-tile kernel with one tree per wave while its tile fits, else the plain kernel."""
+    rng = np.random.default_rng(seed)
+    model, cat_values = _random_oblivious(rng, n_float=n_float, n_cat=n_cat, trees=trees, max_depth=max_depth,
+                                          many_borders=many, scale=float(rng.choice([1.0, -0.5])),
+                                          bias=rng.normal(size=1))
+    x = _random_flat_data(rng, model, cat_values, docs)
+    o = OracleModel(model)
+    g = _evaluator(model, monkeypatch, quad)
+    kernels = g.evaluator().describe_kernels(cb.LAYOUT_FLAT_ROWS, docs)
+    if quad == "1":
+        assert kernels["evaluate"] == "EvalObliviousQuadTileKernel", kernels
+    else:
+        assert kernels["evaluate"] in ("EvalObliviousHalfTileKernel", "EvalObliviousKernel"), kernels
+    np.testing.assert_array_equal(g.quantize_flat(x), o.binarize(x))
+    np.testing.assert_allclose(g.calc_flat(x), o.calc(x), rtol=RTOL, atol=ATOL)
+    for begin, end in ((0, 1), (1, 2), (0, 3), (2, 9), (0, trees - 1), (1, trees), (3, 3), (trees // 2, trees),
+                       (5, 8), (trees - 3, trees)):
         np.testing.assert_allclose(g.calc_flat(x, tree_start=begin, tree_end=end),
                                    o.calc(x, tree_start=begin, tree_end=end), rtol=RTOL, atol=ATOL,
                                    err_msg="trees %d..%d" % (begin, end))
