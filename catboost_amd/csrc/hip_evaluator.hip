@@ -521,9 +521,14 @@ size_t DeepTileLdsBytes(uint32_t rows) {
 }
 
 // LDS of the quad-tile kernel: 64 documents' bins, then per wave the leaf values of four trees (later the partial sums)
-size_t QuadTileLdsBytes(uint32_t rows, int maxd) {
+size_t QuadTileLdsBytes(uint32_t rows, int maxd, uint32_t waves) {
     return ((static_cast<size_t>(rows) * 64 + 15) & ~size_t(15)) +
-           static_cast<size_t>(dev::kTileWaves) * 4 * (size_t(1) << maxd) * sizeof(double);
+           static_cast<size_t>(waves) * 4 * (size_t(1) << maxd) * sizeof(double);
+}
+
+// Waves per workgroup of the quad-tile kernel: eight, or four when the rows leave room for no more; 0: no room
+uint32_t QuadTileWaves(uint32_t rows, int maxd) {
+    return QuadTileLdsBytes(rows, maxd, 8) <= kMaxTileLdsBytes ? 8u : QuadTileLdsBytes(rows, maxd, 4) <= kMaxTileLdsBytes ? 4u : 0u;
 }
 
 // LDS of the pair-tile kernel: 128 documents' bins, then per wave the leaf values of two trees; the same area
@@ -1582,7 +1587,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
                 const int maxd = m.MaxDepth <= 6 ? 6 : 8;
                 const bool pairFits = PairTileLdsBytes(tileRowCount, 8) <= kMaxTileLdsBytes;
                 // four trees per wave on a quarter of a block when the rows do not fit the half tile
-                const bool quadFits = !pairFits && QuadTileLdsBytes(tileRowCount, maxd) <= kMaxTileLdsBytes;
+                const bool quadFits = !pairFits && QuadTileWaves(tileRowCount, maxd) != 0;
                 if (switches.PairTile && tileRowsUsable && (pairFits || quadFits)) {
                     (pairFits ? m.PairRows : m.QuadRows).Upload(rowsInRegisters(pairFits ? 128 : 64));
                     m.TileRowCount = tileRowsSplit ? tileRowCount : m.LayoutBuckets;  // (a model without splits: its one zero bucket)
@@ -2577,20 +2582,21 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
         // the rows do not fit the half tile: quarter blocks, four trees per wave
         const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
         const int maxd = m.MaxDepth <= 6 ? 6 : 8;
-        const size_t lds = QuadTileLdsBytes(m.TileRowCount, maxd);
+        const uint32_t waves = QuadTileWaves(m.TileRowCount, maxd);
+        const size_t lds = QuadTileLdsBytes(m.TileRowCount, maxd, waves);
         CBAMD_ENSURE(4 * blocks < (size_t(1) << 31), "batch is too large for one evaluate launch");
         const auto launch = [&](auto kernel) {
             EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds);
-            hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(4 * blocks)), dim3(64 * dev::kTileWaves), lds, s, bins,
+            hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(4 * blocks)), dim3(64 * waves), lds, s, bins,
                                docCount, m.LayoutBuckets, m.TileMap.Get(), m.TileRowCount,
                                reinterpret_cast<const uint4*>(m.QuadRows.Get()),
                                reinterpret_cast<const double2*>(m.HalfTileLeaves.Get()), m.Bias.Get(), m.Scale, tb, te,
                                results);
         };
         if (maxd == 6) {
-            launch(dev::EvalObliviousQuadTileKernel<6>);
+            waves == 8 ? launch(dev::EvalObliviousQuadTileKernel<6, 8>) : launch(dev::EvalObliviousQuadTileKernel<6, 4>);
         } else {
-            launch(dev::EvalObliviousQuadTileKernel<8>);
+            waves == 8 ? launch(dev::EvalObliviousQuadTileKernel<8, 8>) : launch(dev::EvalObliviousQuadTileKernel<8, 4>);
         }
         HIP_CHECK(hipGetLastError());
         return;

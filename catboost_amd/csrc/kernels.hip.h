@@ -1444,12 +1444,13 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousPairTileKernel(
 // 16 g + 15 walk tree g of a quad of trees, each lane for the four documents of one dword. The rows are pairRows
 // with 64 bytes per row of the tile; rows and leaf values are fetched three rounds ahead, so both tables end with
 // kQuadTreePadding null trees.
-// grid = 4 * doc blocks, block = 64 * kTileWaves threads, dynamic LDS = rows * 64 (rounded up to 16) +
-// kTileWaves * 4 * (1 << MAXD) * 8 bytes (the leaf regions, later the partial sums).
+// WAVES = 8, or 4 when the rows leave LDS for four waves' regions only.
+// grid = 4 * doc blocks, block = 64 * WAVES threads, dynamic LDS = rows * 64 (rounded up to 16) +
+// WAVES * 4 * (1 << MAXD) * 8 bytes (the leaf regions, later the partial sums).
 constexpr int kQuadTreePadding = 4 * kTileWaves * kPairAhead;
 
-template <int MAXD>
-__global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousQuadTileKernel(
+template <int MAXD, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void EvalObliviousQuadTileKernel(
     const uint8_t* __restrict__ bins, size_t docCount, uint32_t bucketCount, const uint32_t* __restrict__ tileMap,
     uint32_t rowCount, const uint4* __restrict__ pairRows, const double2* __restrict__ leaves2,
     const double* __restrict__ bias, double scale, uint32_t treeBegin, uint32_t treeEnd, double* __restrict__ out) {
@@ -1466,11 +1467,11 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousQuadTileKernel(
     const uint32_t tileBytesUsed = rowCount * kWave;  // rowCount = bucketCount without a map
     const uint8_t* src = bins + block * (bucketCount * kWave) * 4 + quarter;
     if (tileMap == nullptr) {
-        for (uint32_t i = tid; i < tileBytesUsed; i += 64 * kTileWaves) {
+        for (uint32_t i = tid; i < tileBytesUsed; i += 64 * WAVES) {
             sTile8[i] = src[4 * i];
         }
     } else {
-        for (uint32_t row = wave; row < rowCount; row += kTileWaves) {
+        for (uint32_t row = wave; row < rowCount; row += WAVES) {
             const uint32_t entry = tileMap[row];
             const uint32_t bin = src[4 * ((entry & 0xffffu) * kWave + lane)];
             sTile8[row * kWave + lane] = static_cast<uint8_t>(MapTileBins(bin, entry >> 16));
@@ -1541,13 +1542,13 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousQuadTileKernel(
             acc[q] = __dadd_rn(acc[q], gathered[q]);                                               \
         }                                                                                          \
         __builtin_amdgcn_sched_barrier(0);                                                         \
-        CBAMD_FETCH_PAIR(k, treeBegin + 4 * (p + kAhead * kTileWaves));                            \
+        CBAMD_FETCH_PAIR(k, treeBegin + 4 * (p + kAhead * WAVES));                            \
         __builtin_amdgcn_sched_barrier(0);                                                         \
         _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                            \
             gathered[q] = sLeafMine[(idx4 >> (8 * q + 8 - MAXD)) & (kLeaves - 1)];                 \
         }                                                                                          \
         __builtin_amdgcn_wave_barrier();                                                           \
-        p += kTileWaves;                                                                           \
+        p += WAVES;                                                                           \
     } while (0)
 
     uint32_t p = wave;
@@ -1558,12 +1559,12 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousQuadTileKernel(
         for (int i = 0; i < kLeafRegs; ++i) {
             pref[k][i] = {0.0, 0.0};
         }
-        CBAMD_FETCH_PAIR(k, treeBegin + 4 * (p + k * kTileWaves));
+        CBAMD_FETCH_PAIR(k, treeBegin + 4 * (p + k * WAVES));
     }
     static_assert(kAhead == 3, "the rounds below are written out for three register sets");
     // whole turns of the three register sets without a branch between the rounds, so that the waits for
     // the loads count only the loads that are older than the one needed
-    while (p + 2 * kTileWaves < pairCount) {
+    while (p + 2 * WAVES < pairCount) {
         CBAMD_PAIR_ROUND(0);
         CBAMD_PAIR_ROUND(1);
         CBAMD_PAIR_ROUND(2);
@@ -1617,7 +1618,7 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousQuadTileKernel(
     if (tid < kWave) {
         double sum = sRed[tid];
 #pragma unroll
-        for (int part = 1; part < 4 * kTileWaves; ++part) {
+        for (int part = 1; part < 4 * WAVES; ++part) {
             sum = __dadd_rn(sum, sRed[part * kWave + tid]);
         }
         const size_t doc = block * kDocsPerBlock + quarter * kWave + tid;

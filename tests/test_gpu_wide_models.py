@@ -207,6 +207,7 @@ def test_deep_trees_on_the_tile_kernel(seed, n_float, n_cat, trees, max_depth, m
     (62, 1500, 6, 602, 8, False, 129),    # one-hot levels; two trees left over
     (63, 1700, 10, 1503, 6, False, 65),   # 64 leaves per tree, 1541 buckets; three trees left over
     (64, 1250, 3, 700, 8, True, 1),       # a feature of 300 borders: two rows for its large bucket; a single document
+    (65, 1900, 4, 1500, 8, False, 300),   # 1766 buckets: LDS for four waves' leaf regions only
 ])
 def test_very_wide_models_against_the_oracle(monkeypatch, quad, seed, n_float, n_cat, trees, max_depth, many, docs):
     """More rows than the half tile holds: a tile of 64 documents with four trees per wave, or (switched off) the
