@@ -30,7 +30,10 @@ Layout of the work:
     unsigned byte compare (bin ^ xorMask) >= splitIdx is then bit 7 of
     majority(x, (x | 0x80) - (splitIdx & 0x7f), splitIdx < 128) taken per byte, x = bin ^ xorMask;
   * the leaf gathers of a tree (four documents per lane) are issued behind its levels and consumed
-    after the levels of the next tree, so their LDS latency is covered; every sum is accumulated in
+    after the levels of the next tree, so their LDS latency is covered. One-dimensional kernels with
+    eight registers to spare keep two sets of leaf values: a tree's gathers go out in one batch right
+    behind the wait for the previous tree's (which sit in the other set and are added behind the batch),
+    so that a gather has a whole tree's instructions to arrive; every sum is accumulated in
     fp64 in tree order, exactly like the CPU evaluator (cpu/evaluator_impl.cpp:362-460), and
     finished as ApplyScaleAndBias does (scale_and_bias.cpp:4-50).
 
@@ -177,10 +180,19 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
         # two sets of four 16-byte loads (first registers of the quads)
         values = [[16, 20, 24, high], [high + 4, high + 8, high + 12, high + 16]]
         assert b0 == 28
+    # second set of leaf values in flight (one-dimensional kernels that have the registers for it): above the
+    # bins; the fused kernels take eight of the registers that only their binarize phase uses
+    two_sets = pitch == 1 and block % 2 == 0 and (fused or vgprs + 8 <= 256)
+    if two_sets:
+        if fused:
+            lw0 = high + 8
+        else:
+            lw0 = vgprs
+            vgprs += 8
     assert vgprs <= 256
 
-    def lv(j, k):
-        return lv0 + 2 * (j * pitch + k)
+    def lv(j, k, other=False):
+        return (lw0 if other else lv0) + 2 * (j * pitch + k)
 
     def ac(j, k):
         return ac0 + 2 * (j * pitch + k)
@@ -201,12 +213,12 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
         for piece in range(count):
             e("  global_load_lds_dwordx4 v2, s[26:27]%s" % (" offset:%d" % (piece * 1024) if piece else ""))
 
-    def add_leaf_values():
+    def add_leaf_values(other=False):
         # sum + leaf as 1.0 * leaf + sum: the same single rounding, and with a constant in src0 the
         # instruction does not depend on the register index that the levels leave in M0
         for j in range(4):
             for k in range(pitch):
-                e("  v_fma_f64 v[%d:%d], 1.0, v[%d:%d], v[%d:%d]" % (ac(j, k), ac(j, k) + 1, lv(j, k), lv(j, k) + 1,
+                e("  v_fma_f64 v[%d:%d], 1.0, v[%d:%d], v[%d:%d]" % (ac(j, k), ac(j, k) + 1, lv(j, k, other), lv(j, k, other) + 1,
                                                                       ac(j, k), ac(j, k) + 1))
 
     def load_rows(regs, tree):
@@ -656,7 +668,7 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
             e("%s_loaded:" % name)
     load_rows(rows_a, 0)
     load_rows(rows_b, 1)
-    for r in range(lv0, ga0):
+    for r in list(range(lv0, ga0)) + (list(range(lw0, lw0 + 8)) if two_sets else []):
         e("  v_mov_b32_e32 v%d, 0" % r)          # leaf values in flight and the sums
     # a launch that continues the sums of earlier trees takes them from `out`
     e("  s_bitcmp1_b32 s15, 1")
@@ -713,24 +725,42 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
                 levels_seven_bit(rows)
             if deep:
                 levels_high(rows)
-            # previous tree's leaf values have arrived (and so has the next tree's row)
-            e("  s_waitcnt lgkmcnt(0)")
-            add_leaf_values()
-            for j in range(4):
+            tree_offset = buf * buf_bytes + i * tree_bytes
+
+            def gather_address(j):
                 if deep:
                     e("  v_mul_u32_u24_sdwa v%d, s23, v%d dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_%d"
                       % (ga0 + j, wd0 + j // 2, j % 2))
                 else:
                     e("  v_mul_u32_u24_sdwa v%d, s23, v3 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_%d"
                       % (ga0 + j, j))
-                tree_offset = buf * buf_bytes + i * tree_bytes
-                if pitch == 1:
-                    e("  ds_read_b64 v[%d:%d], v%d offset:%d" % (lv(j, 0), lv(j, 0) + 1, ga0 + j, tree_offset))
-                else:
-                    for k in range(0, pitch, 2):
-                        e("  ds_read_b128 v[%d:%d], v%d offset:%d" % (lv(j, k), lv(j, k) + 3, ga0 + j,
-                                                                     tree_offset + (k // 2) * leaves * 16))
-            load_rows(rows, buf * block + i + 2)
+            if two_sets:
+                # The trees of a block alternate between the two sets of leaf values (a block has an even number
+                # of trees, so the first tree of a block finds the last one's values in the second set). The wait
+                # sits right in front of the tree's own gathers: the previous tree's had its levels and addresses to
+                # arrive, and so had the next tree's row. Gathers in one batch, sums behind them: interleaved they
+                # took longer (1.137 against 1.090 ms per 4M documents and 1000 trees).
+                mine = i % 2 == 1
+                for j in range(4):
+                    gather_address(j)
+                e("  s_waitcnt lgkmcnt(0)")
+                for j in range(4):
+                    e("  ds_read_b64 v[%d:%d], v%d offset:%d" % (lv(j, 0, mine), lv(j, 0, mine) + 1, ga0 + j, tree_offset))
+                load_rows(rows, buf * block + i + 2)
+                add_leaf_values(not mine)
+            else:
+                # previous tree's leaf values have arrived (and so has the next tree's row)
+                e("  s_waitcnt lgkmcnt(0)")
+                add_leaf_values()
+                for j in range(4):
+                    gather_address(j)
+                    if pitch == 1:
+                        e("  ds_read_b64 v[%d:%d], v%d offset:%d" % (lv(j, 0), lv(j, 0) + 1, ga0 + j, tree_offset))
+                    else:
+                        for k in range(0, pitch, 2):
+                            e("  ds_read_b128 v[%d:%d], v%d offset:%d" % (lv(j, k), lv(j, k) + 3, ga0 + j,
+                                                                         tree_offset + (k // 2) * leaves * 16))
+                load_rows(rows, buf * block + i + 2)
             # copy of the next tree block into the other buffer, spread over this block's trees
             staged = False
             for g in range(len(groups)):
@@ -759,7 +789,7 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
     e("  s_addc_u32 s31, s31, 0")
     e("  s_branch %s_loop" % name)
     e("%s_done:" % name)
-    add_leaf_values()
+    add_leaf_values(two_sets)                # the last tree of a block: second set
     e("  s_set_gpr_idx_off")
     e("  s_bitcmp1_b32 s15, 2")                  # raw sums for a launch that continues them
     e("  s_cbranch_scc1 %s_store" % name)
