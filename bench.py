@@ -4,7 +4,10 @@
 
 A step is one pass of the two kernels (binarize, evaluate) over one batch of synthetic documents
 that already sits in HBM. The default workload is C2: 1000 oblivious trees of depth 8, 200 fp32
-features with 5 % NaN, 4M documents. Prints one JSON line.
+features with 5 % NaN, 4M documents. Prints one JSON line. The default run (C2, no --docs) then gives the other
+four workloads of the baseline (C1, C3, C4, C5 at their full sizes) five steps each, outside the timed region of the
+C2 figure, and reports them under "other_workloads" (kernel times from HIP events, parity of 2000 sampled
+documents against the oracle).
 """
 import argparse
 import json
@@ -152,6 +155,8 @@ def main():
     ap.add_argument("--docs", type=int, default=0, help="override the document count of the workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-end-to-end", action="store_true", help="skip the CalcModelPredictionFlat figure")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="skip the short runs of C1, C3, C4 and C5 that follow the default C2 run")
     ap.add_argument("--check-docs", type=int, default=20000)
     ap.add_argument("--copy-probe-mib", type=int, default=0,
                     help="also run one device-to-device copy of this many MiB (a kernel of known traffic, used to "
@@ -172,6 +177,51 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
 
+    result, ok, context = measure_workload(args.config, args.docs, args.steps, args.warmup, args.check_docs, args.copy_probe_mib)
+    model, info, docs, model_bytes, sample, got = context
+    if not args.no_other_workloads and args.config == "C2" and not args.docs:
+        # the other four workloads of the baseline, outside the timed region of the headline figure: a few steps
+        # each at their full sizes, the same measurement (HIP events around a step's kernels, a sample of the
+        # output against the oracle)
+        del context
+        others = {}
+        for name in ("C1", "C3", "C4", "C5"):
+            r, other_ok, other_context = measure_workload(name, 0, 5, 2, 2000, 0)
+            del other_context
+            torch.cuda.empty_cache()
+            others[name] = {"workload": r["config"]["workload"], "ms_per_step": r["ms_per_step"], "docs_per_sec": r["value"],
+                            "kernel_ms": r["roofline"]["kernel_ms"], "frac": r["roofline"]["frac"],
+                            "kernels": {k: {"name": v["name"], "avg_ms": v["avg_ms"]} for k, v in r["kernels"].items()},
+                            "parity": r["parity"]}
+            ok = ok and other_ok
+        result["other_workloads"] = others
+    if not args.no_end_to_end:
+        result["end_to_end_c_abi"] = end_to_end_c_abi(model, info, docs)
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(model_bytes, info)
+        if info["kind"] == "oblivious" and info["dim"] == 1 and not info["cat_hashes"]:
+            # the sampled documents of the parity check, through the reference's own scalar evaluator
+            ref = reference_standalone(model_bytes, sample, got)
+            if ref is not None:
+                result["cpu_baseline"]["reference_standalone_evaluator"] = ref
+    print(json.dumps(result))
+    if not ok:
+        sys.exit(1)
+
+
+def measure_workload(config, docs_override, steps, warmup, check_docs, copy_probe_mib):
+    """One workload: `warmup` untimed and `steps` timed steps on documents that sit in HBM, and the parity of a
+    sample of the output against the oracle. Returns (the JSON fields, parity ok, what the callers' other legs need)."""
+    import numpy as np
+    import torch
+
+    import catboost_amd as cb
+    from catboost_amd import synthetic as syn
+
+    class args:  # the names the body below uses
+        pass
+    args.config, args.docs, args.steps, args.warmup, args.check_docs, args.copy_probe_mib = (
+        config, docs_override, steps, warmup, check_docs, copy_probe_mib)
     model, info = syn.build_model(args.config)
     model.enable_gpu_evaluation(0)
     docs = args.docs or info["docs"]
@@ -277,18 +327,8 @@ def main():
                                                "max": used_borders[-1]} if used_borders else None},
         "parity": {"checked_docs": int(n_check), "max_abs_err": max_abs, "within_1e-9_rel_1e-12_abs": ok},
     }
-    if not args.no_end_to_end:
-        result["end_to_end_c_abi"] = end_to_end_c_abi(model, info, docs)
-    if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(model_bytes, info)
-        if info["kind"] == "oblivious" and dim == 1 and not info["cat_hashes"]:
-            # the sampled documents of the parity check, through the reference's own scalar evaluator
-            ref = reference_standalone(model_bytes, sample, got)
-            if ref is not None:
-                result["cpu_baseline"]["reference_standalone_evaluator"] = ref
-    print(json.dumps(result))
-    if not ok:
-        sys.exit(1)
+    del x, out
+    return result, ok, (model, info, docs, model_bytes, sample, got)
 
 
 if __name__ == "__main__":

@@ -152,6 +152,8 @@ def load_library():
         "CbHipLastKernelTimes": (ctypes.c_bool, [vp, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float)]),
         "CbHipDescribeKernels": (ctypes.c_bool, [vp, ctypes.c_int, sz, ctypes.c_char_p, sz]),
         "CbHipGetEvaluator": (vp, [vp]),
+        "CbHipEvaluatorSetSmallBatchSlicing": (ctypes.c_bool, [vp, ctypes.c_bool]),
+        "CbHipSetSmallBatchSlicing": (ctypes.c_bool, [vp, ctypes.c_bool]),
         "CbHipSetFeatureLayout": (ctypes.c_bool, [vp, vp, sz, vp, sz, vp, sz]),
         "CbHipLoadModelFromArrays": (ctypes.c_bool, [vp, ctypes.POINTER(ModelArrays)]),
         "CbHipBuildObliviousModel": (ctypes.c_bool, [vp, ctypes.POINTER(ModelArrays), ctypes.c_int32, vp, vp, vp]),
@@ -401,6 +403,10 @@ class DeviceEvaluator:
         _check(self._lib.CbHipLastKernelTimes(self._h, ctypes.byref(a), ctypes.byref(b)))
         return a.value, b.value
 
+    def set_small_batch_slicing(self, enabled):
+        """False: small batches are evaluated in one pass in tree order like large ones (CbHipEvaluatorSetSmallBatchSlicing)."""
+        _check(self._lib.CbHipEvaluatorSetSmallBatchSlicing(self._h, bool(enabled)))
+
 
 class ModelCalcer:
     """Model handle of the model_calcer C API (ModelCalcerWrapper, wrapped_calcer.h:17-110)."""
@@ -566,6 +572,11 @@ class ModelCalcer:
             _check(self._lib.SetPredictionTypeString(self._h, prediction_type.encode()))
         else:
             _check(self._lib.SetPredictionType(self._h, int(prediction_type)))
+
+    def set_small_batch_slicing(self, enabled):
+        """False: small batches are evaluated in one pass in tree order, the CPU evaluator's order of additions,
+        instead of as slices of the trees (CbHipSetSmallBatchSlicing)."""
+        _check(self._lib.CbHipSetSmallBatchSlicing(self._h, bool(enabled)))
 
     def evaluator(self):
         h = self._lib.CbHipGetEvaluator(self._h)

@@ -35,6 +35,7 @@ struct TModelHandle {
     int DeviceId = 0;
     EApiPredictionType PredictionType = APT_RAW_FORMULA_VAL;
     TFeatureLayout Layout;  // IModelEvaluator::SetFeatureLayout, evaluation_interface.h:82
+    bool SmallBatchSlicing = true;  // CbHipSetSmallBatchSlicing
 
     void ResetEvaluator() {
         std::lock_guard<std::mutex> g(EvaluatorLock);
@@ -46,6 +47,9 @@ struct TModelHandle {
         if (!Evaluator) {
             Model.EnsureSupported();
             Evaluator.reset(new THipEvaluator(Model.Trees, DeviceId, &Model.CtrTables, &Layout));
+            if (!SmallBatchSlicing) {
+                Evaluator->SetSmallBatchSlicing(false);
+            }
         }
         return *Evaluator;
     }
@@ -886,6 +890,21 @@ bool CbHipDescribeKernels(CbHipEvaluatorHandle* evaluator, int layout, size_t do
         const std::string text = E(evaluator)->DescribeKernels(layout, docCount);
         CBAMD_ENSURE(text.size() < bufferSize, "description buffer is too small");
         std::memcpy(buffer, text.c_str(), text.size() + 1);
+    });
+}
+
+bool CbHipEvaluatorSetSmallBatchSlicing(CbHipEvaluatorHandle* evaluator, bool enabled) {
+    return Guard([&] { E(evaluator)->SetSmallBatchSlicing(enabled); });
+}
+
+bool CbHipSetSmallBatchSlicing(void* modelHandle, bool enabled) {
+    return Guard([&] {
+        TModelHandle* h = H(modelHandle);
+        std::lock_guard<std::mutex> g(h->EvaluatorLock);
+        h->SmallBatchSlicing = enabled;
+        if (h->Evaluator) {
+            h->Evaluator->SetSmallBatchSlicing(enabled);
+        }
     });
 }
 

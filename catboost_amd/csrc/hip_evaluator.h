@@ -66,8 +66,17 @@ public:
     void EvalQuantizedSlicedDevice(const uint8_t* bins, size_t docCount, double* results, double* partials, void* stream);
     // binarize + evaluate in one launch of a fused kernel, the bins in registers only; false (and nothing
     // launched) when the model, the batch layout or the tree range has no fused kernel
+    // (anyBatchSize: also below the batch size from which the fused launch is the faster one)
     bool EvalRowsFusedDevice(const TFeatureBatch& batch, size_t docCount, size_t treeStart, size_t treeEnd,
-                             double* results, void* stream);
+                             double* results, void* stream, bool anyBatchSize = false);
+    // index of the fused kernel tables that such a call would use (0 flat rows, 1 split rows), -1 when it takes
+    // the two launches: the one test that EvalRowsFusedDevice, the host pipeline and DescribeKernels share
+    int FusedLayoutFor(int layout, size_t stride, size_t docCount, size_t treeStart, size_t treeEnd, bool anyBatchSize) const;
+    // Small batches (fewer than 256 workgroups of the register kernels) are cut into slices of the trees by the
+    // calls that own their scratch memory; off: every sum is one pass in tree order, the CPU evaluator's
+    // order of additions, at the price of the small-batch speed-up. Set it before the calls it should govern.
+    void SetSmallBatchSlicing(bool on);
+    bool SmallBatchSlicing() const;
     void LeafIndexesQuantizedDevice(const uint8_t* bins, size_t docCount, size_t treeStart, size_t treeEnd,
                                     uint32_t* indexes, void* stream);
     // bins in the reference's layout: blocks of 128 docs, [block][bucket][doc in block]
@@ -89,8 +98,9 @@ public:
     void Synchronize(void* stream);
     TKernelTimes LastKernelTimes() const;
     // which kernels a whole-model call (CalcDevice, the host entry points) on docCount documents of the given
-    // layout (TFeatureBatch::ELayout) launches: "fused=<kernel>" or "binarize=<kernel>;evaluate=<kernel>"
-    std::string DescribeKernels(int layout, size_t docCount) const;
+    // layout (TFeatureBatch::ELayout) and row stride (in values; 0: the model's own row width) launches:
+    // "fused=<kernel>" or "binarize=<kernel>;evaluate=<kernel>". Calls for a range of the trees are not described.
+    std::string DescribeKernels(int layout, size_t docCount, size_t stride = 0) const;
 
     // ---- host-resident data: stage -> binarize -> evaluate -> copy back, in document chunks.
     // rows[doc] points at rowLen floats (FlatRows / SplitRows) or columns[f] at docCount floats.

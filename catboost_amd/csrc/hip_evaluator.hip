@@ -309,8 +309,10 @@ const TEvalRegVariant* PickRegVariant(uint32_t buckets, uint32_t dim, uint32_t m
     return best;
 }
 
-// Diagnostic switches, read from the environment when an evaluator is built (cb_hip_evaluator.h lists them).
-// They choose between kernels that give the same results; tests use them to reach every kernel with one model.
+// Diagnostic switches, read from the environment when an evaluator is built (cb_hip_evaluator.h lists them) and
+// only in a process that sets CATBOOST_AMD_TEST_SWITCHES=1: a production process that happens to have one of the
+// names in its environment keeps the default kernels. They choose between kernels that give the same results;
+// tests use them to reach every kernel with one model.
 struct TKernelSwitches {
     bool RegKernel = true;        // CATBOOST_AMD_REG_KERNEL=0: no register-resident assembly kernels
     bool RegSix = true;           // CATBOOST_AMD_REG_SIX=0: no six-bit form of those kernels
@@ -330,6 +332,10 @@ struct TKernelSwitches {
             return v != nullptr && v[0] == '0';
         };
         TKernelSwitches k;
+        const char* gate = std::getenv("CATBOOST_AMD_TEST_SWITCHES");
+        if (gate == nullptr || gate[0] != '1') {
+            return k;
+        }
         k.RegKernel = !off("CATBOOST_AMD_REG_KERNEL");
         k.RegSix = !off("CATBOOST_AMD_REG_SIX");
         k.CtrTile = !off("CATBOOST_AMD_CTR_TILE");
@@ -1102,7 +1108,11 @@ struct THipEvaluator::TImpl {
     TFused Fused[2];
     hipFunction_t FusedFunction = nullptr;
     uint32_t FusedWaves = 0;
-    size_t FusedMinDocs = 0;
+    // Below about one wave per SIMD a fused launch lasts as long as one wave's binarize phase and tree walk,
+    // and two launches (the binarize kernel spreads a block over many waves) are shorter.
+    size_t FusedMinDocs() const {
+        return SmallBatchSlices ? size_t(1024) * dev::kDocsPerBlock : 0;
+    }
     const char* RegKernelName = "";
     const char* FusedKernelName = "";
 
@@ -1132,17 +1142,25 @@ struct THipEvaluator::TImpl {
         bool Busy = false;
 
         THostContext() {
-            HIP_CHECK(hipStreamCreateWithFlags(&Stream, hipStreamNonBlocking));
-            for (auto& e : Ev) {
-                HIP_CHECK(hipEventCreate(&e));
-            }
-            for (auto& slot : Slots) {
-                for (auto& e : slot.Ev) {
+            try {
+                HIP_CHECK(hipStreamCreateWithFlags(&Stream, hipStreamNonBlocking));
+                for (auto& e : Ev) {
                     HIP_CHECK(hipEventCreate(&e));
                 }
+                for (auto& slot : Slots) {
+                    for (auto& e : slot.Ev) {
+                        HIP_CHECK(hipEventCreate(&e));
+                    }
+                }
+            } catch (...) {
+                Release();  // the destructor does not run for a constructor that throws
+                throw;
             }
         }
         ~THostContext() {
+            Release();
+        }
+        void Release() {
             if (Stream) {
                 (void)hipStreamSynchronize(Stream);
             }
@@ -1160,6 +1178,7 @@ struct THipEvaluator::TImpl {
             }
             if (Stream) {
                 (void)hipStreamDestroy(Stream);
+                Stream = nullptr;
             }
         }
         THostContext(const THostContext&) = delete;
@@ -1276,6 +1295,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
     HIP_CHECK(hipSetDevice(deviceId));
     TImpl& m = *Impl;
     m.DeviceId = deviceId;
+    m.SmallBatchSlices = switches.SmallBatch;
     m.NoAllocScratch = NoAllocScratchOfCurrentDevice(deviceId);
     HIP_CHECK(hipStreamCreateWithFlags(&m.Stream, hipStreamNonBlocking));
     TreeCount = trees.GetTreeCount();
@@ -1897,7 +1917,6 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
             m.RegLaunches.push_back(l);
         }
         m.RegKernelUsable = true;
-        m.SmallBatchSlices = switches.SmallBatch;
 
         // ---- fused kernels: float-only one-dimensional models in the 7-bit or six-bit form whose rows are
         // at least sixteen columns wide. The bins registers follow the columns of the rows (a unit = sixteen
@@ -2030,7 +2049,6 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
                 HIP_CHECK(hipModuleGetFunction(&m.FusedFunction, m.RegModule, fused->Name));
                 m.FusedWaves = fused->Waves;
                 m.FusedKernelName = fused->Name;
-                m.FusedMinDocs = switches.SmallBatch ? size_t(1024) * dev::kDocsPerBlock : 0;
             }
             TImpl::TFused& f = m.Fused[layoutIndex];
             f.UnitCount = static_cast<uint32_t>(unitStart.size());
@@ -2795,17 +2813,24 @@ void THipEvaluator::EvalQuantizedSlicedDevice(const uint8_t* bins, size_t docCou
     HIP_CHECK(hipGetLastError());
 }
 
-bool THipEvaluator::EvalRowsFusedDevice(const TFeatureBatch& batch, size_t docCount, size_t treeStart, size_t treeEnd,
-                                        double* results, void* stream) {
-    TImpl& m = *Impl;
-    const int layoutIndex = batch.Layout == TFeatureBatch::FlatRows ? 0 : batch.Layout == TFeatureBatch::SplitRows ? 1 : -1;
+int THipEvaluator::FusedLayoutFor(int layout, size_t stride, size_t docCount, size_t treeStart, size_t treeEnd, bool anyBatchSize) const {
+    const TImpl& m = *Impl;
+    const int layoutIndex = layout == TFeatureBatch::FlatRows ? 0 : layout == TFeatureBatch::SplitRows ? 1 : -1;
     if (layoutIndex < 0 || !m.Fused[layoutIndex].Usable || docCount == 0 || treeStart != 0 || treeEnd != TreeCount ||
-        docCount >= (size_t(1) << 29) || batch.Stride >= (size_t(1) << 20)) {
-        return false;
+        docCount >= (size_t(1) << 29) || stride >= (size_t(1) << 20)) {
+        return -1;
     }
-    // Below about one wave per SIMD a fused launch lasts as long as one wave's binarize phase and tree walk,
-    // and two launches (the binarize kernel spreads a block over many waves) are shorter.
-    if (m.FusedMinDocs > 0 && docCount < m.FusedMinDocs) {
+    if (!anyBatchSize && docCount < m.FusedMinDocs()) {
+        return -1;
+    }
+    return layoutIndex;
+}
+
+bool THipEvaluator::EvalRowsFusedDevice(const TFeatureBatch& batch, size_t docCount, size_t treeStart, size_t treeEnd,
+                                        double* results, void* stream, bool anyBatchSize) {
+    TImpl& m = *Impl;
+    const int layoutIndex = FusedLayoutFor(batch.Layout, batch.Stride, docCount, treeStart, treeEnd, anyBatchSize);
+    if (layoutIndex < 0) {
         return false;
     }
     const TImpl::TFused& f = m.Fused[layoutIndex];
@@ -2839,10 +2864,10 @@ bool THipEvaluator::EvalRowsFusedDevice(const TFeatureBatch& batch, size_t docCo
     return true;
 }
 
-std::string THipEvaluator::DescribeKernels(int layout, size_t docCount) const {
+std::string THipEvaluator::DescribeKernels(int layout, size_t docCount, size_t stride) const {
     const TImpl& m = *Impl;
-    const int fusedIndex = layout == TFeatureBatch::FlatRows ? 0 : layout == TFeatureBatch::SplitRows ? 1 : -1;
-    if (fusedIndex >= 0 && m.Fused[fusedIndex].Usable && docCount >= m.FusedMinDocs) {
+    // whole-model calls only: a call for a range of the trees may take other kernels
+    if (FusedLayoutFor(layout, stride, docCount, 0, TreeCount, false) >= 0) {
         return std::string("fused=") + m.FusedKernelName;
     }
     std::string binarize = m.BinarizeBuckets == 0 ? "none"
@@ -3002,13 +3027,23 @@ void THipEvaluator::CalcDevice(const TFeatureBatch& batch, size_t docCount, size
     SetLastTimes(times);
 }
 
+void THipEvaluator::SetSmallBatchSlicing(bool on) {
+    Impl->SmallBatchSlices = on;
+}
+
+bool THipEvaluator::SmallBatchSlicing() const {
+    return Impl->SmallBatchSlices;
+}
+
 void THipEvaluator::CalcDeviceNoAlloc(const TFeatureBatch& batch, size_t docCount, size_t treeStart, size_t treeEnd,
                                       double* results, void* stream) {
     TImpl& m = *Impl;
-    if (EvalRowsFusedDevice(batch, docCount, treeStart, treeEnd, results, stream)) {
-        return;  // the fused kernel keeps the bins in registers: no buffer at all
-    }
     const size_t maxDocs = kNoAllocScratchBytes / (static_cast<size_t>(m.LayoutBuckets) * dev::kDocsPerBlock) * dev::kDocsPerBlock;
+    // the fused kernel keeps the bins in registers: no buffer at all. A batch whose bins do not fit the fixed
+    // buffer takes it whatever its size (below the size from which it is the faster as well)
+    if (EvalRowsFusedDevice(batch, docCount, treeStart, treeEnd, results, stream, docCount > maxDocs)) {
+        return;
+    }
     CBAMD_ENSURE(docCount <= maxDocs, "batch of " + std::to_string(docCount) + " documents exceeds the fixed bin buffer: at most " +
                                           std::to_string(maxDocs) + " documents per call for this model");
     // every (block, bucket) cell that the evaluate kernels read is written by the binarize kernels of
@@ -3144,8 +3179,10 @@ static void RunPredictionChunk(THipEvaluator& ev, THipEvaluator::TImpl::THostCon
     const size_t dim = static_cast<size_t>(ev.GetApproxDimension());
     const size_t outDim = predictionType == dev::kPredClass ? 1 : dim;
     HIP_CHECK(hipEventRecord(slot.Ev[0], s));
-    if (ev.EvalRowsFusedDevice(batch, n, treeStart, treeEnd, slot.StageResults.Get(), s)) {
+    if (ev.FusedLayoutFor(batch.Layout, batch.Stride, n, treeStart, treeEnd, false) >= 0) {
+        // one launch does both: its whole duration is reported as the evaluate time, as CalcDevice does
         HIP_CHECK(hipEventRecord(slot.Ev[1], s));
+        ev.EvalRowsFusedDevice(batch, n, treeStart, treeEnd, slot.StageResults.Get(), s);
     } else {
         ev.QuantizeDevice(batch, n, ctx.ScratchBins.Get(), s);
         HIP_CHECK(hipEventRecord(slot.Ev[1], s));

@@ -79,15 +79,15 @@ typedef struct CbHipFeatures {
 } CbHipFeatures;
 
 /* Diagnostic switches, read from the environment whenever an evaluator is built (CbHipEvaluatorCreate, the
- * first prediction of a model handle, CbHipSetFeatureLayout). They select between kernels that return the
- * same results and exist for tests and measurements; production callers leave them unset.
+ * first prediction of a model handle, CbHipSetFeatureLayout), and only in a process whose environment has
+ * CATBOOST_AMD_TEST_SWITCHES=1: without it none of the names below is looked at. They select between kernels
+ * that return the same results and exist for tests and measurements.
  *   CATBOOST_AMD_REG_KERNEL=0        no register-resident assembly kernels (the LDS tile kernels instead)
  *   CATBOOST_AMD_REG_SIX=0           no six-bit form of the register-resident kernels
  *   CATBOOST_AMD_REG_MIN_BUCKETS=n   only register-resident kernel shapes that hold n buckets or more
  *   CATBOOST_AMD_REG_SPLIT=0         a float feature with more than 127 used borders sends the model to the mixed
  *                                    (8-bit compare) kernels instead of taking two bins registers
- *   CATBOOST_AMD_SMALL_BATCH=0       no slices of the trees for small batches, fused kernels for every batch size:
- *                                    every sum then has the CPU evaluator's order of additions
+ *   CATBOOST_AMD_SMALL_BATCH=0       the start value of CbHipSetSmallBatchSlicing is "off"
  *   CATBOOST_AMD_LEVEL_ORDER=0       register-resident kernels keep the model's order of a tree's levels
  *   CATBOOST_AMD_FUSED=0             binarize and evaluate always as two launches (no fused kernels)
  *   CATBOOST_AMD_PAIR_TILE=0         wide one-dimensional models (more buckets than an LDS tile of 256 documents
@@ -139,9 +139,13 @@ bool CbHipEvalData(CbHipEvaluatorHandle* evaluator, const CbHipFeatures* deviceF
  * and records no kernel times: it only launches the binarize and evaluate kernels on `hipStream`
  * (NULL = the evaluator's own stream). Fails when CbHipQuantizedBytes(evaluator, docCount) exceeds
  * 32 MiB (the error names the largest document count for the model); a model that runs on a fused
- * kernel keeps its bins in registers, uses no buffer and has no such limit. All calls on one GPU share the
- * array, so calls that overlap there (two streams, two threads, two evaluators) race; calls in stream
- * order on one stream are safe. */
+ * kernel keeps its bins in registers there, uses no buffer and has no such limit (a batch of such a model
+ * that does not fit the buffer takes the fused kernel at any size). The call never cuts the trees into
+ * slices (it has no memory for partial sums): every sum is one pass in tree order, the CPU evaluator's order
+ * of additions, so for small batches it may differ in the last bits from CbHipEvalData with slicing on, and
+ * it has none of that call's small-batch speed-up. All calls on one GPU share the array, so calls that
+ * overlap there (two streams, two threads, two evaluators) race; calls in stream order on one stream are
+ * safe. */
 bool CbHipEvalDataNoAlloc(CbHipEvaluatorHandle* evaluator, const CbHipFeatures* deviceFeatures, size_t docCount,
                           size_t treeStart, size_t treeEnd, double* deviceResults, void* hipStream);
 
@@ -167,13 +171,27 @@ bool CbHipApplyPredictionTypeDevice(CbHipEvaluatorHandle* evaluator, int predict
 bool CbHipSynchronize(CbHipEvaluatorHandle* evaluator, void* hipStream);
 
 /* hipEvent-measured duration of the binarize and evaluate kernels of the last CbHipEvalData or
- * host-level prediction call (summed over its chunks). */
+ * host-level prediction call (summed over its chunks). A call that ran as one fused launch reports the
+ * whole launch as evalMs and 0 as binarizeMs, whatever the entry point. */
 bool CbHipLastKernelTimes(CbHipEvaluatorHandle* evaluator, float* binarizeMs, float* evalMs);
 
 /* Which kernels a whole-model CbHipEvalData (or host entry point) call on docCount documents of `layout`
  * (ECbHipFeatureLayout) launches, as text: "fused=<kernel>" or "binarize=<kernel>;evaluate=<kernel>". For logs
  * and benchmarks; no counterpart in the reference. */
 bool CbHipDescribeKernels(CbHipEvaluatorHandle* evaluator, int layout, size_t docCount, char* buffer, size_t bufferSize);
+
+/* Batches of fewer than 256 workgroups (65 536 to 262 144 documents, by the kernel) are spread over the GPU by
+ * cutting the trees into slices that run side by side; a slice adds its leaves in tree order and the slices'
+ * sums are then added in slice order. The result is the same for every call and every batch size below that
+ * limit, and differs in the last bits (inside 1e-9 relative) from the single pass in tree order that larger
+ * batches, CbHipEvalQuantized and the CPU evaluator make (cpu/evaluator_impl.cpp:362-460; single document:
+ * c_api.cpp:383-384). enabled = false turns the slices off for later calls: every sum is then one pass in tree
+ * order whatever the batch size, at the price of the small-batch speed-up (C2 model, 4096 documents: 0.13
+ * instead of 0.04 ms per call). No counterpart in the reference. The first form acts on a bare evaluator, the
+ * second on a model handle (kept across Load* calls and rebuilt evaluators). Not to be called while another
+ * thread evaluates on the same handle. */
+bool CbHipEvaluatorSetSmallBatchSlicing(CbHipEvaluatorHandle* evaluator, bool enabled);
+bool CbHipSetSmallBatchSlicing(void* modelHandle, bool enabled);
 
 /* ---- extensions on a ModelCalcerHandle (c_api.h) ------------------------------------------ */
 

@@ -54,6 +54,7 @@ def test_library_loaded_is_the_in_tree_hip_build():
     assert cb.ModelCalcer().get_supported_evaluator_types() == [1]  # CBA_FET_GPU only
 
 
+@pytest.mark.both_batch_modes
 @pytest.mark.parametrize("asym", [False, True])
 def test_simple_float_model(asym):
     model = rm.simple_float_model()
@@ -62,6 +63,7 @@ def test_simple_float_model(asym):
     _check_flat(model, rm.DATA, exact=np.arange(8.0))
 
 
+@pytest.mark.both_batch_modes
 @pytest.mark.parametrize("asym", [False, True])
 def test_scale_bias_two_trees(asym):
     model = rm.simple_float_model(tree_count=2, scale=0.5, bias=[0.125])
@@ -74,6 +76,7 @@ def test_scale_bias_two_trees(asym):
     np.testing.assert_array_equal(g.calc_flat(rm.DATA, tree_start=1, tree_end=1), np.zeros(8))
 
 
+@pytest.mark.both_batch_modes
 @pytest.mark.parametrize("asym", [False, True])
 def test_deep_tree(asym):
     model = rm.simple_deep_tree_model(9)
@@ -83,6 +86,7 @@ def test_deep_tree(asym):
     np.testing.assert_array_equal(g.calc_leaf_indexes_flat(rm.deep_tree_data(9)).ravel(), np.arange(512))
 
 
+@pytest.mark.both_batch_modes
 @pytest.mark.parametrize("asym", [False, True])
 def test_multi_value_model(asym):
     model = rm.multi_value_float_model()
@@ -92,6 +96,7 @@ def test_multi_value_model(asym):
     np.testing.assert_array_equal(g.predict_specific_class_flat(rm.DATA[:4], 1), [10., 11., 12., 13.])
 
 
+@pytest.mark.both_batch_modes
 def test_simple_asymmetric_model():
     g, _ = _check_flat(rm.simple_asymmetric_model(), rm.DATA, exact=rm.ASYMMETRIC_PREDICTIONS)
     np.testing.assert_array_equal(g.calc_leaf_indexes_flat(rm.DATA), rm.ASYMMETRIC_LEAF_INDEXES)
@@ -224,6 +229,7 @@ def test_empty_batches(golden_dir):
 
 # ------------------------------------------------------------------- fixtures + goldens ----
 
+@pytest.mark.both_batch_modes
 def test_numeric_only_fixture(golden_dir):
     g = cb.ModelCalcer(os.path.join(golden_dir, "numeric_only_model.cbm"))
     g.enable_gpu_evaluation(0)
@@ -234,6 +240,7 @@ def test_numeric_only_fixture(golden_dir):
     _close(g.calc_single(rm.NUMERIC_ONLY_ROWS[0], []), rm.NUMERIC_ONLY_EXPECTED[:1])
 
 
+@pytest.mark.both_batch_modes
 def test_json_model_format(golden_dir):
     # the json twin of the numeric-only model (CatBoostModelTest.java:181-200) predicts the binary's goldens
     g = cb.ModelCalcer(os.path.join(golden_dir, "numeric_only_model.json"), model_format="json")
@@ -246,6 +253,7 @@ def test_json_model_format(golden_dir):
     _close(g.calc_flat(x), OracleModel(model).calc(x))
 
 
+@pytest.mark.both_batch_modes
 def test_json_model_format_with_ctr_features(golden_dir):
     """Models with CTR features through the json format: bins and predictions equal the oracle's on what
     the format keeps of the model (tests/test_host_logic.py::json_view_of_ctr_model)."""
@@ -271,6 +279,7 @@ def test_json_model_format_with_ctr_features(golden_dir):
     assert checked >= 5
 
 
+@pytest.mark.both_batch_modes
 def test_rust_fixture_with_one_hot_string_cats(golden_dir):
     g = cb.ModelCalcer(os.path.join(golden_dir, "rust_tmp_model.cbm"))
     _close(g.calc(rm.RUST_FLOATS, rm.RUST_CATS), rm.RUST_EXPECTED)
@@ -342,6 +351,7 @@ def _hashed(rows):
     return np.array([[cb.string_cat_feature_hash(c) for c in row] for row in rows], np.int32)
 
 
+@pytest.mark.both_batch_modes
 def test_ctr_goldens_of_the_jvm_tests(golden_dir):
     # CatBoostModelTest.java:457-470, 528-547, 586-601, 720-743; the reference's CUDA evaluator refuses
     # both models (cuda/evaluator.cpp:22-28)
@@ -357,6 +367,7 @@ def test_ctr_goldens_of_the_jvm_tests(golden_dir):
     _close(g.calc_single(rm.JVM_CTR_FLOATS[0], rm.JVM_CTR_CATS[0]), rm.JVM_CTR_EXPECTED[:1])
 
 
+@pytest.mark.both_batch_modes
 def test_ctr_goldens_of_the_rust_and_node_tests(golden_dir):
     g = cb.ModelCalcer(os.path.join(golden_dir, "features_num_cat__dataset_adult.cbm"))
     _close(g.calc(rm.RUST_ADULT_FLOATS, rm.RUST_ADULT_CATS), rm.RUST_ADULT_EXPECTED)
@@ -364,6 +375,7 @@ def test_ctr_goldens_of_the_rust_and_node_tests(golden_dir):
     assert ["%.2f" % v for v in g.calc(rm.NODE_ADULT_FLOATS, rm.NODE_ADULT_CATS)] == rm.NODE_ADULT_EXPECTED_2DP
 
 
+@pytest.mark.both_batch_modes
 def test_ctr_mushroom_labels(golden_dir):
     # CatBoostModelEvaluatorTest.cs:101-127
     g = cb.ModelCalcer(os.path.join(golden_dir, "mushroom_model.cbm"))
@@ -439,6 +451,7 @@ def test_synthetic_ctr_models_of_every_kind(golden_dir, monkeypatch, seed, tile)
         np.testing.assert_array_equal(g.calc_leaf_indexes_flat(flat), o.leaf_indexes(flat))
 
 
+@pytest.mark.both_batch_modes
 @pytest.mark.parametrize("name", ["cat", "nocat"])
 def test_models_that_the_reference_holds_as_exported_cpp(golden_dir, name):
     """The two models that the reference keeps as exported C++ code (tests/golden/make_export_vectors.py):
@@ -662,11 +675,13 @@ def test_device_entry_points_in_a_hip_graph(golden_dir):
             assert torch.equal(out, torch.full_like(out, 1.75))
 
 
+@pytest.mark.both_batch_modes
 def test_querywise_fixture(golden_dir):
     g = cb.ModelCalcer(os.path.join(golden_dir, "features_num__dataset_querywise.cbm"))
     np.testing.assert_allclose(g.calc_flat(rm.querywise_rows()), rm.QUERYWISE_EXPECTED, rtol=1e-12, atol=1e-15)
 
 
+@pytest.mark.both_batch_modes
 def test_iris_fixture(golden_dir):
     path = os.path.join(golden_dir, "iris_model.cbm")
     g = cb.ModelCalcer(path)
@@ -689,6 +704,7 @@ def test_iris_fixture(golden_dir):
     np.testing.assert_allclose(g.calc_flat(feats).reshape(-1, 3).sum(axis=1), 1.0, atol=1e-12)
 
 
+@pytest.mark.both_batch_modes
 @pytest.mark.parametrize("name", ["all", "missed"])
 def test_multiclass_probabilities_of_the_reference_canondata(golden_dir, name):
     """The multi-class model and the 17-digit probability table of the reference's own
@@ -717,6 +733,7 @@ def test_multiclass_probabilities_of_the_reference_canondata(golden_dir, name):
     np.testing.assert_allclose(out.cpu().numpy().reshape(100, dim), expected, rtol=1e-9, atol=1e-12)
 
 
+@pytest.mark.both_batch_modes
 def test_model_of_the_backward_compatibility_test(golden_dir):
     """The old-version three-class model of the reference's test_multiclass_model_backward_compatibility and
     the canonical outputs of `catboost calc` for it (10 digits), through the library."""
@@ -727,6 +744,7 @@ def test_model_of_the_backward_compatibility_test(golden_dir):
         np.testing.assert_allclose(g.calc_flat(v["features"]), v[kind].ravel(), rtol=6e-10, atol=0)
 
 
+@pytest.mark.both_batch_modes
 def test_prediction_types_of_the_reference_unit_test():
     """TestFlatCalcMultiValMultiProba (formula_evaluator_ut.cpp:148-165) through the C API, and the
     one-dimensional types on the two-tree model with scale and bias."""
@@ -749,6 +767,7 @@ def test_prediction_types_of_the_reference_unit_test():
     np.testing.assert_allclose(g.calc_flat(x), 1 / (1 + np.exp(-raw)), rtol=1e-12)
 
 
+@pytest.mark.both_batch_modes
 def test_boston_fixture(golden_dir):
     path = os.path.join(golden_dir, "boston_housing_model.cbm")
     g = cb.ModelCalcer(path)
@@ -1008,6 +1027,7 @@ def test_library_builder_matches_oracle_builder_and_roundtrips():
 
 # --------------------------------------------------------------------- the five workloads ----
 
+@pytest.mark.both_batch_modes
 @pytest.mark.parametrize("name,docs", [("C1", 30000), ("C2", 20000), ("C3", 10000), ("C4", 20000), ("C5", 6000)])
 def test_workload_configs_host_path(name, docs):
     model, info = syn.build_model(name)
@@ -1252,7 +1272,8 @@ def test_c2_full_size_properties():
     ev.eval_quantized(bins.data_ptr(), docs, out2.data_ptr())
     ev.synchronize()
     assert torch.equal(out, out2)
-    # tree sub-ranges (tile kernel) add up to the whole model (scale 1, bias 0 in this workload)
+    # tree sub-ranges (register kernels for the whole tree blocks, the plain kernel for a range's ragged ends) add up to
+    # the whole model (scale 1, bias 0 in this workload)
     trees = model.tree_count
     parts = torch.zeros_like(out)
     part = torch.zeros_like(out)

@@ -53,3 +53,36 @@ def test_small_batches_through_tree_slices(cfg, trees):
         np.testing.assert_array_equal(out.cpu().numpy(), expected)
     else:
         np.testing.assert_allclose(out.cpu().numpy(), expected, rtol=1e-9, atol=1e-12)
+
+
+def test_small_batch_slicing_switched_off_through_the_api():
+    """CbHipSetSmallBatchSlicing / CbHipEvaluatorSetSmallBatchSlicing: with the slices off a small batch is summed in
+    one pass in tree order, the CPU evaluator's bits, through the model handle's host calls and the evaluator's
+    device calls; switched on again the slices are back."""
+    import torch
+
+    model, info = syn.build_model("C2", trees=200)
+    model.enable_gpu_evaluation(0)
+    oracle = OracleModel(read_cbm(model.save_to_buffer()))
+    x = syn.device_features(info, 3000)
+    host = x.cpu().numpy()
+    expected = oracle.calc(host, threads=8)
+    ev = model.evaluator()
+    assert "slices" in ev.describe_kernels(cb.LAYOUT_FLAT_ROWS, 3000)["evaluate"]
+    sliced = model.calc_flat(host)
+    np.testing.assert_allclose(sliced, expected, rtol=1e-9, atol=1e-12)
+    model.set_small_batch_slicing(False)
+    assert "slices" not in str(ev.describe_kernels(cb.LAYOUT_FLAT_ROWS, 3000))   # (this model: the fused kernel at any size)
+    np.testing.assert_array_equal(model.calc_flat(host), expected)
+    out = torch.zeros(3000, dtype=torch.float64, device="cuda:0")
+    torch.cuda.synchronize()
+    ev.eval_data(ev.features(cb.LAYOUT_FLAT_ROWS, x.data_ptr(), x.shape[1]), 3000, out.data_ptr())
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out.cpu().numpy(), expected)
+    # the setting survives a new evaluator of the handle (a feature layout rebuilds it)
+    model.set_feature_layout(None, None, None)
+    np.testing.assert_array_equal(model.calc_flat(host), expected)
+    ev = model.evaluator()
+    ev.set_small_batch_slicing(True)
+    assert "slices" in ev.describe_kernels(cb.LAYOUT_FLAT_ROWS, 3000)["evaluate"]
+    np.testing.assert_array_equal(model.calc_flat(host), sliced)

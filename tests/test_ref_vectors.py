@@ -30,6 +30,7 @@ def test_oracle_reproduces_reference_standalone_evaluator(golden_dir):
     assert n == 3
 
 
+@pytest.mark.both_batch_modes
 @pytest.mark.gpu
 def test_hip_evaluator_reproduces_reference_standalone_evaluator(golden_dir):
     import catboost_amd as cb

@@ -76,3 +76,39 @@ def test_no_alloc_entry_point_refuses_batches_beyond_its_buffer(monkeypatch):
     # the largest batch that fits runs and equals the allocating entry point
     got, expected = _run_both(ev, feats, max_docs, 1)
     assert torch.equal(got, expected)
+
+
+@pytest.mark.small_batch
+def test_no_alloc_entry_point_under_the_default_switches():
+    """With the library's default handling of small batches: a fused model's batch that is too large for the fixed
+    buffer and smaller than the size from which CbHipEvalData itself launches the fused kernel (it must not be
+    refused: the fused kernel needs no buffer), and a model of more than 64 trees whose small batches
+    CbHipEvalData cuts into slices of the trees while the entry point that allocates nothing makes the single
+    pass in tree order: both agree with the oracle, the single pass bit for bit."""
+    import torch
+
+    model, info = syn.build_model("C2", trees=96)
+    model.enable_gpu_evaluation(0)
+    ev = model.evaluator()
+    oracle = OracleModel(read_cbm(model.save_to_buffer()))
+    assert "fused" in ev.describe_kernels(cb.LAYOUT_FLAT_ROWS, 1 << 20)
+    per_block = ev.quantized_bytes(256)
+    max_docs = NO_ALLOC_BYTES // per_block * 256
+    docs = max_docs + 777
+    assert "fused" not in ev.describe_kernels(cb.LAYOUT_FLAT_ROWS, docs)      # CbHipEvalData: two launches at this size
+    x = syn.device_features(info, docs)
+    feats = ev.features(cb.LAYOUT_FLAT_ROWS, x.data_ptr(), x.shape[1])
+    got, expected = _run_both(ev, feats, docs, 1)
+    sample = np.sort(np.random.default_rng(5).choice(docs, 3000, replace=False))
+    want = oracle.calc(x[torch.from_numpy(sample).to("cuda:0")].cpu().numpy(), threads=8)
+    np.testing.assert_array_equal(got.cpu().numpy()[sample], want)               # fused kernel: tree order
+    np.testing.assert_allclose(expected.cpu().numpy()[sample], want, rtol=1e-9, atol=1e-12)
+    # a small batch: slices in CbHipEvalData, one pass here
+    small = 3000
+    assert "slices" in ev.describe_kernels(cb.LAYOUT_FLAT_ROWS, small).get("evaluate", "")
+    part = x[:small].contiguous()
+    feats = ev.features(cb.LAYOUT_FLAT_ROWS, part.data_ptr(), part.shape[1])
+    got, expected = _run_both(ev, feats, small, 1)
+    want = oracle.calc(part.cpu().numpy(), threads=8)
+    np.testing.assert_array_equal(got.cpu().numpy(), want)
+    np.testing.assert_allclose(expected.cpu().numpy(), want, rtol=1e-9, atol=1e-12)
