@@ -522,8 +522,13 @@ uint32_t RowTileWaves(uint32_t buckets, uint32_t maxDepth, int dim) {
 }
 
 // LDS of the deep-tile kernel: 256 documents' bins and the accumulator
-size_t DeepTileLdsBytes(uint32_t rows) {
-    return ((static_cast<size_t>(rows) * 256 + 15) & ~size_t(15)) + dev::kDocsPerBlock * sizeof(double);
+size_t DeepTileLdsBytes(uint32_t rows, int dims) {
+    return ((static_cast<size_t>(rows) * 256 + 15) & ~size_t(15)) + static_cast<size_t>(dims) * dev::kDocsPerBlock * sizeof(double);
+}
+
+// dimensions that a workgroup of the deep-tile kernel sums per walk of the trees
+int DeepTileDims(int dim) {
+    return dim == 1 ? 1 : 2;
 }
 
 // LDS of the quad-tile kernel: 64 documents' bins, then per wave the leaf values of four trees (later the partial sums)
@@ -1041,7 +1046,9 @@ struct THipEvaluator::TImpl {
     TDeviceVec<double> TileLeaves;     // its leaf values: [slice of the dimensions][tree][pair of dimensions][leaf][2]
     size_t TileSliceStride = 0;        // 16-byte pairs of TileLeaves per slice
     TDeviceVec<uint32_t> DeepRows;     // deep-tile kernel (depth 9 to 16): 32 dwords per tree, two halves of the row-tile form
-    TDeviceVec<uint32_t> DeepFirstLeaf;  // and the trees' first leaf values in Leaves
+    TDeviceVec<uint32_t> DeepFirstLeaf;  // and the trees' first leaf values in Leaves (one dimension) or first leaves in DeepLeaves
+    TDeviceVec<double> DeepLeaves;       // several dimensions: [slice of two][tree][leaf][2]
+    uint32_t DeepSliceLeaves = 0;        // leaves of all trees
     TDeviceVec<uint32_t> TileMap;      // rows of the tile of the row-tile or pair-tile kernel when buckets of more than
                                        // 127 values take two; empty: a row per bucket
     uint32_t TileRowCount = 0;
@@ -1470,24 +1477,50 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
     m.Bias.Upload(trees.Bias);
 
     // The kernels that keep a tree's row in registers (two trees per wave on half a tile, one on a whole tile)
-    // compare 7 bits. Their tile has a row per bucket, and two for a float bucket of more than 127 values:
-    // min(bin, 127) and max(bin - 127, 0), which the kernel makes while it copies the bins to LDS (tileMap). A
-    // one-hot bucket of more than 127 values keeps the model off these kernels.
+    // compare 7 bits. Their tile has a row per bucket, and two for a bucket of more than 127 values, which the
+    // kernel makes while it copies the bins to LDS (tileMap): min(bin, 127) and max(bin - 127, 0) for a float
+    // bucket, the bins up to 127 (0 for the others) and bin - 127 from 128 on (0 for the others) for a one-hot bucket.
     std::vector<uint32_t> tileRowOfBucket(offsets.size(), 0), tileMap;
-    bool tileRowsUsable = true, tileRowsSplit = false;
+    const bool tileRowsUsable = true;
+    bool tileRowsSplit = false;
     for (size_t b = 0; b + 1 < offsets.size(); ++b) {
         tileRowOfBucket[b] = static_cast<uint32_t>(tileMap.size());
         if (offsets[b + 1] - offsets[b] <= 127) {
             tileMap.push_back(static_cast<uint32_t>(b));
-        } else if (!(flags[b] & dev::kBucketFlagOneHot)) {
-            tileMap.push_back(static_cast<uint32_t>(b) | (dev::kTileMapLow << 16));
+        } else {
+            const bool oneHot = (flags[b] & dev::kBucketFlagOneHot) != 0;
+            tileMap.push_back(static_cast<uint32_t>(b) | ((oneHot ? dev::kTileMapOneHotLow : dev::kTileMapLow) << 16));
             tileMap.push_back(static_cast<uint32_t>(b) | (dev::kTileMapHigh << 16));
             tileRowsSplit = true;
-        } else {
-            tileRowsUsable = false;
         }
     }
     const uint32_t tileRowCount = static_cast<uint32_t>(tileMap.size());
+    // A level of a tree in those kernels' rows: (row of the tile, xor byte, value added to the four bins, xors)
+    struct TTileLevel {
+        uint32_t Row, Xor, Add;
+        bool IsXor;
+    };
+    const auto tileLevelOf = [&](const TRepackedBin& rb) {
+        TTileLevel level = {tileRowOfBucket[rb.FeatureIndex], 0, 0, false};
+        if (rb.XorMask != 0 || rb.SplitIdx == 0xff) {
+            // one-hot: bin == value, value = ~XorMask; below 128 seven bits of it are enough, a value from 128 on
+            // is looked for as value - 127 in the bucket's second row
+            uint32_t value = ~static_cast<uint32_t>(rb.XorMask) & 0xffu;
+            if (value > 127 && offsets[rb.FeatureIndex + 1] - offsets[rb.FeatureIndex] > 127) {
+                level.Row += 1;
+                value -= 127;
+            }
+            level.Xor = ~value & 0x7fu;
+            level.Add = 0x01010101u;
+            level.IsXor = true;
+        } else if (rb.SplitIdx > 127) {
+            level.Row += 1;  // the bucket's second row holds max(bin - 127, 0)
+            level.Add = (128u - (rb.SplitIdx - 127u)) * 0x01010101u;
+        } else {
+            level.Add = (128u - rb.SplitIdx) * 0x01010101u;
+        }
+        return level;
+    };
     // Their rows: 16 dwords per tree, slot d the byte offset of level d's row in the tile | xor byte << 24, slot
     // 8 + d the value added to the four bins of a dword.
     const auto rowsInRegisters = [&](uint32_t bucketBytes) {
@@ -1496,19 +1529,10 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
             uint32_t* row = rows.data() + t * dev::kPackedTreeDwords;
             bool anyXor = false;
             for (int d = 0; d < trees.TreeSizes[t]; ++d) {
-                const auto& rb = trees.RepackedBins[trees.TreeStartOffsets[t] + d];
-                row[d] = tileRowOfBucket[rb.FeatureIndex] * bucketBytes;
-                if (rb.XorMask != 0 || rb.SplitIdx == 0xff) {
-                    // one-hot: bin == value, value = ~XorMask; 7 bits of it are enough below 128
-                    row[d] |= (static_cast<uint32_t>(rb.XorMask) & 0x7fu) << 24;
-                    row[8 + d] = 0x01010101u;
-                    anyXor = true;
-                } else if (rb.SplitIdx > 127) {
-                    row[d] += bucketBytes;  // the bucket's second row holds max(bin - 127, 0)
-                    row[8 + d] = (128u - (rb.SplitIdx - 127u)) * 0x01010101u;
-                } else {
-                    row[8 + d] = (128u - rb.SplitIdx) * 0x01010101u;
-                }
+                const TTileLevel level = tileLevelOf(trees.RepackedBins[trees.TreeStartOffsets[t] + d]);
+                row[d] = level.Row * bucketBytes | level.Xor << 24;
+                row[8 + d] = level.Add;
+                anyXor = anyXor || level.IsXor;
             }
             if (anyXor) {
                 row[0] |= dev::kPairRowXorFlag;
@@ -2087,36 +2111,50 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         }
     }
 
-    // One-dimensional models of depth 9 to 16 that the register kernels do not take (deeper than 10, one-hot
-    // splits, more registers than they have): the same tile, a tree's levels in two halves of eight, leaf values
-    // gathered from the model's own table (EvalObliviousDeepTileKernel).
-    if (!m.RegKernelUsable && m.Oblivious && m.Dim == 1 && m.MaxDepth > 8 && m.MaxDepth <= 16 && TreeCount > 0 &&
-        switches.RowTile && tileRowsUsable && DeepTileLdsBytes(tileRowsSplit ? tileRowCount : m.LayoutBuckets) <= kMaxTileLdsBytes) {
+    // Models of depth 9 to 16 that the register kernels do not take (deeper than 10, one-hot splits, several
+    // dimensions, more registers than they have): the same tile, a tree's levels in two halves of eight, leaf values
+    // gathered from the model's own table, two dimensions per walk (EvalObliviousDeepTileKernel).
+    if (!m.RegKernelUsable && m.Oblivious && m.MaxDepth > 8 && m.MaxDepth <= 16 && TreeCount > 0 &&
+        switches.RowTile && tileRowsUsable &&
+        DeepTileLdsBytes(tileRowsSplit ? tileRowCount : m.LayoutBuckets, DeepTileDims(m.Dim)) <= kMaxTileLdsBytes) {
         const size_t tableTrees = TreeCount + dev::kPairTreePadding;
         std::vector<uint32_t> rows(tableTrees * 32, 0), first(tableTrees, 0);
         for (size_t t = 0; t < TreeCount; ++t) {
             uint32_t* row = rows.data() + t * 32;
             bool anyXor = false;
             for (int d = 0; d < trees.TreeSizes[t]; ++d) {
-                const auto& rb = trees.RepackedBins[trees.TreeStartOffsets[t] + d];
+                const TTileLevel level = tileLevelOf(trees.RepackedBins[trees.TreeStartOffsets[t] + d]);
                 uint32_t* half = row + (d < 8 ? 0 : 16);
                 const int slot = d % 8;
-                half[slot] = tileRowOfBucket[rb.FeatureIndex] * 256u;
-                if (rb.XorMask != 0 || rb.SplitIdx == 0xff) {
-                    half[slot] |= (static_cast<uint32_t>(rb.XorMask) & 0x7fu) << 24;
-                    half[8 + slot] = 0x01010101u;
-                    anyXor = true;
-                } else if (rb.SplitIdx > 127) {
-                    half[slot] += 256u;
-                    half[8 + slot] = (128u - (rb.SplitIdx - 127u)) * 0x01010101u;
-                } else {
-                    half[8 + slot] = (128u - rb.SplitIdx) * 0x01010101u;
-                }
+                half[slot] = level.Row * 256u | level.Xor << 24;
+                half[8 + slot] = level.Add;
+                anyXor = anyXor || level.IsXor;
             }
             if (anyXor) {
                 row[0] |= dev::kPairRowXorFlag;
             }
             first[t] = firstLeaf[t];
+        }
+        if (m.Dim > 1) {
+            // two dimensions of a leaf side by side, slice after slice
+            const size_t dim = static_cast<size_t>(m.Dim), slices = (dim + 1) / 2;
+            size_t leafCount = 0;
+            for (size_t t = 0; t < TreeCount; ++t) {
+                first[t] = static_cast<uint32_t>(leafCount);
+                leafCount += size_t(1) << trees.TreeSizes[t];
+            }
+            CBAMD_ENSURE(leafCount < (size_t(1) << 31), "too many leaves for the deep-tile kernel");
+            std::vector<double> pairs(slices * leafCount * 2, 0.0);
+            for (size_t t = 0; t < TreeCount; ++t) {
+                const double* values = trees.LeafValues.data() + trees.TreeFirstLeafOffsets[t];
+                for (size_t leaf = 0; leaf < (size_t(1) << trees.TreeSizes[t]); ++leaf) {
+                    for (size_t k = 0; k < dim; ++k) {
+                        pairs[((k / 2) * leafCount + first[t] + leaf) * 2 + k % 2] = values[leaf * dim + k];
+                    }
+                }
+            }
+            m.DeepLeaves.Upload(pairs);
+            m.DeepSliceLeaves = static_cast<uint32_t>(leafCount);
         }
         m.DeepRows.Upload(rows);
         m.DeepFirstLeaf.Upload(first);
@@ -2714,21 +2752,38 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
     }
     if (m.DeepRows.Get() != nullptr) {
         const size_t blocks = (docCount + dev::kDocsPerBlock - 1) / dev::kDocsPerBlock;
-        const size_t lds = DeepTileLdsBytes(m.TileRowCount);
+        const int dims = DeepTileDims(m.Dim);
+        const uint32_t slices = (static_cast<uint32_t>(m.Dim) + dims - 1) / dims;
+        const size_t lds = DeepTileLdsBytes(m.TileRowCount, dims);
         const bool wide = 2 * lds > kMaxTileLdsBytes;  // one workgroup per CU: sixteen waves
+        const dim3 grid(static_cast<uint32_t>(blocks), slices), threads(64 * (wide ? dev::kWideTileWaves : dev::kTileWaves));
         const auto launch = [&](auto kernel) {
             EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds);
-            hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(blocks)), dim3(64 * (wide ? dev::kWideTileWaves : dev::kTileWaves)),
-                               lds, s, reinterpret_cast<const uint32_t*>(bins), docCount, m.LayoutBuckets, m.TileMap.Get(),
-                               m.TileRowCount, reinterpret_cast<const uint4*>(m.DeepRows.Get()), m.DeepFirstLeaf.Get(),
-                               m.Leaves.Get(), m.Bias.Get(), m.Scale, tb, te, results);
+            hipLaunchKernelGGL(kernel, grid, threads, lds, s, reinterpret_cast<const uint32_t*>(bins), docCount, m.LayoutBuckets,
+                               m.TileMap.Get(), m.TileRowCount, reinterpret_cast<const uint4*>(m.DeepRows.Get()),
+                               m.DeepFirstLeaf.Get(), m.Leaves.Get(), m.Bias.Get(), m.Scale, tb, te, results);
         };
-        if (m.MaxDepth <= 12) {
-            wide ? launch(dev::EvalObliviousDeepTileKernel<4, dev::kWideTileWaves>)
-                 : launch(dev::EvalObliviousDeepTileKernel<4, dev::kTileWaves>);
+        const auto launchPairs = [&](auto kernel) {
+            EnsureDynamicLds(reinterpret_cast<const void*>(kernel), lds);
+            hipLaunchKernelGGL(kernel, grid, threads, lds, s, reinterpret_cast<const uint32_t*>(bins), docCount, m.LayoutBuckets,
+                               m.TileMap.Get(), m.TileRowCount, reinterpret_cast<const uint4*>(m.DeepRows.Get()),
+                               m.DeepFirstLeaf.Get(), m.DeepLeaves.Get(), m.Bias.Get(), m.Scale, static_cast<uint32_t>(m.Dim),
+                               m.DeepSliceLeaves, tb, te, results);
+        };
+        if (dims == 1) {
+            if (m.MaxDepth <= 12) {
+                wide ? launch(dev::EvalObliviousDeepTileKernel<4, dev::kWideTileWaves>)
+                     : launch(dev::EvalObliviousDeepTileKernel<4, dev::kTileWaves>);
+            } else {
+                wide ? launch(dev::EvalObliviousDeepTileKernel<8, dev::kWideTileWaves>)
+                     : launch(dev::EvalObliviousDeepTileKernel<8, dev::kTileWaves>);
+            }
+        } else if (m.MaxDepth <= 12) {
+            wide ? launchPairs(dev::EvalObliviousDeepTilePairsKernel<4, dev::kWideTileWaves>)
+                 : launchPairs(dev::EvalObliviousDeepTilePairsKernel<4, dev::kTileWaves>);
         } else {
-            wide ? launch(dev::EvalObliviousDeepTileKernel<8, dev::kWideTileWaves>)
-                 : launch(dev::EvalObliviousDeepTileKernel<8, dev::kTileWaves>);
+            wide ? launchPairs(dev::EvalObliviousDeepTilePairsKernel<8, dev::kWideTileWaves>)
+                 : launchPairs(dev::EvalObliviousDeepTilePairsKernel<8, dev::kTileWaves>);
         }
         HIP_CHECK(hipGetLastError());
         return;

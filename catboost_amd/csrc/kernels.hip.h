@@ -1223,12 +1223,19 @@ constexpr int kPairTreePadding = 2 * kTileWaves * kPairAhead;
 // bucket, bits 16.. what becomes of its bins: 0 as they are, 1 min(bin, 127), 2 max(bin - 127, 0)), byte-parallel.
 // A split "bin >= s" of such a bucket then reads the first row (s <= 127) or the second (with s - 127), and every
 // level of the model is a 7-bit compare.
-constexpr uint32_t kTileMapLow = 1, kTileMapHigh = 2;
+// A one-hot bucket of more than 127 values (bins 1 + index of the value) takes two rows as well: the bins up to 127
+// as they are and 0 for the others (kTileMapOneHotLow), and bin - 127 for the bins from 128 on, 0 for the others
+// (kTileMapHigh does exactly that); "bin == v" reads the first row for v <= 127 and the second, with v - 127,
+// otherwise: both are 7-bit equalities against a value that is not 0.
+constexpr uint32_t kTileMapLow = 1, kTileMapHigh = 2, kTileMapOneHotLow = 3;
 
 __device__ __forceinline__ uint32_t MapTileBins(uint32_t bins4, uint32_t mode) {
     const uint32_t high = bins4 & 0x80808080u;  // bytes above 127
     if (mode == kTileMapLow) {
         return (bins4 | (high - (high >> 7))) & 0x7f7f7f7fu;
+    }
+    if (mode == kTileMapOneHotLow) {
+        return bins4 & ~((high >> 7) * 0xffu);
     }
     if (mode == kTileMapHigh) {
         return ((bins4 & 0x7f7f7f7fu) + 0x01010101u) & ((high >> 7) * 0xffu);
@@ -1948,6 +1955,143 @@ __global__ __launch_bounds__(64 * WAVES) void EvalObliviousDeepTileKernel(
             const size_t doc = block * kDocsPerBlock + q * kWave + lane;
             if (doc < docCount) {
                 out[doc] = Finish(__dadd_rn(sRed[q * kWave + lane], acc[q]), scale, bias[0], treeBegin == 0);
+            }
+        }
+    }
+}
+
+// EvalObliviousDeepTileKernel for models of several dimensions: the same tile, rows and walk; a workgroup sums two
+// dimensions, those from blockIdx.y * 2 on (every slice of the dimensions walks the trees again). `leaves` holds the
+// values slice by slice, [slice][tree][leaf][2] (zeros past the last dimension), `firstLeaf` counts leaves and
+// `sliceLeaves` is the number of leaves of all trees, so that a leaf's two values come with one 16-byte load:
+// gathered as two strided doubles from the model's own table the kernel was no faster than the plain one (the
+// gathers' way through the texture path is what it waits for). A kernel of its own: as a template parameter of
+// the one-dimensional kernel the second dimension cost that kernel 5 %.
+// grid = (doc blocks, ceil(dim / 2)), block = 64 * WAVES, dynamic LDS = rows * 256 (rounded up to 16) + 2 * 256 * 8 bytes.
+template <int HIGH, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void EvalObliviousDeepTilePairsKernel(
+    const uint32_t* __restrict__ bins, size_t docCount, uint32_t bucketCount, const uint32_t* __restrict__ tileMap,
+    uint32_t rowCount, const uint4* __restrict__ deepRows, const uint32_t* __restrict__ firstLeaf,
+    const double* __restrict__ leaves, const double* __restrict__ bias, double scale, uint32_t dim, uint32_t sliceLeaves,
+    uint32_t treeBegin, uint32_t treeEnd, double* __restrict__ out) {
+    static_assert(HIGH == 4 || HIGH == 8, "levels 8..11 or 8..15 in the second half");
+    constexpr int DIMS = 2;
+    const uint32_t d0 = blockIdx.y * DIMS;
+    leaves += static_cast<size_t>(blockIdx.y) * sliceLeaves * 2;
+    extern __shared__ uint32_t sTile[];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const size_t block = blockIdx.x;
+    const uint32_t tileDwords = rowCount * kWave;  // rowCount = bucketCount without a map
+    const uint32_t* src = bins + block * (bucketCount * kWave);
+    if (tileMap == nullptr) {
+        for (uint32_t i = tid; i < tileDwords; i += 64 * WAVES) {
+            sTile[i] = src[i];
+        }
+    } else {
+        for (uint32_t row = wave; row < rowCount; row += WAVES) {
+            const uint32_t entry = tileMap[row];
+            sTile[row * kWave + lane] = MapTileBins(src[(entry & 0xffffu) * kWave + lane], entry >> 16);
+        }
+    }
+    const uint32_t tileBytes = (tileDwords * 4 + 15) & ~15u;
+    double* sRed = reinterpret_cast<double*>(reinterpret_cast<uint8_t*>(sTile) + tileBytes);  // [DIMS][256 documents]
+    const uint8_t* laneTile = reinterpret_cast<const uint8_t*>(sTile) + lane * 4;
+    const uint32_t treeCount = treeEnd - treeBegin;
+    __syncthreads();  // tile is loaded
+
+    double acc[4][DIMS], gathered[4][DIMS];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+#pragma unroll
+        for (int c = 0; c < DIMS; ++c) {
+            acc[q][c] = 0.0;
+            gathered[q][c] = 0.0;
+        }
+    }
+    uint4 rows[2][2][4];
+    uint32_t first[2];
+#define CBAMD_FETCH_DEEP2(k, tree)                                                                  \
+    do {                                                                                           \
+        const uint4* row = deepRows + static_cast<size_t>(tree) * 8;                               \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                            \
+            rows[k][0][i] = row[i];                                                                \
+            rows[k][1][i] = row[4 + i];                                                            \
+        }                                                                                          \
+        first[k] = firstLeaf[tree];                                                                \
+    } while (0)
+#define CBAMD_DEEP_ROUND2(k)                                                                        \
+    do {                                                                                           \
+        uint32_t low4, high4;                                                                      \
+        if (__builtin_amdgcn_readfirstlane(rows[k][0][0].x) & kPairRowXorFlag) {                   \
+            low4 = PairTreeIndexes<true, 8>(laneTile, rows[k][0]);                                 \
+            high4 = PairTreeIndexes<true, HIGH>(laneTile, rows[k][1]);                             \
+        } else {                                                                                   \
+            low4 = PairTreeIndexes<false, 8>(laneTile, rows[k][0]);                                \
+            high4 = PairTreeIndexes<false, HIGH>(laneTile, rows[k][1]);                            \
+        }                                                                                          \
+        const double* treeLeaves = leaves + static_cast<size_t>(__builtin_amdgcn_readfirstlane(first[k])) * DIMS; \
+        _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                            \
+            _Pragma("unroll") for (int c = 0; c < DIMS; ++c) {                                     \
+                acc[q][c] = __dadd_rn(acc[q][c], gathered[q][c]);                                  \
+            }                                                                                      \
+        }                                                                                          \
+        _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                            \
+            const uint32_t leaf = ((low4 >> (8 * q)) & 0xffu) |                                    \
+                                  (((high4 >> (8 * q + 8 - HIGH)) & ((1u << HIGH) - 1)) << 8);     \
+            const double2 pair = reinterpret_cast<const double2*>(treeLeaves)[leaf];               \
+            gathered[q][0] = pair.x;                                                               \
+            gathered[q][1] = pair.y;                                                               \
+        }                                                                                          \
+        CBAMD_FETCH_DEEP2(k, treeBegin + p + 2 * WAVES);                                            \
+        p += WAVES;                                                                                \
+    } while (0)
+
+    uint32_t p = wave;
+    CBAMD_FETCH_DEEP2(0, treeBegin + p);
+    CBAMD_FETCH_DEEP2(1, treeBegin + p + WAVES);
+    while (p + WAVES < treeCount) {
+        CBAMD_DEEP_ROUND2(0);
+        CBAMD_DEEP_ROUND2(1);
+    }
+    if (p < treeCount) {
+        CBAMD_DEEP_ROUND2(0);
+    }
+#undef CBAMD_DEEP_ROUND2
+#undef CBAMD_FETCH_DEEP2
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+#pragma unroll
+        for (int c = 0; c < DIMS; ++c) {
+            acc[q][c] = __dadd_rn(acc[q][c], gathered[q][c]);
+        }
+    }
+    // waves add their partial sums in wave order into the LDS accumulator; the last wave finishes the values
+    // and writes them out (byte q of a lane's dword: document q * 64 + lane)
+    for (uint32_t w = 0; w + 1 < WAVES; ++w) {
+        if (wave == w) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+#pragma unroll
+                for (int c = 0; c < DIMS; ++c) {
+                    double* cell = sRed + c * kDocsPerBlock + q * kWave + lane;
+                    *cell = (w == 0) ? acc[q][c] : __dadd_rn(*cell, acc[q][c]);
+                }
+            }
+        }
+        __syncthreads();
+    }
+    if (wave == WAVES - 1) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const size_t doc = block * kDocsPerBlock + q * kWave + lane;
+#pragma unroll
+            for (int c = 0; c < DIMS; ++c) {
+                if (doc < docCount && d0 + c < dim) {
+                    out[doc * dim + d0 + c] = Finish(__dadd_rn(sRed[c * kDocsPerBlock + q * kWave + lane], acc[q][c]), scale,
+                                                     bias[d0 + c], treeBegin == 0);
+                }
             }
         }
     }

@@ -79,6 +79,8 @@ def _features(cfg):
 
 
 def _cat_cardinalities(cfg, rng):
+    if "cat_cardinality" in cfg:   # every categorical feature with that many values (up to 254 fit a one-hot bucket)
+        return np.full(cfg.get("cats", 0), cfg["cat_cardinality"], dtype=np.int64)
     return rng.integers(2, 11, size=cfg.get("cats", 0))
 
 

@@ -231,3 +231,88 @@ def test_very_wide_models_against_the_oracle(monkeypatch, quad, seed, n_float, n
         np.testing.assert_allclose(g.calc_flat(x, tree_start=begin, tree_end=end),
                                    o.calc(x, tree_start=begin, tree_end=end), rtol=RTOL, atol=ATOL,
                                    err_msg="trees %d..%d" % (begin, end))
+
+
+@pytest.mark.parametrize("seed,dim,n_float,n_cat,trees,max_depth,docs", [
+    (61, 3, 40, 0, 60, 12, 1000),    # twelve levels, three dimensions: two slices of two
+    (62, 2, 30, 5, 25, 16, 513),     # sixteen levels, one-hot levels in either half, one slice
+    (63, 10, 300, 3, 30, 11, 255),   # five slices over a tile of 300 rows
+    (64, 5, 20, 4, 40, 9, 4097),     # depth 9 with one-hot splits and several dimensions
+])
+def test_deep_trees_of_several_dimensions_on_the_tile_kernel(seed, dim, n_float, n_cat, trees, max_depth, docs):
+    """Models of depth 9 to 16 with several dimensions: the deep-tile kernel sums two dimensions per walk of the
+    trees (the plain kernel took these before). Leaf indexes equal the oracle's, predictions within the tolerance."""
+    rng = np.random.default_rng(seed)
+    model, cat_values = _random_oblivious(rng, n_float=n_float, n_cat=n_cat, trees=trees, max_depth=max_depth, dim=dim,
+                                          scale=float(rng.choice([1.0, -0.5])), bias=rng.normal(size=dim))
+    x = _random_flat_data(rng, model, cat_values, docs)
+    o = OracleModel(model)
+    g = cb.ModelCalcer()
+    g.load_from_dict(model)
+    g.enable_gpu_evaluation(0)
+    kernels = g.evaluator().describe_kernels(cb.LAYOUT_FLAT_ROWS, docs)
+    assert kernels["evaluate"] == "EvalObliviousDeepTileKernel", kernels
+    np.testing.assert_array_equal(g.calc_leaf_indexes_flat(x), o.leaf_indexes(x))
+    np.testing.assert_allclose(g.calc_flat(x), o.calc(x), rtol=RTOL, atol=ATOL)
+    for begin, end in ((0, 1), (1, 2), (0, 17), (0, trees - 1), (1, trees), (3, 3), (trees // 2, trees)):
+        np.testing.assert_allclose(g.calc_flat(x, tree_start=begin, tree_end=end),
+                                   o.calc(x, tree_start=begin, tree_end=end), rtol=RTOL, atol=ATOL,
+                                   err_msg="trees %d..%d" % (begin, end))
+
+
+def _model_with_a_large_one_hot_bucket(rng, n_float, trees, max_depth, cardinality, dim=1):
+    """Oblivious model over n_float float features and one categorical feature of `cardinality` values, every one
+    of which some one-hot split tests: the feature's bucket then holds that many values (bins up to `cardinality`)."""
+    from oracle import model_builder as mb
+    from oracle.oracle import integer_cat_feature_hash
+
+    ffs = [mb.float_feature(i, i) for i in range(n_float)]
+    cfs = [mb.cat_feature(0, n_float)]
+    cands = {i: np.unique(rng.normal(size=int(rng.integers(1, 6))).astype(np.float32)) for i in range(n_float)}
+    values = [integer_cat_feature_hash(v) for v in range(cardinality)]
+    tree_list = []
+    for t in range(trees):
+        depth = int(rng.integers(1, max_depth + 1))
+        splits = []
+        for d in range(depth):
+            if rng.random() < 0.3:
+                splits.append(("onehot", 0, int(values[int(rng.integers(0, cardinality))])))
+            else:
+                f = int(rng.integers(0, n_float))
+                splits.append(("float", f, float(rng.choice(cands[f]))))
+        tree_list.append((splits, rng.normal(size=(1 << depth) * dim)))
+    for v in values:
+        tree_list.append(([("onehot", 0, int(v))], rng.normal(size=2 * dim)))
+    return mb.build_oblivious(ffs, cfs, dim, tree_list, scale=0.5, bias=rng.normal(size=dim)), {0: values}
+
+
+@pytest.mark.parametrize("seed,n_float,trees,max_depth,cardinality,dim,kernel", [
+    (71, 300, 200, 8, 200, 1, "EvalObliviousRowTileKernel"),    # values below and above 127 of one bucket
+    (72, 300, 700, 6, 254, 3, "EvalObliviousRowTileKernel"),    # the largest bucket a feature can have, three dimensions
+    (73, 900, 900, 8, 130, 1, "EvalObliviousPairTileKernel"),   # two trees per wave on half a tile
+    (74, 60, 40, 12, 180, 1, "EvalObliviousDeepTileKernel"),    # in either half of a deep tree's levels
+])
+def test_one_hot_bucket_of_more_than_127_values_on_the_tile_kernels(seed, n_float, trees, max_depth, cardinality, dim, kernel):
+    """A one-hot bucket of more than 127 values takes two rows of the tile (the bins up to 127, and bin - 127 from
+    128 on), so that "bin == value" stays a 7-bit compare: such models ran on the half-tile or the plain kernel
+    before. Bins and leaf indexes equal the oracle's, predictions within the tolerance."""
+    rng = np.random.default_rng(seed)
+    model, cat_values = _model_with_a_large_one_hot_bucket(rng, n_float, trees, max_depth, cardinality, dim)
+    docs = 3000
+    x = _random_flat_data(rng, model, cat_values, docs)
+    o = OracleModel(model)
+    g = cb.ModelCalcer()
+    g.load_from_dict(model)
+    g.enable_gpu_evaluation(0)
+    kernels = g.evaluator().describe_kernels(cb.LAYOUT_FLAT_ROWS, docs)
+    assert kernels["evaluate"] == kernel, kernels
+    bins = o.binarize(x)
+    assert bins.max() > 127
+    np.testing.assert_array_equal(g.quantize_flat(x), bins)
+    np.testing.assert_array_equal(g.calc_leaf_indexes_flat(x), o.leaf_indexes(x))
+    np.testing.assert_allclose(g.calc_flat(x), o.calc(x), rtol=RTOL, atol=ATOL)
+    total = len(model["tree_sizes"])
+    for begin, end in ((0, 1), (1, 2), (0, 17), (3, 3), (total // 2, total)):
+        np.testing.assert_allclose(g.calc_flat(x, tree_start=begin, tree_end=end),
+                                   o.calc(x, tree_start=begin, tree_end=end), rtol=RTOL, atol=ATOL,
+                                   err_msg="trees %d..%d" % (begin, end))
