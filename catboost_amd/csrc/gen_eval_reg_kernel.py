@@ -182,7 +182,10 @@ def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
         assert b0 == 28
     # second set of leaf values in flight (one-dimensional kernels that have the registers for it): above the
     # bins; the fused kernels take eight of the registers that only their binarize phase uses
-    two_sets = pitch == 1 and block % 2 == 0 and (fused or vgprs + 8 <= 256)
+    def waves_per_simd(registers):
+        return 512 // ((registers + 7) // 8 * 8)
+    # (not where the eight registers would cost a wave per SIMD: the 96-register shape runs four)
+    two_sets = pitch == 1 and block % 2 == 0 and (fused or (vgprs + 8 <= 256 and waves_per_simd(vgprs + 8) == waves_per_simd(vgprs)))
     if two_sets:
         if fused:
             lw0 = high + 8
