@@ -1687,6 +1687,11 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
                 entries.reserve(compactEntries.size());
                 values.reserve(valuesByEntry.size());
                 for (const TNsUnit& unit : bestUnits) {
+                    // a wave copies a unit sixteen bytes per lane: every unit starts at a multiple of four entries
+                    while (entries.size() % 4 != 0) {
+                        entries.push_back(255u);
+                        values.insert(values.end(), static_cast<size_t>(m.Dim), 0.0);
+                    }
                     const uint32_t first = static_cast<uint32_t>(entries.size());
                     uint32_t start[dev::kNsUnitTrees] = {};
                     uint32_t count = 0;
@@ -1709,9 +1714,14 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
                     units.insert(units.end(), row, row + 8);
                 }
                 m.NsUnitCount = static_cast<uint32_t>(bestUnits.size());
-                m.NsCompactEntries.Upload(entries);
-                m.NsCompactRows.Upload(units);
                 m.NsEntryCount = static_cast<uint32_t>(entries.size());
+                {
+                    // ... in whole regions, whatever the unit's size: spare entries behind the last unit
+                    std::vector<uint32_t> padded(entries);
+                    padded.resize(entries.size() + m.NsLdsShape.Entries, 255u);
+                    m.NsCompactEntries.Upload(padded);
+                }
+                m.NsCompactRows.Upload(units);
                 if (m.Dim > 1) {
                     // [slice of the dimensions][entry][dimension of the slice], zeros past the last dimension
                     const uint32_t dims = NsLdsDims(m.Dim), slices = (static_cast<uint32_t>(m.Dim) + dims - 1) / dims;

@@ -2373,8 +2373,8 @@ __global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
     const uint4* __restrict__ unitRows, uint32_t unitCount, const double* __restrict__ valuesByEntry,
     const double* __restrict__ bias, double scale, uint32_t dim, uint32_t entryCount, uint32_t treeBegin,
     uint32_t treeEnd, double* __restrict__ out) {
-    constexpr int kFetch = ENTRIES / kWave;
-    static_assert(ENTRIES <= kNsLdsEntries && ENTRIES % kWave == 0, "a region holds whole rounds of a wave's copy");
+    constexpr int kFetch = ENTRIES / (4 * kWave);  // rounds of a wave's copy, sixteen bytes per lane
+    static_assert(ENTRIES <= kNsLdsEntries && ENTRIES % (4 * kWave) == 0, "a region holds whole rounds of a wave's copy");
     extern __shared__ uint32_t sTile[];
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & (kWave - 1);
@@ -2391,16 +2391,26 @@ __global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
     const uint32_t bucketMask = 0x3ff00u;
     __syncthreads();  // tile is loaded
 
-    uint32_t fetched[kFetch];
-#define CBAMD_FETCH_UNIT(rowValue)                                                   \
-    do {                                                                             \
-        const uint32_t fFirst = __builtin_amdgcn_readfirstlane((rowValue).x);        \
-        const uint32_t fCount = __builtin_amdgcn_readfirstlane((rowValue).z);        \
-        _Pragma("unroll") for (int i = 0; i < kFetch; ++i) {                         \
-            if (static_cast<uint32_t>(i) * kWave < fCount) {                         \
-                fetched[i] = entries[fFirst + min(i * kWave + lane, fCount - 1)];    \
-            }                                                                        \
-        }                                                                            \
+    // A unit's entries come as whole rounds, whatever its size: a unit starts at a multiple of four entries and
+    // the table ends with ENTRIES spare ones, so the copy needs neither a bound nor a branch (entries past the
+    // unit's are never followed).
+    using TEntries4 = uint32_t __attribute__((ext_vector_type(4)));
+    TEntries4 fetched[kFetch];
+#define CBAMD_STORE_UNIT()                                                                                  \
+    do {                                                                                                    \
+        _Pragma("unroll") for (int i = 0; i < kFetch; ++i) {                                                \
+            reinterpret_cast<TEntries4*>(sEntries)[i * kWave + lane] = fetched[i];                          \
+        }                                                                                                   \
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                                              \
+        __builtin_amdgcn_wave_barrier();                                                                    \
+    } while (0)
+#define CBAMD_FETCH_UNIT(rowValue)                                                                          \
+    do {                                                                                                    \
+        const uint32_t fFirst = __builtin_amdgcn_readfirstlane((rowValue).x);                               \
+        const TEntries4* fSource = reinterpret_cast<const TEntries4*>(entries + fFirst) + lane;             \
+        _Pragma("unroll") for (int i = 0; i < kFetch; ++i) {                                                \
+            fetched[i] = fSource[i * kWave];                                                                \
+        }                                                                                                   \
     } while (0)
 
     double acc[4][DIMS];
@@ -2411,15 +2421,21 @@ __global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
             acc[j][k] = 0.0;
         }
     }
-    // one dimension: a unit's values are requested behind its walk and added after the next unit's
-    double pending[kNsUnitTrees][4];
+    // one dimension: a unit's values are requested behind its walk and added behind the next unit's. Two sets
+    // of them take turns (the loop below is written out for two units), so that the loads of one unit never
+    // wait for registers that the sums of the unit before still read.
+    double pending[2][kNsUnitTrees][4];
 #pragma unroll
-    for (int g = 0; g < kNsUnitTrees; ++g) {
+    for (int p = 0; p < 2; ++p) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            pending[g][j] = 0.0;
+        for (int g = 0; g < kNsUnitTrees; ++g) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                pending[p][g][j] = 0.0;
+            }
         }
     }
+    int lastSet = -1;  // the set whose values are not added yet
     const uint32_t d0 = blockIdx.y * DIMS;
     const double* sliceValues = valuesByEntry + static_cast<size_t>(blockIdx.y) * entryCount * DIMS;
     uint32_t u = wave;
@@ -2429,10 +2445,9 @@ __global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
         row2 = unitRows[2 * u + 1];
         CBAMD_FETCH_UNIT(row);
     }
-    while (u < unitCount) {
+    const auto walkUnit = [&](double (&mineSet)[kNsUnitTrees][4], const double (&otherSet)[kNsUnitTrees][4]) {
         const uint32_t first = __builtin_amdgcn_readfirstlane(row.x);
         const uint32_t height = __builtin_amdgcn_readfirstlane(row.y);
-        const uint32_t count = __builtin_amdgcn_readfirstlane(row.z);
         const uint32_t packed = __builtin_amdgcn_readfirstlane(row2.x);
         const uint32_t trees = packed >> 16;
         // trees the unit does not have walk its first tree again; their values are not added
@@ -2450,14 +2465,7 @@ __global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
         }
         if (anyWanted) {
             // the previous unit's reads were issued before these stores and LDS serves one wave in order
-#pragma unroll
-            for (int i = 0; i < kFetch; ++i) {
-                if (static_cast<uint32_t>(i) * kWave < count) {
-                    sEntries[i * kWave + lane] = fetched[i];
-                }
-            }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
+            CBAMD_STORE_UNIT();
         }
         const uint32_t uNext = u + WAVES;
         uint4 rowNext = make_uint4(0, 0, 0, 0), row2Next = make_uint4(0, 0, 0, 0);
@@ -2512,7 +2520,7 @@ __global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
             for (int g = 0; g < kNsUnitTrees; ++g) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    acc[j][0] = __dadd_rn(acc[j][0], pending[g][j]);
+                    acc[j][0] = __dadd_rn(acc[j][0], otherSet[g][j]);
                 }
             }
 #pragma unroll
@@ -2520,12 +2528,12 @@ __global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
                 if (wanted[g]) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        pending[g][j] = valuesByEntry[first + idx[g][j]];
+                        mineSet[g][j] = valuesByEntry[first + idx[g][j]];
                     }
                 } else {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        pending[g][j] = 0.0;
+                        mineSet[g][j] = 0.0;
                     }
                 }
             }
@@ -2553,14 +2561,29 @@ __global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
         u = uNext;
         row = rowNext;
         row2 = row2Next;
+    };
+    while (u < unitCount) {
+        walkUnit(pending[0], pending[1]);
+        lastSet = 0;
+        if (u >= unitCount) {
+            break;
+        }
+        walkUnit(pending[1], pending[0]);
+        lastSet = 1;
     }
 #undef CBAMD_FETCH_UNIT
+#undef CBAMD_STORE_UNIT
     if constexpr (DIMS == 1) {
 #pragma unroll
-        for (int g = 0; g < kNsUnitTrees; ++g) {
+        for (int p = 0; p < 2; ++p) {
+            if (lastSet == p) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                acc[j][0] = __dadd_rn(acc[j][0], pending[g][j]);
+                for (int g = 0; g < kNsUnitTrees; ++g) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        acc[j][0] = __dadd_rn(acc[j][0], pending[p][g][j]);
+                    }
+                }
             }
         }
     }
