@@ -2474,16 +2474,30 @@ __global__ __launch_bounds__(64 * WAVES) void EvalNonSymmetricLdsKernel(
             row2Next = unitRows[2 * uNext + 1];
             CBAMD_FETCH_UNIT(rowNext);
         }
+        // The first step starts at the root for all four documents of a lane: one read of the children, one of the
+        // four bins (a terminal root selects itself like any other terminal entry, so the step is safe for a tree
+        // of one leaf).
         uint32_t entry[kNsUnitTrees][4];
 #pragma unroll
         for (int g = 0; g < kNsUnitTrees; ++g) {
             const uint32_t rootEntry = anyWanted ? sEntries[start[g]] : 0u;
+            if (anyWanted && height > 0) {
+                const uint64_t pair = LdsLoad<uint64_t>(__builtin_amdgcn_alignbit(wave, rootEntry, 19));
+                uint32_t binAddr;
+                asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(binAddr) : "v"(rootEntry), "s"(bucketMask), "v"(laneOff));
+                const uint32_t bins4 = LdsLoad<uint32_t>(binAddr);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                entry[g][j] = rootEntry;
+                for (int j = 0; j < 4; ++j) {
+                    entry[g][j] = static_cast<uint32_t>(((bins4 >> (8 * j)) & 0xffu) >= (rootEntry & 0xffu) ? pair >> 32 : pair);
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    entry[g][j] = rootEntry;
+                }
             }
         }
-        for (uint32_t step = 0; step < (anyWanted ? height : 0u); ++step) {
+        for (uint32_t step = 1; step < (anyWanted ? height : 0u); ++step) {
             uint64_t pair[kNsUnitTrees][4];  // the two children of a chain's node, left in the low half
             uint32_t bin[kNsUnitTrees][4];
 #pragma unroll
