@@ -1040,7 +1040,7 @@ struct THipEvaluator::TImpl {
     TDeviceVec<uint32_t> PackedTrees;  // tile kernel: 16 dwords per oblivious tree of depth <= 8
     TDeviceVec<uint32_t> PackedMixed;  // half-tile kernel: packed rows in the form chosen per tree
     TDeviceVec<double> HalfTileLeaves; // half-tile kernel: 64 or 256 leaf values per tree at a fixed pitch
-    TDeviceVec<uint32_t> PairRows;     // pair-tile kernel: 16 dwords per tree, empty when the model does not qualify
+    TDeviceVec<uint32_t> PairRows;     // pair-tile kernel: 8 dwords per tree, empty when the model does not qualify
     TDeviceVec<uint32_t> QuadRows;     // quad-tile kernel: the same with 64 bytes per row of the tile
     TDeviceVec<uint32_t> TileRows;     // row-tile kernel (whole tile, one tree per wave): the same with 256 bytes per bucket
     TDeviceVec<double> TileLeaves;     // its leaf values: [slice of the dimensions][tree][pair of dimensions][leaf][2]
@@ -1541,6 +1541,27 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         return rows;
     };
 
+    // The pair-tile kernel's rows: 8 dwords per tree, a level's row offset (128-byte rows), xor byte (bits 0-6) and
+    // the byte added to the bins (bits 24-31) in one dword
+    const auto packedPairRows = [&]() {
+        constexpr uint32_t kDwords = 8;
+        std::vector<uint32_t> rows((trees.GetTreeCount() + dev::kQuadTreePadding) * kDwords, 0);
+        for (size_t t = 0; t < trees.GetTreeCount(); ++t) {
+            uint32_t* row = rows.data() + t * kDwords;
+            bool anyXor = false;
+            for (int d = 0; d < trees.TreeSizes[t]; ++d) {
+                const TTileLevel level = tileLevelOf(trees.RepackedBins[trees.TreeStartOffsets[t] + d]);
+                CBAMD_ENSURE(level.Row < 1024 && level.Xor < 128 && (level.Add & 0xffu) <= 128, "level does not fit the packed row");
+                row[d] = level.Row * 128u | level.Xor | (level.Add & 0xffu) << 24;
+                anyXor = anyXor || level.IsXor;
+            }
+            if (anyXor) {
+                row[0] |= dev::kPairRowXorFlag;
+            }
+        }
+        return rows;
+    };
+
     // 7-bit compares need every bin and split index to fit 7 bits and no xor mask
     m.PackedSevenBit = m.Oblivious && !m.HasOneHot && m.MaxBucketValues <= 127;
     if (m.Oblivious && m.MaxDepth <= 8) {
@@ -1633,7 +1654,11 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
                 // four trees per wave on a quarter of a block when the rows do not fit the half tile
                 const bool quadFits = !pairFits && QuadTileWaves(tileRowCount, maxd) != 0;
                 if (switches.PairTile && tileRowsUsable && (pairFits || quadFits)) {
-                    (pairFits ? m.PairRows : m.QuadRows).Upload(rowsInRegisters(pairFits ? 128 : 64));
+                    if (pairFits) {
+                        m.PairRows.Upload(packedPairRows());
+                    } else {
+                        m.QuadRows.Upload(rowsInRegisters(64));
+                    }
                     m.TileRowCount = tileRowsSplit ? tileRowCount : m.LayoutBuckets;  // (a model without splits: its one zero bucket)
                     if (tileRowsSplit) {
                         m.TileMap.Upload(tileMap);

@@ -1203,10 +1203,12 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousHalfTileKernel(
 // and one byte-parallel compare for 2 x 128 (tree, document) pairs instead of 128. Needs every bin of the
 // tile below 128 (the 7-bit compare; a one-hot level xors first: (bin ^ (~value & 0x7f)) + 1 carries into
 // bit 7 exactly when bin == value).
-// `pairRows` holds 16 dwords per tree: slot d = byte offset of level d's bucket in the tile (bucket * 128)
-// | xor byte << 24, slot 0 also bit 23 when some level of the tree xors; slot 8 + d = the value added to all
-// four bytes. Levels past the tree's depth are zero (bucket 0, add 0: never true). A lane keeps its tree's
-// row in registers (four 16-byte loads, the same addresses for the 32 lanes of a group) and the wave
+// `pairRows` holds 8 dwords per tree, one per level: byte offset of the level's bucket in the tile (bucket * 128,
+// bits 7-16) | xor byte (bits 0-6) | the value added to each of the four bins << 24, slot 0 also bit 23 when some
+// level of the tree xors (PackedPairTreeIndexes). Levels past the tree's depth are zero (bucket 0, add 0: never
+// true). A lane keeps its tree's row in registers (two 16-byte loads, the same addresses for the 32 lanes of a
+// group; with offsets and values to add as a dword each the row took four, and the kernel, which is bound by the
+// bytes its lanes receive over the vector memory path, 49 ms instead of 41 on 10M documents x 5000 trees) and the wave
 // publishes the two trees' leaf values, which are contiguous in `leaves` (1 << MAXD doubles per tree), in its
 // own LDS region. Waves take the pairs round robin; a last tree without a partner is done by wave 0 with both
 // groups on the same tree and only the first one adding. Partial sums (one per wave and group) are added in a
@@ -1241,6 +1243,37 @@ __device__ __forceinline__ uint32_t MapTileBins(uint32_t bins4, uint32_t mode) {
         return ((bins4 & 0x7f7f7f7fu) + 0x01010101u) & ((high >> 7) * 0xffu);
     }
     return bins4;
+}
+
+// The same walk on a tree's row in its packed form, one dword per level: bits 7-16 the byte offset of the level's
+// row in a tile of 128-byte rows, bits 0-6 the xor byte, bits 24-31 the value added to each of the four bins (bit
+// 23 of slot 0: some level of the tree xors). laneOffset is the lane's offset inside a row; the tile starts at LDS
+// address 0 (the kernel has no other LDS). A pair of trees then costs a lane two 16-byte loads instead of four:
+// the pair-tile kernel is bound by the bytes that the vector memory path delivers to its lanes.
+template <bool XOR, int MAXD>
+__device__ __forceinline__ uint32_t PackedPairTreeIndexes(uint32_t laneOffset, const uint4 (&desc)[2]) {
+    const uint32_t levels[8] = {desc[0].x, desc[0].y, desc[0].z, desc[0].w, desc[1].x, desc[1].y, desc[1].z, desc[1].w};
+    uint32_t a[MAXD];
+#pragma unroll
+    for (int d = 0; d < MAXD; ++d) {
+        a[d] = *reinterpret_cast<const __attribute__((address_space(3))) uint32_t*>((levels[d] & 0x1ff80u) | laneOffset);
+    }
+    // one wait for the eight reads (lgkmcnt 0, the other counters untouched)
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_sched_barrier(0);
+    uint32_t idx4 = 0;
+#pragma unroll
+    for (int d = 0; d < MAXD; ++d) {
+        uint32_t v = a[d];
+        if (XOR) {
+            const uint32_t x = levels[d] & 0x7fu;
+            v ^= __builtin_amdgcn_perm(x, x, 0u);  // the xor byte four times
+        }
+        const uint32_t adds = __builtin_amdgcn_perm(levels[d], levels[d], 0x03030303u);  // byte 3 four times
+        idx4 = ((v + adds) & 0x80808080u) | (idx4 >> 1);
+    }
+    return idx4;
 }
 
 template <bool XOR, int MAXD>
@@ -1280,6 +1313,10 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousPairTileKernel(
     constexpr uint32_t kLeaves = 1u << MAXD;
     constexpr int kLeafRegs = MAXD == 8 ? 4 : 1;  // 16-byte pieces of a pair's 2 * kLeaves leaf values per lane
     static_assert(MAXD == 8 || MAXD == 6, "64 or 256 leaves per tree");
+    // s_waitcnt that lets the loads of two pairs (two 16-byte pieces of a row and kLeafRegs of leaf values each)
+    // stay in flight: vmcnt in bits 0-3 and 14-15, the other counters untouched
+    constexpr int kLoadsBehind = 2 * (2 + kLeafRegs);
+    constexpr int kWaitForOldestPair = (kLoadsBehind & 0xf) | ((kLoadsBehind >> 4) << 14) | 0x0f70;
     extern __shared__ uint32_t sTile[];
     uint16_t* sTile16 = reinterpret_cast<uint16_t*>(sTile);
     const uint32_t tid = threadIdx.x;
@@ -1305,23 +1342,23 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousPairTileKernel(
     double* leafArea = reinterpret_cast<double*>(reinterpret_cast<uint8_t*>(sTile) + tileBytes);
     double2* sLeafWave2 = reinterpret_cast<double2*>(leafArea + wave * 2 * kLeaves);
     const double* sLeafMine = leafArea + wave * 2 * kLeaves + group * kLeaves;
-    const uint8_t* laneTile = reinterpret_cast<const uint8_t*>(sTile) + (lane & 31) * 4;
+    const uint32_t laneOffset = (lane & 31) * 4;
     __syncthreads();  // tile is loaded
 
     const uint32_t treeCount = treeEnd - treeBegin;
     const uint32_t pairCount = treeCount / 2;
     double acc[4] = {0.0, 0.0, 0.0, 0.0};
     constexpr int kAhead = kPairAhead;
-    uint4 rows[kAhead][4];
+    uint4 rows[kAhead][2];
     double2 pref[kAhead][kLeafRegs];
     // what a lane fetches of the pair that starts at tree `first`: its group's row and its pieces of the
     // two trees' leaf values
-    const uint4* myRows = pairRows + group * 4;
+    const uint4* myRows = pairRows + group * 2;
     const double2* myLeaves = leaves2 + lane;
 #define CBAMD_FETCH_PAIR(k, first)                                                                 \
     do {                                                                                           \
-        const uint4* row = myRows + static_cast<size_t>(first) * 4;                                \
-        _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                            \
+        const uint4* row = myRows + static_cast<size_t>(first) * 2;                                \
+        _Pragma("unroll") for (int i = 0; i < 2; ++i) {                                            \
             rows[k][i] = row[i];                                                                   \
         }                                                                                          \
         const double2* values = myLeaves + static_cast<size_t>(first) * (kLeaves / 2);             \
@@ -1341,9 +1378,9 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousPairTileKernel(
         const uint32_t flags =                                                                     \
             __builtin_amdgcn_readlane(rows[k][0].x, 0) | __builtin_amdgcn_readlane(rows[k][0].x, 32); \
         if (flags & kPairRowXorFlag) {                                                             \
-            idx4 = PairTreeIndexes<true, MAXD>(laneTile, rows[k]);                                 \
+            idx4 = PackedPairTreeIndexes<true, MAXD>(laneOffset, rows[k]);                         \
         } else {                                                                                   \
-            idx4 = PairTreeIndexes<false, MAXD>(laneTile, rows[k]);                                \
+            idx4 = PackedPairTreeIndexes<false, MAXD>(laneOffset, rows[k]);                        \
         }                                                                                          \
     } while (0)
 
@@ -1354,8 +1391,8 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousPairTileKernel(
 #define CBAMD_PAIR_ROUND(k)                                                                        \
     do {                                                                                           \
         uint32_t idx4;                                                                             \
-        /* one wait for this pair's eight loads: the sixteen of the two pairs behind it stay in flight */ \
-        __builtin_amdgcn_s_waitcnt(0x4f70);                                                        \
+        /* one wait for this pair's loads: those of the two pairs behind it stay in flight */     \
+        __builtin_amdgcn_s_waitcnt(kWaitForOldestPair);                                            \
         __builtin_amdgcn_sched_barrier(0);                                                         \
         CBAMD_PUBLISH_AND_WALK(k, idx4);                                                           \
         _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                            \
@@ -1401,9 +1438,9 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousPairTileKernel(
     }
     if ((treeCount & 1) && wave == 0) {
         // the last tree has no partner: both groups walk it (its row and its leaf values twice), the first adds
-        const uint4* row = pairRows + static_cast<size_t>(treeEnd - 1) * 4;
+        const uint4* row = pairRows + static_cast<size_t>(treeEnd - 1) * 2;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < 2; ++i) {
             rows[0][i] = row[i];
         }
         const double2* values = leaves2 + static_cast<size_t>(treeEnd - 1) * (kLeaves / 2);
@@ -2321,9 +2358,12 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalNonSymmetricTileKernel(
 // and the compare only selects: one LDS round trip per level. A terminal entry points at its own
 // pair and compares so that it selects itself (even index: splitIdx 255, false for every bin;
 // odd index: splitIdx 0, true for every bin, which no real split has). The next unit's entries
-// are fetched into registers while the current unit is walked. valuesByEntry holds the leaf
-// value of every terminal entry, indexed like `entries`; a unit's values are requested behind
-// its walk and added after the next unit's walk.
+// are fetched into registers while the current unit is walked: sixteen bytes per lane and whole rounds of
+// the wave, with neither bounds nor branches - every unit starts at a multiple of four entries and `entries`
+// ends with ENTRIES spare ones (a copy written with a test per round cost a taken branch each way per round,
+// a tenth of the kernel's time). valuesByEntry holds the leaf value of every terminal entry, indexed like
+// `entries`; a unit's values are requested behind its walk and added after the next unit's walk, two sets of
+// registers taking turns.
 // unitRows: 8 dwords per unit: first entry, height of the tallest tree, number of entries, first entry of the
 // second tree relative to the unit's, that of the third tree | number of trees << 16, and the model's numbers
 // of the three trees: a call for the trees [treeBegin, treeEnd) adds the values of those only and passes over
