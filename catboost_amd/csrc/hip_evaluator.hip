@@ -1041,6 +1041,7 @@ struct THipEvaluator::TImpl {
     TDeviceVec<uint32_t> PackedMixed;  // half-tile kernel: packed rows in the form chosen per tree
     TDeviceVec<double> HalfTileLeaves; // half-tile kernel: 64 or 256 leaf values per tree at a fixed pitch
     TDeviceVec<uint32_t> PairRows;     // pair-tile kernel: 8 dwords per tree, empty when the model does not qualify
+    bool PairSix = false;              // ... in the six-bit form (every bin below 64)
     TDeviceVec<uint32_t> QuadRows;     // quad-tile kernel: the same with 64 bytes per row of the tile
     TDeviceVec<uint32_t> TileRows;     // row-tile kernel (whole tile, one tree per wave): the same with 256 bytes per bucket
     TDeviceVec<double> TileLeaves;     // its leaf values: [slice of the dimensions][tree][pair of dimensions][leaf][2]
@@ -1543,7 +1544,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
 
     // The pair-tile kernel's rows: 8 dwords per tree, a level's row offset (128-byte rows), xor byte (bits 0-6) and
     // the byte added to the bins (bits 24-31) in one dword
-    const auto packedPairRows = [&]() {
+    const auto packedPairRows = [&](bool six) {
         constexpr uint32_t kDwords = 8;
         std::vector<uint32_t> rows((trees.GetTreeCount() + dev::kQuadTreePadding) * kDwords, 0);
         for (size_t t = 0; t < trees.GetTreeCount(); ++t) {
@@ -1552,7 +1553,17 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
             for (int d = 0; d < trees.TreeSizes[t]; ++d) {
                 const TTileLevel level = tileLevelOf(trees.RepackedBins[trees.TreeStartOffsets[t] + d]);
                 CBAMD_ENSURE(level.Row < 1024 && level.Xor < 128 && (level.Add & 0xffu) <= 128, "level does not fit the packed row");
-                row[d] = level.Row * 128u | level.Xor | (level.Add & 0xffu) << 24;
+                uint32_t xorByte = level.Xor, addByte = level.Add & 0xffu;
+                if (six && d % 2 == 0) {
+                    // the six-bit form of an even level: its result goes to bit 6 of the byte
+                    if (level.IsXor) {
+                        xorByte &= 0x3fu;
+                    } else {
+                        CBAMD_ENSURE(addByte > 64, "split index beyond the six-bit form");
+                        addByte -= 64;
+                    }
+                }
+                row[d] = level.Row * 128u | xorByte | addByte << 24;
                 anyXor = anyXor || level.IsXor;
             }
             if (anyXor) {
@@ -1655,7 +1666,9 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
                 const bool quadFits = !pairFits && QuadTileWaves(tileRowCount, maxd) != 0;
                 if (switches.PairTile && tileRowsUsable && (pairFits || quadFits)) {
                     if (pairFits) {
-                        m.PairRows.Upload(packedPairRows());
+                        // every bin below 64: the walk joins two levels at a time
+                        m.PairSix = m.MaxBucketValues <= 63 && !tileRowsSplit && switches.RegSix;
+                        m.PairRows.Upload(packedPairRows(m.PairSix));
                     } else {
                         m.QuadRows.Upload(rowsInRegisters(64));
                     }
@@ -2708,9 +2721,9 @@ void THipEvaluator::EvalQuantizedDevice(const uint8_t* bins, size_t docCount, si
                                    results);
             };
             if (maxd == 6) {
-                launch(dev::EvalObliviousPairTileKernel<6>);
+                m.PairSix ? launch(dev::EvalObliviousPairTileKernel<6, true>) : launch(dev::EvalObliviousPairTileKernel<6, false>);
             } else {
-                launch(dev::EvalObliviousPairTileKernel<8>);
+                m.PairSix ? launch(dev::EvalObliviousPairTileKernel<8, true>) : launch(dev::EvalObliviousPairTileKernel<8, false>);
             }
             HIP_CHECK(hipGetLastError());
             return;

@@ -1250,7 +1250,11 @@ __device__ __forceinline__ uint32_t MapTileBins(uint32_t bins4, uint32_t mode) {
 // 23 of slot 0: some level of the tree xors). laneOffset is the lane's offset inside a row; the tile starts at LDS
 // address 0 (the kernel has no other LDS). A pair of trees then costs a lane two 16-byte loads instead of four:
 // the pair-tile kernel is bound by the bytes that the vector memory path delivers to its lanes.
-template <bool XOR, int MAXD>
+// SIX: every bin of the tile is below 64. The even levels then carry the byte (64 - split), so that their result
+// lands in bit 6 while the following level's lands in bit 7, and a pair of levels joins the index with one shift
+// and two bit-field inserts: eighteen instructions for eight levels where the one-level-at-a-time form takes
+// twenty-four (a one-hot level on an even position xors with the low six bits of its mask).
+template <bool XOR, int MAXD, bool SIX>
 __device__ __forceinline__ uint32_t PackedPairTreeIndexes(uint32_t laneOffset, const uint4 (&desc)[2]) {
     const uint32_t levels[8] = {desc[0].x, desc[0].y, desc[0].z, desc[0].w, desc[1].x, desc[1].y, desc[1].z, desc[1].w};
     uint32_t a[MAXD];
@@ -1262,7 +1266,7 @@ __device__ __forceinline__ uint32_t PackedPairTreeIndexes(uint32_t laneOffset, c
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_waitcnt(0xc07f);
     __builtin_amdgcn_sched_barrier(0);
-    uint32_t idx4 = 0;
+    uint32_t r[MAXD];
 #pragma unroll
     for (int d = 0; d < MAXD; ++d) {
         uint32_t v = a[d];
@@ -1270,8 +1274,24 @@ __device__ __forceinline__ uint32_t PackedPairTreeIndexes(uint32_t laneOffset, c
             const uint32_t x = levels[d] & 0x7fu;
             v ^= __builtin_amdgcn_perm(x, x, 0u);  // the xor byte four times
         }
-        const uint32_t adds = __builtin_amdgcn_perm(levels[d], levels[d], 0x03030303u);  // byte 3 four times
-        idx4 = ((v + adds) & 0x80808080u) | (idx4 >> 1);
+        r[d] = v + __builtin_amdgcn_perm(levels[d], levels[d], 0x03030303u);  // byte 3 four times
+    }
+    uint32_t idx4 = 0;
+    if constexpr (SIX) {
+        static_assert(MAXD % 2 == 0, "levels in pairs");
+#pragma unroll
+        for (int d = 0; d < MAXD; d += 2) {
+            // bit 7 of the odd level, bit 6 of the even one; below them what is left of the even level's sum, which
+            // only the first pair lets through: those six bits leave the byte with the shifts that follow (MAXD 8)
+            // or end below the six bits that index the leaves (MAXD 6)
+            const uint32_t pair = (r[d + 1] & 0x80808080u) | (r[d] & 0x7f7f7f7fu);
+            idx4 = d == 0 ? pair : (pair & 0xc0c0c0c0u) | ((idx4 >> 2) & 0x3f3f3f3fu);
+        }
+    } else {
+#pragma unroll
+        for (int d = 0; d < MAXD; ++d) {
+            idx4 = (r[d] & 0x80808080u) | (idx4 >> 1);
+        }
     }
     return idx4;
 }
@@ -1305,7 +1325,7 @@ __device__ __forceinline__ uint32_t PairTreeIndexes(const uint8_t* laneTile, con
     return idx4;
 }
 
-template <int MAXD>
+template <int MAXD, bool SIX>
 __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousPairTileKernel(
     const uint16_t* __restrict__ bins, size_t docCount, uint32_t bucketCount, const uint32_t* __restrict__ tileMap,
     uint32_t rowCount, const uint4* __restrict__ pairRows, const double2* __restrict__ leaves2,
@@ -1378,9 +1398,9 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousPairTileKernel(
         const uint32_t flags =                                                                     \
             __builtin_amdgcn_readlane(rows[k][0].x, 0) | __builtin_amdgcn_readlane(rows[k][0].x, 32); \
         if (flags & kPairRowXorFlag) {                                                             \
-            idx4 = PackedPairTreeIndexes<true, MAXD>(laneOffset, rows[k]);                         \
+            idx4 = PackedPairTreeIndexes<true, MAXD, SIX>(laneOffset, rows[k]);                    \
         } else {                                                                                   \
-            idx4 = PackedPairTreeIndexes<false, MAXD>(laneOffset, rows[k]);                        \
+            idx4 = PackedPairTreeIndexes<false, MAXD, SIX>(laneOffset, rows[k]);                   \
         }                                                                                          \
     } while (0)
 
