@@ -43,7 +43,7 @@ def _check(tag, g, o, x):
 
 def _tree_model_case(seed, rng, asymmetric):
     dim = int(rng.choice([1, 1, 1, 2, 3, 5, 10, 20]))
-    n_float = int(rng.choice([1, 2, 7, 30, 100, 130, 200, 209, 224, 250, 400]))
+    n_float = int(rng.choice([1, 2, 7, 30, 100, 130, 200, 209, 224, 250, 400, 700, 1100]))
     n_cat = int(rng.choice([0, 0, 1, 2, 5]))
     trees = int(rng.choice([1, 2, 17, 40, 150, 400]))
     max_depth = int(rng.choice([1, 3, 6, 8, 10, 12]))
