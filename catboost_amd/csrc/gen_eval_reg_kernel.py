@@ -87,6 +87,7 @@ LDS_BUFFER_LIMIT = 32 * 1024
 # hip_evaluator.hip lists the same variants
 SHAPES = [
     (224, 4, 1, 256), (208, 4, 1, 256), (200, 4, 1, 256), (96, 8, 1, 256),
+    (96, 8, 1, 64),
     (192, 4, 2, 64), (160, 4, 4, 64), (128, 4, 6, 64),
     (192, 4, 2, 256), (160, 4, 4, 256), (128, 4, 6, 256),
 ]

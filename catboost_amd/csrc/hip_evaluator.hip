@@ -200,6 +200,7 @@ struct TEvalRegVariant {
 };
 constexpr TEvalRegVariant kEvalRegVariants[] = {
     {96, 8, 1, 256, false, false, "cbamd_eval_reg_b96_w8_p1_l256"},
+    {96, 8, 1, 64, false, false, "cbamd_eval_reg_b96_w8_p1_l64"},
     {200, 4, 1, 256, false, false, "cbamd_eval_reg_b200_w4_p1_l256"},
     {208, 4, 1, 256, false, false, "cbamd_eval_reg_b208_w4_p1_l256"},
     {224, 4, 1, 256, false, false, "cbamd_eval_reg_b224_w4_p1_l256"},
@@ -210,6 +211,7 @@ constexpr TEvalRegVariant kEvalRegVariants[] = {
     {160, 4, 4, 256, false, false, "cbamd_eval_reg_b160_w4_p4_l256"},
     {128, 4, 6, 256, false, false, "cbamd_eval_reg_b128_w4_p6_l256"},
     {96, 8, 1, 256, true, false, "cbamd_eval_reg_b96_w8_p1_l256_m"},
+    {96, 8, 1, 64, true, false, "cbamd_eval_reg_b96_w8_p1_l64_m"},
     {200, 4, 1, 256, true, false, "cbamd_eval_reg_b200_w4_p1_l256_m"},
     {208, 4, 1, 256, true, false, "cbamd_eval_reg_b208_w4_p1_l256_m"},
     {224, 4, 1, 256, true, false, "cbamd_eval_reg_b224_w4_p1_l256_m"},
@@ -220,6 +222,7 @@ constexpr TEvalRegVariant kEvalRegVariants[] = {
     {160, 4, 4, 256, true, false, "cbamd_eval_reg_b160_w4_p4_l256_m"},
     {128, 4, 6, 256, true, false, "cbamd_eval_reg_b128_w4_p6_l256_m"},
     {96, 8, 1, 256, false, true, "cbamd_eval_reg_b96_w8_p1_l256_s"},
+    {96, 8, 1, 64, false, true, "cbamd_eval_reg_b96_w8_p1_l64_s"},
     {200, 4, 1, 256, false, true, "cbamd_eval_reg_b200_w4_p1_l256_s"},
     {208, 4, 1, 256, false, true, "cbamd_eval_reg_b208_w4_p1_l256_s"},
     {224, 4, 1, 256, false, true, "cbamd_eval_reg_b224_w4_p1_l256_s"},
@@ -294,7 +297,10 @@ const TEvalRegVariant* PickRegVariant(uint32_t buckets, uint32_t dim, uint32_t m
             break;
         }
         for (const auto& v : kEvalRegVariants) {
-            const uint32_t leaves = maxDepth > 8 ? 1024u : dim > 1 && maxDepth <= 6 && !onePerLaunch ? 64u : 256u;
+            // trees of depth <= 6: 64 leaf rows and six levels. One-dimensional models only on the 96-register
+            // shape: wider ones keep the eight-level kernels, whose fused forms they can take
+            const bool shallow = maxDepth <= 6 && !onePerLaunch && (dim > 1 || (buckets <= 96 && minVariantBuckets <= 96));
+            const uint32_t leaves = maxDepth > 8 ? 1024u : shallow ? 64u : 256u;
             if (buckets > v.Buckets || v.Buckets < minVariantBuckets || (dim == 1 || onePerLaunch) != (v.Pitch == 1) ||
                 v.Leaves != leaves || v.Mixed != mixed || v.Six != six) {
                 continue;
