@@ -321,7 +321,7 @@ const TEvalRegVariant* PickRegVariant(uint32_t buckets, uint32_t dim, uint32_t m
 // tests use them to reach every kernel with one model.
 struct TKernelSwitches {
     bool RegKernel = true;        // CATBOOST_AMD_REG_KERNEL=0: no register-resident assembly kernels
-    bool RegSix = true;           // CATBOOST_AMD_REG_SIX=0: no six-bit form of those kernels
+    bool RegSix = true;           // CATBOOST_AMD_REG_SIX=0: no six-bit form of those kernels, nor of the pair-tile kernel
     bool CtrTile = true;          // CATBOOST_AMD_CTR_TILE=0: the plain CTR kernel instead of the tile kernel
     uint32_t RegMinBuckets = 0;   // CATBOOST_AMD_REG_MIN_BUCKETS=n: only register kernels that hold n buckets or more
     bool Fused = true;            // CATBOOST_AMD_FUSED=0: binarize and evaluate always as two launches

@@ -83,7 +83,7 @@ typedef struct CbHipFeatures {
  * CATBOOST_AMD_TEST_SWITCHES=1: without it none of the names below is looked at. They select between kernels
  * that return the same results and exist for tests and measurements.
  *   CATBOOST_AMD_REG_KERNEL=0        no register-resident assembly kernels (the LDS tile kernels instead)
- *   CATBOOST_AMD_REG_SIX=0           no six-bit form of the register-resident kernels
+ *   CATBOOST_AMD_REG_SIX=0           no six-bit form of the register-resident kernels and of the pair-tile kernel
  *   CATBOOST_AMD_REG_MIN_BUCKETS=n   only register-resident kernel shapes that hold n buckets or more
  *   CATBOOST_AMD_REG_SPLIT=0         a float feature with more than 127 used borders sends the model to the mixed
  *                                    (8-bit compare) kernels instead of taking two bins registers
