@@ -1213,7 +1213,9 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousHalfTileKernel(
 // own LDS region. Waves take the pairs round robin; a last tree without a partner is done by wave 0 with both
 // groups on the same tree and only the first one adding. Partial sums (one per wave and group) are added in a
 // fixed order at the end. The fetches run kPairAhead rounds ahead of the walk without looking at the tree range:
-// both tables end with kPairTreePadding trees' worth of zeros.
+// both tables end with kPairTreePadding trees' worth of zeros. The LDS reads of a pair's levels are issued a round
+// before the arithmetic on them, behind the previous pair's leaf values going into the region, so a round's
+// instructions never wait for reads of its own (a null tree's levels read row 0).
 // With `tileMap` the tile has rowCount rows (MapTileBins) and the offsets in pairRows name rows, not buckets.
 // grid = 2 * doc blocks, block = 64 * kTileWaves threads, dynamic LDS = rows * 128 (rounded up to 16) +
 // kTileWaves * 2 * max(1 << MAXD, 128) * 8 bytes (the leaf regions, later the partial sums).
@@ -1296,6 +1298,47 @@ __device__ __forceinline__ uint32_t PackedPairTreeIndexes(uint32_t laneOffset, c
     return idx4;
 }
 
+// The two halves of PackedPairTreeIndexes for a kernel that keeps the reads of a tree's levels one round ahead of
+// the arithmetic on them: the reads alone, and the walk on what they returned.
+template <int MAXD>
+__device__ __forceinline__ void ReadPackedPairLevels(uint32_t laneOffset, const uint4 (&desc)[2], uint32_t (&a)[MAXD]) {
+    const uint32_t levels[8] = {desc[0].x, desc[0].y, desc[0].z, desc[0].w, desc[1].x, desc[1].y, desc[1].z, desc[1].w};
+#pragma unroll
+    for (int d = 0; d < MAXD; ++d) {
+        a[d] = *reinterpret_cast<const __attribute__((address_space(3))) uint32_t*>((levels[d] & 0x1ff80u) | laneOffset);
+    }
+}
+
+template <bool XOR, int MAXD, bool SIX>
+__device__ __forceinline__ uint32_t WalkPackedPairLevels(const uint32_t (&a)[MAXD], const uint4 (&desc)[2]) {
+    const uint32_t levels[8] = {desc[0].x, desc[0].y, desc[0].z, desc[0].w, desc[1].x, desc[1].y, desc[1].z, desc[1].w};
+    uint32_t r[MAXD];
+#pragma unroll
+    for (int d = 0; d < MAXD; ++d) {
+        uint32_t v = a[d];
+        if (XOR) {
+            const uint32_t x = levels[d] & 0x7fu;
+            v ^= __builtin_amdgcn_perm(x, x, 0u);  // the xor byte four times
+        }
+        r[d] = v + __builtin_amdgcn_perm(levels[d], levels[d], 0x03030303u);  // byte 3 four times
+    }
+    uint32_t idx4 = 0;
+    if constexpr (SIX) {
+        static_assert(MAXD % 2 == 0, "levels in pairs");
+#pragma unroll
+        for (int d = 0; d < MAXD; d += 2) {
+            const uint32_t pair = (r[d + 1] & 0x80808080u) | (r[d] & 0x7f7f7f7fu);
+            idx4 = d == 0 ? pair : (pair & 0xc0c0c0c0u) | ((idx4 >> 2) & 0x3f3f3f3fu);
+        }
+    } else {
+#pragma unroll
+        for (int d = 0; d < MAXD; ++d) {
+            idx4 = (r[d] & 0x80808080u) | (idx4 >> 1);
+        }
+    }
+    return idx4;
+}
+
 template <bool XOR, int MAXD>
 __device__ __forceinline__ uint32_t PairTreeIndexes(const uint8_t* laneTile, const uint4 (&desc)[4]) {
     const uint32_t offs[8] = {desc[0].x, desc[0].y, desc[0].z, desc[0].w, desc[1].x, desc[1].y, desc[1].z, desc[1].w};
@@ -1335,8 +1378,13 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousPairTileKernel(
     static_assert(MAXD == 8 || MAXD == 6, "64 or 256 leaves per tree");
     // s_waitcnt that lets the loads of two pairs (two 16-byte pieces of a row and kLeafRegs of leaf values each)
     // stay in flight: vmcnt in bits 0-3 and 14-15, the other counters untouched
-    constexpr int kLoadsBehind = 2 * (2 + kLeafRegs);
+    // (of the pair behind the oldest, its row has to be there as well: its levels are read a round early)
+    constexpr int kLoadsBehind = kLeafRegs + (2 + kLeafRegs);
     constexpr int kWaitForOldestPair = (kLoadsBehind & 0xf) | ((kLoadsBehind >> 4) << 14) | 0x0f70;
+    // s_waitcnt for the level reads of this round: the previous round's gathers and this round's stores were issued
+    // behind them (LDS serves a wave's requests in order); vmcnt and expcnt untouched
+    constexpr int kWaitForLevelReads = 0xc07f | ((4 + kLeafRegs) << 8);
+    constexpr int kWaitForGathers = 0xc07f | ((kLeafRegs + MAXD) << 8);
     extern __shared__ uint32_t sTile[];
     uint16_t* sTile16 = reinterpret_cast<uint16_t*>(sTile);
     const uint32_t tid = threadIdx.x;
@@ -1381,10 +1429,13 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousPairTileKernel(
         _Pragma("unroll") for (int i = 0; i < 2; ++i) {                                            \
             rows[k][i] = row[i];                                                                   \
         }                                                                                          \
+        /* the row first: the round before the pair's own waits for it alone */                   \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
         const double2* values = myLeaves + static_cast<size_t>(first) * (kLeaves / 2);             \
         _Pragma("unroll") for (int i = 0; i < kLeafRegs; ++i) {                                    \
             pref[k][i] = values[i * kWave];                                                        \
         }                                                                                          \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
     } while (0)
     // the pair's leaf values into the wave's LDS region (the previous pair's gathers were issued before these
     // stores and LDS serves one wave's requests in order), then the levels: four leaf indexes per lane
@@ -1408,13 +1459,36 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousPairTileKernel(
     // reads are under way; the registers of this pair take the pair kAhead rounds ahead as soon as every level
     // has read them (the loads then land in those registers), and the gathers go out last.
     double gathered[4] = {0.0, 0.0, 0.0, 0.0};
+    uint32_t levelBins[kAhead][MAXD];  // what the reads of a pair's levels returned, issued a round before their use
 #define CBAMD_PAIR_ROUND(k)                                                                        \
     do {                                                                                           \
+        constexpr int kn = (k + 1) % kAhead;                                                       \
         uint32_t idx4;                                                                             \
-        /* one wait for this pair's loads: those of the two pairs behind it stay in flight */     \
+        /* one wait for this pair's loads and the next pair's row: the later loads stay in flight */ \
         __builtin_amdgcn_s_waitcnt(kWaitForOldestPair);                                            \
         __builtin_amdgcn_sched_barrier(0);                                                         \
-        CBAMD_PUBLISH_AND_WALK(k, idx4);                                                           \
+        _Pragma("unroll") for (int i = 0; i < kLeafRegs; ++i) {                                    \
+            sLeafWave2[i * kWave + lane] = pref[k][i];                                             \
+        }                                                                                          \
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                                     \
+        __builtin_amdgcn_wave_barrier();                                                           \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+        __builtin_amdgcn_s_waitcnt(kWaitForLevelReads);                                            \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+        /* the next pair's levels are read while this pair's are worked on */                     \
+        ReadPackedPairLevels<MAXD>(laneOffset, rows[kn], levelBins[kn]);                           \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+        const uint32_t flags =                                                                     \
+            __builtin_amdgcn_readlane(rows[k][0].x, 0) | __builtin_amdgcn_readlane(rows[k][0].x, 32); \
+        if (flags & kPairRowXorFlag) {                                                             \
+            idx4 = WalkPackedPairLevels<true, MAXD, SIX>(levelBins[k], rows[k]);                   \
+        } else {                                                                                   \
+            idx4 = WalkPackedPairLevels<false, MAXD, SIX>(levelBins[k], rows[k]);                  \
+        }                                                                                          \
+        /* the previous round's gathers: this round's stores and reads were issued behind them */ \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
+        __builtin_amdgcn_s_waitcnt(kWaitForGathers);                                               \
+        __builtin_amdgcn_sched_barrier(0);                                                         \
         _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                            \
             acc[q] = __dadd_rn(acc[q], gathered[q]);                                               \
         }                                                                                          \
@@ -1439,6 +1513,15 @@ __global__ __launch_bounds__(64 * kTileWaves) void EvalObliviousPairTileKernel(
         CBAMD_FETCH_PAIR(k, treeBegin + 2 * (p + k * kTileWaves));
     }
     static_assert(kAhead == 3, "the rounds below are written out for three register sets");
+#pragma unroll
+    for (int k = 1; k < kAhead; ++k) {
+#pragma unroll
+        for (int d = 0; d < MAXD; ++d) {
+            levelBins[k][d] = 0;
+        }
+    }
+    ReadPackedPairLevels<MAXD>(laneOffset, rows[0], levelBins[0]);  // the first pair's levels
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // (so that the rounds' waits need not cover this way into the loop)
     // whole turns of the three register sets without a branch between the rounds, so that the waits for
     // the loads count only the loads that are older than the one needed
     while (p + 2 * kTileWaves < pairCount) {
