@@ -249,6 +249,8 @@ struct TFusedVariant {
     const char* Name;
 };
 constexpr TFusedVariant kFusedVariants[] = {
+    {64, 8, false, "cbamd_fused_b64_w8"},
+    {64, 8, true, "cbamd_fused_b64_w8_s"},
     {208, 4, false, "cbamd_fused_b208_w4"},
     {208, 4, true, "cbamd_fused_b208_w4_s"},
 };
@@ -1999,10 +2001,22 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         // ---- fused kernels: float-only one-dimensional models in the 7-bit or six-bit form whose rows are
         // at least sixteen columns wide. The bins registers follow the columns of the rows (a unit = sixteen
         // consecutive columns = sixteen registers), so the level rows are rewritten per row layout.
-        // (models that fit the 96-register shape stay on two launches: their evaluate kernel runs at four waves per
-        // SIMD, a fused one at three, and is the faster - measured on 50 and 90 buckets)
-        const bool fusedCandidate = switches.Fused && !regMapped && !variant->Mixed && variant->Pitch == 1 && variant->Waves == 4 && variant->Leaves == 256 && m.Dim == 1 && !m.HasCats &&
-                                    m.CtrCount == 0 && m.BinarizeBuckets == BucketCount && BucketCount > 0;
+        // Models of the 96-register shape take the fused kernel of 64 bins registers when their units fit it (112
+        // registers: four waves per SIMD like their evaluate kernel); with more units they stay on two launches
+        // (a fused kernel of 96 bins registers would run at three waves per SIMD and is the slower - measured on
+        // 50 and 90 buckets). The fused kernels walk eight levels on 256 leaf rows per tree: a model on the
+        // six-level kernel gets a leaf table of that pitch for them (its level rows have the eight slots anyway).
+        const bool fusedCandidate = switches.Fused && !regMapped && !variant->Mixed && variant->Pitch == 1 && variant->Leaves <= 256 && m.Dim == 1 && !m.HasCats &&
+                                    m.CtrCount == 0 && m.BinarizeBuckets == BucketCount && BucketCount > 0 &&
+                                    (TreeCount / block + 3) * block * 256 * 8 + 16 * kFusedImageBytes < (uint64_t(1) << 32) - (1u << 20);
+        std::vector<double> fusedLeaves;  // 256 rows per tree
+        if (fusedCandidate && variant->Leaves == 64) {
+            fusedLeaves.assign(tableTrees * 256, 0.0);
+            for (size_t t = 0; t < TreeCount; ++t) {
+                std::copy(leaves.begin() + t * 64, leaves.begin() + (t + 1) * 64, fusedLeaves.begin() + t * 256);
+            }
+        }
+        const std::vector<double>& fusedLeafTable = variant->Leaves == 64 ? fusedLeaves : leaves;
         for (int layoutIndex = 0; layoutIndex < 2 && fusedCandidate; ++layoutIndex) {
             const std::vector<uint32_t>& columns = layoutIndex == 0 ? srcFlat : srcSplit;
             const size_t rowWidth = layoutIndex == 0 ? m.FlatVectorSize : m.MinFloatSize;
@@ -2034,7 +2048,9 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
             }
             const TFusedVariant* fused = nullptr;
             for (const auto& v : kFusedVariants) {
-                if (v.Six == variant->Six && unitStart.size() * kFusedUnitColumns <= v.Buckets && !fused) {
+                // (the wide fused shape is for the models of the wide evaluate kernels)
+                if (v.Six == variant->Six && unitStart.size() * kFusedUnitColumns <= v.Buckets && !fused &&
+                    (variant->Waves == 4 || v.Buckets == 64)) {
                     fused = &v;
                 }
             }
@@ -2079,7 +2095,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
             for (size_t u = 0; u < unitStart.size(); ++u) {
                 units[(static_cast<size_t>(maxUnits) + 1) * kFusedUnitDwords + u] = unitStart[u] * 4;
             }
-            std::vector<uint8_t> table(images * kFusedImageBytes + leaves.size() * sizeof(double), 0);
+            std::vector<uint8_t> table(images * kFusedImageBytes + fusedLeafTable.size() * sizeof(double), 0);
             for (uint32_t slot = 0; slot < fused->Buckets; ++slot) {
                 const uint32_t unit = slot / kFusedUnitColumns, column = slot % kFusedUnitColumns;
                 uint32_t* record = units.data() + static_cast<size_t>(unit) * kFusedUnitDwords;
@@ -2110,7 +2126,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
                     lut[c] = static_cast<uint8_t>(fused->Six ? start * 4 : start);  // the six-bit form stores byte offsets
                 }
             }
-            std::memcpy(table.data() + images * kFusedImageBytes, leaves.data(), leaves.size() * sizeof(double));
+            std::memcpy(table.data() + images * kFusedImageBytes, fusedLeafTable.data(), fusedLeafTable.size() * sizeof(double));
             // level rows of the same form as the register kernel's, naming bins registers of this layout
             std::vector<uint32_t> fusedRows(rows);
             for (size_t t = 0; t < TreeCount; ++t) {

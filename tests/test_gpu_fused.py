@@ -1,9 +1,10 @@
 """The fused kernels (binarize + evaluate in one launch, the bins in registers only) against the two-launch
 path and the oracle. Needs an MI355X.
 
-CbHipEvalData and the host entry points take the fused kernel for float-only one-dimensional oblivious
-models of more than 96 buckets whose rows are at least sixteen columns wide; CATBOOST_AMD_FUSED=0 keeps an evaluator on the two
-launches. Both add the leaves in tree order in fp64: results must be equal bit for bit, and within
+CbHipEvalData and the host entry points take a fused kernel for float-only one-dimensional oblivious
+models whose rows are at least sixteen columns wide and whose used columns make at most four units of sixteen
+(the kernel of 64 bins registers) or which have more than 96 buckets (the kernel of 208); CATBOOST_AMD_FUSED=0
+keeps an evaluator on the two launches. Both add the leaves in tree order in fp64: results must be equal bit for bit, and within
 1e-9 relative / 1e-12 absolute of the oracle.
 """
 import numpy as np
@@ -56,7 +57,8 @@ def _compare(model_bytes, x, monkeypatch, stride=None):
 
 
 @pytest.mark.parametrize("cfg,trees,docs", [("C2", 50, 1), ("C2", 50, 255), ("C2", 50, 257), ("C2", 64, 5000),
-                                             ("C2", 1000, 20000), ("C2", 200, 30011)])
+                                             ("C2", 1000, 20000), ("C2", 200, 30011),
+                                             ("C1", 200, 5000), ("C1", 37, 1), ("C1", 37, 2049)])
 def test_fused_equals_two_launches(cfg, trees, docs, monkeypatch):
     model, info = syn.build_model(cfg, trees=trees)
     x = syn.host_features(info, docs, seed=3)
@@ -129,6 +131,34 @@ def test_fused_shallow_trees_and_mixed_depths(monkeypatch):
     model = mb.build_oblivious(feats, [], 1, trees)
     x = rng.normal(size=(3001, columns)).astype(np.float32)
     _compare(_bytes(model), x, monkeypatch)
+
+
+@pytest.mark.parametrize("columns,used_count,depth,max_borders", [(16, 16, 8, 120), (23, 9, 8, 40), (64, 64, 6, 30),
+                                                                  (50, 50, 8, 126), (300, 40, 7, 60), (61, 33, 3, 5)])
+def test_fused_small_models(columns, used_count, depth, max_borders, monkeypatch):
+    """Models of at most four units: the fused kernel of 64 bins registers, in its seven-bit form (a feature
+    with more than 63 borders) and its six-bit form, behind the six-level and the eight-level evaluate kernels'
+    tables, with used columns far apart (300 columns, 40 of them used in three clusters) and a last unit that is
+    moved back into the row."""
+    rng = np.random.default_rng(columns * 1000 + used_count)
+    if columns == 300:
+        used = sorted(set(range(3, 17)) | set(range(140, 153)) | set(range(287, 300)))
+    else:
+        used = sorted(rng.choice(columns, size=used_count, replace=False).tolist())
+    model = _random_model(rng, columns, used, trees=150, depth=depth,
+                          borders_of=lambda f: rng.normal(0, 1, size=rng.integers(1, max_borders + 1)),
+                          nan_true=set(used[::3]))
+    x = rng.normal(0, 1.5, size=(4099, columns)).astype(np.float32)
+    for f in used:
+        b = np.asarray(model["float_features"][f]["borders"], np.float32)
+        rows = rng.integers(0, x.shape[0], size=100)
+        x[rows, f] = rng.choice(b, size=100)
+    x[rng.random(x.shape) < 0.03] = np.nan
+    x[rng.random(x.shape) < 0.01] = np.inf
+    (fm, fev), _ = _evaluators(_bytes(model), monkeypatch)
+    assert fev.describe_kernels(cb.LAYOUT_FLAT_ROWS, x.shape[0]).get("fused", "").startswith("cbamd_fused_b64_w8")
+    _compare(_bytes(model), x, monkeypatch)
+    _compare(_bytes(model), x[:300], monkeypatch, stride=columns + 3)
 
 
 def test_fused_split_rows_layout(monkeypatch):
