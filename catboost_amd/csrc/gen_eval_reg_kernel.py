@@ -96,10 +96,10 @@ DEEP_SHAPES = [(208, 4, 1, 1024), (96, 8, 1, 1024)]
 VARIANTS = [shape + (mixed, six) for mixed, six in ((False, False), (False, True), (True, False)) for shape in SHAPES]
 VARIANTS += [shape + (False, six) for six in (False, True) for shape in DEEP_SHAPES]
 # shapes of the fused kernels (one dimension, 256 leaf rows), each in a plain and a six-bit form. The wide shape,
-# and one of 64 bins registers that still runs four waves per SIMD (112 registers); a model of 65 to 96 buckets
-# runs its separate evaluate kernel at four waves per SIMD, which a fused kernel of 96 bins registers (144: three)
-# does not match: measured, two launches are the faster there.
-FUSED_SHAPES = [(208, 4), (64, 8)]
+# and two of 64 and 80 bins registers that still run four waves per SIMD (112 and 128 registers); a model of more
+# units, up to 96 buckets, runs its separate evaluate kernel at four waves per SIMD, which a fused kernel of 96
+# bins registers (144: three) does not match: measured, two launches are the faster there.
+FUSED_SHAPES = [(208, 4), (64, 8), (80, 8)]
 FUSED_MAX_STEPS = 4
 FUSED_EXTRA_SETS = 1
 FUSED_UNIT_DWORDS = 40

@@ -3,7 +3,7 @@ path and the oracle. Needs an MI355X.
 
 CbHipEvalData and the host entry points take a fused kernel for float-only one-dimensional oblivious
 models whose rows are at least sixteen columns wide and whose used columns make at most four units of sixteen
-(the kernel of 64 bins registers) or which have more than 96 buckets (the kernel of 208); CATBOOST_AMD_FUSED=0
+or five (the kernels of 64 and 80 bins registers) or which have more than 96 buckets (the kernel of 208); CATBOOST_AMD_FUSED=0
 keeps an evaluator on the two launches. Both add the leaves in tree order in fp64: results must be equal bit for bit, and within
 1e-9 relative / 1e-12 absolute of the oracle.
 """
@@ -133,13 +133,15 @@ def test_fused_shallow_trees_and_mixed_depths(monkeypatch):
     _compare(_bytes(model), x, monkeypatch)
 
 
-@pytest.mark.parametrize("columns,used_count,depth,max_borders", [(16, 16, 8, 120), (23, 9, 8, 40), (64, 64, 6, 30),
-                                                                  (50, 50, 8, 126), (300, 40, 7, 60), (61, 33, 3, 5)])
-def test_fused_small_models(columns, used_count, depth, max_borders, monkeypatch):
-    """Models of at most four units: the fused kernel of 64 bins registers, in its seven-bit form (a feature
-    with more than 63 borders) and its six-bit form, behind the six-level and the eight-level evaluate kernels'
-    tables, with used columns far apart (300 columns, 40 of them used in three clusters) and a last unit that is
-    moved back into the row."""
+@pytest.mark.parametrize("columns,used_count,depth,max_borders,shape",
+                         [(16, 16, 8, 120, 64), (23, 9, 8, 40, 64), (64, 64, 6, 30, 64), (50, 50, 8, 126, 64),
+                          (300, 40, 7, 60, 64), (61, 33, 3, 5, 64), (80, 80, 8, 100, 80), (70, 70, 6, 30, 80),
+                          (77, 60, 5, 126, 80)])
+def test_fused_small_models(columns, used_count, depth, max_borders, shape, monkeypatch):
+    """Models of at most four or five units: the fused kernels of 64 and 80 bins registers, in their seven-bit
+    form (a feature with more than 63 borders) and their six-bit form, behind the six-level and the eight-level
+    evaluate kernels' tables, with used columns far apart (300 columns, 40 of them used in three clusters) and a
+    last unit that is moved back into the row."""
     rng = np.random.default_rng(columns * 1000 + used_count)
     if columns == 300:
         used = sorted(set(range(3, 17)) | set(range(140, 153)) | set(range(287, 300)))
@@ -156,7 +158,7 @@ def test_fused_small_models(columns, used_count, depth, max_borders, monkeypatch
     x[rng.random(x.shape) < 0.03] = np.nan
     x[rng.random(x.shape) < 0.01] = np.inf
     (fm, fev), _ = _evaluators(_bytes(model), monkeypatch)
-    assert fev.describe_kernels(cb.LAYOUT_FLAT_ROWS, x.shape[0]).get("fused", "").startswith("cbamd_fused_b64_w8")
+    assert fev.describe_kernels(cb.LAYOUT_FLAT_ROWS, x.shape[0]).get("fused", "").startswith("cbamd_fused_b%d_w8" % shape)
     _compare(_bytes(model), x, monkeypatch)
     _compare(_bytes(model), x[:300], monkeypatch, stride=columns + 3)
 
