@@ -100,6 +100,9 @@ VARIANTS += [shape + (False, six) for six in (False, True) for shape in DEEP_SHA
 # units, up to 96 buckets, runs its separate evaluate kernel at four waves per SIMD, which a fused kernel of 96
 # bins registers (144: three) does not match: measured, two launches are the faster there.
 FUSED_SHAPES = [(208, 4), (64, 8), (80, 8)]
+# The two small shapes also in a form that walks six levels ("_d6": models of depth <= 6; the leaf tables keep the
+# 256 rows per tree that the border images' buffers are sized for, the index reaches the first 64 of them).
+FUSED_SIX_LEVEL_BUCKETS = 96
 FUSED_MAX_STEPS = 4
 FUSED_EXTRA_SETS = 1
 FUSED_UNIT_DWORDS = 40
@@ -118,9 +121,9 @@ def fused_chunks(buckets, six):
     return chunks + chunks % 2
 
 
-def kernel_name(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
+def kernel_name(buckets, waves, pitch, leaves, mixed, six=False, fused=False, levels=None):
     if fused:
-        return "cbamd_fused_b%d_w%d%s" % (buckets, waves, "_s" if six else "")
+        return "cbamd_fused_b%d_w%d%s%s" % (buckets, waves, "_d6" if levels == 6 else "", "_s" if six else "")
     return "cbamd_eval_reg_b%d_w%d_p%d_l%d%s" % (buckets, waves, pitch, leaves, "_m" if mixed else "_s" if six else "")
 
 
@@ -132,11 +135,12 @@ def tree_block(pitch, leaves):
     return block
 
 
-def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False):
+def gen_kernel(buckets, waves, pitch, leaves, mixed, six=False, fused=False, levels=None):
     assert not (mixed and six)
     assert not fused or (pitch == 1 and leaves == 256 and not mixed and buckets % 16 == 0)
-    name = kernel_name(buckets, waves, pitch, leaves, mixed, six, fused)
-    depth = {64: 6, 256: 8, 1024: 10}[leaves]
+    assert levels is None or (fused and levels == 6)
+    name = kernel_name(buckets, waves, pitch, leaves, mixed, six, fused, levels)
+    depth = levels or {64: 6, 256: 8, 1024: 10}[leaves]
     deep = depth > 8                      # levels 8 and 9 go into a second index word
     assert not deep or (pitch == 1 and not mixed and not fused)
     row_dwords = 32 if mixed or deep else 16      # level table of a tree
@@ -906,9 +910,10 @@ def generate():
         metas.append(meta)
     for buckets, waves in FUSED_SHAPES:
         for six in (False, True):
-            text, meta = gen_kernel(buckets, waves, 1, 256, False, six, fused=True)
-            parts.append(text)
-            metas.append(meta)
+            for levels in (None, 6) if buckets <= FUSED_SIX_LEVEL_BUCKETS else (None,):
+                text, meta = gen_kernel(buckets, waves, 1, 256, False, six, fused=True, levels=levels)
+                parts.append(text)
+                metas.append(meta)
     parts.append(".amdgpu_metadata")
     parts.append("---")
     parts.append("amdhsa.kernels:")

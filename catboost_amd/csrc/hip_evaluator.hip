@@ -241,20 +241,26 @@ constexpr TEvalRegVariant kEvalRegVariants[] = {
 constexpr int kRegMaxDepth = 10;  // deepest tree of the register kernels (one-dimensional models; 8 otherwise)
 
 // Fused kernels (binarize + evaluate in one launch, bins only ever in registers): shapes of
-// gen_eval_reg_kernel.py's FUSED_SHAPES, each in a plain and a six-bit form.
+// gen_eval_reg_kernel.py's FUSED_SHAPES, each in a plain and a six-bit form; the small shapes also in a form that
+// walks six levels instead of eight (models of depth <= 6), listed before the eight-level form of their shape.
 struct TFusedVariant {
     uint32_t Buckets;  // bins registers = 16 per unit of sixteen columns
     uint32_t Waves;
     bool Six;
+    uint32_t Levels;
     const char* Name;
 };
 constexpr TFusedVariant kFusedVariants[] = {
-    {64, 8, false, "cbamd_fused_b64_w8"},
-    {64, 8, true, "cbamd_fused_b64_w8_s"},
-    {80, 8, false, "cbamd_fused_b80_w8"},
-    {80, 8, true, "cbamd_fused_b80_w8_s"},
-    {208, 4, false, "cbamd_fused_b208_w4"},
-    {208, 4, true, "cbamd_fused_b208_w4_s"},
+    {64, 8, false, 6, "cbamd_fused_b64_w8_d6"},
+    {64, 8, true, 6, "cbamd_fused_b64_w8_d6_s"},
+    {64, 8, false, 8, "cbamd_fused_b64_w8"},
+    {64, 8, true, 8, "cbamd_fused_b64_w8_s"},
+    {80, 8, false, 6, "cbamd_fused_b80_w8_d6"},
+    {80, 8, true, 6, "cbamd_fused_b80_w8_d6_s"},
+    {80, 8, false, 8, "cbamd_fused_b80_w8"},
+    {80, 8, true, 8, "cbamd_fused_b80_w8_s"},
+    {208, 4, false, 8, "cbamd_fused_b208_w4"},
+    {208, 4, true, 8, "cbamd_fused_b208_w4_s"},
 };
 constexpr uint32_t kFusedUnitColumns = 16;
 constexpr uint32_t kFusedUnitDwords = 40;   // sixteen lo, sixteen scale, flags, padding
@@ -2006,15 +2012,12 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
         // Models of the 96-register shape take the fused kernel of 64 or 80 bins registers when their units fit it (112
         // and 128 registers: four waves per SIMD like their evaluate kernel); with more units they stay on two launches
         // (a fused kernel of 96 bins registers would run at three waves per SIMD and is the slower - measured on
-        // 50 and 90 buckets). The fused kernels walk eight levels on 256 leaf rows per tree: a model on the
-        // six-level kernel gets a leaf table of that pitch for them (its level rows have the eight slots anyway) - as
-        // long as it has few trees per feature: the two levels and the larger tables cost the fused launch
-        // 0.04 ms per 1000 trees and million documents against the six-level kernel, the bins' round trip that it
-        // saves 0.0006 ms per feature and million documents (4M documents x 1000 trees of depth 6 over 70 features:
-        // 1.19 ms fused against 1.15; C1, 200 trees over 50 features: 0.109 against 0.127).
+        // 50 and 90 buckets). The fused kernels copy 256 leaf rows per tree: a model on the six-level kernel gets
+        // a leaf table of that pitch for them (its level rows have the eight slots anyway) and the form of the
+        // fused kernel that walks six levels (4M documents x 1000 trees of depth 6 over 70 features: 1.06 ms
+        // against 1.15 on two launches; with the eight-level walk 1.19).
         const bool fusedCandidate = switches.Fused && !regMapped && !variant->Mixed && variant->Pitch == 1 && variant->Leaves <= 256 && m.Dim == 1 && !m.HasCats &&
                                     m.CtrCount == 0 && m.BinarizeBuckets == BucketCount && BucketCount > 0 &&
-                                    (variant->Leaves == 256 || TreeCount <= 8 * BucketCount) &&
                                     (TreeCount / block + 3) * block * 256 * 8 + 16 * kFusedImageBytes < (uint64_t(1) << 32) - (1u << 20);
         std::vector<double> fusedLeaves;  // 256 rows per tree
         if (fusedCandidate && variant->Leaves == 64) {
@@ -2057,7 +2060,7 @@ THipEvaluator::THipEvaluator(const TModelTrees& trees, int deviceId, const std::
             for (const auto& v : kFusedVariants) {
                 // (the wide fused shape is for the models of the wide evaluate kernels)
                 if (v.Six == variant->Six && unitStart.size() * kFusedUnitColumns <= v.Buckets && !fused &&
-                    (variant->Waves == 4 || v.Buckets <= 80)) {
+                    (variant->Waves == 4 || v.Buckets <= 80) && m.MaxDepth <= v.Levels) {
                     fused = &v;
                 }
             }

@@ -140,7 +140,7 @@ def test_fused_shallow_trees_and_mixed_depths(monkeypatch):
 def test_fused_small_models(columns, used_count, depth, max_borders, shape, monkeypatch):
     """Models of at most four or five units: the fused kernels of 64 and 80 bins registers, in their seven-bit
     form (a feature with more than 63 borders) and their six-bit form, behind the six-level and the eight-level
-    evaluate kernels' tables, with used columns far apart (300 columns, 40 of them used in three clusters) and a
+    evaluate kernels' tables (the fused kernel then walks six or eight levels), with used columns far apart (300 columns, 40 of them used in three clusters) and a
     last unit that is moved back into the row."""
     rng = np.random.default_rng(columns * 1000 + used_count)
     if columns == 300:
@@ -158,7 +158,9 @@ def test_fused_small_models(columns, used_count, depth, max_borders, shape, monk
     x[rng.random(x.shape) < 0.03] = np.nan
     x[rng.random(x.shape) < 0.01] = np.inf
     (fm, fev), _ = _evaluators(_bytes(model), monkeypatch)
-    assert fev.describe_kernels(cb.LAYOUT_FLAT_ROWS, x.shape[0]).get("fused", "").startswith("cbamd_fused_b%d_w8" % shape)
+    name = fev.describe_kernels(cb.LAYOUT_FLAT_ROWS, x.shape[0]).get("fused", "")
+    assert name.startswith("cbamd_fused_b%d_w8" % shape)
+    assert ("_d6" in name) == (depth <= 6), "models of depth <= 6 take the form that walks six levels"
     _compare(_bytes(model), x, monkeypatch)
     _compare(_bytes(model), x[:300], monkeypatch, stride=columns + 3)
 

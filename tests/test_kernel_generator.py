@@ -55,11 +55,13 @@ def _copies(lines, wave, lane, wave_bytes):
 def test_staging_copies_stay_inside_the_tables(fused):
     gen = _generator()
     if fused:
-        cases = [(buckets, waves, 1, 256, False, six, True) for buckets, waves in gen.FUSED_SHAPES for six in (False, True)]
+        cases = [(buckets, waves, 1, 256, False, six, True, levels) for buckets, waves in gen.FUSED_SHAPES
+                 for six in (False, True)
+                 for levels in ((None, 6) if buckets <= gen.FUSED_SIX_LEVEL_BUCKETS else (None,))]
     else:
-        cases = [variant + (False,) for variant in gen.VARIANTS]
-    for buckets, waves, pitch, leaves, mixed, six, is_fused in cases:
-        text, _ = gen.gen_kernel(buckets, waves, pitch, leaves, mixed, six, fused=is_fused)
+        cases = [variant + (False, None) for variant in gen.VARIANTS]
+    for buckets, waves, pitch, leaves, mixed, six, is_fused, levels in cases:
+        text, _ = gen.gen_kernel(buckets, waves, pitch, leaves, mixed, six, fused=is_fused, levels=levels)
         lines = text.split("\n")
         block = gen.tree_block(pitch, leaves)
         buf_bytes = block * leaves * pitch * 8
