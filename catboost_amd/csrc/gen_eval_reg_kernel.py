@@ -100,9 +100,9 @@ VARIANTS += [shape + (False, six) for six in (False, True) for shape in DEEP_SHA
 # units, up to 96 buckets, runs its separate evaluate kernel at four waves per SIMD, which a fused kernel of 96
 # bins registers (144: three) does not match: measured, two launches are the faster there.
 FUSED_SHAPES = [(208, 4), (64, 8), (80, 8)]
-# The two small shapes also in a form that walks six levels ("_d6": models of depth <= 6; the leaf tables keep the
-# 256 rows per tree that the border images' buffers are sized for, the index reaches the first 64 of them).
-FUSED_SIX_LEVEL_BUCKETS = 96
+# Every shape also in a form that walks six levels ("_d6": models of depth <= 6; the leaf tables keep the 256 rows
+# per tree that the border images' buffers are sized for, the index reaches the first 64 of them).
+FUSED_SIX_LEVEL_BUCKETS = 208
 FUSED_MAX_STEPS = 4
 FUSED_EXTRA_SETS = 1
 FUSED_UNIT_DWORDS = 40

@@ -241,8 +241,8 @@ constexpr TEvalRegVariant kEvalRegVariants[] = {
 constexpr int kRegMaxDepth = 10;  // deepest tree of the register kernels (one-dimensional models; 8 otherwise)
 
 // Fused kernels (binarize + evaluate in one launch, bins only ever in registers): shapes of
-// gen_eval_reg_kernel.py's FUSED_SHAPES, each in a plain and a six-bit form; the small shapes also in a form that
-// walks six levels instead of eight (models of depth <= 6), listed before the eight-level form of their shape.
+// gen_eval_reg_kernel.py's FUSED_SHAPES, each in a plain and a six-bit form, and each of these in a form that
+// walks six levels instead of eight (models of depth <= 6), listed before the eight-level form of its shape.
 struct TFusedVariant {
     uint32_t Buckets;  // bins registers = 16 per unit of sixteen columns
     uint32_t Waves;
@@ -259,6 +259,8 @@ constexpr TFusedVariant kFusedVariants[] = {
     {80, 8, true, 6, "cbamd_fused_b80_w8_d6_s"},
     {80, 8, false, 8, "cbamd_fused_b80_w8"},
     {80, 8, true, 8, "cbamd_fused_b80_w8_s"},
+    {208, 4, false, 6, "cbamd_fused_b208_w4_d6"},
+    {208, 4, true, 6, "cbamd_fused_b208_w4_d6_s"},
     {208, 4, false, 8, "cbamd_fused_b208_w4"},
     {208, 4, true, 8, "cbamd_fused_b208_w4_s"},
 };

@@ -165,6 +165,23 @@ def test_fused_small_models(columns, used_count, depth, max_borders, shape, monk
     _compare(_bytes(model), x[:300], monkeypatch, stride=columns + 3)
 
 
+@pytest.mark.parametrize("max_depth,borders", [(6, 40), (5, 100), (7, 40)])
+def test_fused_wide_models_by_depth(max_depth, borders, monkeypatch):
+    """The fused kernel of 208 bins registers in its six-level form (models of depth <= 6) and its eight-level
+    form, six-bit and seven-bit."""
+    rng = np.random.default_rng(max_depth * 100 + borders)
+    columns = 170
+    used = list(range(columns))
+    feats_borders = {f: rng.normal(0, 1, size=rng.integers(1, borders + 1)) for f in used}
+    model = _random_model(rng, columns, used, trees=90, depth=max_depth, borders_of=lambda f: feats_borders[f])
+    x = rng.normal(0, 1.5, size=(2500, columns)).astype(np.float32)
+    x[rng.random(x.shape) < 0.02] = np.nan
+    (fm, fev), _ = _evaluators(_bytes(model), monkeypatch)
+    name = fev.describe_kernels(cb.LAYOUT_FLAT_ROWS, x.shape[0]).get("fused", "")
+    assert name.startswith("cbamd_fused_b208_w4") and ("_d6" in name) == (max_depth <= 6)
+    _compare(_bytes(model), x, monkeypatch)
+
+
 def test_fused_split_rows_layout(monkeypatch):
     """Separate float rows (the Index positions of the model's features, which need not be their flat positions)
     take the fused kernel of their own unit tables."""
